@@ -1,0 +1,151 @@
+"""GPU parity of the module-1 drop-in (YiTu_GNN_kernel.forward / backward /
+forward_gin / backward_gin / SAG) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import ATOL_BF16, RTOL_BF16, assert_close, powerlaw_graph, random_csr
+from yitu_amd import YiTu_GNN_kernel as K
+from yitu_amd.data import graphgen
+
+pytestmark = pytest.mark.gpu
+
+PS, DW, WPB = 32, 32, 8  # tuning knobs of the reference signature (ignored by the kernels)
+
+
+def _graph_args(indptr, indices, dev):
+    pp, p2n = K.build_part(PS, indptr)
+    return (indptr.to(dev), indices.to(dev), graphgen.gcn_norm(indptr).to(dev), pp.to(dev),
+            p2n.to(dev))
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 4, 33, 64, 100, 128, 130, 256, 260, 512, 1030, 2052])
+def test_sag_all_row_widths(dev, dim):
+    n = 257
+    indptr, indices = random_csr(n, n, 0.04, dim, hub_rows=(7,), hub_degree=150, empty_rows=(0, 5))
+    x = torch.randn(n, dim, generator=torch.Generator().manual_seed(dim))
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    got = K.SAG(x.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert_close(got, oracle.sag(x.numpy(), indptr, indices), what="SAG dim=%d" % dim)
+    assert torch.all(got[0] == 0) and torch.all(got[5] == 0)
+
+
+@pytest.mark.parametrize("hub_degree", [511, 512, 513, 1024, 1025, 3000])
+@pytest.mark.parametrize("dim", [64, 128, 36])
+def test_hub_rows_take_the_chunked_path(dev, hub_degree, dim):
+    """Rows with >= 512 edges are summed by the workgroup-per-chunk kernels."""
+    n = 4096
+    indptr, indices = random_csr(n, n, 0.002, hub_degree, hub_rows=(1, 4000, 4095),
+                                 hub_degree=hub_degree, empty_rows=(2,))
+    x = torch.randn(n, dim, generator=torch.Generator().manual_seed(1))
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    w = torch.eye(dim)
+    got = K.forward(x.to(dev), w.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)[0]
+    want = oracle.gcn_forward(x.numpy(), w.numpy(), indptr, indices, deg.cpu().numpy())
+    assert_close(got, want, what="hub=%d dim=%d" % (hub_degree, dim))
+
+
+@pytest.mark.parametrize("fin,fout", [(16, 64), (64, 128), (50, 7)])
+def test_gcn_forward_backward(dev, fin, fout):
+    indptr, indices = powerlaw_graph(12, 60000, 3)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(fin)
+    x = torch.randn(n, fin, generator=g)
+    w = torch.randn(fin, fout, generator=g) / 8
+    dy = torch.randn(n, fout, generator=g)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    out = K.forward(x.to(dev), w.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert isinstance(out, list) and len(out) == 1
+    s = deg.cpu().numpy()
+    assert_close(out[0], oracle.gcn_forward(x.numpy(), w.numpy(), indptr, indices, s))
+    dx, dw = K.backward(dy.to(dev), x.to(dev), w.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)
+    want_dx, want_dw = oracle.gcn_backward(dy.numpy(), x.numpy(), w.numpy(), indptr, indices, s)
+    assert_close(dx, want_dx)
+    # dW sums n = 4096 products per element: scale the absolute bar accordingly
+    assert_close(dw, want_dw, atol=1e-4 * np.sqrt(n))
+
+
+def test_gin_forward_backward(dev):
+    indptr, indices = powerlaw_graph(11, 30000, 4)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(n, 48, generator=g)
+    w = torch.randn(48, 20, generator=g) / 8
+    dy = torch.randn(n, 20, generator=g)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    out, agg = K.forward_gin(x.to(dev), w.to(dev), rp, ci, 0.5, pp, p2n, PS, DW, WPB)
+    want_out, want_agg = oracle.gin_forward(x.numpy(), w.numpy(), indptr, indices, 0.5)
+    assert_close(agg, want_agg)
+    assert_close(out, want_out, atol=2e-4)
+    dx, dw = K.backward_gin(dy.to(dev), agg, w.to(dev), rp, ci, 0.5, pp, p2n, PS, DW, WPB)
+    want_dx, want_dw = oracle.gin_backward(dy.numpy(), want_agg, w.numpy(), indptr, indices, 0.5)
+    assert_close(dx, want_dx, atol=2e-4)
+    assert_close(dw, want_dw, atol=1e-4 * np.sqrt(n) * 4)
+
+
+@pytest.mark.parametrize("dim", [8, 128, 100, 264])
+def test_bf16_input_fp32_accumulate(dev, dim):
+    indptr, indices = powerlaw_graph(12, 80000, 5)
+    n = indptr.numel() - 1
+    xb = torch.randn(n, dim, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    got = K._aggregate(xb.to(dev), rp, ci, deg, 1.0)
+    bits = xb.view(torch.int16).numpy().view(np.uint16)
+    want = oracle.row_agg_bf16(bits, indptr, indices, deg.cpu().numpy(), oracle.MODE_GCN)
+    assert got.dtype == torch.float32
+    assert_close(got, want, rtol=RTOL_BF16, atol=ATOL_BF16)
+    # the inputs are exactly representable, so the fp32 bar holds as well
+    assert_close(got, want)
+
+
+def test_results_are_bitwise_reproducible(dev):
+    indptr, indices = powerlaw_graph(13, 200000, 6)
+    n = indptr.numel() - 1
+    x = torch.randn(n, 64, generator=torch.Generator().manual_seed(3)).to(dev)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    a = K.SAG(x, rp, ci, deg, pp, p2n, PS, DW, WPB)
+    b = K.SAG(x, rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert torch.equal(a, b)
+
+
+def test_linearity_and_row_block_invariance_at_scale(dev):
+    """Size-independent properties on a 2^17-node power-law graph: linear in x,
+    and a row's result does not depend on which other rows are in the launch."""
+    src, dst = graphgen.rmat(17, 3_000_000, 7, self_loops=True, device=dev)
+    n = 1 << 17
+    rp, ci = graphgen.csr_by_destination(src, dst, n)
+    deg = graphgen.gcn_norm(rp)
+    g = torch.Generator(device=dev).manual_seed(1)
+    x1 = torch.randn(n, 128, generator=g, device=dev)
+    x2 = torch.randn(n, 128, generator=g, device=dev)
+    f = lambda x: K._aggregate(x, rp, ci, deg, 1.0)
+    y1, y2, y12 = f(x1), f(x2), f(x1 + 2 * x2)
+    assert_close(y12, y1 + 2 * y2, atol=2e-4)
+    lo, hi = 1000, 50000
+    sub_rp = (rp[lo:hi + 1] - rp[lo]).contiguous()
+    sub_ci = ci[rp[lo].item():rp[hi].item()].contiguous()
+    out = torch.empty(hi - lo, 128, device=dev)
+    from yitu_amd import _lib
+    ws = _lib.workspace(_lib.lib().yitu_spmm_workspace_bytes(_lib.c_i64(sub_ci.numel()),
+                                                             _lib.c_i64(128)), dev)
+    y_unscaled = K._aggregate(x1, rp, ci, None, 1.0)
+    rc = _lib.lib().yitu_agg_csr(_lib.ptr(out), _lib.ptr(x1), 0, _lib.ptr(sub_rp), _lib.ptr(sub_ci),
+                                 _lib.ptr(None), _lib.c_i64(hi - lo), _lib.c_i64(n),
+                                 _lib.c_i64(sub_ci.numel()), _lib.c_i64(128), _lib.c_f32(1.0),
+                                 _lib.c_i64(-1), _lib.ptr(ws), _lib.c_size(ws.numel()),
+                                 _lib.stream_ptr(dev))
+    _lib.check(rc, "yitu_agg_csr")
+    assert torch.equal(out, y_unscaled[lo:hi])
+
+
+def test_rejects_cpu_tensors_and_bad_dtypes(dev):
+    indptr, indices = random_csr(10, 10, 0.3, 0)
+    x = torch.randn(10, 4)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    with pytest.raises(RuntimeError):
+        K.SAG(x, rp, ci, deg, pp, p2n, PS, DW, WPB)  # CPU features
+    with pytest.raises(RuntimeError):
+        K.SAG(x.to(dev), rp.long(), ci, deg, pp, p2n, PS, DW, WPB)
+    with pytest.raises(RuntimeError):
+        K.SAG(x.to(dev).t(), rp, ci, deg, pp, p2n, PS, DW, WPB)  # not contiguous

@@ -1,0 +1,108 @@
+"""ctypes binding of libyitu_hip.so and the small amount of torch plumbing
+(device pointers, current stream, cached workspace) shared by the op modules.
+
+There is no CPU fallback: if the library is missing or a tensor is not on a HIP
+device the call raises.
+"""
+import ctypes
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libyitu_hip.so")
+_lib = None
+_lock = threading.Lock()
+
+c_i64 = ctypes.c_int64
+c_int = ctypes.c_int
+c_f32 = ctypes.c_float
+c_size = ctypes.c_size_t
+c_ptr = ctypes.c_void_p
+
+
+def lib():
+    """Loads the HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        "libyitu_hip.so is not built; run `python -m yitu_amd.build` "
+                        "(there is no CPU fallback)")
+                l = ctypes.CDLL(LIB_PATH)
+                l.yitu_last_error.restype = ctypes.c_char_p
+                _lib = l
+    return _lib
+
+
+def _declare(name, restype=ctypes.c_int):
+    fn = getattr(lib(), name)
+    fn.restype = restype
+    return fn
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = lib().yitu_last_error().decode("utf-8", "replace")
+        raise RuntimeError("%s failed (code %d): %s" % (what, rc, msg))
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    if t is None:
+        return c_ptr(0)
+    return c_ptr(t.data_ptr())
+
+
+def stream_ptr(device):
+    return c_ptr(torch.cuda.current_stream(device).cuda_stream)
+
+
+def require_device(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("expected a tensor on the GPU (HIP device), got %s" % t.device)
+        if not t.is_contiguous():
+            raise RuntimeError("expected a contiguous tensor")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("tensors live on different devices: %s vs %s" % (dev, t.device))
+    return dev
+
+
+def require_dtype(t, dtype, name):
+    if t.dtype != dtype:
+        raise RuntimeError("%s must be %s, got %s" % (name, dtype, t.dtype))
+
+
+def workspace(n_bytes, device):
+    """Scratch buffer for one call; the caching allocator makes this cheap and
+    stream-ordered reuse keeps concurrent ops on one stream from colliding."""
+    n = max(int(n_bytes), 256)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+# Widest-row cache: the kernels skip their hub-row machinery when they are told
+# that no row reaches the hub threshold. Computed once per indptr tensor.
+_max_degree = {}
+
+
+def max_degree(indptr):
+    key = (indptr.data_ptr(), indptr.numel(), indptr._version, str(indptr.device))
+    v = _max_degree.get(key)
+    if v is None:
+        if indptr.numel() <= 1:
+            v = 0
+        else:
+            v = int((indptr[1:] - indptr[:-1]).max().item())
+        if len(_max_degree) > 64:
+            _max_degree.clear()
+        _max_degree[key] = v
+    return v

@@ -1,0 +1,71 @@
+// extern "C" surface of libyitu_hip.so (declared in include/yitu_hip.h).
+#include "../../include/yitu_hip.h"
+
+#include "spmm_rows.hpp"
+
+using namespace yitu;
+
+#define YITU_API extern "C" __attribute__((visibility("default")))
+
+YITU_API const char *yitu_last_error(void) { return last_error(); }
+YITU_API int yitu_abi_version(void) { return 1; }
+
+YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len) {
+    return hub_workspace_bytes(nnz, row_len);
+}
+
+YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_t *row_pointers,
+                          const int32_t *column_index, const float *degrees, int64_t n_rows,
+                          int64_t n_src, int64_t nnz, int64_t dim, float alpha,
+                          int64_t max_degree, void *workspace, size_t workspace_bytes,
+                          void *stream) {
+    YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0 && dim >= 0, "negative size");
+    if (n_rows == 0 || dim == 0) return 0;
+    YITU_REQUIRE(out && row_pointers, "null output or row_pointers");
+    YITU_REQUIRE(nnz == 0 || (x && column_index), "null input with nnz > 0");
+    YITU_REQUIRE(n_rows < INT32_MAX && n_src < INT32_MAX && dim < (1 << 20), "size out of range");
+    SpmmParams p{};
+    p.indptr = row_pointers;
+    p.indices = column_index;
+    p.feat = x;
+    p.out = out;
+    p.scale_row = degrees;
+    p.scale_col = degrees;
+    p.n_rows = (int)n_rows;
+    p.L = (int)dim;
+    p.F = (int)dim;
+    p.H = 1;
+    p.col_mask = 0x7fffffff;
+    p.alpha = alpha;
+    p.xcd_remap = 0;
+    return launch_spmm(p, degrees ? W_DEGPROD : W_NONE, x_is_bf16 != 0, nnz, max_degree, workspace,
+                       workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *indptr,
+                               const int32_t *indices, const float *features, int64_t n_dst,
+                               int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
+                               int64_t max_degree, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+    YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
+                 "negative size");
+    if (n_dst == 0 || n_heads * n_features == 0) return 0;
+    YITU_REQUIRE(out && indptr, "null output or indptr");
+    YITU_REQUIRE(nnz == 0 || (values && indices && features), "null input with nnz > 0");
+    YITU_REQUIRE(n_dst < INT32_MAX && n_src <= (1 << 24) && n_heads * n_features < (1 << 20),
+                 "size out of range (columns are 24-bit)");
+    SpmmParams p{};
+    p.indptr = indptr;
+    p.indices = indices;
+    p.feat = features;
+    p.out = out;
+    p.values = values;
+    p.n_rows = (int)n_dst;
+    p.L = (int)(n_heads * n_features);
+    p.F = (int)n_features;
+    p.H = (int)n_heads;
+    p.col_mask = 0xffffff;
+    p.alpha = 1.0f;
+    return launch_spmm(p, W_EDGEHEAD, false, nnz, max_degree, workspace, workspace_bytes,
+                       static_cast<hipStream_t>(stream));
+}
