@@ -73,6 +73,82 @@ int yitu_spmm_forward(float *out_device, const float *values_device, const int32
                       int64_t max_degree, void *workspace_device, size_t workspace_bytes,
                       void *stream);
 
+/*
+ * spmm_backward (entry.cpp:92-104; spmm_cuda.cu:24-42,64-86):
+ *   grad_a[i,h]   = sum_k grad_out[row_i,h,k] * features[col_i,h,k]
+ *   grad_x[c,h,k] = sum_{i: col_i = c} grad_out[row_i,h,k] * values[i,h]
+ * Either output may be NULL to skip it. grad_x is computed as a gather over
+ * the transposed structure (t_* from yitu_csr_transpose, required when grad_x
+ * is requested) instead of the reference's 2*E*H*F float atomics; both outputs
+ * are fully written and bitwise reproducible. max_degree / max_degree_t: widest
+ * row of the CSR / of its transpose if known, else -1.
+ * Workspace: yitu_spmm_workspace_bytes(nnz, H*F).
+ */
+int yitu_spmm_backward(float *grad_a_device, float *grad_x_device, const float *values_device,
+                       const int32_t *indptr_device, const int32_t *indices_device,
+                       const float *features_device, const float *grad_out_device,
+                       const int32_t *t_indptr_device, const int32_t *t_rows_device,
+                       const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
+                       int64_t n_heads, int64_t n_features, int64_t max_degree,
+                       int64_t max_degree_t, void *workspace_device, size_t workspace_bytes,
+                       void *stream);
+
+/*
+ * sddmm_forward (entry.cpp:106-116; sddmm_cuda.cu:5-33,69-89):
+ *   attn[i,h] = softmax over {i' in row r with the same bid} of
+ *               leaky_relu(query[bid,r,h] + key[col,h], 0.2),
+ *   bid = indices[i] >> 24, col = indices[i] & 0xffffff.
+ * query [n_bid,n_dst,H], key [n_src,H], attn [nnz,H] (every entry is written).
+ * The softmax subtracts the running maximum; the reference does not
+ * (sddmm_cuda.cu:15-21) and overflows for logits above ~88.
+ */
+size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid);
+int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
+                       const int32_t *indices_device, const float *query_device,
+                       const float *key_device, int64_t n_dst, int64_t n_src, int64_t nnz,
+                       int64_t n_heads, int64_t n_bid, int64_t max_degree, void *workspace_device,
+                       size_t workspace_bytes, void *stream);
+
+/*
+ * sddmm_backward (entry.cpp:118-134; sddmm_cuda.cu:36-67,91-118):
+ *   gv[i,h] = attn (grad_out - sum_j attn_j grad_out_j) * (x < 0 ? 0.2 : 1)
+ *   grad_query[bid,r,h] = sum_i gv ;  grad_key[col,h] = sum_{i: col_i = col} gv
+ * grad_query and grad_key are fully written. Two forms of the grad_key sum:
+ *   t_indptr == NULL: float atomics (as the reference; order not reproducible);
+ *   t_indptr, t_perm from yitu_csr_transpose and grad_edge_device [nnz,H]
+ *   scratch: gv is stored per edge and summed by a gather over the transposed
+ *   structure (bitwise reproducible).
+ */
+int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float *grad_edge_device,
+                        const int32_t *indptr_device, const int32_t *indices_device,
+                        const float *query_device, const float *key_device,
+                        const float *attn_device, const float *grad_out_device,
+                        const int32_t *t_indptr_device, const int32_t *t_perm_device,
+                        int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
+                        int64_t max_degree, void *workspace_device, size_t workspace_bytes,
+                        void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Graph preparation                                                           */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * By-source (transposed) view of a CSR, built once per graph on the device.
+ * The reference has no such step: its backward kernels scatter with atomics
+ * (spmm_cuda.cu:33-38, sddmm_cuda.cu:59-63); this turns those scatters into
+ * gathers. For the stable order of a canonical CSR:
+ *   t_indptr [n_cols+1]: edges of source c are t_indptr[c] .. t_indptr[c+1]-1
+ *   t_rows   [nnz]     : destination row of each of them (ascending per source)
+ *   t_perm   [nnz]     : its position in the original indices/values arrays
+ * col_mask selects the column bits of indices (0xffffff for packed graph_ext
+ * indices, 0x7fffffff for plain ones).
+ */
+size_t yitu_csr_transpose_workspace_bytes(int64_t nnz, int64_t n_cols);
+int yitu_csr_transpose(int32_t *t_indptr_device, int32_t *t_rows_device, int32_t *t_perm_device,
+                       const int32_t *indptr_device, const int32_t *indices_device, int64_t n_rows,
+                       int64_t n_cols, int64_t nnz, int32_t col_mask, void *workspace_device,
+                       size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

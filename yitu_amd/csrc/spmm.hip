@@ -15,13 +15,18 @@ void set_error(const char *fmt, ...) {
 }
 const char *last_error() { return g_error; }
 
-__global__ void zero_hub_counters_kernel(HubCounters *c) {
-    if (threadIdx.x == 0) {
-        c->n_items = 0;
-        c->n_rows = 0;
-        c->overflow = 0;
-        c->pad = 0;
-    }
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(float *p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) p[i] = 0.0f;
+}
+
+int fill_zero(float *p, int64_t n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int grid = (int)std::min<int64_t>(ceil_div(n, kBlock), 8192);
+    fill_zero_kernel<<<grid, kBlock, 0, stream>>>(p, n);
+    YITU_LAUNCH_CHECK();
+    return 0;
 }
 
 // A hub row has >= kHubThreshold edges and yields ceil(deg / kHubChunk) items,
@@ -32,7 +37,7 @@ static inline int64_t hub_max_items(int64_t nnz) { return nnz / kHubChunk + hub_
 size_t hub_workspace_bytes(int64_t nnz, int64_t L) {
     size_t b = 256;  // counters
     b += align_up(sizeof(int4) * (size_t)hub_max_rows(nnz), 256);
-    b += align_up(sizeof(int2) * (size_t)hub_max_items(nnz), 256);
+    b += align_up(sizeof(int4) * (size_t)hub_max_items(nnz), 256);
     b += align_up(sizeof(float) * (size_t)hub_max_items(nnz) * (size_t)L, 256);
     return b;
 }
@@ -50,8 +55,8 @@ int hub_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t
     q.max_items = (int)hub_max_items(nnz);
     q.rows = reinterpret_cast<int4 *>(w);
     w += align_up(sizeof(int4) * (size_t)q.max_rows, 256);
-    q.items = reinterpret_cast<int2 *>(w);
-    w += align_up(sizeof(int2) * (size_t)q.max_items, 256);
+    q.items = reinterpret_cast<int4 *>(w);
+    w += align_up(sizeof(int4) * (size_t)q.max_items, 256);
     q.partial = reinterpret_cast<float *>(w);
     return 0;
 }

@@ -38,7 +38,7 @@ struct HubCounters {
 struct HubQueue {
     HubCounters *counters;  // zeroed before the row kernel
     int4 *rows;             // {row, first_item, n_chunks, 0}
-    int2 *items;            // {row, chunk}
+    int4 *items;            // {row, chunk, index into rows[], 0}
     float *partial;         // [n_items, L]
     int max_rows;
     int max_items;
@@ -63,6 +63,27 @@ struct SpmmParams {
     int xcd_remap;
     HubQueue hub;
 };
+
+// Appends a hub row and its ceil(deg / kHubChunk) chunk items to the queue.
+// Called by all lanes of the wave that owns the row.
+__device__ __forceinline__ void queue_hub_row(const HubQueue &q, int row, int deg) {
+    const int lane = lane_id();
+    const int n_chunks = (deg + kHubChunk - 1) / kHubChunk;
+    int first = 0, slot_r = 0;
+    if (lane == 0) {
+        first = atomicAdd(&q.counters->n_items, n_chunks);
+        slot_r = atomicAdd(&q.counters->n_rows, 1);
+    }
+    first = __shfl(first, 0, kWave);
+    slot_r = __shfl(slot_r, 0, kWave);
+    if (slot_r < q.max_rows && first + n_chunks <= q.max_items) {
+        if (lane == 0) q.rows[slot_r] = make_int4(row, first, n_chunks, 0);
+        for (int c = lane; c < n_chunks; c += kWave)
+            q.items[first + c] = make_int4(row, c, slot_r, 0);
+    } else if (lane == 0) {
+        atomicExch(&q.counters->overflow, 1);
+    }
+}
 
 // One step of the edge loop: every slot of the wave picks its edge (step + slot)
 // out of the batch held one-per-lane in my_col / my_w / my_vrow and loads that
@@ -112,7 +133,6 @@ __device__ __forceinline__ void accumulate_edges(float (&acc)[KT][VEC], const Sp
                                                  int e_beg, int e_end, int c0) {
     constexpr int SLOTS = kWave / G;
     const int lane = lane_id();
-    const int slot = lane / G;
     const int sub = lane % G;
     const TIN *__restrict__ feat = static_cast<const TIN *>(p.feat);
 
@@ -197,20 +217,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
 
     if (deg >= p.hub_threshold) {
         // queue the row for the chunked kernels; nothing is written here
-        const int n_chunks = (deg + kHubChunk - 1) / kHubChunk;
-        int first = 0, slot_r = 0;
-        if (lane == 0) {
-            first = atomicAdd(&p.hub.counters->n_items, n_chunks);
-            slot_r = atomicAdd(&p.hub.counters->n_rows, 1);
-        }
-        first = __shfl(first, 0, kWave);
-        slot_r = __shfl(slot_r, 0, kWave);
-        if (slot_r < p.hub.max_rows && first + n_chunks <= p.hub.max_items) {
-            if (lane == 0) p.hub.rows[slot_r] = make_int4(row, first, n_chunks, 0);
-            for (int c = lane; c < n_chunks; c += kWave) p.hub.items[first + c] = make_int2(row, c);
-        } else if (lane == 0) {
-            atomicExch(&p.hub.counters->overflow, 1);
-        }
+        queue_hub_row(p.hub, row, deg);
         return;
     }
 
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(kBlock) void spmm_hub_items_kernel(SpmmParams p) {
     const int n_items = min(p.hub.counters->n_items, p.hub.max_items);
 
     for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
-        const int2 it = p.hub.items[item];
+        const int4 it = p.hub.items[item];
         const int row = it.x;
         const int beg = p.indptr[row] + it.y * kHubChunk;
         const int end = min(p.indptr[row + 1], beg + kHubChunk);
@@ -314,7 +321,14 @@ __global__ __launch_bounds__(kBlock) void spmm_hub_reduce_kernel(SpmmParams p) {
     }
 }
 
-__global__ void zero_hub_counters_kernel(HubCounters *c);
+static __global__ void zero_hub_counters_kernel(HubCounters *c) {
+    if (threadIdx.x == 0) {
+        c->n_items = 0;
+        c->n_rows = 0;
+        c->overflow = 0;
+        c->pad = 0;
+    }
+}
 
 // Host side: carve the queue out of a caller-provided workspace.
 size_t hub_workspace_bytes(int64_t nnz, int64_t L);
@@ -325,5 +339,7 @@ int hub_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t
 int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max_degree_hint,
                 void *workspace, size_t workspace_bytes, hipStream_t stream);
 const char *last_error();
+// Zero-fill by kernel (safe to record into a captured graph, unlike a memset node).
+int fill_zero(float *p, int64_t n, hipStream_t stream);
 
 }  // namespace yitu

@@ -1,0 +1,229 @@
+"""Drop-in for the reference's ``graph_ext`` extension module
+(YiTu_GNN/YiTu_H/src/entry.cpp:184-193): ``spmm_forward/backward``,
+``sddmm_forward/backward``, ``hfused_forward/backward``, ``b2gemm`` and
+``b2gemm_backward`` with the reference's argument order, dtype checks
+(CHECK_INPUT: device + contiguous + exact dtype, common.h:6-12) and return
+arity, backed by libyitu_hip.so.
+
+Observable differences from the reference:
+  * any number of destination rows works (the reference launches
+    ``dim3(n_heads, n_nodes)`` and silently returns zeros above 65,535 rows,
+    spmm_cuda.cu:57);
+  * the edge softmax subtracts the row maximum (the reference does not,
+    sddmm_cuda.cu:15-21); equal within tolerance wherever the reference does
+    not overflow;
+  * backward scatters are gathers over a transposed structure that is built on
+    the device once per graph and cached on the ``indices`` tensor: results are
+    bitwise reproducible, unlike the reference's float atomics;
+  * ``hfused_backward`` returns ``[grad_a, grad_x, grad_query, grad_key]``; the
+    reference version drops the first two and mis-indexes heads
+    (hfused_cuda.cu:59,186) and is unreachable from its Python side.
+"""
+import weakref
+
+import torch
+
+from . import _lib
+from ._lib import c_i64, c_int, c_size, check, ptr, stream_ptr
+
+COL_MASK = 0xFFFFFF
+
+
+def _check(t, dtype, name, dim=None):
+    # CHECK_INPUT(x, dtype) of the reference (common.h:6-12)
+    _lib.require_device(t)
+    _lib.require_dtype(t, dtype, name)
+    if dim is not None and t.dim() != dim:
+        raise RuntimeError("%s must be %d-D, got %d-D" % (name, dim, t.dim()))
+
+
+def _size_fn(name):
+    fn = getattr(_lib.lib(), name)
+    fn.restype = c_size
+    return fn
+
+
+# --------------------------------------------------------------------------- #
+# transposed structure, cached per (indptr, indices) pair
+# --------------------------------------------------------------------------- #
+class _Transposed:
+    __slots__ = ("t_indptr", "t_rows", "t_perm", "max_degree_t", "n_src")
+
+
+_transposed = {}
+
+
+def transposed(indptr, indices, n_src):
+    """By-source view (t_indptr, t_rows, t_perm) of a packed CSR, built on the
+    device on first use and kept for as long as ``indices`` is alive."""
+    key = (id(indices), indices.data_ptr(), indices._version, indptr.data_ptr(), int(n_src))
+    hit = _transposed.get(key)
+    if hit is not None:
+        return hit
+    dev = indices.device
+    n_rows = indptr.numel() - 1
+    nnz = indices.numel()
+    t = _Transposed()
+    t.n_src = int(n_src)
+    t.t_indptr = torch.empty(n_src + 1, dtype=torch.int32, device=dev)
+    t.t_rows = torch.empty(nnz, dtype=torch.int32, device=dev)
+    t.t_perm = torch.empty(nnz, dtype=torch.int32, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_csr_transpose_workspace_bytes")(c_i64(nnz), c_i64(n_src)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_csr_transpose(ptr(t.t_indptr), ptr(t.t_rows), ptr(t.t_perm), ptr(indptr),
+                                           ptr(indices), c_i64(n_rows), c_i64(n_src), c_i64(nnz),
+                                           c_int(COL_MASK), ptr(ws), c_size(ws.numel()),
+                                           stream_ptr(dev))
+    check(rc, "yitu_csr_transpose")
+    t.max_degree_t = _lib.max_degree(t.t_indptr)
+    _transposed[key] = t
+    weakref.finalize(indices, _transposed.pop, key, None)
+    return t
+
+
+# --------------------------------------------------------------------------- #
+# SpMM
+# --------------------------------------------------------------------------- #
+def spmm_forward(values, indptr, indices, features):
+    """out[r,h,k] = sum_i values[i,h] * features[col_i,h,k] (entry.cpp:80-90)."""
+    _check(values, torch.float32, "values", 2)
+    _check(indptr, torch.int32, "indptr", 1)
+    _check(indices, torch.int32, "indices", 1)
+    _check(features, torch.float32, "features", 3)
+    dev = _lib.require_device(values, indptr, indices, features)
+    n_dst = indptr.numel() - 1
+    n_src, h, f = features.shape
+    nnz = indices.numel()
+    if values.shape[0] != nnz or values.shape[1] != h:
+        raise RuntimeError("values must be [n_edges, n_heads]")
+    out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
+    maxdeg = _lib.max_degree(indptr)
+    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 512 else 0
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_spmm_forward(ptr(out), ptr(values), ptr(indptr), ptr(indices),
+                                          ptr(features), c_i64(n_dst), c_i64(n_src), c_i64(nnz),
+                                          c_i64(h), c_i64(f), c_i64(maxdeg), ptr(ws),
+                                          c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_spmm_forward")
+    return out
+
+
+def spmm_backward(values, indptr, indices, features, grad_out):
+    """Returns [grad_a [E,H], grad_x [Ns,H,F]] (entry.cpp:92-104)."""
+    _check(values, torch.float32, "values", 2)
+    _check(indptr, torch.int32, "indptr", 1)
+    _check(indices, torch.int32, "indices", 1)
+    _check(features, torch.float32, "features", 3)
+    _check(grad_out, torch.float32, "grad_out", 3)
+    dev = _lib.require_device(values, indptr, indices, features, grad_out)
+    n_dst = indptr.numel() - 1
+    n_src, h, f = features.shape
+    nnz = indices.numel()
+    if grad_out.shape[0] != n_dst or grad_out.shape[1] != h or grad_out.shape[2] != f:
+        raise RuntimeError("grad_out must be [n_dst, n_heads, n_features]")
+    grad_a = torch.empty_like(values)
+    grad_x = torch.empty_like(features)
+    tr = transposed(indptr, indices, n_src)
+    maxdeg = _lib.max_degree(indptr)
+    need = 0
+    if max(maxdeg, tr.max_degree_t) >= 512:
+        need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f))
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_spmm_backward(ptr(grad_a), ptr(grad_x), ptr(values), ptr(indptr),
+                                           ptr(indices), ptr(features), ptr(grad_out),
+                                           ptr(tr.t_indptr), ptr(tr.t_rows), ptr(tr.t_perm),
+                                           c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h), c_i64(f),
+                                           c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(ws),
+                                           c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_spmm_backward")
+    return [grad_a, grad_x]
+
+
+# --------------------------------------------------------------------------- #
+# SDDMM + LeakyReLU + edge softmax
+# --------------------------------------------------------------------------- #
+def _sddmm_shapes(indptr, indices, query, key):
+    _check(indptr, torch.int32, "indptr", 1)
+    _check(indices, torch.int32, "indices", 1)
+    _check(query, torch.float32, "query", 3)
+    _check(key, torch.float32, "key", 2)
+    if query.size(-1) != key.size(-1):
+        raise RuntimeError("query and key disagree on the number of heads")
+    if query.size(1) != indptr.numel() - 1:
+        raise RuntimeError("query.size(1) must equal the number of destination rows")
+    if query.size(0) > 16:
+        raise RuntimeError("at most 16 query blocks (the block tag is 4 bits wide)")
+    return indptr.numel() - 1, key.size(0), indices.numel(), key.size(1), query.size(0)
+
+
+def sddmm_forward(indptr, indices, query, key):
+    """attn[i,h] = softmax_{row, bid}(leaky_relu(query[bid,r,h] + key[col,h], 0.2)) (entry.cpp:106-116)."""
+    n_dst, n_src, nnz, h, n_bid = _sddmm_shapes(indptr, indices, query, key)
+    dev = _lib.require_device(indptr, indices, query, key)
+    attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    maxdeg = _lib.max_degree(indptr)
+    need = 0
+    if maxdeg >= 512:
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_sddmm_forward(ptr(attn), ptr(indptr), ptr(indices), ptr(query), ptr(key),
+                                           c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
+                                           c_i64(n_bid), c_i64(maxdeg), ptr(ws), c_size(ws.numel()),
+                                           stream_ptr(dev))
+    check(rc, "yitu_sddmm_forward")
+    return attn
+
+
+def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, deterministic=True):
+    """Returns [grad_query, grad_key] (entry.cpp:118-134). ``deterministic=False``
+    selects the float-atomic scatter for grad_key (the reference's form)."""
+    n_dst, n_src, nnz, h, n_bid = _sddmm_shapes(indptr, indices, query, key)
+    _check(attn_values, torch.float32, "attn_values", 2)
+    _check(grad_out, torch.float32, "grad_out", 2)
+    if attn_values.shape != (nnz, h) or grad_out.shape != attn_values.shape:
+        raise RuntimeError("attn_values and grad_out must be [n_edges, n_heads]")
+    dev = _lib.require_device(indptr, indices, query, key, attn_values, grad_out)
+    grad_query = torch.empty_like(query)
+    grad_key = torch.empty_like(key)
+    maxdeg = _lib.max_degree(indptr)
+    tr = transposed(indptr, indices, n_src) if deterministic else None
+    grad_edge = torch.empty_like(attn_values) if deterministic else None
+    need = 0
+    if maxdeg >= 512 or (tr is not None and tr.max_degree_t >= 512):
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_sddmm_backward(
+            ptr(grad_query), ptr(grad_key), ptr(grad_edge), ptr(indptr), ptr(indices), ptr(query),
+            ptr(key), ptr(attn_values), ptr(grad_out), ptr(tr.t_indptr if tr else None),
+            ptr(tr.t_perm if tr else None), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
+            c_i64(n_bid), c_i64(maxdeg), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_sddmm_backward")
+    return [grad_query, grad_key]
+
+
+# --------------------------------------------------------------------------- #
+# horizontally fused SpMM || SDDMM
+# --------------------------------------------------------------------------- #
+def hfused_forward(spmm_values, spmm_indptr, spmm_indices, spmm_features, sddmm_indptr,
+                   sddmm_indices, sddmm_query, sddmm_key):
+    """An SpMM on graph A and an SDDMM+softmax on graph B with equal row counts
+    (entry.cpp:136-155; hfused_cuda.cu:96-137). Returns [spmm_out, attn]."""
+    if spmm_indptr.numel() != sddmm_indptr.numel():
+        raise RuntimeError("the two graphs must have the same number of rows")
+    out = spmm_forward(spmm_values, spmm_indptr, spmm_indices, spmm_features)
+    attn = sddmm_forward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key)
+    return [out, attn]
+
+
+def hfused_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad, sddmm_indptr,
+                    sddmm_indices, sddmm_query, sddmm_key, sddmm_attn, sddmm_grad):
+    """Union of the two backward ops (entry.cpp:157-182) with the correct
+    arithmetic: returns [grad_a, grad_x, grad_query, grad_key]."""
+    grad_a, grad_x = spmm_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad)
+    grad_q, grad_k = sddmm_backward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key, sddmm_attn,
+                                    sddmm_grad)
+    return [grad_a, grad_x, grad_q, grad_k]

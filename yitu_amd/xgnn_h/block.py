@@ -1,0 +1,70 @@
+"""CSR holder and multi-relation CSR packing (xgnn_h/block.py)."""
+from typing import List
+
+import torch
+
+
+class Block:
+    """``size = [n_dst, n_src]``, ``adj_sparse = [indptr, indices]`` (block.py:5-33)."""
+
+    def __init__(self, size: list, adj: list, right_norm=None):
+        self.size = size
+        self.adj_sparse = adj
+        self.right_norm = right_norm
+
+    def to(self, device):
+        self.adj_sparse = [self.adj_sparse[0].to(device), self.adj_sparse[1].to(device)]
+        if self.right_norm is not None:
+            self.right_norm = self.right_norm.to(device)
+        return self
+
+    def num_edges(self):
+        indices = self.adj_sparse[1]
+        assert indices.dim() == 1
+        return indices.numel()
+
+    def num_src_nodes(self):
+        return self.size[1]
+
+    def num_dst_nodes(self):
+        indptr = self.adj_sparse[0]
+        assert indptr.dim() == 1
+        assert self.size[0] == indptr.size(0) - 1
+        return self.size[0]
+
+
+def stitch_csr(block_list: List[Block]):
+    """Row-wise concatenation of up to 16 blocks with equal row counts
+    (block.py:36-67): block b's columns are shifted by the source counts of
+    blocks 0..b-1 and tagged ``(b << 24) + col``. The reference walks every edge
+    in a Python loop; this is the same integer result from vectorised tensor ops
+    on whichever device the blocks live on."""
+    lens = [blk.size[0] for blk in block_list]
+    n_rows = min(lens)
+    assert len(lens) <= 16
+    assert min(lens) == max(lens)
+    dev = block_list[0].adj_sparse[0].device
+    rows, keys, blk_of = [], [], []
+    cursor = 0
+    for bid, blk in enumerate(block_list):
+        indptr, indices = blk.adj_sparse
+        assert indptr.numel() == n_rows + 1
+        deg = (indptr[1:] - indptr[:-1]).to(torch.int64)
+        col = indices.to(torch.int64) + cursor
+        if col.numel():
+            assert int(col.max()) <= 2 ** 24
+        rows.append(torch.repeat_interleave(torch.arange(n_rows, device=dev), deg))
+        keys.append((bid << 24) + col)
+        blk_of.append(torch.full((col.numel(),), bid, dtype=torch.int64, device=dev))
+        cursor += blk.size[1]
+    rows = torch.cat(rows)
+    keys = torch.cat(keys)
+    blk_of = torch.cat(blk_of)
+    # order: by row, then by block, keeping each block's own edge order (stable)
+    order = torch.argsort(rows * 16 + blk_of, stable=True)
+    new_indices = keys[order].to(torch.int32)
+    counts = torch.bincount(rows, minlength=n_rows)
+    new_indptr = torch.zeros(n_rows + 1, dtype=torch.int64, device=dev)
+    new_indptr[1:] = torch.cumsum(counts, 0)
+    n_cols = sum(blk.size[1] for blk in block_list)
+    return Block(size=[n_rows, n_cols], adj=[new_indptr.to(torch.int32), new_indices])
