@@ -118,6 +118,7 @@ int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
  *   t_indptr, t_perm from yitu_csr_transpose and grad_edge_device [nnz,H]
  *   scratch: gv is stored per edge and summed by a gather over the transposed
  *   structure (bitwise reproducible).
+ * max_degree / max_degree_t: widest row of the CSR / of its transpose, or -1.
  */
 int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float *grad_edge_device,
                         const int32_t *indptr_device, const int32_t *indices_device,
@@ -125,8 +126,8 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
                         const float *attn_device, const float *grad_out_device,
                         const int32_t *t_indptr_device, const int32_t *t_perm_device,
                         int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                        int64_t max_degree, void *workspace_device, size_t workspace_bytes,
-                        void *stream);
+                        int64_t max_degree, int64_t max_degree_t, void *workspace_device,
+                        size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */

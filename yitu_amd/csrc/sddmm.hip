@@ -550,8 +550,8 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
                                  const float *key, const float *attn, const float *grad_out,
                                  const int32_t *t_indptr, const int32_t *t_perm, int64_t n_dst,
                                  int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                 int64_t max_degree, void *workspace, size_t workspace_bytes,
-                                 void *stream_) {
+                                 int64_t max_degree, int64_t max_degree_t, void *workspace,
+                                 size_t workspace_bytes, void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
@@ -598,7 +598,7 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
         sp.H = 1;
         sp.col_mask = 0x7fffffff;
         sp.alpha = 1.0f;
-        return launch_spmm(sp, W_NONE, false, nnz, -1, workspace, workspace_bytes, stream);
+        return launch_spmm(sp, W_NONE, false, nnz, max_degree_t, workspace, workspace_bytes, stream);
     }
     return 0;
 }

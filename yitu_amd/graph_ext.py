@@ -200,7 +200,8 @@ def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, determini
             ptr(grad_query), ptr(grad_key), ptr(grad_edge), ptr(indptr), ptr(indices), ptr(query),
             ptr(key), ptr(attn_values), ptr(grad_out), ptr(tr.t_indptr if tr else None),
             ptr(tr.t_perm if tr else None), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-            c_i64(n_bid), c_i64(maxdeg), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+            c_i64(n_bid), c_i64(maxdeg), c_i64(tr.max_degree_t if tr else -1), ptr(ws),
+            c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_sddmm_backward")
     return [grad_query, grad_key]
 
