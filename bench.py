@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse message-passing hot path on one MI355X.
+
+Default workload (``c3_spmm_f32``): the large GCN SpMM of the baseline's third
+configuration -- R-MAT graph, 2^21 nodes, 63 M drawn edges (deduplicated, self
+loops added), CSR by destination, features [N,128] fp32, edge weight
+1/sqrt(d_i d_j). One step = forward aggregation of X plus backward aggregation
+of dY (the reference's backward applies the same CSR, YiTu_GNN_kernel.cu:447-461),
+both through the C ABI (yitu_agg_csr). ``value`` = edges / second with the
+reference's definition: n_edges / (time of forward + backward)
+(YiTu_GNN/YiTu_H/test/bench_macro.py:371-391). Inputs are resident in HBM before
+the timed region.
+
+Prints ONE JSON line on stdout. Other workloads: ``--workload c3_spmm_bf16``,
+``c2_gat_f32``, ``c1_gcn_f32``.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+# HBM bytes per aggregation call measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (two runs, each scaled by the same counter's reading for a 1 GiB copy kernel);
+# the summaries live under profiles/. None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def build_c3(dev, scale=21, draws=63_000_000, seed=20242):
+    from yitu_amd.data import graphgen
+    src, dst = graphgen.rmat(scale, draws, seed, self_loops=True, device=dev)
+    n = 1 << scale
+    rp, ci = graphgen.csr_by_destination(src, dst, n)
+    del src, dst
+    return n, rp, ci, graphgen.gcn_norm(rp)
+
+
+def agg_call(out, x, rp, ci, deg, ws, maxdeg):
+    from yitu_amd import _lib
+    n, dim = x.shape
+    rc = _lib.lib().yitu_agg_csr(
+        _lib.ptr(out), _lib.ptr(x), _lib.c_int(1 if x.dtype == torch.bfloat16 else 0), _lib.ptr(rp),
+        _lib.ptr(ci), _lib.ptr(deg), _lib.c_i64(rp.numel() - 1), _lib.c_i64(n),
+        _lib.c_i64(ci.numel()), _lib.c_i64(dim), _lib.c_f32(1.0), _lib.c_i64(maxdeg), _lib.ptr(ws),
+        _lib.c_size(ws.numel()), _lib.stream_ptr(x.device))
+    _lib.check(rc, "yitu_agg_csr")
+
+
+def cpu_baseline_spmm(rp, ci, deg, x, dy):
+    """The oracle's float/OpenMP restatement on the host cores, full workload."""
+    import oracle
+    rp_h, ci_h, deg_h = rp.cpu().numpy(), ci.cpu().numpy(), deg.cpu().numpy()
+    x_h, dy_h = x.float().cpu().numpy(), dy.float().cpu().numpy()
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    oracle.row_agg(x_h[:1024], rp_h[:1025] - rp_h[0], ci_h[:rp_h[1024]], deg_h, oracle.MODE_GCN,
+                   f64=False)  # warm-up: loads the library, spins up the team
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        oracle.row_agg(x_h, rp_h, ci_h, deg_h, oracle.MODE_GCN, f64=False)
+        oracle.row_agg(dy_h, rp_h, ci_h, deg_h, oracle.MODE_GCN, f64=False)
+        times.append(time.perf_counter() - t0)
+    t = min(times)
+    return {"value": ci_h.shape[0] / t, "unit": "edges/s", "cores": cores, "kind": "port",
+            "sample": "full workload (2^21 nodes, %d edges, F=128), fwd+bwd, best of 2, "
+                      "OpenMP float restatement oracle/yitu_oracle.c" % ci_h.shape[0],
+            "seconds": t}
+
+
+def run_spmm(args, dev, bf16):
+    from yitu_amd import _lib
+    n, rp, ci, deg = build_c3(dev)
+    nnz = ci.numel()
+    dim = 128
+    g = torch.Generator(device=dev).manual_seed(20242)
+    x = torch.randn(n, dim, generator=g, device=dev)
+    dy = torch.randn(n, dim, generator=g, device=dev)
+    if bf16:
+        x, dy = x.to(torch.bfloat16), dy.to(torch.bfloat16)
+    out = torch.empty(n, dim, device=dev)
+    dx = torch.empty(n, dim, device=dev)
+    maxdeg = int((rp[1:] - rp[:-1]).max().item())
+    fn = _lib.lib().yitu_spmm_workspace_bytes
+    fn.restype = _lib.c_size
+    ws = torch.empty(int(fn(_lib.c_i64(nnz), _lib.c_i64(dim))), dtype=torch.uint8, device=dev)
+
+    def step(events=None):
+        for src_t, dst_t in ((x, out), (dy, dx)):
+            if events is not None:
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+            agg_call(dst_t, src_t, rp, ci, deg, ws, maxdeg)
+            if events is not None:
+                e1.record()
+                events.append((e0, e1))
+
+    for _ in range(args.warmup):
+        step()
+    _sync()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(events)
+    _sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    call_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
+
+    b_in = 2 if bf16 else 4
+    alg = 4 * (n + 1) + 4 * nnz + 4 * n + b_in * n * dim + 4 * n * dim  # per aggregation call
+    achieved = alg / (call_ms * 1e-3) / 1e9
+    name = "c3_spmm_bf16" if bf16 else "c3_spmm_f32"
+    res = {
+        "metric": "SpMM edges/sec (GCN aggregation fwd+bwd, n_edges / step time)",
+        "value": nnz / (ms_per_step * 1e-3),
+        "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16-in/f32-acc" if bf16 else "f32", "data": "synthetic",
+        "config": {"workload": name, "graph": "R-MAT scale 21 (a,b,c,d)=(.57,.19,.19,.05), "
+                   "63M draws dedup + self loops, CSR by destination", "n_nodes": n,
+                   "n_edges": nnz, "max_in_degree": maxdeg, "feature_dim": dim,
+                   "step": "aggregate(X) + aggregate(dY), same CSR, W = I"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "kernel": "one yitu_agg_csr call = zero_hub_counters + spmm_rows_kernel + "
+                               "spmm_hub_items_kernel + spmm_hub_reduce_kernel",
+                     "kernel_ms": call_ms, "algorithmic_bytes": alg,
+                     "gather_bytes_no_reuse": nnz * dim * b_in},
+    }
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline_spmm(rp, ci, deg, x, dy)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3_spmm_f32")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.workload == "c3_spmm_f32":
+        res = run_spmm(args, dev, bf16=False)
+    elif args.workload == "c3_spmm_bf16":
+        res = run_spmm(args, dev, bf16=True)
+    else:
+        sys.exit("unknown workload %s" % args.workload)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()
