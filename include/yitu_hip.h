@@ -130,6 +130,46 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
                         size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Fused GAT attention (composition of the two ops above in one pass)          */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * No single reference entry point: the reference lowers a GAT layer to
+ * sddmm_forward followed by spmm_forward (xgnn_h/executor.py:22-40,
+ * test/common/model.py:96-106). This computes the same composition
+ *   attn = sddmm_forward(indptr, indices, query[None], key)     (n_bid = 1)
+ *   out  = spmm_forward(attn, indptr, indices, features)
+ * reading each destination row once. attn_device [nnz,H] receives the
+ * probabilities for the backward pass; it may be NULL when the shape takes the
+ * fused kernel (n_features % 4 == 0, n_heads <= 64, 16-byte aligned pointers).
+ */
+size_t yitu_gat_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_features);
+int yitu_gat_forward(float *out_device, float *attn_device, const int32_t *indptr_device,
+                     const int32_t *indices_device, const float *query_device,
+                     const float *key_device, const float *features_device, int64_t n_dst,
+                     int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
+                     int64_t max_degree, void *workspace_device, size_t workspace_bytes,
+                     void *stream);
+
+/*
+ * Backward of the composition (spmm_backward then sddmm_backward,
+ * xgnn_h/sparse.py:22-35,67-81) in one call, given grad_out [n_dst,H,F]:
+ * grad_query [n_dst,H], grad_key [n_src,H], grad_features [n_src,H,F], all
+ * fully written, no atomics. The two scratch buffers are [nnz,H] floats.
+ */
+int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
+                      float *grad_features_device, float *grad_attn_scratch_device,
+                      float *grad_edge_scratch_device, const int32_t *indptr_device,
+                      const int32_t *indices_device, const float *query_device,
+                      const float *key_device, const float *features_device,
+                      const float *attn_device, const float *grad_out_device,
+                      const int32_t *t_indptr_device, const int32_t *t_rows_device,
+                      const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
+                      int64_t n_heads, int64_t n_features, int64_t max_degree,
+                      int64_t max_degree_t, void *workspace_device, size_t workspace_bytes,
+                      void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */
 /* ------------------------------------------------------------------------- */
 

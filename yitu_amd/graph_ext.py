@@ -228,3 +228,64 @@ def hfused_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_
     grad_q, grad_k = sddmm_backward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key, sddmm_attn,
                                     sddmm_grad)
     return [grad_a, grad_x, grad_q, grad_k]
+
+
+# --------------------------------------------------------------------------- #
+# fused GAT attention (extension: the composition sddmm_forward -> spmm_forward)
+# --------------------------------------------------------------------------- #
+def gat_forward(indptr, indices, query, key, features):
+    """Returns [out [Nd,H,F], attn [E,H]] = the reference's two-op GAT lowering
+    (sddmm_forward then spmm_forward, n_bid = 1) in one pass per destination row."""
+    _check(indptr, torch.int32, "indptr", 1)
+    _check(indices, torch.int32, "indices", 1)
+    _check(query, torch.float32, "query", 2)
+    _check(key, torch.float32, "key", 2)
+    _check(features, torch.float32, "features", 3)
+    dev = _lib.require_device(indptr, indices, query, key, features)
+    n_dst = indptr.numel() - 1
+    n_src, h, f = features.shape
+    nnz = indices.numel()
+    if query.shape != (n_dst, h) or key.shape != (n_src, h):
+        raise RuntimeError("query must be [n_dst, H] and key [n_src, H]")
+    out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
+    attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    maxdeg = _lib.max_degree(indptr)
+    need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f)) if maxdeg >= 512 else 0
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gat_forward(ptr(out), ptr(attn), ptr(indptr), ptr(indices), ptr(query),
+                                         ptr(key), ptr(features), c_i64(n_dst), c_i64(n_src),
+                                         c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(ws),
+                                         c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_gat_forward")
+    return [out, attn]
+
+
+def gat_backward(indptr, indices, query, key, features, attn, grad_out):
+    """Returns [grad_query, grad_key, grad_features] of gat_forward's ``out``."""
+    _check(grad_out, torch.float32, "grad_out", 3)
+    _check(attn, torch.float32, "attn", 2)
+    dev = _lib.require_device(indptr, indices, query, key, features, attn, grad_out)
+    n_dst = indptr.numel() - 1
+    n_src, h, f = features.shape
+    nnz = indices.numel()
+    tr = transposed(indptr, indices, n_src)
+    grad_q = torch.empty_like(query)
+    grad_k = torch.empty_like(key)
+    grad_x = torch.empty_like(features)
+    s1 = torch.empty_like(attn)
+    s2 = torch.empty_like(attn)
+    maxdeg = _lib.max_degree(indptr)
+    need = 0
+    if max(maxdeg, tr.max_degree_t) >= 512:
+        need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f))
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gat_backward(
+            ptr(grad_q), ptr(grad_k), ptr(grad_x), ptr(s1), ptr(s2), ptr(indptr), ptr(indices),
+            ptr(query), ptr(key), ptr(features), ptr(attn), ptr(grad_out), ptr(tr.t_indptr),
+            ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
+            c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(ws), c_size(ws.numel()),
+            stream_ptr(dev))
+    check(rc, "yitu_gat_backward")
+    return [grad_q, grad_k, grad_x]

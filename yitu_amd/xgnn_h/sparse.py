@@ -100,3 +100,30 @@ def hfused_spddmm(spmm_block: block.Block, spmm_values, spmm_x, sddmm_block: blo
         sddmm_query = sddmm_query.unsqueeze(0)
     return HFUSEDFunction.apply(spmm_block.adj_sparse, spmm_values, spmm_x,
                                 sddmm_block.adj_sparse, sddmm_query, sddmm_key)
+
+
+class FusedGATFunction(autograd.Function):
+    """The vertical fusion the reference's optimizer stops short of:
+    ``gspmm(blk, fused_gsddmm(blk, q, k), x)`` as one op, forward and backward."""
+
+    @staticmethod
+    def forward(ctx, adj_sparse, query, key, x):
+        indptr, indices = adj_sparse
+        out, attn = graph_ext.gat_forward(indptr, indices, query, key, x)
+        ctx.adj_sparse = adj_sparse
+        ctx.save_for_backward(query, key, x, attn)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        indptr, indices = ctx.adj_sparse
+        query, key, x, attn = ctx.saved_tensors
+        grad_q, grad_k, grad_x = graph_ext.gat_backward(indptr, indices, query, key, x, attn,
+                                                        grad_out.contiguous())
+        return None, grad_q, grad_k, grad_x
+
+
+def fused_gat(block: block.Block, query: torch.Tensor, key: torch.Tensor, x: torch.Tensor):
+    """query [n_dst, H], key [n_src, H], x [n_src, H, F] -> [n_dst, H, F]."""
+    assert x.dim() == 3 and query.dim() == 2 and key.dim() == 2
+    return FusedGATFunction.apply(block.adj_sparse, query, key, x)
