@@ -146,6 +146,73 @@ def run_spmm(args, dev, bf16):
     return res
 
 
+def run_gat(args, dev):
+    """Second configuration: GAT attention, 4 heads x 64, R-MAT 2^18 nodes, 13 M draws
+    (deduplicated), fp32. One step = fused forward (SDDMM + LeakyReLU + edge softmax +
+    aggregate, attn saved) + backward (grad of x', q, k), through the C ABI. The dense
+    per-head projections q = <a_dst, x'>, k = <a_src, x'> are outside the timed step."""
+    from yitu_amd import graph_ext
+    from yitu_amd.data import graphgen
+    scale, draws, h, f = 18, 13_000_000, 4, 64
+    n = 1 << scale
+    src, dst = graphgen.rmat(scale, draws, 20241, device=dev)
+    rp, ci = graphgen.csr_by_destination(src, dst, n)
+    del src, dst
+    nnz = ci.numel()
+    g = torch.Generator(device=dev).manual_seed(20241)
+    x = torch.randn(n, h, f, generator=g, device=dev)
+    a_src = torch.randn(h, f, generator=g, device=dev) * 0.1
+    a_dst = torch.randn(h, f, generator=g, device=dev) * 0.1
+    q = torch.einsum("nhf,hf->nh", x, a_dst).contiguous()
+    k = torch.einsum("nhf,hf->nh", x, a_src).contiguous()
+    gy = torch.randn(n, h, f, generator=g, device=dev)
+    graph_ext.transposed(rp, ci, n)  # one-time graph preparation, outside the timed region
+
+    ev = {"fwd": [], "bwd": []}
+
+    def step(timed):
+        es = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        es[0].record()
+        out, attn = graph_ext.gat_forward(rp, ci, q, k, x)
+        es[1].record()
+        graph_ext.gat_backward(rp, ci, q, k, x, attn, gy)
+        es[2].record()
+        if timed:
+            ev["fwd"].append((es[0], es[1]))
+            ev["bwd"].append((es[1], es[2]))
+
+    for _ in range(args.warmup):
+        step(False)
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    _sync()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    fwd_ms = sum(a.elapsed_time(b) for a, b in ev["fwd"]) / args.steps
+    bwd_ms = sum(a.elapsed_time(b) for a, b in ev["bwd"]) / args.steps
+    alg_fwd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h + 8 * n * h * f
+    alg_bwd = (2 * 4 * n * h * f + 4 * nnz * h + 8 * nnz + 8 * (n + 1) + 4 * nnz
+               + 4 * n * h * f + 8 * n * h)
+    return {
+        "metric": "GAT attention fwd+bwd (fused SDDMM+LeakyReLU+softmax+aggregate), edges/sec",
+        "value": nnz / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "c2_gat_f32", "graph": "R-MAT scale 18, 13M draws dedup, CSR by "
+                   "destination", "n_nodes": n, "n_edges": nnz, "heads": h, "head_dim": f},
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "roofline": {"bound": "hbm", "achieved": alg_fwd / (fwd_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("c2_gat_f32"),
+                     "kernel": "yitu_gat_forward (gat_fwd_rows_kernel + hub kernels)",
+                     "kernel_ms": fwd_ms, "algorithmic_bytes": alg_fwd,
+                     "bwd_achieved": alg_bwd / (bwd_ms * 1e-3) / 1e9,
+                     "bwd_algorithmic_bytes": alg_bwd},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,6 +220,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3_spmm_f32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="default workload only")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)")
@@ -162,8 +230,17 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "c3_spmm_f32":
         res = run_spmm(args, dev, bf16=False)
+        if not args.no_extra:
+            # the other single-GPU configurations ride along as extra fields
+            args.no_cpu = True
+            slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
+                                                "roofline") if k in r}
+            res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
+                            "c2_gat_f32": slim(run_gat(args, dev))}
     elif args.workload == "c3_spmm_bf16":
         res = run_spmm(args, dev, bf16=True)
+    elif args.workload == "c2_gat_f32":
+        res = run_gat(args, dev)
     else:
         sys.exit("unknown workload %s" % args.workload)
     print(json.dumps(res))
