@@ -170,6 +170,43 @@ int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Dense products on the matrix cores (fp32 MFMA)                              */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * C[m,n] (+)= op(A)[m,k] . op(B)[k,n], row-major, fp32. trans_a: A is stored
+ * [k,m]; trans_b: B is stored [n,k]. Replaces the torch::mm (cuBLAS SGEMM)
+ * calls around the aggregation kernels: X.W (YiTu_GNN_kernel.cu:276,606),
+ * G.W^T and X^T.G (cu:471-472,715-716). Products with few output tiles and a long
+ * inner dimension (X^T.G) are split along k over the chip; the slabs go to the
+ * workspace (yitu_sgemm_workspace_bytes; NULL = no split) and are summed in a
+ * fixed order.
+ */
+size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems);
+int yitu_sgemm(float *c_device, const float *a_device, const float *b_device, int64_t m, int64_t n,
+               int64_t k, int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldc,
+               int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
+
+/*
+ * b2gemm (entry.cpp:56-64; fc_cuda.cu:4-75): y_a = x . w_a^T, y_b = x . w_b^T
+ * as one grouped launch. x [n,k], w_* [m,k], y_* [n,m], contiguous.
+ */
+int yitu_b2gemm(float *y_a_device, float *y_b_device, const float *x_device,
+                const float *w_a_device, const float *w_b_device, int64_t n, int64_t k, int64_t m,
+                void *stream);
+
+/*
+ * b2gemm_backward (entry.cpp:66-78; fc_cuda.cu:77-215):
+ * dw_* [m,k] = grad_*^T . x ; dx [n,k] = grad_a . w_a + grad_b . w_b.
+ * Workspace: yitu_sgemm_workspace_bytes(m, k, n, 2).
+ */
+int yitu_b2gemm_backward(float *dx_device, float *dw_a_device, float *dw_b_device,
+                         const float *x_device, const float *w_a_device, const float *w_b_device,
+                         const float *grad_a_device, const float *grad_b_device, int64_t n,
+                         int64_t k, int64_t m, void *workspace_device, size_t workspace_bytes,
+                         void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */
 /* ------------------------------------------------------------------------- */
 

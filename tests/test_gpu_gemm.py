@@ -1,0 +1,94 @@
+"""GPU parity of the MFMA fp32 GEMM entry points (yitu_sgemm, yitu_b2gemm,
+yitu_b2gemm_backward) against double-precision products."""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+import oracle
+from helpers import assert_close
+from yitu_amd import graph_ext
+from yitu_amd.xgnn_h import bundle
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref(a, b, ta, tb):
+    a64, b64 = a.double(), b.double()
+    return ((a64.t() if ta else a64) @ (b64.t() if tb else b64)).float()
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (7, 5, 3), (128, 128, 16), (130, 257, 33),
+                                   (256, 128, 256), (1000, 40, 100), (64, 300, 1)])
+def test_sgemm_all_layouts(dev, ta, tb, m, n, k):
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + k)
+    a = torch.randn((k, m) if ta else (m, k), generator=g)
+    b = torch.randn((n, k) if tb else (k, n), generator=g)
+    got = graph_ext.sgemm(a.to(dev), b.to(dev), ta, tb)
+    assert_close(got, _ref(a, b, ta, tb), atol=1e-4 * max(1.0, np.sqrt(k) / 4),
+                 what="m=%d n=%d k=%d ta=%s tb=%s" % (m, n, k, ta, tb))
+
+
+def test_sgemm_split_k_long_inner_dimension(dev):
+    """dW = X^T G with K = number of nodes: few tiles, split along K, fixed-order reduce."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(70001, 96, generator=g)
+    gy = torch.randn(70001, 130, generator=g)
+    got = graph_ext.sgemm(x.to(dev), gy.to(dev), True, False)
+    assert_close(got, _ref(x, gy, True, False), atol=1e-4 * np.sqrt(70001))
+    again = graph_ext.sgemm(x.to(dev), gy.to(dev), True, False)
+    assert torch.equal(got, again)
+
+
+def test_sgemm_typed_gemm_shape(dev):
+    """[n_t, 256] x [256, 256] of the heterogeneous configuration (fast path)."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(1 << 15, 256, generator=g)
+    w = torch.randn(256, 256, generator=g) * 0.02
+    assert_close(graph_ext.sgemm(x.to(dev), w.to(dev)), _ref(x, w, False, False))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_check_bundle(dev, seed):
+    """test_kernel.py:187-233 with seeded shapes: b2gemm vs two bias-free Linear layers,
+    outputs and all three gradients, through GEMMBundleFunction."""
+    rng = np.random.default_rng(seed)
+    n, k, m = int(rng.integers(8, 1025)), int(rng.integers(8, 257)), int(rng.integers(1, 33))
+    torch.manual_seed(seed)
+    x = torch.randn(n, k, device=dev, requires_grad=True)
+    fc1 = nn.Linear(k, m, bias=False).to(dev)
+    fc2 = nn.Linear(k, m, bias=False).to(dev)
+    y1, y2 = fc1(x), fc2(x)
+    torch.sum(y1 + y2).backward()
+    gx1, g1, g2 = x.grad.clone(), fc1.weight.grad.clone(), fc2.weight.grad.clone()
+    x.grad.zero_()
+    fc1.zero_grad()
+    fc2.zero_grad()
+    y3, y4 = bundle.GEMMBundleFunction.apply(x, fc1.weight, fc2.weight, fc1.bias, fc2.bias)
+    torch.sum(y3 + y4).backward()
+    assert torch.allclose(y1, y3, atol=1e-3) and torch.allclose(y2, y4, atol=1e-3)
+    assert torch.allclose(g1, fc1.weight.grad, atol=1e-3)
+    assert torch.allclose(g2, fc2.weight.grad, atol=1e-3)
+    assert torch.allclose(gx1, x.grad, atol=1e-3)
+
+
+def test_b2gemm_against_oracle(dev):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4096, 256, generator=g)
+    wa = torch.randn(256, 256, generator=g) * 0.02
+    wb = torch.randn(256, 256, generator=g) * 0.02
+    ga = torch.randn(4096, 256, generator=g)
+    gb = torch.randn(4096, 256, generator=g)
+    ya, yb = graph_ext.b2gemm(x.to(dev), wa.to(dev), wb.to(dev))
+    want_a, want_b = oracle.b2gemm(x.numpy(), wa.numpy(), wb.numpy())
+    assert_close(ya, want_a)
+    assert_close(yb, want_b)
+    dx, dwa, dwb = graph_ext.b2gemm_backward(x.to(dev), wa.to(dev), wb.to(dev), ga.to(dev),
+                                             gb.to(dev))
+    want_dx, want_dwa, want_dwb = oracle.b2gemm_backward(x.numpy(), wa.numpy(), wb.numpy(),
+                                                         ga.numpy(), gb.numpy())
+    assert_close(dx, want_dx)
+    assert_close(dwa, want_dwa, atol=1e-4 * 64)
+    assert_close(dwb, want_dwb, atol=1e-4 * 64)

@@ -20,6 +20,12 @@ from . import _lib
 from ._lib import c_f32, c_i64, c_int, c_size, check, ptr, stream_ptr
 
 
+def _mm(a, b, trans_a=False, trans_b=False):
+    """Dense fp32 product on the matrix cores (the reference calls torch::mm)."""
+    from .graph_ext import sgemm
+    return sgemm(a.contiguous(), b.contiguous(), trans_a, trans_b)
+
+
 def _check_inputs(*tensors):
     # CHECK_INPUT of the reference: CUDA + contiguous (YiTu_GNN.cpp:65-69)
     return _lib.require_device(*tensors)
@@ -67,7 +73,7 @@ def forward(input, weight, row_pointers, column_index, degrees, part_pointers, p
             dimWorker, warpPerBlock):
     """GCN: out = aggregate_{s_i s_j}(X.W) (YiTu_GNN.cpp:94-117; cu:264-317). Returns [out]."""
     _check_inputs(input, weight, row_pointers, column_index, degrees, part_pointers, part2Node)
-    tmp = torch.mm(input, weight)
+    tmp = _mm(input, weight)
     return [_aggregate(tmp, row_pointers, column_index, degrees, 1.0)]
 
 
@@ -78,7 +84,7 @@ def backward(d_output, X, W, row_pointers, column_index, degrees, part_pointers,
     cu:422-475). Returns [d_input, d_weight]."""
     _check_inputs(d_output, X, W, row_pointers, column_index, degrees, part_pointers, part2Node)
     g = _aggregate(d_output, row_pointers, column_index, degrees, 1.0)
-    return [torch.mm(g, W.t()), torch.mm(X.t(), g)]
+    return [_mm(g, W, trans_b=True), _mm(X, g, trans_a=True)]
 
 
 def forward_gin(input, weight, row_pointers, column_index, epsilon, part_pointers, part2Node,
@@ -86,7 +92,7 @@ def forward_gin(input, weight, row_pointers, column_index, epsilon, part_pointer
     """GIN: A = eps * sum_j X[j]; out = A.W (YiTu_GNN.cpp:150-172; cu:563-618). Returns [out, A]."""
     _check_inputs(input, weight, row_pointers, column_index, part_pointers, part2Node)
     agg = _aggregate(input, row_pointers, column_index, None, float(epsilon))
-    return [torch.mm(agg, weight), agg]
+    return [_mm(agg, weight), agg]
 
 
 def backward_gin(d_output, X, W, row_pointers, column_index, epsilon, part_pointers, part2Node,
@@ -94,8 +100,8 @@ def backward_gin(d_output, X, W, row_pointers, column_index, epsilon, part_point
     """GIN backward: dW = X^T.dY (X is the saved aggregate), dX = eps * sum_j (dY.W^T)[j]
     (YiTu_GNN.cpp:177-201; cu:701-751). Returns [d_input, d_weight]."""
     _check_inputs(d_output, X, W, row_pointers, column_index, part_pointers, part2Node)
-    d_weight = torch.mm(X.t(), d_output)
-    g = torch.mm(d_output, W.t())
+    d_weight = _mm(X, d_output, trans_a=True)
+    g = _mm(d_output, W, trans_b=True)
     return [_aggregate(g, row_pointers, column_index, None, float(epsilon)), d_weight]
 
 

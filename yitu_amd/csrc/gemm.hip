@@ -1,0 +1,364 @@
+// fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32) for the dense
+// products of the heterogeneous path (two Linear layers sharing one input,
+// fc_cuda.cu) and the X.W / G.W^T / X^T.G products around the GCN / GIN
+// aggregation (YiTu_GNN_kernel.cu:276,471-472,606,715-716).
+//
+//   C[M,N] (+)= A[M,K] . B[K,N],  element (i,k) of A at A + i*a_si + k*a_sk,
+//                                  element (k,j) of B at B + k*b_sk + j*b_sj,
+// one of each stride pair being 1, C row-major. Up to 8 problems that share
+// N, K and the strides are grouped into one launch (blockIdx.z).
+//
+// Tiling: 128x128 output tile per 256-thread workgroup, each of the 4 waves
+// owns 64x64 = 2x2 MFMA tiles (64 accumulator registers); K advances in steps
+// of 16 through double-buffered LDS tiles stored K-major, so an MFMA operand
+// read is 32 consecutive floats per half wave (conflict free). Operands that
+// are K-contiguous in memory are transposed on their way into LDS. The next
+// K-step's global loads are issued before the current step's MFMAs.
+#include "../../include/yitu_hip.h"
+#include "spmm_rows.hpp"
+
+namespace yitu {
+
+constexpr int BM = 128, BN = 128, BK = 16, LDP = 132;  // LDP: padded LDS row (floats)
+constexpr int kMaxGroup = 8;
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+struct GemmProblem {
+    const float *A;
+    const float *B;
+    float *C;
+    int M;
+};
+
+struct GemmParams {
+    GemmProblem prob[kMaxGroup];
+    int n_prob;
+    int N, K;
+    int64_t a_si, a_sk, b_sk, b_sj;
+    int ldc;
+    int accumulate;  // C += A.B instead of C = A.B
+    // split-K: blockIdx.z = problem * n_split + split; split s covers K range
+    // [s * k_chunk, min(K, (s+1) * k_chunk)) and writes its own [M, N] slab of
+    // `partial` (slab index = blockIdx.z, all problems sized by max_m)
+    int n_split, k_chunk, max_m;
+    float *partial;
+};
+
+// Loads this thread's 8 elements of a [128 x 16] operand tile into regs.
+// KCONT: the operand is contiguous along K (thread owns 8 consecutive k of one row),
+// otherwise contiguous along the row dimension (8 consecutive rows of one k).
+template <bool KCONT, bool FAST>
+__device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict__ base,
+                                          int64_t s_row, int64_t s_k, int row0, int k0, int n_rows,
+                                          int K) {
+    const int t = threadIdx.x;
+    if constexpr (KCONT) {
+        const int row = row0 + (t >> 1), k = k0 + (t & 1) * 8;
+        const float *p = base + (int64_t)row * s_row + k;
+        if constexpr (FAST) {
+            const float4 a = *reinterpret_cast<const float4 *>(p);
+            const float4 b = *reinterpret_cast<const float4 *>(p + 4);
+            r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
+            r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = (row < n_rows && k + i < K) ? p[i] : 0.0f;
+        }
+    } else {
+        const int k = k0 + (t >> 4), row = row0 + (t & 15) * 8;
+        const float *p = base + (int64_t)k * s_k + row;
+        if constexpr (FAST) {
+            const float4 a = *reinterpret_cast<const float4 *>(p);
+            const float4 b = *reinterpret_cast<const float4 *>(p + 4);
+            r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
+            r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = (k < K && row + i < n_rows) ? p[i] : 0.0f;
+        }
+    }
+}
+
+template <bool KCONT>
+__device__ __forceinline__ void store_tile(float (*tile)[LDP], const float (&r)[8]) {
+    const int t = threadIdx.x;
+    if constexpr (KCONT) {
+        const int row = t >> 1, k = (t & 1) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; i++) tile[k + i][row] = r[i];
+    } else {
+        const int k = t >> 4, row = (t & 15) * 8;
+        *reinterpret_cast<float4 *>(&tile[k][row]) = make_float4(r[0], r[1], r[2], r[3]);
+        *reinterpret_cast<float4 *>(&tile[k][row + 4]) = make_float4(r[4], r[5], r[6], r[7]);
+    }
+}
+
+template <bool A_KCONT, bool B_KCONT, bool FAST>
+__global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
+    __shared__ float As[2][BK][LDP];
+    __shared__ float Bs[2][BK][LDP];
+    const GemmProblem pr = p.prob[blockIdx.z / p.n_split];
+    const int split = blockIdx.z % p.n_split;
+    const int kb = split * p.k_chunk, ke = min(p.K, kb + p.k_chunk);
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (m0 >= pr.M) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int l32 = lane & 31, lk = lane >> 5;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    float ra[8], rb[8];
+    load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb, pr.M, ke);
+    load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb, p.N, ke);
+    store_tile<A_KCONT>(As[0], ra);
+    store_tile<B_KCONT>(Bs[0], rb);
+    __syncthreads();
+
+    const int n_steps = (ke - kb + BK - 1) / BK;
+    for (int s = 0; s < n_steps; s++) {
+        const int cur = s & 1;
+        if (s + 1 < n_steps) {
+            load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb + (s + 1) * BK, pr.M, ke);
+            load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb + (s + 1) * BK, p.N, ke);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            const float a0 = As[cur][kk + lk][wm + l32];
+            const float a1 = As[cur][kk + lk][wm + 32 + l32];
+            const float b0 = Bs[cur][kk + lk][wn + l32];
+            const float b1 = Bs[cur][kk + lk][wn + 32 + l32];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (s + 1 < n_steps) {
+            // the other buffer was last read in step s-1, before the barrier below
+            store_tile<A_KCONT>(As[cur ^ 1], ra);
+            store_tile<B_KCONT>(Bs[cur ^ 1], rb);
+        }
+        __syncthreads();
+    }
+
+    // accumulator element 4*jj + ii of tile (i, j) is C[8*jj + 4*(lane/32) + ii][lane % 32]
+    float *cbase = pr.C;
+    int ldc = p.ldc;
+    bool accumulate = p.accumulate != 0;
+    if (p.n_split > 1) {
+        cbase = p.partial + (size_t)blockIdx.z * p.max_m * p.N;
+        ldc = p.N;
+        accumulate = false;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = n0 + wn + 32 * j + l32;
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+                for (int ii = 0; ii < 4; ii++) {
+                    const int row = m0 + wm + 32 * i + 8 * jj + 4 * lk + ii;
+                    if (FAST || (row < pr.M && col < p.N)) {
+                        float *c = cbase + (int64_t)row * ldc + col;
+                        const float v = acc[i][j][4 * jj + ii];
+                        *c = accumulate ? *c + v : v;
+                    }
+                }
+        }
+}
+
+// C (+)= sum over splits of the partial slabs, in split order (reproducible)
+__global__ __launch_bounds__(256) void sgemm_splitk_reduce_kernel(GemmParams p) {
+    const GemmProblem pr = p.prob[blockIdx.y];
+    const int64_t total = (int64_t)pr.M * p.N;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total;
+         e += (int64_t)gridDim.x * 256) {
+        const int row = (int)(e / p.N), col = (int)(e % p.N);
+        float s = 0.0f;
+        for (int z = 0; z < p.n_split; z++)
+            s += p.partial[((size_t)(blockIdx.y * p.n_split + z) * p.max_m + row) * p.N + col];
+        float *c = pr.C + (int64_t)row * p.ldc + col;
+        *c = p.accumulate ? *c + s : s;
+    }
+}
+
+// Few output tiles and a long inner dimension (dW = X^T.G with K = number of
+// nodes): split K so the whole chip works, partials summed by a second kernel.
+static void choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
+    p.n_split = 1;
+    p.k_chunk = ((p.K + BK - 1) / BK) * BK;
+    p.max_m = max_m;
+    const int64_t tiles = ceil_div(p.N, BN) * ceil_div(max_m, BM) * p.n_prob;
+    if (tiles >= 256 || p.K < 4096) return;
+    int64_t want = std::min<int64_t>(ceil_div(p.K, 1024), ceil_div(1024, tiles));
+    const int64_t slab = (int64_t)max_m * p.N * sizeof(float) * p.n_prob;
+    want = std::min<int64_t>(want, slab > 0 ? (int64_t)(workspace_bytes / slab) : 1);
+    if (want <= 1) return;
+    p.k_chunk = (int)(ceil_div(ceil_div(p.K, want), BK) * BK);
+    p.n_split = (int)ceil_div(p.K, p.k_chunk);
+}
+
+template <bool A_KCONT, bool B_KCONT>
+static int sgemm_launch(const GemmParams &p, int max_m, hipStream_t stream) {
+    bool fast = p.N % BN == 0 && p.K % BK == 0;
+    for (int i = 0; i < p.n_prob; i++) {
+        fast = fast && p.prob[i].M % BM == 0 && aligned16(p.prob[i].A) && aligned16(p.prob[i].B);
+    }
+    // vector loads also need every row / k-line to start 16-byte aligned
+    fast = fast && (A_KCONT ? p.a_si % 4 == 0 : p.a_sk % 4 == 0) &&
+           (B_KCONT ? p.b_sj % 4 == 0 : p.b_sk % 4 == 0);
+    dim3 grid((unsigned)ceil_div(p.N, BN), (unsigned)ceil_div(max_m, BM),
+              (unsigned)(p.n_prob * p.n_split));
+    if (fast)
+        sgemm_mfma_kernel<A_KCONT, B_KCONT, true><<<grid, 256, 0, stream>>>(p);
+    else
+        sgemm_mfma_kernel<A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    if (p.n_split > 1) {
+        dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)max_m * p.N, 256), 2048),
+                (unsigned)p.n_prob);
+        sgemm_splitk_reduce_kernel<<<rg, 256, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+// trans_a: A is given as [K, M] row-major (else [M, K]); trans_b: B is given as
+// [N, K] row-major (else [K, N]).
+int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, void *workspace,
+                  size_t workspace_bytes, hipStream_t stream) {
+    int max_m = 0;
+    for (int i = 0; i < p.n_prob; i++) max_m = std::max(max_m, p.prob[i].M);
+    if (max_m == 0 || p.N == 0) return 0;
+    choose_split(p, max_m, workspace ? workspace_bytes : 0);
+    p.partial = static_cast<float *>(workspace);
+    if (p.K == 0) {
+        if (p.accumulate) return 0;
+        // empty inner dimension: C = 0
+        for (int i = 0; i < p.n_prob; i++) {
+            if (p.ldc == p.N) {
+                int rc = fill_zero(p.prob[i].C, (int64_t)p.prob[i].M * p.N, stream);
+                if (rc) return rc;
+            } else {
+                for (int r = 0; r < p.prob[i].M; r++) {
+                    int rc = fill_zero(p.prob[i].C + (int64_t)r * p.ldc, p.N, stream);
+                    if (rc) return rc;
+                }
+            }
+        }
+        return 0;
+    }
+    if (trans_a) {  // element (i,k) at A[k*lda + i]: contiguous along rows
+        p.a_si = 1;
+        p.a_sk = lda;
+    } else {
+        p.a_si = lda;
+        p.a_sk = 1;
+    }
+    if (trans_b) {  // element (k,j) at B[j*ldb + k]: contiguous along K
+        p.b_sk = 1;
+        p.b_sj = ldb;
+    } else {
+        p.b_sk = ldb;
+        p.b_sj = 1;
+    }
+    if (!trans_a && trans_b) return sgemm_launch<true, true>(p, max_m, stream);
+    if (!trans_a && !trans_b) return sgemm_launch<true, false>(p, max_m, stream);
+    if (trans_a && !trans_b) return sgemm_launch<false, false>(p, max_m, stream);
+    return sgemm_launch<false, true>(p, max_m, stream);
+}
+
+}  // namespace yitu
+
+using namespace yitu;
+#define YITU_API extern "C" __attribute__((visibility("default")))
+
+// Enough for the widest split the policy picks: 1024 / tiles slabs of [m, n].
+YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems) {
+    const int64_t tiles = ceil_div(n, BN) * ceil_div(m, BM) * n_problems;
+    if (tiles <= 0 || tiles >= 256 || k < 4096) return 256;
+    const int64_t splits = std::min<int64_t>(ceil_div(k, 1024), ceil_div(1024, tiles));
+    return align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256);
+}
+
+YITU_API int yitu_sgemm(float *c, const float *a, const float *b, int64_t m, int64_t n, int64_t k,
+                        int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldc,
+                        int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    YITU_REQUIRE(m >= 0 && n >= 0 && k >= 0, "negative size");
+    if (m == 0 || n == 0) return 0;
+    YITU_REQUIRE(c && (k == 0 || (a && b)), "null operand");
+    YITU_REQUIRE(m < INT32_MAX && n < INT32_MAX && k < INT32_MAX && ldc >= n, "size out of range");
+    YITU_REQUIRE(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n), "leading dimension too small");
+    GemmParams p{};
+    p.prob[0] = GemmProblem{a, b, c, (int)m};
+    p.n_prob = 1;
+    p.N = (int)n;
+    p.K = (int)k;
+    p.ldc = (int)ldc;
+    p.accumulate = accumulate;
+    return sgemm_grouped(p, trans_a != 0, trans_b != 0, (int)lda, (int)ldb, workspace,
+                         workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_b2gemm(float *y_a, float *y_b, const float *x, const float *w_a,
+                         const float *w_b, int64_t n, int64_t k, int64_t m, void *stream) {
+    YITU_REQUIRE(n >= 0 && k >= 0 && m >= 0, "negative size");
+    if (n == 0 || m == 0) return 0;
+    YITU_REQUIRE(y_a && y_b && (k == 0 || (x && w_a && w_b)), "null operand");
+    YITU_REQUIRE(n < INT32_MAX && k < INT32_MAX && m < INT32_MAX, "size out of range");
+    GemmParams p{};
+    p.prob[0] = GemmProblem{x, w_a, y_a, (int)n};
+    p.prob[1] = GemmProblem{x, w_b, y_b, (int)n};
+    p.n_prob = 2;
+    p.N = (int)m;
+    p.K = (int)k;
+    p.ldc = (int)m;
+    return sgemm_grouped(p, false, true, (int)k, (int)k, nullptr, 0,
+                         static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_b2gemm_backward(float *dx, float *dw_a, float *dw_b, const float *x,
+                                  const float *w_a, const float *w_b, const float *grad_a,
+                                  const float *grad_b, int64_t n, int64_t k, int64_t m,
+                                  void *workspace, size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n >= 0 && k >= 0 && m >= 0, "negative size");
+    YITU_REQUIRE(n < INT32_MAX && k < INT32_MAX && m < INT32_MAX, "size out of range");
+    YITU_REQUIRE(dx && dw_a && dw_b, "null output");
+    // dw_* [m,k] = grad_*^T [m,n] . x [n,k]: one grouped launch of two problems
+    if (m > 0 && k > 0) {
+        GemmParams p{};
+        p.prob[0] = GemmProblem{grad_a, x, dw_a, (int)m};
+        p.prob[1] = GemmProblem{grad_b, x, dw_b, (int)m};
+        p.n_prob = 2;
+        p.N = (int)k;
+        p.K = (int)n;
+        p.ldc = (int)k;
+        int rc = sgemm_grouped(p, true, false, (int)m, (int)k, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+    }
+    // dx [n,k] = grad_a [n,m] . w_a [m,k] + grad_b . w_b
+    if (n > 0 && k > 0) {
+        for (int pass = 0; pass < 2; pass++) {
+            GemmParams p{};
+            p.prob[0] = GemmProblem{pass ? grad_b : grad_a, pass ? w_b : w_a, dx, (int)n};
+            p.n_prob = 1;
+            p.N = (int)k;
+            p.K = (int)m;
+            p.ldc = (int)k;
+            p.accumulate = pass;
+            int rc = sgemm_grouped(p, false, false, (int)m, (int)k, nullptr, 0, stream);
+            if (rc) return rc;
+        }
+    }
+    return 0;
+}

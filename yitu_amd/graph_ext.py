@@ -231,6 +231,73 @@ def hfused_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_
 
 
 # --------------------------------------------------------------------------- #
+# two Linear layers sharing one input
+# --------------------------------------------------------------------------- #
+def b2gemm(x, w_a, w_b):
+    """Returns [y_a, y_b] = [x . w_a^T, x . w_b^T] (entry.cpp:56-64) on the matrix cores."""
+    _check(x, torch.float32, "x", 2)
+    _check(w_a, torch.float32, "w_a", 2)
+    _check(w_b, torch.float32, "w_b", 2)
+    if w_a.shape != w_b.shape or w_a.size(1) != x.size(1):
+        raise RuntimeError("w_a and w_b must both be [m, k] with k = x.size(1)")
+    dev = _lib.require_device(x, w_a, w_b)
+    n, k = x.shape
+    m = w_a.size(0)
+    y_a = torch.empty((n, m), dtype=torch.float32, device=dev)
+    y_b = torch.empty((n, m), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_b2gemm(ptr(y_a), ptr(y_b), ptr(x), ptr(w_a), ptr(w_b), c_i64(n),
+                                    c_i64(k), c_i64(m), stream_ptr(dev))
+    check(rc, "yitu_b2gemm")
+    return [y_a, y_b]
+
+
+def b2gemm_backward(x, w_a, w_b, grad_a, grad_b):
+    """Returns [dx, dw_a, dw_b] (entry.cpp:66-78)."""
+    for t, name in ((x, "x"), (w_a, "w_a"), (w_b, "w_b"), (grad_a, "grad_a"), (grad_b, "grad_b")):
+        _check(t, torch.float32, name, 2)
+    if grad_a.shape != grad_b.shape or w_a.shape != w_b.shape:
+        raise RuntimeError("the two halves of the bundle must have equal shapes")
+    dev = _lib.require_device(x, w_a, w_b, grad_a, grad_b)
+    n, k = x.shape
+    m = w_a.size(0)
+    if grad_a.shape != (n, m):
+        raise RuntimeError("grad_* must be [n, m]")
+    dx = torch.empty_like(x)
+    dw_a = torch.empty_like(w_a)
+    dw_b = torch.empty_like(w_b)
+    ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(c_i64(m), c_i64(k), c_i64(n),
+                                                               c_i64(2)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_b2gemm_backward(ptr(dx), ptr(dw_a), ptr(dw_b), ptr(x), ptr(w_a),
+                                             ptr(w_b), ptr(grad_a), ptr(grad_b), c_i64(n), c_i64(k),
+                                             c_i64(m), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_b2gemm_backward")
+    return [dx, dw_a, dw_b]
+
+
+def sgemm(a, b, trans_a=False, trans_b=False):
+    """op(a) . op(b) in fp32 on the matrix cores; a, b contiguous 2-D."""
+    _check(a, torch.float32, "a", 2)
+    _check(b, torch.float32, "b", 2)
+    dev = _lib.require_device(a, b)
+    m, k = (a.size(1), a.size(0)) if trans_a else (a.size(0), a.size(1))
+    kb, n = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
+    if k != kb:
+        raise RuntimeError("inner dimensions differ: %d vs %d" % (k, kb))
+    c = torch.empty((m, n), dtype=torch.float32, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(c_i64(m), c_i64(n), c_i64(k),
+                                                               c_i64(1)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_sgemm(ptr(c), ptr(a), ptr(b), c_i64(m), c_i64(n), c_i64(k),
+                                   c_int(int(trans_a)), c_int(int(trans_b)), c_i64(a.size(1)),
+                                   c_i64(b.size(1)), c_i64(n), c_int(0), ptr(ws), c_size(ws.numel()),
+                                   stream_ptr(dev))
+    check(rc, "yitu_sgemm")
+    return c
+
+
+# --------------------------------------------------------------------------- #
 # fused GAT attention (extension: the composition sddmm_forward -> spmm_forward)
 # --------------------------------------------------------------------------- #
 def gat_forward(indptr, indices, query, key, features):
