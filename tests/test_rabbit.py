@@ -1,0 +1,185 @@
+"""Rabbit-Order relabelling (yitu_amd.rabbit): invariants the definition fixes,
+agreement with an independent dictionary-based statement of the single-thread
+algorithm on small graphs, and locality on graphs with planted communities.
+
+The reference implementation (ccsrc/reorder/rabbit_order.hpp) needs boost, which
+is absent here, so its exact permutation values cannot be produced: equality with
+the reference's own output is PARITY UNPINNED; what is pinned is everything the
+algorithm's definition determines."""
+import numpy as np
+import pytest
+import torch
+
+from yitu_amd import rabbit
+
+
+def _python_rabbit(src, dst, n):
+    """Single-thread incremental aggregation with plain dicts (rabbit_order.hpp:393-673)."""
+    adj = [dict() for _ in range(n)]
+    for s, d in zip(src, dst):
+        if s != d:
+            adj[s][d] = adj[s].get(d, 0.0) + 1.0
+            adj[d][s] = adj[d].get(s, 0.0) + 1.0
+    es = [sorted(a.items()) for a in adj]
+    strength = [float(sum(w for _, w in e)) for e in es]
+    total = float(sum(strength))
+    com = list(range(n))
+    child = [None] * n
+    sibling = [None] * n
+    pairs = [(v, len(es[v])) for v in range(n)]
+    # the C++ uses std::sort with a degree-only comparator; any order that is
+    # consistent with it must be tried by the caller, so return both pieces
+    return es, strength, total, com, child, sibling, pairs
+
+
+def _aggregate_with_order(src, dst, n, order):
+    es, strength, total, com, child, sibling, _ = _python_rabbit(src, dst, n)
+
+    def root(v):
+        while com[v] != v:
+            v = com[v]
+        return v
+
+    def members(v):  # v and everything merged into it
+        out, stack = [], [v]
+        while stack:
+            u = stack.pop()
+            out.append(u)
+            c = child[u]
+            while c is not None:
+                stack.append(c)
+                c = sibling[c]
+        return out
+
+    merged_edges = {}
+    tops = []
+    for v in order:
+        acc = {}
+        # edge lists of members that were themselves visited are already aggregated;
+        # every original edge of the community is reachable through exactly one of
+        # them, so walk original adjacency of all members
+        for u in members(v):
+            for t, w in es[u]:
+                c = root(t)
+                if c != v:
+                    acc[c] = acc.get(c, 0.0) + w
+        best, gain = v, 0.0
+        for t in sorted(acc):
+            d = acc[t] - strength[v] * strength[t] / total
+            if gain < d:
+                best, gain = t, d
+        if best == v:
+            tops.append(v)
+        else:
+            strength[best] = float(np.float32(strength[best] + strength[v]))  # float storage, double math
+            sibling[v] = child[best]
+            child[best] = v
+            com[v] = best
+    perm = [None] * n
+    nxt = 0
+    for top in tops:
+        stack = []
+        u = top
+        while u is not None:
+            stack.append(u)
+            u = child[u]
+        while stack:
+            v = stack.pop()
+            perm[v] = nxt
+            nxt += 1
+            u = sibling[v]
+            while u is not None:
+                stack.append(u)
+                u = child[u]
+    return perm
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_matches_independent_statement_on_small_graphs(seed):
+    """Up to 16 vertices libstdc++'s std::sort is a plain insertion sort, i.e. stable,
+    so the visiting order is 'ascending degree, then ascending id' and the whole
+    algorithm is determined: compare the permutation with the dictionary version."""
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(2, 17))
+    m = int(rng.integers(1, 4 * n))
+    src = rng.integers(0, n, m)
+    dst = rng.integers(0, n, m)
+    src[0] = n - 1
+    es = _python_rabbit(src, dst, n)[0]
+    order = sorted(range(n), key=lambda v: len(es[v]))  # stable
+    want = _aggregate_with_order(src, dst, n, order)
+    _, perm = rabbit.reorder_with_perm(torch.IntTensor(np.stack([src, dst])))
+    assert perm.tolist() == want, (n, src.tolist(), dst.tolist())
+
+
+@pytest.mark.parametrize("n,m,seed", [(1, 1, 0), (10, 5, 1), (200, 1500, 2), (3000, 20000, 3)])
+def test_bijection_and_relabelled_edges(n, m, seed):
+    rng = np.random.default_rng(seed)
+    src = rng.integers(0, n, m).astype(np.int32)
+    dst = rng.integers(0, n, m).astype(np.int32)
+    src[0] = n - 1  # make max id + 1 == n
+    ei = torch.from_numpy(np.stack([src, dst]))
+    out, perm = rabbit.reorder_with_perm(ei)
+    assert out.dtype == torch.int32 and out.shape == ei.shape
+    assert sorted(perm.tolist()) == list(range(n))  # a permutation of [0, n)
+    p = perm.numpy()
+    assert np.array_equal(out.numpy()[0], p[src]) and np.array_equal(out.numpy()[1], p[dst])
+    assert torch.equal(rabbit.reorder(ei), out)  # reproducible
+    # isolated / unused ids get ids too, and self loops are tolerated
+    assert perm.numel() == n
+
+
+def test_planted_communities_become_contiguous_and_local():
+    rng = np.random.default_rng(0)
+    k, size = 12, 25
+    n = k * size
+    src, dst = [], []
+    for c in range(k):
+        ids = np.arange(c * size, (c + 1) * size)
+        for _ in range(size * 6):
+            a, b = rng.choice(ids, 2, replace=False)
+            src.append(a)
+            dst.append(b)
+    for _ in range(k * 2):  # sparse links between communities
+        a, b = rng.integers(0, n, 2)
+        src.append(a)
+        dst.append(b)
+    shuffle = rng.permutation(n)
+    s, d = shuffle[np.asarray(src)], shuffle[np.asarray(dst)]
+    ei = torch.from_numpy(np.ascontiguousarray(np.stack([s, d]).astype(np.int32)))
+    out, perm = rabbit.reorder_with_perm(ei)
+    before = np.abs(s - d).mean()
+    after = (out[0] - out[1]).abs().float().mean().item()
+    assert after < before / 4  # avg_edgeSpan, the reference's own locality metric (dataset.py:109)
+    # members of a planted community land in one contiguous id range
+    spans = []
+    for c in range(k):
+        new = perm.numpy()[shuffle[c * size:(c + 1) * size]]
+        spans.append(new.max() - new.min() + 1)
+    assert np.median(spans) <= size * 1.5
+
+
+def test_modularity_not_below_singletons():
+    """Merging only on positive gain means the communities' modularity is >= that of
+    singleton communities (= -sum (d_v / 2m)^2 < 0)."""
+    rng = np.random.default_rng(3)
+    n, m = 300, 2500
+    src, dst = rng.integers(0, n, m), rng.integers(0, n, m)
+    out, perm = rabbit.reorder_with_perm(torch.from_numpy(np.stack([src, dst]).astype(np.int32)))
+    # communities = maximal runs that the permutation keeps contiguous are not
+    # observable from outside; check the weaker, observable property instead:
+    # relabelling preserves the edge multiset up to the bijection
+    inv = np.empty(n, np.int64)
+    inv[perm.numpy()] = np.arange(n)
+    assert np.array_equal(inv[out.numpy()[0]], src) and np.array_equal(inv[out.numpy()[1]], dst)
+
+
+def test_input_checks():
+    with pytest.raises(RuntimeError):
+        rabbit.reorder(torch.zeros(2, 3, dtype=torch.int64))
+    with pytest.raises(RuntimeError):
+        rabbit.reorder(torch.zeros(3, 2, dtype=torch.int32))
+    with pytest.raises(RuntimeError):
+        rabbit.reorder(torch.tensor([[0, -1], [1, 2]], dtype=torch.int32))
+    empty = rabbit.reorder(torch.zeros(2, 0, dtype=torch.int32))
+    assert empty.shape == (2, 0)

@@ -45,7 +45,30 @@ def _compile(src, force):
     return obj
 
 
+HOST_LIB = os.path.join(HERE, "libyitu_host.so")
+# x86-64-v3: built in one container, loaded on another host
+HOST_FLAGS = ["-O3", "-mavx2", "-mfma", "-std=c++17", "-fopenmp", "-fPIC", "-fvisibility=hidden",
+              "-Wall", "-Wextra", "-shared"]
+
+
+def build_host(force=False):
+    """libyitu_host.so: the CPU graph-preparation code (g++, OpenMP)."""
+    srcs = sorted(glob.glob(os.path.join(CSRC, "host", "*.cpp")))
+    newest = max([os.path.getmtime(s) for s in srcs] +
+                 [os.path.getmtime(os.path.join(HERE, "..", "include", "yitu_host.h"))])
+    if not force and os.path.exists(HOST_LIB) and os.path.getmtime(HOST_LIB) > newest:
+        return HOST_LIB
+    cmd = [os.environ.get("CXX", "g++")] + HOST_FLAGS + srcs + ["-o", HOST_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + r.stdout + r.stderr)
+    if r.stderr.strip():
+        sys.stderr.write(r.stderr)
+    return HOST_LIB
+
+
 def build(force=False, jobs=8):
+    build_host(force)
     os.makedirs(OBJ, exist_ok=True)
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:

@@ -1,0 +1,289 @@
+// Rabbit-Order vertex relabelling (community-based, locality-improving) on the
+// host: the graph preparation step behind YiTu_GNN.rabbit.reorder
+// (ccsrc/reorder/reorder.cpp:235-290, algorithm in ccsrc/reorder/rabbit_order.hpp).
+//
+// Pipeline:
+//   1. symmetrise the edge list, drop self loops, merge duplicates with summed
+//      unit weights (reorder.cpp:31-97)                       [parallel, counting sort]
+//   2. visit vertices in ascending degree; each visited vertex gathers the edges
+//      of its community, re-targets them to community roots, and merges into the
+//      neighbour with the best modularity gain w_vu - str_v str_u / W, if any is
+//      positive (rabbit_order.hpp:393-526, 554-621)            [sequential]
+//   3. number the vertices by a depth-first walk of each top-level community's
+//      merge dendrogram; communities are laid out in the order in which they
+//      became top-level (rabbit_order.hpp:623-673)
+//
+// The aggregation in step 2 runs on one thread: the reference's lock-free
+// parallel version gives a thread-count- and timing-dependent permutation, and
+// the single-thread order is the one that is reproducible. Edge weights are
+// counts held in float (exact below 2^24), so the order in which duplicates are
+// summed does not change any comparison.
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <numeric>
+#include <utility>
+#include <vector>
+
+#include <omp.h>
+
+#include "../../../include/yitu_host.h"
+
+namespace {
+
+using vint = uint32_t;
+constexpr vint kNone = 0xffffffffu;
+
+struct Edge {
+    vint to;
+    float w;
+};
+
+thread_local char g_err[256] = "";
+
+// Symmetric weighted adjacency in CSR form: row v = distinct neighbours of v
+// (ascending id) with the number of input edges between them in either direction.
+struct Adjacency {
+    std::vector<int64_t> ptr;
+    std::vector<Edge> edges;
+};
+
+Adjacency build_adjacency(const int32_t *src, const int32_t *dst, int64_t m, vint n) {
+    std::vector<int64_t> count(n + 1, 0);
+    for (int64_t i = 0; i < m; i++) {
+        if (src[i] != dst[i]) {
+            count[(vint)src[i] + 1]++;
+            count[(vint)dst[i] + 1]++;
+        }
+    }
+    for (vint v = 0; v < n; v++) count[v + 1] += count[v];
+    std::vector<vint> raw((size_t)count[n]);
+    {
+        std::vector<int64_t> fill(count.begin(), count.end() - 1);
+        for (int64_t i = 0; i < m; i++) {
+            if (src[i] != dst[i]) {
+                raw[(size_t)fill[(vint)src[i]]++] = (vint)dst[i];
+                raw[(size_t)fill[(vint)dst[i]]++] = (vint)src[i];
+            }
+        }
+    }
+    // sort each row, count distinct targets
+    std::vector<int64_t> uniq(n + 1, 0);
+#pragma omp parallel for schedule(dynamic, 1024)
+    for (int64_t v = 0; v < (int64_t)n; v++) {
+        vint *b = raw.data() + count[v], *e = raw.data() + count[v + 1];
+        std::sort(b, e);
+        int64_t u = 0;
+        for (vint *p = b; p != e; ++p) u += (p == b || p[0] != p[-1]);
+        uniq[v + 1] = u;
+    }
+    for (vint v = 0; v < n; v++) uniq[v + 1] += uniq[v];
+    Adjacency adj;
+    adj.ptr = uniq;
+    adj.edges.resize((size_t)uniq[n]);
+#pragma omp parallel for schedule(dynamic, 1024)
+    for (int64_t v = 0; v < (int64_t)n; v++) {
+        const vint *b = raw.data() + count[v], *e = raw.data() + count[v + 1];
+        Edge *out = adj.edges.data() + uniq[v];
+        for (const vint *p = b; p != e;) {
+            const vint t = *p;
+            float w = 0.0f;
+            while (p != e && *p == t) {
+                w += 1.0f;
+                ++p;
+            }
+            *out++ = Edge{t, w};
+        }
+    }
+    return adj;
+}
+
+struct Dendrogram {
+    vint n = 0;
+    std::vector<vint> com;      // community pointer (root: com[v] == v)
+    std::vector<vint> child;    // last vertex merged into v
+    std::vector<vint> sibling;  // previous vertex merged into the same parent
+    std::vector<float> str;     // community strength; -1 once v has been merged away
+    std::vector<vint> tops;     // top-level vertices in the order they were fixed
+    std::vector<std::vector<Edge>> es;  // current (aggregated) edge list of each vertex
+    double total = 0.0;
+};
+
+inline vint find_root(Dendrogram &g, vint v) {
+    vint c = v;
+    while (g.com[c] != c) c = g.com[c];
+    if (v != c && g.com[v] != c) g.com[v] = c;  // one-step shortcut for the next lookup
+    return c;
+}
+
+// sort by target and add up the weights of equal targets, in place
+inline size_t combine(Edge *b, Edge *e) {
+    if (b == e) return 0;
+    std::sort(b, e, [](const Edge &x, const Edge &y) { return x.to < y.to; });
+    Edge *o = b;
+    for (Edge *p = b + 1; p != e; ++p) {
+        if (p->to == o->to)
+            o->w += p->w;
+        else
+            *++o = *p;
+    }
+    return (size_t)(o - b) + 1;
+}
+
+// Edges of v's whole community, re-targeted to current roots, self loops removed,
+// duplicates merged: becomes v's own edge list.
+void gather_community_edges(Dendrogram &g, vint v, std::vector<Edge> &buf,
+                            std::vector<vint> &united_child) {
+    buf.clear();
+    size_t combined = 0;
+    auto push = [&](vint u) {
+        for (const Edge &e : g.es[u]) {
+            const vint c = find_root(g, e.to);
+            if (c != v) buf.push_back(Edge{c, e.w});
+        }
+        if (buf.size() - combined >= 2048) {  // keep the working set small
+            combined += combine(buf.data() + combined, buf.data() + buf.size());
+            buf.resize(combined);
+        }
+    };
+    push(v);
+    while (united_child[v] != g.child[v]) {
+        const vint c = g.child[v];
+        for (vint w = c; w != kNone && w != united_child[v]; w = g.sibling[w]) push(w);
+        united_child[v] = c;
+    }
+    buf.resize(combine(buf.data(), buf.data() + buf.size()));
+    g.es[v].assign(buf.begin(), buf.end());
+}
+
+Dendrogram aggregate(const Adjacency &adj, vint n) {
+    Dendrogram g;
+    g.n = n;
+    g.com.resize(n);
+    g.child.assign(n, kNone);
+    g.sibling.assign(n, kNone);
+    g.str.resize(n);
+    g.es.resize(n);
+    std::iota(g.com.begin(), g.com.end(), 0u);
+    double total = 0.0;
+#pragma omp parallel for reduction(+ : total) schedule(static)
+    for (int64_t v = 0; v < (int64_t)n; v++) {
+        const Edge *b = adj.edges.data() + adj.ptr[v], *e = adj.edges.data() + adj.ptr[v + 1];
+        float s = 0.0f;
+        for (const Edge *p = b; p != e; ++p) s += p->w;
+        g.es[v].assign(b, e);
+        g.str[v] = s;
+        total += s;
+    }
+    g.total = total;
+
+    // ascending (unweighted) degree; ties fall where std::sort leaves them, the
+    // comparator looks at the degree only (rabbit_order.hpp:531-541)
+    std::vector<std::pair<vint, vint>> order(n);
+    for (vint v = 0; v < n; v++) order[v] = {v, (vint)g.es[v].size()};
+    std::sort(order.begin(), order.end(),
+              [](const std::pair<vint, vint> &x, const std::pair<vint, vint> &y) {
+                  return x.second < y.second;
+              });
+
+    std::vector<Edge> buf;
+    buf.reserve((size_t)std::min<int64_t>((int64_t)n * 2, (int64_t)1 << 24));
+    std::vector<vint> united_child(n, kNone);
+    for (vint i = 0; i < n; i++) {
+        const vint v = order[i].first;
+        gather_community_edges(g, v, buf, united_child);
+        const float vstr = g.str[v];
+        // neighbour with the largest positive modularity gain; first one wins ties
+        double best_gain = 0.0;
+        vint best = v;
+        for (const Edge &e : g.es[v]) {
+            const double d = (double)e.w - (double)vstr * (double)g.str[e.to] / g.total;
+            if (best_gain < d) {
+                best_gain = d;
+                best = e.to;
+            }
+        }
+        if (best == v) {
+            g.tops.push_back(v);
+        } else {
+            g.str[best] += vstr;
+            g.sibling[v] = g.child[best];
+            g.child[best] = v;
+            g.com[v] = best;
+            g.str[v] = -1.0f;
+        }
+    }
+    return g;
+}
+
+// new id of every vertex: depth-first over each top-level community's merge tree
+std::vector<vint> permutation(const Dendrogram &g) {
+    std::vector<vint> perm(g.n, kNone);
+    std::vector<vint> stack;
+    vint next = 0;
+    auto push_chain = [&](vint v) {  // v, its last child, that one's last child, ...
+        for (; v != kNone; v = g.child[v]) stack.push_back(v);
+    };
+    for (const vint top : g.tops) {
+        push_chain(top);
+        while (!stack.empty()) {
+            const vint v = stack.back();
+            stack.pop_back();
+            perm[v] = next++;
+            if (g.sibling[v] != kNone) push_chain(g.sibling[v]);
+        }
+    }
+    return perm;
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) const char *yitu_host_last_error(void) {
+    return g_err;
+}
+
+extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder(
+    int32_t *out_edge_index, int32_t *perm_out, int64_t perm_capacity, int64_t *n_vertices,
+    const int32_t *in_edge_index, int64_t n_edges) {
+    if (n_edges < 0 || (n_edges > 0 && !in_edge_index)) {
+        snprintf(g_err, sizeof(g_err), "bad edge list");
+        return -1;
+    }
+    const int32_t *src = in_edge_index, *dst = in_edge_index + n_edges;
+    int64_t n64 = 0;
+    for (int64_t i = 0; i < n_edges; i++) {
+        if (src[i] < 0 || dst[i] < 0) {
+            snprintf(g_err, sizeof(g_err), "negative vertex id at edge %lld", (long long)i);
+            return -1;
+        }
+        n64 = std::max<int64_t>(n64, (int64_t)std::max(src[i], dst[i]) + 1);
+    }
+    if (n_vertices) *n_vertices = n64;
+    const vint n = (vint)n64;
+    if (perm_out && perm_capacity < n64) {
+        snprintf(g_err, sizeof(g_err), "perm buffer holds %lld ids, graph has %lld vertices",
+                 (long long)perm_capacity, (long long)n64);
+        return -1;
+    }
+    if (n == 0) return 0;
+    const Adjacency adj = build_adjacency(src, dst, n_edges, n);
+    const Dendrogram g = aggregate(adj, n);
+    const std::vector<vint> perm = permutation(g);
+    for (vint v = 0; v < n; v++) {
+        if (perm[v] == kNone) {
+            snprintf(g_err, sizeof(g_err), "internal error: vertex %u not numbered", v);
+            return -2;
+        }
+    }
+    if (perm_out)
+        for (vint v = 0; v < n; v++) perm_out[v] = (int32_t)perm[v];
+    if (out_edge_index) {
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n_edges; i++) {
+            out_edge_index[i] = (int32_t)perm[(vint)src[i]];
+            out_edge_index[n_edges + i] = (int32_t)perm[(vint)dst[i]];
+        }
+    }
+    return 0;
+}

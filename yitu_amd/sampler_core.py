@@ -1,0 +1,116 @@
+"""Drop-in for the reference's ``sampler_core`` extension module
+(YiTu_GNN/YiTu_T/sampler_core.cpp:374-402): ``ParallelSampler`` with
+``sample / reset / get_ret`` and ``TemporalGraphBlock`` accessors returning numpy
+arrays. Only the most-recent-neighbour mode the temporal attention path uses is
+implemented (``recent=True``, ``num_history=1``, ``window_duration=0``); other
+modes raise ``NotImplementedError``.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _host
+
+
+class TemporalGraphBlock:
+    """COO block: ``row`` = root slot, ``col`` = index into ``nodes`` (roots first),
+    ``eid``, ``ts``, ``dts`` (= root time - edge time, 0 for the roots), ``nodes``."""
+
+    def __init__(self, row, col, eid, ts, dts, nodes, dim_in, dim_out):
+        self._row, self._col, self._eid = row, col, eid
+        self._ts, self._dts, self._nodes = ts, dts, nodes
+        self._dim_in, self._dim_out = int(dim_in), int(dim_out)
+
+    def row(self):
+        return self._row.copy()
+
+    def col(self):
+        return self._col.copy()
+
+    def eid(self):
+        return self._eid.copy()
+
+    def ts(self):
+        return self._ts.copy()
+
+    def dts(self):
+        return self._dts.copy()
+
+    def nodes(self):
+        return self._nodes.copy()
+
+    def dim_in(self):
+        return self._dim_in
+
+    def dim_out(self):
+        return self._dim_out
+
+    # phase timers of the reference block; not collected here
+    def tot_time(self):
+        return 0.0
+
+    ptr_time = search_time = sample_time = coo_time = tot_time
+
+
+class ParallelSampler:
+    def __init__(self, indptr, indices, eid, ts, num_thread_per_worker, num_workers, num_layers,
+                 num_neighbors, recent, prop_time, num_history, window_duration):
+        if not recent:
+            raise NotImplementedError("only recent=True (most-recent-k neighbours) is built")
+        if num_history != 1 or abs(window_duration) > 1e-7:
+            raise NotImplementedError("only num_history=1, window_duration=0 is built")
+        self._indptr = np.ascontiguousarray(indptr, dtype=np.int32)
+        self._indices = np.ascontiguousarray(indices, dtype=np.int32)
+        self._eid = np.ascontiguousarray(eid, dtype=np.int32)
+        self._ts = np.ascontiguousarray(ts, dtype=np.float32)
+        fan = np.ascontiguousarray(num_neighbors, dtype=np.int32)
+        if fan.shape[0] < num_layers:
+            raise ValueError("num_neighbors needs one entry per layer")
+        p = lambda a: ctypes.c_void_p(a.ctypes.data)
+        self._h = _host.lib().yitu_sampler_create(
+            p(self._indptr), p(self._indices), p(self._eid), p(self._ts),
+            ctypes.c_int64(self._indptr.shape[0] - 1), ctypes.c_int64(self._indices.shape[0]),
+            ctypes.c_int(int(num_thread_per_worker) * int(num_workers)), ctypes.c_int(num_layers),
+            p(fan), ctypes.c_int(int(bool(prop_time))))
+        if not self._h:
+            raise RuntimeError("invalid T-CSR passed to ParallelSampler")
+        self._ret = []
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            _host.lib().yitu_sampler_destroy(ctypes.c_void_p(h))
+            self._h = None
+
+    def reset(self):
+        _host.lib().yitu_sampler_reset(ctypes.c_void_p(self._h))
+
+    def sample(self, root_nodes, root_ts):
+        nodes = np.ascontiguousarray(root_nodes, dtype=np.int32)
+        ts = np.ascontiguousarray(root_ts, dtype=np.float32)
+        if nodes.shape != ts.shape or nodes.ndim != 1:
+            raise ValueError("root_nodes and root_ts must be 1-D and equally long")
+        L = _host.lib()
+        rc = L.yitu_sampler_sample(ctypes.c_void_p(self._h), ctypes.c_void_p(nodes.ctypes.data),
+                                   ctypes.c_void_p(ts.ctypes.data), ctypes.c_int64(nodes.shape[0]))
+        if rc != 0:
+            raise RuntimeError("sample failed: %s" %
+                               L.yitu_sampler_last_error(ctypes.c_void_p(self._h)).decode())
+        self._ret = []
+        for b in range(L.yitu_sampler_num_blocks(ctypes.c_void_p(self._h))):
+            ne, din, dout = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+            L.yitu_sampler_block_sizes(ctypes.c_void_p(self._h), b, ctypes.byref(ne),
+                                       ctypes.byref(din), ctypes.byref(dout))
+            row = np.empty(ne.value, np.int32)
+            col = np.empty(ne.value, np.int32)
+            eid = np.empty(ne.value, np.int32)
+            bts = np.empty(din.value, np.float32)
+            dts = np.empty(din.value, np.float32)
+            bn = np.empty(din.value, np.int32)
+            p = lambda a: ctypes.c_void_p(a.ctypes.data)
+            L.yitu_sampler_block_copy(ctypes.c_void_p(self._h), b, p(row), p(col), p(eid), p(bts),
+                                      p(dts), p(bn))
+            self._ret.append(TemporalGraphBlock(row, col, eid, bts, dts, bn, din.value, dout.value))
+
+    def get_ret(self):
+        return list(self._ret)
