@@ -77,7 +77,9 @@ int yitu_spmm_forward(float *out_device, const float *values_device, const int32
  * spmm_backward (entry.cpp:92-104; spmm_cuda.cu:24-42,64-86):
  *   grad_a[i,h]   = sum_k grad_out[row_i,h,k] * features[col_i,h,k]
  *   grad_x[c,h,k] = sum_{i: col_i = c} grad_out[row_i,h,k] * values[i,h]
- * Either output may be NULL to skip it. grad_x is computed as a gather over
+ * Either output may be NULL to skip it (values may then be NULL for grad_a
+ * alone, which is the plain per-edge dot product of a destination row with a
+ * source row). grad_x is computed as a gather over
  * the transposed structure (t_* from yitu_csr_transpose, required when grad_x
  * is requested) instead of the reference's 2*E*H*F float atomics; both outputs
  * are fully written and bitwise reproducible. max_degree / max_degree_t: widest

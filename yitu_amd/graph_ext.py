@@ -141,6 +141,33 @@ def spmm_backward(values, indptr, indices, features, grad_out):
     return [grad_a, grad_x]
 
 
+def edge_dot(indptr, indices, dst_feat, src_feat):
+    """e[i,h] = <dst_feat[row_i,h,:], src_feat[col_i,h,:]> for every edge i: the
+    SDDMM-dot inside spmm_backward (spmm_cuda.cu:33-35) as an op of its own."""
+    _check(indptr, torch.int32, "indptr", 1)
+    _check(indices, torch.int32, "indices", 1)
+    _check(dst_feat, torch.float32, "dst_feat", 3)
+    _check(src_feat, torch.float32, "src_feat", 3)
+    dev = _lib.require_device(indptr, indices, dst_feat, src_feat)
+    n_dst = indptr.numel() - 1
+    n_src, h, f = src_feat.shape
+    nnz = indices.numel()
+    if dst_feat.shape != (n_dst, h, f):
+        raise RuntimeError("dst_feat must be [n_dst, H, F] matching src_feat's H and F")
+    out = torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    maxdeg = _lib.max_degree(indptr)
+    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 512 else 0
+    ws = _lib.workspace(need, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_spmm_backward(ptr(out), ptr(None), ptr(None), ptr(indptr), ptr(indices),
+                                           ptr(src_feat), ptr(dst_feat), ptr(None), ptr(None),
+                                           ptr(None), c_i64(n_dst), c_i64(n_src), c_i64(nnz),
+                                           c_i64(h), c_i64(f), c_i64(maxdeg), c_i64(-1), ptr(ws),
+                                           c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_spmm_backward")
+    return out
+
+
 # --------------------------------------------------------------------------- #
 # SDDMM + LeakyReLU + edge softmax
 # --------------------------------------------------------------------------- #

@@ -1,0 +1,2 @@
+"""Temporal neighbour attention (YiTu_GNN/YiTu_T/layers.py) over the HIP ops."""
+from .layers import TemporalBlock, TimeEncode, TransfomerAttentionLayer  # noqa: F401

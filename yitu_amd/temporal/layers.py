@@ -1,0 +1,141 @@
+"""Time encoding and the temporal attention layer (YiTu_GNN/YiTu_T/layers.py:6-17,
+39-142) without DGL: the message-flow block is the sampler's COO output, the
+edge softmax / weighted sum run on the graph_ext kernels.
+
+The reference computes the attention core with DGL ops that are not part of its
+own tree (dgl.ops.edge_softmax, update_all(copy_src, sum), layers.py:131-135);
+their arithmetic is restated here as
+    logits = sum_d Q[dst] * K[e]          (per-edge dot, H heads)
+    att    = softmax over each destination's edges of LeakyReLU_0.2(logits)
+    agg    = sum_e att[e] * V[e]
+"""
+import numpy as np
+import torch
+
+from .. import graph_ext
+from ..xgnn_h import block as xblock
+from ..xgnn_h import sparse
+
+
+class TimeEncode(torch.nn.Module):
+    """cos(t * w + b), w_i = 10^(-9 i / (dim - 1)), b = 0, both trainable (layers.py:6-17)."""
+
+    def __init__(self, dim):
+        super().__init__()
+        self.dim = dim
+        self.w = torch.nn.Linear(1, dim)
+        self.w.weight = torch.nn.Parameter(
+            torch.from_numpy(1 / 10 ** np.linspace(0, 9, dim, dtype=np.float32)).reshape(dim, -1))
+        self.w.bias = torch.nn.Parameter(torch.zeros(dim))
+
+    def forward(self, t):
+        return torch.cos(self.w(t.reshape((-1, 1))))
+
+
+class TemporalBlock:
+    """What the layer needs of a sampled block: ``n_dst`` roots, edges sorted by
+    root slot, one new source node per edge (as sampler_core emits them).
+    ``h`` holds the node features [n_dst + n_edges, dim_node_feat] (roots first),
+    ``dt`` the per-edge time deltas, ``f`` optional edge features."""
+
+    def __init__(self, row, n_dst, dt, h=None, f=None, device="cuda"):
+        dev = torch.device(device)
+        row = torch.as_tensor(np.asarray(row), dtype=torch.int64)
+        if row.numel() and not bool((row[1:] >= row[:-1]).all()):
+            raise ValueError("edges must be grouped by destination (ascending root slot)")
+        counts = torch.bincount(row, minlength=n_dst)
+        indptr = torch.zeros(n_dst + 1, dtype=torch.int64)
+        indptr[1:] = torch.cumsum(counts, 0)
+        self.n_dst = int(n_dst)
+        self.n_edges = int(row.numel())
+        self.row = row.to(dev)
+        self.blk = xblock.Block([n_dst, self.n_edges],
+                                [indptr.to(torch.int32),
+                                 torch.arange(self.n_edges, dtype=torch.int32)]).to(dev)
+        self.dt = torch.as_tensor(np.asarray(dt), dtype=torch.float32).to(dev)
+        self.h = h
+        self.f = f
+
+    @staticmethod
+    def from_sampler(tgb, memory=None, device="cuda"):
+        """Builds the block from a ``TemporalGraphBlock`` and gathers node features
+        from a ``[num_nodes, dim]`` table by node id (the reference's prepare_input)."""
+        n_dst = tgb.dim_out()
+        h = None
+        if memory is not None:
+            ids = torch.as_tensor(tgb.nodes(), dtype=torch.int64, device=memory.device)
+            h = memory[ids].to(device)
+        return TemporalBlock(tgb.row(), n_dst, tgb.dts()[n_dst:], h=h, device=device)
+
+    def num_edges(self):
+        return self.n_edges
+
+    def num_dst_nodes(self):
+        return self.n_dst
+
+
+class TransfomerAttentionLayer(torch.nn.Module):
+    """layers.py:39-142, the non-``combined`` branches. Parameter names and shapes
+    are the reference's, so its state_dicts load unchanged."""
+
+    def __init__(self, dim_node_feat, dim_edge_feat, dim_time, num_head, dropout, att_dropout,
+                 dim_out, combined=False):
+        super().__init__()
+        if combined:
+            raise NotImplementedError("combined=True is not built")
+        self.num_head = num_head
+        self.dim_node_feat = dim_node_feat
+        self.dim_edge_feat = dim_edge_feat
+        self.dim_time = dim_time
+        self.dim_out = dim_out
+        self.dropout = torch.nn.Dropout(dropout)
+        self.att_dropout = torch.nn.Dropout(att_dropout)
+        self.att_act = torch.nn.LeakyReLU(0.2)
+        if dim_time > 0:
+            self.time_enc = TimeEncode(dim_time)
+        if dim_node_feat + dim_time > 0:
+            self.w_q = torch.nn.Linear(dim_node_feat + dim_time, dim_out)
+        self.w_k = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
+        self.w_v = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
+        self.w_out = torch.nn.Linear(dim_node_feat + dim_out, dim_out)
+        self.layer_norm = torch.nn.LayerNorm(dim_out)
+
+    def forward(self, b: TemporalBlock):
+        assert self.dim_time + self.dim_node_feat + self.dim_edge_feat > 0
+        dev = self.w_k.weight.device
+        n_dst = b.num_dst_nodes()
+        if b.num_edges() == 0:
+            return torch.zeros((n_dst, self.dim_out), device=dev)
+        parts_q, parts_kv = [], []
+        if self.dim_node_feat > 0:
+            parts_q.append(b.h[:n_dst])
+            parts_kv.append(b.h[n_dst:])
+        if self.dim_edge_feat > 0:
+            parts_kv.append(b.f)
+        if self.dim_time > 0:
+            parts_kv.append(self.time_enc(b.dt))
+            parts_q.append(self.time_enc(torch.zeros(n_dst, dtype=torch.float32, device=dev)))
+        kv_in = torch.cat(parts_kv, dim=1)
+        head_dim = self.dim_out // self.num_head
+        if parts_q:
+            Q = self.w_q(torch.cat(parts_q, dim=1))
+        else:  # edge features only (layers.py:104-107)
+            Q = torch.ones((n_dst, self.dim_out), device=dev)
+        K = self.w_k(kv_in).reshape(-1, self.num_head, head_dim).contiguous()
+        V = self.w_v(kv_in).reshape(-1, self.num_head, head_dim).contiguous()
+        Q = Q.reshape(n_dst, self.num_head, head_dim).contiguous()
+        # att = edge_softmax(LeakyReLU(sum_d Q*K)); fused_gsddmm applies LeakyReLU(0.2) +
+        # softmax to (query + key): query = 0, key = the dot-product logits, one key per edge
+        logits = sparse.edge_dot(b.blk, Q, K)
+        zeros = torch.zeros((n_dst, self.num_head), device=dev)
+        if logits.requires_grad:
+            att = sparse.fused_gsddmm(b.blk, zeros.requires_grad_(), logits)
+        else:
+            att = graph_ext.sddmm_forward(b.blk.adj_sparse[0], b.blk.adj_sparse[1],
+                                          zeros.unsqueeze(0), logits)
+        att = self.att_dropout(att)
+        agg = sparse.gspmm(b.blk, att, V).reshape(n_dst, self.dim_out)
+        rst = torch.cat([agg, b.h[:n_dst]], dim=1) if self.dim_node_feat != 0 else agg
+        rst = self.w_out(rst)
+        rst = torch.nn.functional.relu(self.dropout(rst))
+        return self.layer_norm(rst)

@@ -127,3 +127,30 @@ def fused_gat(block: block.Block, query: torch.Tensor, key: torch.Tensor, x: tor
     """query [n_dst, H], key [n_src, H], x [n_src, H, F] -> [n_dst, H, F]."""
     assert x.dim() == 3 and query.dim() == 2 and key.dim() == 2
     return FusedGATFunction.apply(block.adj_sparse, query, key, x)
+
+
+class EdgeDotFunction(autograd.Function):
+    """e[i,h] = <dst[row_i,h,:], src[col_i,h,:]> (dot-product attention logits).
+    Backward: grad_dst = SpMM of grad_e with src, grad_src by the transposed gather."""
+
+    @staticmethod
+    def forward(ctx, adj_sparse, dst_feat, src_feat):
+        indptr, indices = adj_sparse
+        ctx.adj_sparse = adj_sparse
+        ctx.save_for_backward(dst_feat, src_feat)
+        return graph_ext.edge_dot(indptr, indices, dst_feat, src_feat)
+
+    @staticmethod
+    def backward(ctx, grad_e):
+        indptr, indices = ctx.adj_sparse
+        dst_feat, src_feat = ctx.saved_tensors
+        grad_e = grad_e.contiguous()
+        grad_dst = graph_ext.spmm_forward(grad_e, indptr, indices, src_feat)
+        # grad_src[c] = sum_{i: col_i = c} grad_e[i] * dst[row_i]: spmm_backward's grad_x
+        # with dst_feat in the role of grad_out
+        _, grad_src = graph_ext.spmm_backward(grad_e, indptr, indices, src_feat, dst_feat)
+        return None, grad_dst, grad_src
+
+
+def edge_dot(block: block.Block, dst_feat: torch.Tensor, src_feat: torch.Tensor):
+    return EdgeDotFunction.apply(block.adj_sparse, dst_feat, src_feat)
