@@ -1,0 +1,83 @@
+"""GCN / GAT / heterogeneous layers on the GPU against dense torch algebra, the
+method of the reference's test_allclose.py (GCN layer == D_in^-1 A X W^T) and
+test_kernel.py (GAT attention == masked dense softmax)."""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from helpers import assert_close, random_csr
+from yitu_amd.xgnn_h import block as xblock
+from yitu_amd.xgnn_h import convert, layers
+
+pytestmark = pytest.mark.gpu
+
+
+def test_gcn_layer_equals_dense_right_norm(dev):
+    """test_allclose.py:24-30,53-62: y = D_in^-1 A (X W^T + b)."""
+    torch.manual_seed(0)
+    n, fin, fout = 300, 40, 24
+    indptr, indices = random_csr(n, n, 0.03, 1, empty_rows=(7,))
+    blk = xblock.Block([n, n], [indptr, indices]).to(dev)
+    norm = layers.right_norm(blk)
+    layer = layers.GCNLayer(fin, fout).to(dev)
+    x = torch.randn(n, fin, device=dev, requires_grad=True)
+    y = layer(blk, norm, x)
+    w = torch.randn_like(y)
+    (y * w).sum().backward()
+    got = [y.detach(), x.grad.clone(), layer.fc.weight.grad.clone()]
+    x.grad = None
+    layer.zero_grad()
+    dense = convert.to_dense(n, n, [indptr, indices], torch.ones(indices.numel())).to(dev)
+    deg = dense.sum(1, keepdim=True)
+    yd = torch.where(deg > 0, 1.0 / deg.clamp(min=1), torch.zeros_like(deg)) * (dense @ layer.fc(x))
+    (yd * w).sum().backward()
+    assert torch.all(got[0][7] == 0)
+    for a, b in zip(got, [yd.detach(), x.grad, layer.fc.weight.grad]):
+        assert_close(a, b, atol=2e-4)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_gat_layer_equals_dense_attention(dev, fused):
+    torch.manual_seed(1)
+    n, fin, f, h = 257, 30, 16, 4
+    indptr, indices = random_csr(n, n, 0.04, 2, hub_rows=(3,), hub_degree=200)
+    blk = xblock.Block([n, n], [indptr, indices]).to(dev)
+    layer = layers.GATLayer(fin, f, h, fused=fused).to(dev)
+    x = torch.randn(n, fin, device=dev, requires_grad=True)
+    y = layer(blk, x)
+    w = torch.randn_like(y)
+    (y * w).sum().backward()
+    got = [y.detach(), x.grad.clone()] + [p.grad.clone() for p in layer.parameters()]
+    x.grad = None
+    layer.zero_grad()
+    adj = convert.to_dense(n, n, [indptr, indices], torch.ones(indices.numel())).to(dev)
+    hv = layer.linear_v(x)
+    q, k = layer.linear_q(hv), layer.linear_k(hv)
+    e = nn.functional.leaky_relu(q[:, None, :] + k[None, :, :], 0.2)
+    e = torch.where(adj[:, :, None] > 0, e, torch.full_like(e, -1e38))
+    a = torch.softmax(e.permute(2, 0, 1), dim=-1) * adj[None]
+    yd = torch.bmm(a, hv.view(n, h, f).transpose(0, 1)).transpose(0, 1).mean(dim=1)
+    (yd * w).sum().backward()
+    want = [yd.detach(), x.grad] + [p.grad for p in layer.parameters()]
+    for a_, b_ in zip(got, want):
+        assert_close(a_, b_, rtol=1e-4, atol=5e-4)
+
+
+def test_hetero_conv_mean_over_relations(dev):
+    torch.manual_seed(2)
+    sizes = {"a": 50, "b": 70}
+    rels = [("a", "r0", "b"), ("b", "r1", "b"), ("b", "r2", "a")]
+    hgraph, norms = {}, {}
+    for i, (s, e, d) in enumerate(rels):
+        ip, ix = random_csr(sizes[d], sizes[s], 0.1, 10 + i)
+        blk = xblock.Block([sizes[d], sizes[s]], [ip, ix]).to(dev)
+        hgraph[(s, e, d)] = blk
+        norms[str((s, e, d))] = layers.right_norm(blk)
+    conv = layers.HeteroGraphConv({e: layers.GCNLayer(12, 8) for _, e, _ in rels}).to(dev)
+    xs = {t: torch.randn(n, 12, device=dev) for t, n in sizes.items()}
+    out = conv(hgraph, xs, norms)
+    b0 = conv.convs["r0"](hgraph[rels[0]], norms[str(rels[0])], (xs["a"], xs["b"]))
+    b1 = conv.convs["r1"](hgraph[rels[1]], norms[str(rels[1])], (xs["b"], xs["b"]))
+    assert_close(out["b"], (b0 + b1) / 2)
+    assert out["a"].shape == (50, 8)
