@@ -30,8 +30,8 @@ int yitu_abi_version(void);
 /* Module 1: YiTu_GNN.YiTu_GNN_kernel  (ccsrc/kernel/YiTu_GNN.cpp:247-258)     */
 /* ------------------------------------------------------------------------- */
 
-/* Scratch for the aggregation / SpMM kernels: queue and partial sums of rows
- * with >= 512 edges. row_len = floats per feature row. */
+/* Scratch for the aggregation / SpMM kernels: queue, band-sort buffers and
+ * partial sums of the rows with >= 64 edges. row_len = floats per feature row. */
 size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len);
 
 /*

@@ -51,7 +51,7 @@ def _aggregate(x, row_pointers, column_index, degrees, alpha):
     ws_bytes = _lib.lib().yitu_spmm_workspace_bytes
     ws_bytes.restype = c_size
     maxdeg = _lib.max_degree(row_pointers)
-    need = ws_bytes(c_i64(nnz), c_i64(dim)) if maxdeg >= 512 else 0
+    need = ws_bytes(c_i64(nnz), c_i64(dim)) if maxdeg >= 64 else 0
     ws = _lib.workspace(need, x.device)
     with torch.cuda.device(x.device):
         rc = fn(ptr(out), ptr(x), c_int(1 if x.dtype == torch.bfloat16 else 0), ptr(row_pointers),

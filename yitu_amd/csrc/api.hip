@@ -32,6 +32,7 @@ YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_
     p.scale_row = degrees;
     p.scale_col = degrees;
     p.n_rows = (int)n_rows;
+    p.n_src = (int)n_src;
     p.L = (int)dim;
     p.F = (int)dim;
     p.H = 1;
@@ -61,6 +62,7 @@ YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *i
     p.out = out;
     p.values = values;
     p.n_rows = (int)n_dst;
+    p.n_src = (int)n_src;
     p.L = (int)(n_heads * n_features);
     p.F = (int)n_features;
     p.H = (int)n_heads;

@@ -309,7 +309,7 @@ static int gat_fwd_launch(GatParams &p, const GatWorkspace &g, bool with_hub, hi
     rp.L = p.L;
     rp.alpha = 1.0f;
     rp.hub = p.hub;
-    spmm_hub_reduce_kernel<W_NONE>
+    spmm_hub_reduce_kernel<W_NONE, 4>
         <<<(int)std::min<int64_t>(p.hub.max_rows, 1024), kBlock, 0, stream>>>(rp);
     YITU_LAUNCH_CHECK();
     return 0;
@@ -383,6 +383,7 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
         p.hub.partial = g.partial;
         p.hub.max_rows = g.max_rows;
         p.hub.max_items = g.max_items;
+        p.hub.chunk = kHubChunk;
         p.rowstat = g.rowstat;
     }
     const int lanes = (int)(L / 4);

@@ -32,6 +32,7 @@ static int sddmm_setup(SddmmParams &p, int64_t nnz, int64_t max_degree, void *wo
     w += 256;
     p.hub.max_rows = (int)sd_max_rows(nnz);
     p.hub.max_items = (int)sd_max_items(nnz);
+    p.hub.chunk = kHubChunk;
     p.hub.rows = reinterpret_cast<int4 *>(w);
     w += align_up(sizeof(int4) * (size_t)p.hub.max_rows, 256);
     p.hub.items = reinterpret_cast<int4 *>(w);
@@ -204,6 +205,7 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
         sp.feat = grad_edge;
         sp.out = grad_key;
         sp.n_rows = (int)n_src;
+        sp.n_src = (int)nnz;
         sp.L = sp.F = (int)n_heads;
         sp.H = 1;
         sp.col_mask = 0x7fffffff;

@@ -201,7 +201,7 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
             nnz >= kHubThreshold && !(max_degree >= 0 && max_degree < kHubThreshold);
         p.hub_threshold = with_hub ? kHubThreshold : 0x7fffffff;
         if (with_hub) {
-            int rc = hub_queue_init(p.hub, workspace, workspace_bytes, nnz, L);
+            int rc = hub512_queue_init(p.hub, workspace, workspace_bytes, nnz);
             if (rc) return rc;
         }
         int rc;
@@ -224,6 +224,7 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
         sp.values = values;
         sp.eperm = t_perm;
         sp.n_rows = (int)n_src;
+        sp.n_src = (int)n_dst;
         sp.L = (int)L;
         sp.F = (int)n_features;
         sp.H = (int)n_heads;

@@ -98,7 +98,7 @@ def spmm_forward(values, indptr, indices, features):
         raise RuntimeError("values must be [n_edges, n_heads]")
     out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 512 else 0
+    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 64 else 0
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_spmm_forward(ptr(out), ptr(values), ptr(indptr), ptr(indices),
@@ -127,7 +127,7 @@ def spmm_backward(values, indptr, indices, features, grad_out):
     tr = transposed(indptr, indices, n_src)
     maxdeg = _lib.max_degree(indptr)
     need = 0
-    if max(maxdeg, tr.max_degree_t) >= 512:
+    if max(maxdeg, tr.max_degree_t) >= 64:
         need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
@@ -156,7 +156,7 @@ def edge_dot(indptr, indices, dst_feat, src_feat):
         raise RuntimeError("dst_feat must be [n_dst, H, F] matching src_feat's H and F")
     out = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 512 else 0
+    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 64 else 0
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_spmm_backward(ptr(out), ptr(None), ptr(None), ptr(indptr), ptr(indices),
@@ -192,7 +192,7 @@ def sddmm_forward(indptr, indices, query, key):
     attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
     need = 0
-    if maxdeg >= 512:
+    if maxdeg >= 64:
         need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
@@ -219,7 +219,7 @@ def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, determini
     tr = transposed(indptr, indices, n_src) if deterministic else None
     grad_edge = torch.empty_like(attn_values) if deterministic else None
     need = 0
-    if maxdeg >= 512 or (tr is not None and tr.max_degree_t >= 512):
+    if maxdeg >= 64 or (tr is not None and tr.max_degree_t >= 64):
         need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
@@ -344,7 +344,7 @@ def gat_forward(indptr, indices, query, key, features):
     out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
     attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f)) if maxdeg >= 512 else 0
+    need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f)) if maxdeg >= 64 else 0
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_gat_forward(ptr(out), ptr(attn), ptr(indptr), ptr(indices), ptr(query),
@@ -371,7 +371,7 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out):
     s2 = torch.empty_like(attn)
     maxdeg = _lib.max_degree(indptr)
     need = 0
-    if max(maxdeg, tr.max_degree_t) >= 512:
+    if max(maxdeg, tr.max_degree_t) >= 64:
         need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
