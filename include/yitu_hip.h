@@ -27,12 +27,36 @@ const char *yitu_last_error(void);
 int yitu_abi_version(void);
 
 /* ------------------------------------------------------------------------- */
+/* Row plan (per graph, built once)                                            */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * The counterpart of the reference's neighbour-group partition build_part
+ * (ccsrc/kernel/YiTu_GNN.cpp:203-245), which its callers compute once per graph
+ * and pass to every op as part_pointers / part2Node: rows with >= 64 edges are
+ * cut into items of 64 edges, listed in ascending order of the source id in the
+ * middle of each item. The gather kernels (aggregation, SpMM, per-edge dot, GAT
+ * aggregate) run one wave per item in that order, which keeps the hot rows of
+ * the feature table in L2. The plan depends on (indptr, indices) only.
+ * Every op that takes `plan_device` also accepts NULL and then builds a
+ * temporary plan in its workspace on each call.
+ * col_mask selects the column bits of indices (0xffffff for packed graph_ext
+ * indices, 0x7fffffff for plain ones).
+ */
+size_t yitu_plan_bytes(int64_t nnz);
+size_t yitu_plan_workspace_bytes(int64_t nnz);
+int yitu_plan_build(void *plan_device, size_t plan_bytes, const int32_t *indptr_device,
+                    const int32_t *indices_device, int64_t n_rows, int64_t n_src, int64_t nnz,
+                    int32_t col_mask, void *workspace_device, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Module 1: YiTu_GNN.YiTu_GNN_kernel  (ccsrc/kernel/YiTu_GNN.cpp:247-258)     */
 /* ------------------------------------------------------------------------- */
 
-/* Scratch for the aggregation / SpMM kernels: queue, band-sort buffers and
- * partial sums of the rows with >= 64 edges. row_len = floats per feature row. */
-size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len);
+/* Scratch for the aggregation / SpMM kernels: partial sums of the rows with
+ * >= 64 edges, plus a temporary row plan when the call is given none
+ * (with_plan = 0). row_len = floats per feature row. */
+size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with_plan);
 
 /*
  * CSR neighbour aggregation, the kernel inside
@@ -48,14 +72,14 @@ size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len);
  * accumulation and out [n_rows, dim] are fp32. Every row of out is written
  * (empty rows get zeros), without atomics: results are bitwise reproducible.
  * The neighbour-group arguments of the reference (part_pointers, part2Node,
- * partSize, dimWorker, warpPerBlock) have no counterpart: the row split is
- * done on the device per call. max_degree: widest row if known, else -1.
+ * partSize, dimWorker, warpPerBlock) are replaced by the row plan (or nothing).
+ * max_degree: widest row if known, else -1.
  */
 int yitu_agg_csr(float *out_device, const void *x_device, int x_is_bf16,
                  const int32_t *row_pointers_device, const int32_t *column_index_device,
                  const float *degrees_device, int64_t n_rows, int64_t n_src, int64_t nnz,
-                 int64_t dim, float alpha, int64_t max_degree, void *workspace_device,
-                 size_t workspace_bytes, void *stream);
+                 int64_t dim, float alpha, int64_t max_degree, const void *plan_device,
+                 void *workspace_device, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Module 2: graph_ext  (YiTu_GNN/YiTu_H/src/entry.cpp:184-193)                */
@@ -65,13 +89,13 @@ int yitu_agg_csr(float *out_device, const void *x_device, int x_is_bf16,
  * spmm_forward (entry.cpp:80-90; spmm_cuda.cu:4-21,44-62):
  *   out[r,h,k] = sum_{i in row r} values[i,h] * features[indices[i] & 0xffffff, h, k]
  * values [nnz,H], features [n_src,H,F], out [n_dst,H,F], all fp32.
- * Workspace: yitu_spmm_workspace_bytes(nnz, H*F).
+ * Workspace: yitu_spmm_workspace_bytes(nnz, H*F, plan != NULL).
  */
 int yitu_spmm_forward(float *out_device, const float *values_device, const int32_t *indptr_device,
                       const int32_t *indices_device, const float *features_device, int64_t n_dst,
                       int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                      int64_t max_degree, void *workspace_device, size_t workspace_bytes,
-                      void *stream);
+                      int64_t max_degree, const void *plan_device, void *workspace_device,
+                      size_t workspace_bytes, void *stream);
 
 /*
  * spmm_backward (entry.cpp:92-104; spmm_cuda.cu:24-42,64-86):
@@ -83,8 +107,9 @@ int yitu_spmm_forward(float *out_device, const float *values_device, const int32
  * the transposed structure (t_* from yitu_csr_transpose, required when grad_x
  * is requested) instead of the reference's 2*E*H*F float atomics; both outputs
  * are fully written and bitwise reproducible. max_degree / max_degree_t: widest
- * row of the CSR / of its transpose if known, else -1.
- * Workspace: yitu_spmm_workspace_bytes(nnz, H*F).
+ * row of the CSR / of its transpose if known, else -1. plan_device /
+ * plan_t_device: row plans of (indptr, indices) and of (t_indptr, t_rows), or NULL.
+ * Workspace: yitu_spmm_workspace_bytes(nnz, H*F, both plans given).
  */
 int yitu_spmm_backward(float *grad_a_device, float *grad_x_device, const float *values_device,
                        const int32_t *indptr_device, const int32_t *indices_device,
@@ -92,8 +117,8 @@ int yitu_spmm_backward(float *grad_a_device, float *grad_x_device, const float *
                        const int32_t *t_indptr_device, const int32_t *t_rows_device,
                        const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
                        int64_t n_heads, int64_t n_features, int64_t max_degree,
-                       int64_t max_degree_t, void *workspace_device, size_t workspace_bytes,
-                       void *stream);
+                       int64_t max_degree_t, const void *plan_device, const void *plan_t_device,
+                       void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
  * sddmm_forward (entry.cpp:106-116; sddmm_cuda.cu:5-33,69-89):
@@ -104,7 +129,7 @@ int yitu_spmm_backward(float *grad_a_device, float *grad_x_device, const float *
  * The softmax subtracts the running maximum; the reference does not
  * (sddmm_cuda.cu:15-21) and overflows for logits above ~88.
  */
-size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid);
+size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid, int with_plan);
 int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
                        const int32_t *indices_device, const float *query_device,
                        const float *key_device, int64_t n_dst, int64_t n_src, int64_t nnz,
@@ -121,6 +146,7 @@ int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
  *   scratch: gv is stored per edge and summed by a gather over the transposed
  *   structure (bitwise reproducible).
  * max_degree / max_degree_t: widest row of the CSR / of its transpose, or -1.
+ * plan_t_device: row plan of the transposed structure (gather form only), or NULL.
  */
 int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float *grad_edge_device,
                         const int32_t *indptr_device, const int32_t *indices_device,
@@ -128,8 +154,8 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
                         const float *attn_device, const float *grad_out_device,
                         const int32_t *t_indptr_device, const int32_t *t_perm_device,
                         int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                        int64_t max_degree, int64_t max_degree_t, void *workspace_device,
-                        size_t workspace_bytes, void *stream);
+                        int64_t max_degree, int64_t max_degree_t, const void *plan_t_device,
+                        void *workspace_device, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Fused GAT attention (composition of the two ops above in one pass)          */
@@ -145,13 +171,14 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
  * probabilities for the backward pass; it may be NULL when the shape takes the
  * fused kernel (n_features % 4 == 0, n_heads <= 64, 16-byte aligned pointers).
  */
-size_t yitu_gat_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_features);
+size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads, int64_t n_features,
+                                int with_plans);
 int yitu_gat_forward(float *out_device, float *attn_device, const int32_t *indptr_device,
                      const int32_t *indices_device, const float *query_device,
                      const float *key_device, const float *features_device, int64_t n_dst,
                      int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                     int64_t max_degree, void *workspace_device, size_t workspace_bytes,
-                     void *stream);
+                     int64_t max_degree, const void *plan_device, void *workspace_device,
+                     size_t workspace_bytes, void *stream);
 
 /*
  * Backward of the composition (spmm_backward then sddmm_backward,
@@ -168,8 +195,8 @@ int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       const int32_t *t_indptr_device, const int32_t *t_rows_device,
                       const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
                       int64_t n_heads, int64_t n_features, int64_t max_degree,
-                      int64_t max_degree_t, void *workspace_device, size_t workspace_bytes,
-                      void *stream);
+                      int64_t max_degree_t, const void *plan_device, const void *plan_t_device,
+                      void *workspace_device, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Dense products on the matrix cores (fp32 MFMA)                              */

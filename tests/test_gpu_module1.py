@@ -31,10 +31,11 @@ def test_sag_all_row_widths(dev, dim):
     assert torch.all(got[0] == 0) and torch.all(got[5] == 0)
 
 
-@pytest.mark.parametrize("hub_degree", [511, 512, 513, 1024, 1025, 3000])
+@pytest.mark.parametrize("hub_degree", [63, 64, 65, 127, 128, 129, 511, 1025, 3000])
 @pytest.mark.parametrize("dim", [64, 128, 36])
-def test_hub_rows_take_the_chunked_path(dev, hub_degree, dim):
-    """Rows with >= 512 edges are summed by the workgroup-per-chunk kernels."""
+def test_long_rows_take_the_planned_item_path(dev, hub_degree, dim):
+    """Rows with >= 64 edges are cut into 64-edge items (one wave each, band order);
+    single-item rows are written directly, the others through partial rows."""
     n = 4096
     indptr, indices = random_csr(n, n, 0.002, hub_degree, hub_rows=(1, 4000, 4095),
                                  hub_degree=hub_degree, empty_rows=(2,))
@@ -99,6 +100,25 @@ def test_bf16_input_fp32_accumulate(dev, dim):
     assert_close(got, want)
 
 
+def test_with_and_without_row_plan_agree_bitwise(dev):
+    """The cached row plan and the temporary one built per call give identical bits."""
+    from yitu_amd import _lib
+    indptr, indices = powerlaw_graph(13, 200000, 8)
+    n = indptr.numel() - 1
+    x = torch.randn(n, 64, generator=torch.Generator().manual_seed(4)).to(dev)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    with_plan = K._aggregate(x, rp, ci, deg, 1.0)
+    out = torch.empty_like(with_plan)
+    ws = _lib.workspace(_lib.size_fn("yitu_spmm_workspace_bytes")(
+        _lib.c_i64(ci.numel()), _lib.c_i64(64), _lib.c_int(0)), dev)
+    rc = _lib.lib().yitu_agg_csr(_lib.ptr(out), _lib.ptr(x), 0, _lib.ptr(rp), _lib.ptr(ci),
+                                 _lib.ptr(deg), _lib.c_i64(n), _lib.c_i64(n), _lib.c_i64(ci.numel()),
+                                 _lib.c_i64(64), _lib.c_f32(1.0), _lib.c_i64(-1), _lib.ptr(None),
+                                 _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
+    _lib.check(rc, "yitu_agg_csr")
+    assert torch.equal(out, with_plan)
+
+
 def test_results_are_bitwise_reproducible(dev):
     indptr, indices = powerlaw_graph(13, 200000, 6)
     n = indptr.numel() - 1
@@ -127,14 +147,15 @@ def test_linearity_and_row_block_invariance_at_scale(dev):
     sub_ci = ci[rp[lo].item():rp[hi].item()].contiguous()
     out = torch.empty(hi - lo, 128, device=dev)
     from yitu_amd import _lib
-    ws = _lib.workspace(_lib.lib().yitu_spmm_workspace_bytes(_lib.c_i64(sub_ci.numel()),
-                                                             _lib.c_i64(128)), dev)
+    # no row plan is passed: the call builds a temporary one in its workspace
+    ws = _lib.workspace(_lib.size_fn("yitu_spmm_workspace_bytes")(
+        _lib.c_i64(sub_ci.numel()), _lib.c_i64(128), _lib.c_int(0)), dev)
     y_unscaled = K._aggregate(x1, rp, ci, None, 1.0)
     rc = _lib.lib().yitu_agg_csr(_lib.ptr(out), _lib.ptr(x1), 0, _lib.ptr(sub_rp), _lib.ptr(sub_ci),
                                  _lib.ptr(None), _lib.c_i64(hi - lo), _lib.c_i64(n),
                                  _lib.c_i64(sub_ci.numel()), _lib.c_i64(128), _lib.c_f32(1.0),
-                                 _lib.c_i64(-1), _lib.ptr(ws), _lib.c_size(ws.numel()),
-                                 _lib.stream_ptr(dev))
+                                 _lib.c_i64(-1), _lib.ptr(None), _lib.ptr(ws),
+                                 _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
     _lib.check(rc, "yitu_agg_csr")
     assert torch.equal(out, y_unscaled[lo:hi])
 

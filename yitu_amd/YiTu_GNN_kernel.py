@@ -5,7 +5,8 @@ return arity, backed by the gfx950 kernels of libyitu_hip.so.
 Differences from the reference that callers can observe:
   * the neighbour-group arguments (part_pointers, part2Node, partSize,
     dimWorker, warpPerBlock) are accepted and validated for device/contiguity
-    like the others but do not steer the kernels: rows are split on the device;
+    like the others but do not steer the kernels: their role is played by a row
+    plan that is built on the device on first use of a graph and cached;
   * outputs live on the input's device (the reference allocates ``forward``'s
     output on the default CUDA device, YiTu_GNN_kernel.cu:278);
   * failures raise ``RuntimeError`` instead of ``exit(-1)`` (cu:309-314);
@@ -47,17 +48,17 @@ def _aggregate(x, row_pointers, column_index, degrees, alpha):
     if degrees is not None and degrees.numel() < max(n_rows, n_src):
         raise RuntimeError("degrees is shorter than the number of nodes")
     out = torch.empty((n_rows, dim), dtype=torch.float32, device=x.device)
-    fn = _lib.lib().yitu_agg_csr
-    ws_bytes = _lib.lib().yitu_spmm_workspace_bytes
-    ws_bytes.restype = c_size
     maxdeg = _lib.max_degree(row_pointers)
-    need = ws_bytes(c_i64(nnz), c_i64(dim)) if maxdeg >= 64 else 0
+    plan = _lib.row_plan(row_pointers, column_index, n_src, 0x7FFFFFFF)
+    need = _lib.size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(dim), c_int(1)) \
+        if plan is not None else 0
     ws = _lib.workspace(need, x.device)
     with torch.cuda.device(x.device):
-        rc = fn(ptr(out), ptr(x), c_int(1 if x.dtype == torch.bfloat16 else 0), ptr(row_pointers),
-                ptr(column_index), ptr(degrees), c_i64(n_rows), c_i64(n_src), c_i64(nnz),
-                c_i64(dim), c_f32(alpha), c_i64(maxdeg), ptr(ws), c_size(ws.numel()),
-                stream_ptr(x.device))
+        rc = _lib.lib().yitu_agg_csr(
+            ptr(out), ptr(x), c_int(1 if x.dtype == torch.bfloat16 else 0), ptr(row_pointers),
+            ptr(column_index), ptr(degrees), c_i64(n_rows), c_i64(n_src), c_i64(nnz), c_i64(dim),
+            c_f32(alpha), c_i64(maxdeg), ptr(plan), ptr(ws), c_size(ws.numel()),
+            stream_ptr(x.device))
     check(rc, "yitu_agg_csr")
     return out
 

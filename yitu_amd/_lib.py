@@ -7,6 +7,7 @@ device the call raises.
 import ctypes
 import os
 import threading
+import weakref
 
 import torch
 
@@ -106,3 +107,41 @@ def max_degree(indptr):
             _max_degree.clear()
         _max_degree[key] = v
     return v
+
+
+# Row plans (band-ordered items of the long rows) are a function of the graph
+# only: built on the device on first use and kept while the index tensor lives.
+_plans = {}
+
+
+def row_plan(indptr, indices, n_src, col_mask):
+    """Device buffer holding the row plan of (indptr, indices), or None when no
+    row reaches the planning threshold."""
+    if max_degree(indptr) < 64:
+        return None
+    key = (id(indices), indices.data_ptr(), indices._version, indptr.data_ptr(), int(n_src),
+           int(col_mask))
+    hit = _plans.get(key)
+    if hit is not None:
+        return hit
+    L = lib()
+    L.yitu_plan_bytes.restype = c_size
+    L.yitu_plan_workspace_bytes.restype = c_size
+    dev = indices.device
+    nnz = indices.numel()
+    plan = torch.empty(int(L.yitu_plan_bytes(c_i64(nnz))), dtype=torch.uint8, device=dev)
+    ws = workspace(L.yitu_plan_workspace_bytes(c_i64(nnz)), dev)
+    with torch.cuda.device(dev):
+        rc = L.yitu_plan_build(ptr(plan), c_size(plan.numel()), ptr(indptr), ptr(indices),
+                               c_i64(indptr.numel() - 1), c_i64(n_src), c_i64(nnz), c_int(col_mask),
+                               ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_plan_build")
+    _plans[key] = plan
+    weakref.finalize(indices, _plans.pop, key, None)
+    return plan
+
+
+def size_fn(name):
+    fn = getattr(lib(), name)
+    fn.restype = c_size
+    return fn

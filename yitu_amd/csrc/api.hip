@@ -10,15 +10,15 @@ using namespace yitu;
 YITU_API const char *yitu_last_error(void) { return last_error(); }
 YITU_API int yitu_abi_version(void) { return 1; }
 
-YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len) {
-    return hub_workspace_bytes(nnz, row_len);
+YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with_plan) {
+    return spmm_workspace_bytes(nnz, row_len, with_plan != 0);
 }
 
 YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_t *row_pointers,
                           const int32_t *column_index, const float *degrees, int64_t n_rows,
                           int64_t n_src, int64_t nnz, int64_t dim, float alpha,
-                          int64_t max_degree, void *workspace, size_t workspace_bytes,
-                          void *stream) {
+                          int64_t max_degree, const void *plan, void *workspace,
+                          size_t workspace_bytes, void *stream) {
     YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0 && dim >= 0, "negative size");
     if (n_rows == 0 || dim == 0) return 0;
     YITU_REQUIRE(out && row_pointers, "null output or row_pointers");
@@ -38,16 +38,15 @@ YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_
     p.H = 1;
     p.col_mask = 0x7fffffff;
     p.alpha = alpha;
-    p.xcd_remap = 0;
-    return launch_spmm(p, degrees ? W_DEGPROD : W_NONE, x_is_bf16 != 0, nnz, max_degree, workspace,
-                       workspace_bytes, static_cast<hipStream_t>(stream));
+    return launch_spmm(p, degrees ? W_DEGPROD : W_NONE, x_is_bf16 != 0, nnz, max_degree, plan,
+                       workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *indptr,
                                const int32_t *indices, const float *features, int64_t n_dst,
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                               int64_t max_degree, void *workspace, size_t workspace_bytes,
-                               void *stream) {
+                               int64_t max_degree, const void *plan, void *workspace,
+                               size_t workspace_bytes, void *stream) {
     YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
                  "negative size");
     if (n_dst == 0 || n_heads * n_features == 0) return 0;
@@ -68,6 +67,7 @@ YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *i
     p.H = (int)n_heads;
     p.col_mask = 0xffffff;
     p.alpha = 1.0f;
-    return launch_spmm(p, W_EDGEHEAD, false, nnz, max_degree, workspace, workspace_bytes,
+    return launch_spmm(p, W_EDGEHEAD, false, nnz, max_degree, plan, workspace, workspace_bytes,
                        static_cast<hipStream_t>(stream));
 }
+

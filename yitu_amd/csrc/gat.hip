@@ -11,27 +11,22 @@
 //            computed exactly once in the (edge, head) lane layout, stored to
 //            attn (one contiguous run), then broadcast lane-to-lane to the
 //            (slot, column) layout that gathers x[col] tiles and accumulates.
-// Hub rows: chunk statistics and their per-row combine reuse the SDDMM kernels,
-// a chunk-apply kernel writes attn and per-chunk partial rows, the SpMM reduce
-// kernel adds those in chunk order.
+// Rows of 64 or more edges take the row plan's band-ordered 64-edge items:
+// item statistics, per-row merge, item apply (attn + partial rows), and the SpMM
+// reduce kernel, which adds a row's partials in a fixed order.
 #include "../../include/yitu_hip.h"
 #include "sddmm_kernels.hpp"
 
 namespace yitu {
 
 struct GatParams {
-    const int32_t *indptr;
-    const int32_t *indices;
+    SpmmParams sp;       // indptr, indices, feat = x [n_src, L], out, n_rows, L, F, H, plan, partial
     const float *query;  // [n_dst, H]
     const float *key;    // [n_src, H]
-    const float *feat;   // [n_src, L]
-    float *out;          // [n_dst, L]
     float *attn;         // [nnz, H] or null
-    int n_dst, L, F, H;
     int HP;              // heads rounded up to a power of two (<= 64)
-    int hub_threshold;
-    HubQueue hub;          // hub.partial: per-item partial rows [item][L]
-    const float *rowstat;  // [hub row][H][3]: max, 1/sum
+    float *item_stats;   // [plan item id][H][2]: (max, sum) of the item's logits
+    float *row_stats;    // [n_dst][H][2]: (max, 1/sum) of the planned rows
 };
 
 // (max, sum) over the lanes that share lane % hp, hp a runtime power of two
@@ -43,51 +38,47 @@ __device__ __forceinline__ MaxSum ms_wave_rt(MaxSum a, int hp) {
     return a;
 }
 
-__device__ __forceinline__ MaxSum gat_stats(const GatParams &p, int e_beg, int e_end, float qv) {
+// Softmax statistics of the n edges in window lanes [first, first + n) for this
+// lane's head (lane % HP), in the (edge, head) lane layout.
+__device__ __forceinline__ MaxSum gat_stats_window(const GatParams &p, const EdgeWindow &win,
+                                                   int first, int n, float qv) {
     const int lane = lane_id();
     const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int H = p.sp.H;
     MaxSum a = ms_init();
-    if (hl < p.H) {
-        for (int e = e_beg + esub; e < e_end; e += eps) {
-            const int col = p.indices[e] & kColMask;
-            a = ms_push(a, leaky(qv + p.key[(size_t)col * p.H + hl]));
-        }
+    for (int k0 = 0; k0 < n; k0 += eps) {
+        const int k = k0 + esub;
+        const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+        if (k < n && hl < H) a = ms_push(a, leaky(qv + p.key[(size_t)col * H + hl]));
     }
     return a;
 }
 
-// Phase B over edges [e_beg, e_end): writes attn and accumulates the weighted
-// feature tiles of column block c0. m / inv are this lane's head statistics in
-// the (edge, head) layout (lane % HP = head).
+// Phase B for the n edges in window lanes [first, first + n) (CSR edges e0 ...):
+// every (edge, head) probability is computed once in the (edge, head) layout,
+// stored to attn, then broadcast to the (slot, column) layout that gathers the
+// x[col] tiles. m / inv are this lane's head statistics (lane % HP = head).
 template <int VEC, int G, int KT>
-__device__ __forceinline__ void gat_accumulate(float (&acc)[KT][VEC], const GatParams &p,
-                                               int e_beg, int e_end, int c0, float qv, float m,
-                                               float inv, bool write_attn) {
+__device__ __forceinline__ void gat_apply_window(float (&acc)[KT][VEC], const GatParams &p,
+                                                 const TileLanes<VEC, G, KT, W_EDGEHEAD> &tl,
+                                                 const EdgeWindow &win, int first, int n, int e0,
+                                                 float qv, float m, float inv, bool write_attn) {
     constexpr int SLOTS = kWave / G;
     constexpr int UNROLL = KT >= 4 ? 2 : 4;
     const int lane = lane_id();
-    const int slot = lane / G, sub = lane % G;
+    const int slot = lane / G;
     const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
-    const float *__restrict__ feat = p.feat;
+    const int H = p.sp.H, L = p.sp.L;
+    const float *__restrict__ feat = static_cast<const float *>(p.sp.feat);
 
-    int off[KT], head[KT];
-    bool live[KT];
-#pragma unroll
-    for (int t = 0; t < KT; t++) {
-        off[t] = c0 + (t * G + sub) * VEC;
-        live[t] = off[t] < p.L;
-        if (!live[t]) off[t] = 0;
-        head[t] = off[t] / p.F;
-    }
-
-    for (int e0 = e_beg; e0 < e_end; e0 += eps) {
-        const int nb = min(eps, e_end - e0);
-        const int e = e0 + esub;
-        const int col = p.indices[min(e, e_end - 1)] & kColMask;
+    for (int k0 = 0; k0 < n; k0 += eps) {
+        const int nb = min(eps, n - k0);
+        const int k = k0 + esub;
+        const int col = __shfl(win.col, first + min(k, n - 1), kWave);
         float pv = 0.0f;
-        if (e < e_end && hl < p.H) {
-            pv = expf(leaky(qv + p.key[(size_t)col * p.H + hl]) - m) * inv;
-            if (write_attn) p.attn[(size_t)e * p.H + hl] = pv;
+        if (k < n && hl < H) {
+            pv = expf(leaky(qv + p.key[(size_t)col * H + hl]) - m) * inv;
+            if (write_attn) p.attn[(size_t)(e0 + k) * H + hl] = pv;
         }
         for (int j0 = 0; j0 < nb; j0 += SLOTS * UNROLL) {
             float v[UNROLL][KT][VEC];
@@ -96,18 +87,17 @@ __device__ __forceinline__ void gat_accumulate(float (&acc)[KT][VEC], const GatP
             for (int u = 0; u < UNROLL; u++) {
                 const int ej = j0 + u * SLOTS + slot;
                 const bool valid = ej < nb;
-                const int src = valid ? ej * p.HP : 0;  // lane holding edge ej (head 0)
+                const int src = valid ? ej * p.HP : 0;  // lane holding edge ej, head 0
                 const int c = __shfl(col, src, kWave);
 #pragma unroll
                 for (int t = 0; t < KT; t++) {
-                    const float wt = __shfl(pv, src + head[t], kWave);
-                    w[u][t] = (valid && live[t]) ? wt : 0.0f;
+                    const float wt = __shfl(pv, src + tl.head[t], kWave);
+                    w[u][t] = (valid && tl.live[t]) ? wt : 0.0f;
                 }
-                // steps wholly past the sub-batch load nothing (wave-uniform test)
-                if (j0 + u * SLOTS < nb) {
+                if (j0 + u * SLOTS < nb) {  // wave-uniform: steps past the sub-batch load nothing
 #pragma unroll
                     for (int t = 0; t < KT; t++)
-                        RowLoad<VEC, float>::ld(feat + (size_t)c * p.L + off[t], v[u][t]);
+                        RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
                 } else {
 #pragma unroll
                     for (int t = 0; t < KT; t++)
@@ -125,93 +115,174 @@ __device__ __forceinline__ void gat_accumulate(float (&acc)[KT][VEC], const GatP
     }
 }
 
+// Short rows, fully fused: a wave walks kRowsPerWave rows; per row statistics,
+// then probabilities + aggregate, all from the sliding edge window.
 template <int VEC, int G, int KT>
-__global__ __launch_bounds__(kBlock) void gat_fwd_rows_kernel(GatParams p) {
+__global__ __launch_bounds__(kBlock) void gat_rows_kernel(GatParams p) {
     const int lane = lane_id();
-    const int row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-    if (row >= p.n_dst) return;
-    const int beg = p.indptr[row], end = p.indptr[row + 1];
-    const int deg = end - beg;
-    if (deg >= p.hub_threshold) {
-        queue_hub_row(p.hub, row, deg);
-        return;
-    }
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
     const int sub = lane % G, slot = lane / G;
     const int hl = lane & (p.HP - 1);
-    float qv = 0.0f, m = 0.0f, inv = 0.0f;
-    if (deg > 0) {
-        qv = hl < p.H ? p.query[(size_t)row * p.H + hl] : 0.0f;
-        MaxSum a = ms_wave_rt(gat_stats(p, beg, end, qv), p.HP);
-        m = a.m;
-        inv = 1.0f / a.s;
-    }
-    for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
-        float acc[KT][VEC];
-#pragma unroll
-        for (int t = 0; t < KT; t++)
-#pragma unroll
-            for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
+    const int H = p.sp.H, L = p.sp.L;
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int row = r0 + i;
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int deg = end - beg;
+        if (deg >= p.sp.plan.threshold) continue;
+        float qv = 0.0f, m = 0.0f, inv = 0.0f;
         if (deg > 0) {
-            gat_accumulate<VEC, G, KT>(acc, p, beg, end, c0, qv, m, inv, p.attn && c0 == 0);
-            fold_slots<VEC, G, KT>(acc);
+            qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
+            MaxSum a = ms_init();
+            for (int b = beg; b < end; b += kWave) {
+                const int n = min(kWave, end - b);
+                if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                    load_window<W_NONE>(win, p.sp, b, limit);
+                a = ms_merge(a, gat_stats_window(p, win, b - win.base, n, qv));
+            }
+            a = ms_wave_rt(a, p.HP);
+            m = a.m;
+            inv = 1.0f / a.s;
         }
-        if (slot == 0) {
+        for (int c0 = 0; c0 < L; c0 += G * VEC * KT) {
+            const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+            float acc[KT][VEC];
 #pragma unroll
-            for (int t = 0; t < KT; t++) {
-                const int o = c0 + (t * G + sub) * VEC;
-                if (o < p.L) store_row<VEC>(p.out + (size_t)row * p.L + o, acc[t]);
+            for (int t = 0; t < KT; t++)
+#pragma unroll
+                for (int k = 0; k < VEC; k++) acc[t][k] = 0.0f;
+            for (int b = beg; b < end; b += kWave) {
+                const int n = min(kWave, end - b);
+                if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                    load_window<W_NONE>(win, p.sp, b, limit);
+                gat_apply_window<VEC, G, KT>(acc, p, tl, win, b - win.base, n, b, qv, m, inv,
+                                             p.attn && c0 == 0);
+            }
+            if (deg > 0) fold_slots<VEC, G, KT>(acc);
+            if (slot == 0) {
+#pragma unroll
+                for (int t = 0; t < KT; t++) {
+                    const int o = c0 + (t * G + sub) * VEC;
+                    if (o < L) store_row<VEC>(p.sp.out + (size_t)row * L + o, acc[t]);
+                }
             }
         }
     }
 }
 
-template <int VEC, int G, int KT>
-__global__ __launch_bounds__(kBlock) void gat_fwd_hub_apply_kernel(GatParams p) {
-    __shared__ float red[kWavesPerBlock][G * VEC * KT];
-    if (p.hub.counters->overflow) return;
-    const int n_items = min(p.hub.counters->n_items, p.hub.max_items);
-    const int lane = lane_id(), wave = threadIdx.x / kWave;
-    const int sub = lane % G, slot = lane / G;
+// Long rows, step 1: (max, sum) of every plan item.
+__global__ __launch_bounds__(kBlock) void gat_item_stats_kernel(GatParams p) {
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
-    constexpr int kPerWave = kHubChunk / kWavesPerBlock;
-    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
-        const int4 it = p.hub.items[item];
-        const int row = it.x;
-        const int beg = p.indptr[row] + it.y * kHubChunk;
-        const int end = min(p.indptr[row + 1], beg + kHubChunk);
-        const int wbeg = min(end, beg + wave * kPerWave), wend = min(end, wbeg + kPerWave);
-        float qv = 0.0f, m = 0.0f, inv = 0.0f;
-        if (hl < p.H) {
-            qv = p.query[(size_t)row * p.H + hl];
-            const float *rs = p.rowstat + ((size_t)it.z * p.H + hl) * 3;
-            m = rs[0];
-            inv = rs[1];
-        }
-        for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
-            float acc[KT][VEC];
+    const int H = p.sp.H;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
 #pragma unroll
-            for (int t = 0; t < KT; t++)
-#pragma unroll
-                for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
-            if (wend > wbeg) {
-                gat_accumulate<VEC, G, KT>(acc, p, wbeg, wend, c0, qv, m, inv, p.attn && c0 == 0);
-                fold_slots<VEC, G, KT>(acc);
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (j >= n_here) break;
+            const int beg = __shfl(my_rec.x, j, kWave), end = __shfl(my_rec.y, j, kWave);
+            const int item = __shfl(my_rec.z, j, kWave);
+            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            EdgeWindow win;
+            load_window<W_NONE>(win, p.sp, beg, end);
+            const float qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
+            MaxSum a = ms_wave_rt(gat_stats_window(p, win, 0, end - beg, qv), p.HP);
+            if (lane < p.HP && lane < H) {
+                p.item_stats[((size_t)item * H + lane) * 2] = a.m;
+                p.item_stats[((size_t)item * H + lane) * 2 + 1] = a.s;
             }
-            __syncthreads();
-            if (slot == 0) {
+        }
+    }
+}
+
+// Step 2: merge the item statistics of every planned row in item order.
+__global__ __launch_bounds__(kBlock) void gat_row_combine_kernel(GatParams p) {
+    if (p.sp.plan.counters->overflow) return;
+    const int n_rows = min(p.sp.plan.counters->n_rows, p.sp.plan.max_rows);
+    const int H = p.sp.H;
+    const int64_t total = (int64_t)n_rows * H;
+    for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < total;
+         t += (int64_t)gridDim.x * kBlock) {
+        const int4 r = p.sp.plan.rows[t / H];
+        const int h = (int)(t % H);
+        MaxSum a = ms_init();
+        for (int c = 0; c < r.z; c++) {
+            const float *st = p.item_stats + ((size_t)(r.y + c) * H + h) * 2;
+            a = ms_merge(a, MaxSum{st[0], st[1]});
+        }
+        p.row_stats[((size_t)r.x * H + h) * 2] = a.m;
+        p.row_stats[((size_t)r.x * H + h) * 2 + 1] = 1.0f / a.s;
+    }
+}
+
+// Step 3: probabilities and weighted aggregate of every item, in band order.
+template <int VEC, int G, int KT>
+__global__ __launch_bounds__(kBlock) void gat_item_apply_kernel(GatParams p) {
+    const int lane = lane_id();
+    const int sub = lane % G, slot = lane / G;
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int hl = lane & (p.HP - 1);
+    const int H = p.sp.H, L = p.sp.L;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int e_beg[kItemsPerWave], n_edges[kItemsPerWave], item_id[kItemsPerWave],
+            row_tag[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            e_beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            item_id[j] = __shfl(my_rec.z, j, kWave);
+            row_tag[j] = __shfl(my_rec.w, j, kWave);
+            n_edges[j] = j < n_here ? end - e_beg[j] : 0;
+            if (n_edges[j] > 0) load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;
+            const bool single = row_tag[j] < 0;
+            const int row = row_tag[j] & 0x7fffffff;
+            float qv = 0.0f, m = 0.0f, inv = 0.0f;
+            if (hl < H) {
+                qv = p.query[(size_t)row * H + hl];
+                m = p.row_stats[((size_t)row * H + hl) * 2];
+                inv = p.row_stats[((size_t)row * H + hl) * 2 + 1];
+            }
+            float *dst = single ? p.sp.out + (size_t)row * L
+                                : p.sp.partial + (size_t)item_id[j] * L;
+            for (int c0 = 0; c0 < L; c0 += G * VEC * KT) {
+                const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+                float acc[KT][VEC];
 #pragma unroll
                 for (int t = 0; t < KT; t++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) red[wave][(t * G + sub) * VEC + i] = acc[t][i];
-            }
-            __syncthreads();
-            for (int e = threadIdx.x; e < G * VEC * KT; e += kBlock) {
-                const int o = c0 + e;
-                if (o < p.L) {
-                    float s = red[0][e];
+                    for (int k = 0; k < VEC; k++) acc[t][k] = 0.0f;
+                gat_apply_window<VEC, G, KT>(acc, p, tl, win[j], 0, n_edges[j], e_beg[j], qv, m,
+                                             inv, p.attn && c0 == 0);
+                fold_slots<VEC, G, KT>(acc);
+                if (slot == 0) {
 #pragma unroll
-                    for (int w = 1; w < kWavesPerBlock; w++) s += red[w][e];
-                    p.hub.partial[(size_t)item * p.L + o] = s;
+                    for (int t = 0; t < KT; t++) {
+                        const int o = c0 + (t * G + sub) * VEC;
+                        if (o < L) store_row<VEC>(dst + o, acc[t]);
+                    }
                 }
             }
         }
@@ -219,98 +290,32 @@ __global__ __launch_bounds__(kBlock) void gat_fwd_hub_apply_kernel(GatParams p) 
 }
 
 // ---- host side ----------------------------------------------------------------
-static inline int64_t gat_max_rows(int64_t nnz) { return nnz / kHubThreshold + 1; }
-static inline int64_t gat_max_items(int64_t nnz) { return nnz / kHubChunk + gat_max_rows(nnz) + 1; }
-
-struct GatWorkspace {
-    HubCounters *counters;
-    int4 *rows, *items;
-    float *stats;    // [item][H][3]
-    float *rowstat;  // [hub row][H][3]
-    float *partial;  // [item][L]
-    int max_rows, max_items;
-};
-
-static size_t gat_ws_bytes(int64_t nnz, int64_t H, int64_t L) {
-    size_t b = 256;
-    b += 2 * align_up(sizeof(int4) * (size_t)gat_max_items(nnz), 256);
-    b += align_up(sizeof(float) * 3 * (size_t)(gat_max_items(nnz) * H), 256);
-    b += align_up(sizeof(float) * 3 * (size_t)(gat_max_rows(nnz) * H), 256);
-    b += align_up(sizeof(float) * (size_t)(gat_max_items(nnz) * L), 256);
-    return b;
-}
-
-static void gat_ws_carve(GatWorkspace &g, void *workspace, int64_t nnz, int64_t H, int64_t L) {
-    char *w = static_cast<char *>(workspace);
-    g.max_rows = (int)gat_max_rows(nnz);
-    g.max_items = (int)gat_max_items(nnz);
-    g.counters = reinterpret_cast<HubCounters *>(w);
-    w += 256;
-    g.rows = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)g.max_items, 256);
-    g.items = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)g.max_items, 256);
-    g.stats = reinterpret_cast<float *>(w);
-    w += align_up(sizeof(float) * 3 * (size_t)g.max_items * H, 256);
-    g.rowstat = reinterpret_cast<float *>(w);
-    w += align_up(sizeof(float) * 3 * (size_t)g.max_rows * H, 256);
-    g.partial = reinterpret_cast<float *>(w);
-}
-
-template <int HP>
-static int gat_hub_stats_launch(const SddmmParams &sp, hipStream_t stream) {
-    sddmm_fwd_hub_stats_kernel<HP>
-        <<<(int)std::min<int64_t>(sp.hub.max_items, 4096), kBlock, 0, stream>>>(sp);
-    YITU_LAUNCH_CHECK();
-    sddmm_fwd_hub_combine_kernel<<<(int)std::min<int64_t>(sp.hub.max_rows, 512), kBlock, 0,
-                                   stream>>>(sp);
-    YITU_LAUNCH_CHECK();
-    return 0;
+// workspace beyond the plan: item statistics, row statistics, partial rows
+static size_t gat_own_bytes(int64_t n_dst, int64_t nnz, int64_t H, int64_t L) {
+    return align_up(sizeof(float) * 2 * (size_t)(plan_max_items(nnz) * H), 256) +
+           align_up(sizeof(float) * 2 * (size_t)(n_dst * H), 256) +
+           align_up(sizeof(float) * (size_t)(plan_max_items(nnz) * L), 256);
 }
 
 template <int VEC, int G, int KT>
-static int gat_fwd_launch(GatParams &p, const GatWorkspace &g, bool with_hub, hipStream_t stream) {
-    if (with_hub) {
-        zero_hub_counters_kernel<<<1, kWave, 0, stream>>>(g.counters);
-        YITU_LAUNCH_CHECK();
-    }
-    gat_fwd_rows_kernel<VEC, G, KT>
-        <<<(int)ceil_div(p.n_dst, kWavesPerBlock), kBlock, 0, stream>>>(p);
+static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
+    gat_rows_kernel<VEC, G, KT>
+        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    if (!with_hub) return 0;
-    // chunk statistics + per-row combine: the SDDMM hub kernels on the same queue
-    SddmmParams sp{};
-    sp.indptr = p.indptr;
-    sp.indices = p.indices;
-    sp.query = p.query;
-    sp.key = p.key;
-    sp.n_dst = p.n_dst;
-    sp.H = p.H;
-    sp.n_bid = 1;
-    sp.hub = p.hub;
-    sp.hub.partial = g.stats;
-    sp.rowstat = g.rowstat;
-    int rc;
-    switch (p.HP) {
-        case 1: rc = gat_hub_stats_launch<1>(sp, stream); break;
-        case 2: rc = gat_hub_stats_launch<2>(sp, stream); break;
-        case 4: rc = gat_hub_stats_launch<4>(sp, stream); break;
-        case 8: rc = gat_hub_stats_launch<8>(sp, stream); break;
-        case 16: rc = gat_hub_stats_launch<16>(sp, stream); break;
-        case 32: rc = gat_hub_stats_launch<32>(sp, stream); break;
-        default: rc = gat_hub_stats_launch<64>(sp, stream); break;
-    }
-    if (rc) return rc;
-    gat_fwd_hub_apply_kernel<VEC, G, KT>
-        <<<(int)std::min<int64_t>(p.hub.max_items, 4096), kBlock, 0, stream>>>(p);
+    if (!has_items) return 0;
+    const int item_grid = (int)std::min<int64_t>(
+        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+    gat_item_stats_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    SpmmParams rp{};
-    rp.out = p.out;
-    rp.L = p.L;
-    rp.alpha = 1.0f;
-    rp.hub = p.hub;
-    spmm_hub_reduce_kernel<W_NONE, 4>
-        <<<(int)std::min<int64_t>(p.hub.max_rows, 1024), kBlock, 0, stream>>>(rp);
+    gat_row_combine_kernel<<<(int)std::min<int64_t>(
+                                 ceil_div((int64_t)p.sp.plan.max_rows * p.sp.H, kBlock), 4096),
+                             kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    gat_item_apply_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    p.sp.alpha = 1.0f;
+    spmm_reduce_kernel<W_NONE, 4>
+        <<<(int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16), kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
     return 0;
 }
@@ -320,19 +325,21 @@ static int gat_fwd_launch(GatParams &p, const GatWorkspace &g, bool with_hub, hi
 using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
-YITU_API size_t yitu_gat_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_features) {
+YITU_API size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads,
+                                         int64_t n_features, int with_plans) {
     const int64_t L = n_heads * n_features;
-    size_t b = gat_ws_bytes(nnz, n_heads, L);
-    b = std::max(b, (size_t)yitu_spmm_workspace_bytes(nnz, L));
-    b = std::max(b, (size_t)yitu_sddmm_workspace_bytes(nnz, n_heads, 1));
-    return b;
+    size_t b = gat_own_bytes(n_dst, nnz, n_heads, L) + (with_plans ? 0 : plan_temp_bytes(nnz));
+    b = std::max(b, (size_t)yitu_spmm_workspace_bytes(nnz, L, with_plans));
+    b = std::max(b, (size_t)yitu_sddmm_workspace_bytes(nnz, n_heads, 1, with_plans));
+    return b + 256;
 }
 
 YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
                               const int32_t *indices, const float *query, const float *key,
                               const float *features, int64_t n_dst, int64_t n_src, int64_t nnz,
                               int64_t n_heads, int64_t n_features, int64_t max_degree,
-                              void *workspace, size_t workspace_bytes, void *stream_) {
+                              const void *plan, void *workspace, size_t workspace_bytes,
+                              void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
                  "negative size");
@@ -351,47 +358,48 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
                                     1, max_degree, workspace, workspace_bytes, stream_);
         if (rc) return rc;
         return yitu_spmm_forward(out, attn, indptr, indices, features, n_dst, n_src, nnz, n_heads,
-                                 n_features, max_degree, workspace, workspace_bytes, stream_);
+                                 n_features, max_degree, plan, workspace, workspace_bytes,
+                                 stream_);
     }
     GatParams p{};
-    p.indptr = indptr;
-    p.indices = indices;
+    p.sp.indptr = indptr;
+    p.sp.indices = indices;
+    p.sp.feat = features;
+    p.sp.out = out;
+    p.sp.n_rows = (int)n_dst;
+    p.sp.n_src = (int)n_src;
+    p.sp.L = (int)L;
+    p.sp.F = (int)n_features;
+    p.sp.H = (int)n_heads;
+    p.sp.col_mask = kColMask;
+    p.sp.alpha = 1.0f;
     p.query = query;
     p.key = key;
-    p.feat = features;
-    p.out = out;
     p.attn = attn;
-    p.n_dst = (int)n_dst;
-    p.L = (int)L;
-    p.F = (int)n_features;
-    p.H = (int)n_heads;
     p.HP = 1;
-    while (p.HP < p.H) p.HP <<= 1;
-    const bool with_hub = nnz >= kHubThreshold && !(max_degree >= 0 && max_degree < kHubThreshold);
-    p.hub_threshold = with_hub ? kHubThreshold : 0x7fffffff;
-    GatWorkspace g{};
-    if (with_hub) {
-        const size_t need = gat_ws_bytes(nnz, n_heads, L);
-        YITU_REQUIRE(workspace && workspace_bytes >= need, "workspace too small: need %zu bytes",
-                     need);
-        YITU_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
-                     "workspace must be 256-byte aligned");
-        gat_ws_carve(g, workspace, nnz, n_heads, L);
-        p.hub.counters = g.counters;
-        p.hub.rows = g.rows;
-        p.hub.items = g.items;
-        p.hub.partial = g.partial;
-        p.hub.max_rows = g.max_rows;
-        p.hub.max_items = g.max_items;
-        p.hub.chunk = kHubChunk;
-        p.rowstat = g.rowstat;
+    while (p.HP < p.sp.H) p.HP <<= 1;
+    bool has_items = false;
+    void *rest = nullptr;
+    size_t rest_bytes = 0;
+    int rc = plan_resolve(p.sp.plan, has_items, plan, indptr, indices, n_dst, n_src, nnz, kColMask,
+                          max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
+    if (rc) return rc;
+    if (has_items) {
+        const size_t need = gat_own_bytes(n_dst, nnz, n_heads, L);
+        YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes", need);
+        char *w = static_cast<char *>(rest);
+        p.item_stats = reinterpret_cast<float *>(w);
+        w += align_up(sizeof(float) * 2 * (size_t)(plan_max_items(nnz) * n_heads), 256);
+        p.row_stats = reinterpret_cast<float *>(w);
+        w += align_up(sizeof(float) * 2 * (size_t)(n_dst * n_heads), 256);
+        p.sp.partial = reinterpret_cast<float *>(w);
     }
     const int lanes = (int)(L / 4);
-    if (lanes <= 16) return gat_fwd_launch<4, 16, 1>(p, g, with_hub, stream);
-    if (lanes <= 32) return gat_fwd_launch<4, 32, 1>(p, g, with_hub, stream);
-    if (lanes <= 64) return gat_fwd_launch<4, 64, 1>(p, g, with_hub, stream);
-    if (lanes <= 128) return gat_fwd_launch<4, 64, 2>(p, g, with_hub, stream);
-    return gat_fwd_launch<4, 64, 4>(p, g, with_hub, stream);
+    if (lanes <= 16) return gat_fwd_launch<4, 16, 1>(p, has_items, stream);
+    if (lanes <= 32) return gat_fwd_launch<4, 32, 1>(p, has_items, stream);
+    if (lanes <= 64) return gat_fwd_launch<4, 64, 1>(p, has_items, stream);
+    if (lanes <= 128) return gat_fwd_launch<4, 64, 2>(p, has_items, stream);
+    return gat_fwd_launch<4, 64, 4>(p, has_items, stream);
 }
 
 YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_features,
@@ -401,8 +409,9 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                                const float *grad_out, const int32_t *t_indptr,
                                const int32_t *t_rows, const int32_t *t_perm, int64_t n_dst,
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                               int64_t max_degree, int64_t max_degree_t, void *workspace,
-                               size_t workspace_bytes, void *stream) {
+                               int64_t max_degree, int64_t max_degree_t, const void *plan,
+                               const void *plan_t, void *workspace, size_t workspace_bytes,
+                               void *stream) {
     YITU_REQUIRE(grad_query && grad_key && grad_features, "null output");
     YITU_REQUIRE(nnz == 0 || (grad_attn_scratch && grad_edge_scratch),
                  "gat_backward needs two [nnz, H] scratch buffers");
@@ -412,12 +421,12 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
     // gather of grad_out over the transposed structure
     int rc = yitu_spmm_backward(grad_attn_scratch, grad_features, attn, indptr, indices, features,
                                 grad_out, t_indptr, t_rows, t_perm, n_dst, n_src, nnz, n_heads,
-                                n_features, max_degree, max_degree_t, workspace, workspace_bytes,
-                                stream);
+                                n_features, max_degree, max_degree_t, plan, plan_t, workspace,
+                                workspace_bytes, stream);
     if (rc) return rc;
     // softmax + LeakyReLU backward; grad_key gathered over the transposed structure
     return yitu_sddmm_backward(grad_query, grad_key, grad_edge_scratch, indptr, indices, query,
                                key, attn, grad_attn_scratch, t_indptr, t_perm, n_dst, n_src, nnz,
-                               n_heads, 1, max_degree, max_degree_t, workspace, workspace_bytes,
-                               stream);
+                               n_heads, 1, max_degree, max_degree_t, plan_t, workspace,
+                               workspace_bytes, stream);
 }

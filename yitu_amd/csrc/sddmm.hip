@@ -114,9 +114,11 @@ static int sddmm_bwd_dispatch(const SddmmParams &p, bool with_hub, hipStream_t s
 using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
-YITU_API size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid) {
-    // the backward's gather pass reuses the buffer as an SpMM hub queue
-    return std::max(sddmm_ws_bytes(nnz, n_heads, n_bid), hub_workspace_bytes(nnz, n_heads));
+YITU_API size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid,
+                                           int with_plan) {
+    // the backward's gather pass reuses the buffer as SpMM workspace
+    return std::max(sddmm_ws_bytes(nnz, n_heads, n_bid),
+                    spmm_workspace_bytes(nnz, n_heads, with_plan != 0));
 }
 
 static int sddmm_check(const int32_t *indptr, const int32_t *indices, const float *query,
@@ -161,8 +163,8 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
                                  const float *key, const float *attn, const float *grad_out,
                                  const int32_t *t_indptr, const int32_t *t_perm, int64_t n_dst,
                                  int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                 int64_t max_degree, int64_t max_degree_t, void *workspace,
-                                 size_t workspace_bytes, void *stream_) {
+                                 int64_t max_degree, int64_t max_degree_t, const void *plan_t,
+                                 void *workspace, size_t workspace_bytes, void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
@@ -210,7 +212,9 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
         sp.H = 1;
         sp.col_mask = 0x7fffffff;
         sp.alpha = 1.0f;
-        return launch_spmm(sp, W_NONE, false, nnz, max_degree_t, workspace, workspace_bytes, stream);
+        // the plan of the transposed structure fits: same row bounds, other columns
+        return launch_spmm(sp, W_NONE, false, nnz, max_degree_t, plan_t, workspace,
+                           workspace_bytes, stream);
     }
     return 0;
 }

@@ -1,10 +1,4 @@
 // Instantiation table and host-side launch logic of the row-split SpMM.
-#include <hip/hip_runtime.h>
-
-#include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
-
 #include "spmm_rows.hpp"
 
 #include <cstdarg>
@@ -35,69 +29,10 @@ int fill_zero(float *p, int64_t n, hipStream_t stream) {
     return 0;
 }
 
-// A queued row has >= threshold edges and yields ceil(deg / chunk) items, so
-// rows <= nnz / threshold and items <= nnz / chunk + rows.
-static inline int64_t hub_max_rows(int64_t nnz) { return nnz / kAggThreshold + 1; }
-static inline int64_t hub_max_items(int64_t nnz) { return nnz / kAggChunk + hub_max_rows(nnz) + 1; }
-
-static size_t sort_temp_bytes(int64_t n) {
-    size_t bytes = 0;
-    uint32_t *k = nullptr;
-    int32_t *v = nullptr;
-    (void)rocprim::radix_sort_pairs(nullptr, bytes, k, k, v, v, (size_t)n, 0, 16);
-    return bytes;
-}
-
-size_t hub_workspace_bytes(int64_t nnz, int64_t L) {
-    const size_t items = (size_t)hub_max_items(nnz);
-    size_t b = 256;  // counters
-    b += align_up(sizeof(int4) * (size_t)hub_max_rows(nnz), 256);
-    b += align_up(sizeof(int4) * items, 256);
-    b += 4 * align_up(sizeof(int32_t) * items, 256);  // sort keys / values, in and out
-    b += align_up(sizeof(int4) * items, 256);         // band-ordered item records
-    b += align_up(sort_temp_bytes((int64_t)items), 256);
-    b += align_up(sizeof(float) * items * (size_t)L, 256);
-    return b;
-}
-
-struct HubSortBuffers {
-    uint32_t *keys_in, *keys_out;
-    int32_t *vals_in;
-    int4 *records;
-    void *temp;
-    size_t temp_bytes;
-};
-
-static int hub_queue_init(HubQueue &q, HubSortBuffers &sb, void *workspace, size_t workspace_bytes,
-                          int64_t nnz, int64_t L) {
-    YITU_REQUIRE(workspace != nullptr && workspace_bytes >= hub_workspace_bytes(nnz, L),
-                 "workspace too small: need %zu bytes, got %zu", hub_workspace_bytes(nnz, L),
-                 workspace_bytes);
-    YITU_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
-                 "workspace must be 256-byte aligned");
-    char *w = static_cast<char *>(workspace);
-    q.counters = reinterpret_cast<HubCounters *>(w);
-    w += 256;
-    q.max_rows = (int)hub_max_rows(nnz);
-    q.max_items = (int)hub_max_items(nnz);
-    q.chunk = kAggChunk;
-    q.rows = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)q.max_rows, 256);
-    q.items = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)q.max_items, 256);
-    const size_t arr = align_up(sizeof(int32_t) * (size_t)q.max_items, 256);
-    sb.keys_in = reinterpret_cast<uint32_t *>(w);
-    sb.keys_out = reinterpret_cast<uint32_t *>(w + arr);
-    sb.vals_in = reinterpret_cast<int32_t *>(w + 2 * arr);
-    q.order = reinterpret_cast<int32_t *>(w + 3 * arr);
-    w += 4 * arr;
-    sb.records = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)q.max_items, 256);
-    sb.temp = w;
-    sb.temp_bytes = sort_temp_bytes(q.max_items);
-    w += align_up(sb.temp_bytes, 256);
-    q.partial = reinterpret_cast<float *>(w);
-    return 0;
+size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan) {
+    size_t b = align_up(sizeof(float) * (size_t)plan_max_items(nnz) * (size_t)L, 256);
+    if (!with_plan) b += plan_temp_bytes(nnz);
+    return b + 256;
 }
 
 // Queue of (row, 512-edge chunk) items without partial rows, for kernels whose
@@ -124,103 +59,86 @@ int hub512_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int6
 }
 
 template <int VEC, int G, int KT, int WMODE, typename TIN>
-static int launch_variant(const SpmmParams &p, const HubSortBuffers &sb, bool with_hub,
-                          hipStream_t stream) {
+static int launch_variant(const SpmmParams &p, bool has_items, hipStream_t stream) {
     const int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave);
-    if (with_hub) {
-        zero_hub_counters_kernel<<<1, kWave, 0, stream>>>(p.hub.counters);
-        YITU_LAUNCH_CHECK();
-    }
     spmm_rows_kernel<VEC, G, KT, WMODE, TIN><<<grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    if (with_hub) {
-        // order the items by the band of the feature table they read
-        int bits = 1;
-        while (((int64_t)1 << bits) < p.n_src) bits++;
-        spmm_hub_keys_kernel<<<(int)ceil_div(p.hub.max_items, kBlock), kBlock, 0, stream>>>(
-            p, sb.keys_in, sb.vals_in, std::max(0, bits - 16));
+    if (has_items) {
+        const int item_grid = (int)std::min<int64_t>(
+            ceil_div(p.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+        spmm_items_kernel<VEC, G, KT, WMODE, TIN><<<item_grid, kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
-        size_t temp_bytes = sb.temp_bytes;
-        YITU_HIP(rocprim::radix_sort_pairs(sb.temp, temp_bytes, sb.keys_in, sb.keys_out, sb.vals_in,
-                                           p.hub.order, (size_t)p.hub.max_items, 0, 16, stream));
-        spmm_hub_records_kernel<<<(int)ceil_div(p.hub.max_items, kBlock), kBlock, 0, stream>>>(
-            p, sb.records);
-        YITU_LAUNCH_CHECK();
-        const int hub_grid = (int)std::min<int64_t>(
-            ceil_div(p.hub.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
-        spmm_hub_items_kernel<VEC, G, KT, WMODE, TIN>
-            <<<hub_grid, kBlock, 0, stream>>>(p, sb.records);
-        YITU_LAUNCH_CHECK();
-        const int red_grid = (int)std::min<int64_t>(p.hub.max_rows, 1 << 16);
+        const int red_grid = (int)std::min<int64_t>(p.plan.max_rows, 1 << 16);
         constexpr int RV = VEC >= 4 ? 4 : VEC;  // VEC | L whenever this variant is chosen
         if (p.L % RV == 0)
-            spmm_hub_reduce_kernel<WMODE, RV><<<red_grid, kBlock, 0, stream>>>(p);
+            spmm_reduce_kernel<WMODE, RV><<<red_grid, kBlock, 0, stream>>>(p);
         else
-            spmm_hub_reduce_kernel<WMODE, 1><<<red_grid, kBlock, 0, stream>>>(p);
+            spmm_reduce_kernel<WMODE, 1><<<red_grid, kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
     }
     return 0;
 }
 
 template <int WMODE, typename TIN, int VEC>
-static int dispatch_shape(const SpmmParams &p, const HubSortBuffers &sb, bool with_hub,
-                          hipStream_t stream) {
+static int dispatch_shape(const SpmmParams &p, bool with_hub, hipStream_t stream) {
     const int lanes = (p.L + VEC - 1) / VEC;
     if constexpr (VEC >= 4) {
-        if (lanes <= 16) return launch_variant<VEC, 16, 1, WMODE, TIN>(p, sb, with_hub, stream);
-        if (lanes <= 32) return launch_variant<VEC, 32, 1, WMODE, TIN>(p, sb, with_hub, stream);
-        if (lanes <= 64) return launch_variant<VEC, 64, 1, WMODE, TIN>(p, sb, with_hub, stream);
-        if (lanes <= 128) return launch_variant<VEC, 64, 2, WMODE, TIN>(p, sb, with_hub, stream);
-        if constexpr (VEC == 4) return launch_variant<VEC, 64, 4, WMODE, TIN>(p, sb, with_hub, stream);
-        return launch_variant<VEC, 64, 2, WMODE, TIN>(p, sb, with_hub, stream);
+        if (lanes <= 16) return launch_variant<VEC, 16, 1, WMODE, TIN>(p, with_hub, stream);
+        if (lanes <= 32) return launch_variant<VEC, 32, 1, WMODE, TIN>(p, with_hub, stream);
+        if (lanes <= 64) return launch_variant<VEC, 64, 1, WMODE, TIN>(p, with_hub, stream);
+        if (lanes <= 128) return launch_variant<VEC, 64, 2, WMODE, TIN>(p, with_hub, stream);
+        if constexpr (VEC == 4) return launch_variant<VEC, 64, 4, WMODE, TIN>(p, with_hub, stream);
+        return launch_variant<VEC, 64, 2, WMODE, TIN>(p, with_hub, stream);
     } else {
-        if (lanes <= 64) return launch_variant<VEC, 64, 1, WMODE, TIN>(p, sb, with_hub, stream);
-        return launch_variant<VEC, 64, 4, WMODE, TIN>(p, sb, with_hub, stream);
+        if (lanes <= 64) return launch_variant<VEC, 64, 1, WMODE, TIN>(p, with_hub, stream);
+        return launch_variant<VEC, 64, 4, WMODE, TIN>(p, with_hub, stream);
     }
 }
 
 template <int WMODE>
-static int dispatch_type(const SpmmParams &p, const HubSortBuffers &sb, bool bf16_in,
-                         bool with_hub, hipStream_t stream) {
+static int dispatch_type(const SpmmParams &p, bool bf16_in, bool with_hub, hipStream_t stream) {
     // a lane's VEC elements must stay inside one head and one aligned vector
     const int unit = WMODE == W_EDGEHEAD ? p.F : p.L;
     if constexpr (WMODE != W_EDGEHEAD) {
       if (bf16_in) {
         if (unit % 8 == 0 && aligned16(p.feat) && aligned16(p.out))
-            return dispatch_shape<WMODE, bf16_t, 8>(p, sb, with_hub, stream);
-        return dispatch_shape<WMODE, bf16_t, 1>(p, sb, with_hub, stream);
+            return dispatch_shape<WMODE, bf16_t, 8>(p, with_hub, stream);
+        return dispatch_shape<WMODE, bf16_t, 1>(p, with_hub, stream);
       }
     }
     if (unit % 4 == 0 && aligned16(p.feat) && aligned16(p.out))
-        return dispatch_shape<WMODE, float, 4>(p, sb, with_hub, stream);
+        return dispatch_shape<WMODE, float, 4>(p, with_hub, stream);
     if (unit % 2 == 0 && aligned16(p.feat) && aligned16(p.out))
-        return dispatch_shape<WMODE, float, 2>(p, sb, with_hub, stream);
-    return dispatch_shape<WMODE, float, 1>(p, sb, with_hub, stream);
+        return dispatch_shape<WMODE, float, 2>(p, with_hub, stream);
+    return dispatch_shape<WMODE, float, 1>(p, with_hub, stream);
 }
 
 int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max_degree_hint,
-                void *workspace, size_t workspace_bytes, hipStream_t stream) {
+                const void *plan, void *workspace, size_t workspace_bytes, hipStream_t stream) {
     if (p.n_rows == 0 || p.L == 0) return 0;
     YITU_REQUIRE(nnz < (int64_t)1 << 31 && (int64_t)p.n_rows * p.L < ((int64_t)1 << 40),
                  "problem exceeds the int32 edge-index range");
-    // No row can reach the hub threshold when the whole graph (or its widest
-    // row, if the caller knows it) is smaller: skip the queue and its kernels.
-    bool with_hub = nnz >= kAggThreshold;
-    if (max_degree_hint >= 0 && max_degree_hint < kAggThreshold) with_hub = false;
-    p.hub_threshold = with_hub ? kAggThreshold : 0x7fffffff;
-    HubSortBuffers sb{};
+    bool with_hub = false;
+    void *rest = nullptr;
+    size_t rest_bytes = 0;
+    int rc = plan_resolve(p.plan, with_hub, plan, p.indptr, p.indices, p.n_rows, p.n_src, nnz,
+                          p.col_mask, max_degree_hint, workspace, workspace_bytes, &rest,
+                          &rest_bytes, stream);
+    if (rc) return rc;
+    p.partial = nullptr;
     if (with_hub) {
-        int rc = hub_queue_init(p.hub, sb, workspace, workspace_bytes, nnz, p.L);
-        if (rc) return rc;
-    } else {
-        p.hub = HubQueue{};
+        const size_t need = sizeof(float) * (size_t)p.plan.max_items * (size_t)p.L;
+        YITU_REQUIRE(rest && rest_bytes >= need,
+                     "workspace too small for the partial rows: need %zu more bytes, got %zu", need,
+                     rest_bytes);
+        p.partial = static_cast<float *>(rest);
     }
     switch (wmode) {
-        case W_NONE: return dispatch_type<W_NONE>(p, sb, bf16_in, with_hub, stream);
-        case W_DEGPROD: return dispatch_type<W_DEGPROD>(p, sb, bf16_in, with_hub, stream);
+        case W_NONE: return dispatch_type<W_NONE>(p, bf16_in, with_hub, stream);
+        case W_DEGPROD: return dispatch_type<W_DEGPROD>(p, bf16_in, with_hub, stream);
         case W_EDGEHEAD:
             YITU_REQUIRE(!bf16_in, "edge-weighted SpMM takes fp32 features");
-            return dispatch_type<W_EDGEHEAD>(p, sb, false, with_hub, stream);
+            return dispatch_type<W_EDGEHEAD>(p, false, with_hub, stream);
     }
     set_error("unknown weight mode %d", wmode);
     return -1;

@@ -10,87 +10,79 @@
 namespace yitu {
 
 struct DotParams {
-    const int32_t *indptr;
-    const int32_t *indices;
-    const float *feat;      // [n_src, L]
+    SpmmParams sp;          // indptr, indices, feat, n_rows, L, F, H, col_mask, plan
     const float *grad_out;  // [n_dst, L]
     float *grad_a;          // [nnz, H]
-    int n_rows, L, F, H;
-    int lph;       // lanes per head (F / VEC) when that is a power of two <= G, else 0
-    int hub_threshold;
-    HubQueue hub;  // only the row/item lists are used
+    int lph;  // lanes per head (F / VEC) when that is a power of two <= G, else 0
 };
 
-// Dot products for edges [e_beg, e_end) of `row`; gt holds the row's grad_out tile.
-template <int VEC, int G, int KT>
-__device__ __forceinline__ void dot_edges(const DotParams &p, int row, int e_beg, int e_end) {
+// Dot products of the row's grad_out tile `gt` with the n edges in window lanes
+// [first, first + n); edge k of them is CSR edge e0 + k.
+template <int VEC, int G, int KT, int UNROLL = (KT >= 4 ? 2 : 4)>
+__device__ __forceinline__ void dot_window(const DotParams &p, const float (&gt)[KT][VEC],
+                                           const TileLanes<VEC, G, KT, W_EDGEHEAD> &tl,
+                                           const EdgeWindow &win, int first, int n, int e0,
+                                           int c0) {
     constexpr int SLOTS = kWave / G;
     const int lane = lane_id();
     const int slot = lane / G, sub = lane % G;
-    const float *__restrict__ feat = p.feat;
+    const float *__restrict__ feat = static_cast<const float *>(p.sp.feat);
+    const int L = p.sp.L, F = p.sp.F, H = p.sp.H;
+    // heads present in this column tile, for the generic reduction
+    const int h_lo = c0 / F;
+    const int h_hi = min(H - 1, (min(L, c0 + G * VEC * KT) - 1) / F);
 
-    for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
-        int off[KT], head[KT];
-        bool live[KT];
-        float gt[KT][VEC];
+    for (int s0 = 0; s0 < n; s0 += SLOTS * UNROLL) {
+        float v[UNROLL][KT][VEC];
+        // all gathers of the group first
 #pragma unroll
-        for (int t = 0; t < KT; t++) {
-            off[t] = c0 + (t * G + sub) * VEC;
-            live[t] = off[t] < p.L;
-            if (!live[t]) off[t] = 0;
-            head[t] = off[t] / p.F;
-            RowLoad<VEC, float>::ld(p.grad_out + (size_t)row * p.L + off[t], gt[t]);
-            if (!live[t])
+        for (int u = 0; u < UNROLL; u++) {
+            const int k = min(s0 + u * SLOTS + slot, n - 1);
+            const int c = __shfl(win.col, first + k, kWave);
+            if (s0 + u * SLOTS < n) {  // wave-uniform
 #pragma unroll
-                for (int i = 0; i < VEC; i++) gt[t][i] = 0.0f;
+                for (int t = 0; t < KT; t++)
+                    RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+            }
         }
-        // first head of this column tile, used by the generic reduction
-        const int h_lo = c0 / p.F;
-        const int h_hi = min(p.H - 1, (min(p.L, c0 + G * VEC * KT) - 1) / p.F);
-
-        for (int base = e_beg; base < e_end; base += kWave) {
-            const int n = min(kWave, e_end - base);
-            const int my_col = p.indices[base + min(lane, n - 1)] & 0xffffff;
-            for (int s = 0; s < n; s += SLOTS) {
-                const int src = s + slot;
-                const bool valid = src < n;
-                const int c = __shfl(my_col, src, kWave);
-                float part[KT];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            if (s0 + u * SLOTS >= n) break;  // wave-uniform
+            const int k = s0 + u * SLOTS + slot;
+            const bool valid = k < n;
+            const size_t e = (size_t)(e0 + min(k, n - 1));
+            float part[KT];
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                float d = 0.0f;
+#pragma unroll
+                for (int i = 0; i < VEC; i++) d += gt[t][i] * v[u][t][i];
+                part[t] = d;
+            }
+            if (p.lph > 0) {
+                // a head is lph consecutive lanes of one tile
 #pragma unroll
                 for (int t = 0; t < KT; t++) {
-                    float v[VEC];
-                    RowLoad<VEC, float>::ld(feat + (size_t)c * p.L + off[t], v);
+                    float d = part[t];
+                    for (int o = p.lph >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                    if (valid && tl.live[t] && (sub & (p.lph - 1)) == 0)
+                        p.grad_a[e * H + tl.head[t]] = d;
+                }
+            } else {
+                // generic shapes: one masked reduction per head present in the tile
+                for (int h = h_lo; h <= h_hi; h++) {
                     float d = 0.0f;
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) d += gt[t][i] * v[i];
-                    part[t] = d;
-                }
-                const size_t e = (size_t)(base + src);
-                if (p.lph > 0 && p.lph <= G) {
-                    // a head is lph consecutive lanes of one tile
-#pragma unroll
-                    for (int t = 0; t < KT; t++) {
-                        float d = part[t];
-                        for (int o = p.lph >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
-                        if (valid && live[t] && (sub & (p.lph - 1)) == 0)
-                            p.grad_a[e * p.H + head[t]] = d;
-                    }
-                } else {
-                    // generic shapes: one masked reduction per head present in the tile
-                    for (int h = h_lo; h <= h_hi; h++) {
-                        float d = 0.0f;
-#pragma unroll
-                        for (int t = 0; t < KT; t++)
-                            if (live[t] && head[t] == h) d += part[t];
-                        d = group_sum<G>(d);
-                        if (valid && sub == 0) {
-                            float *dst = p.grad_a + e * p.H + h;
-                            // a head that started in an earlier column pass keeps its partial
-                            if (h * p.F < c0)
-                                *dst += d;
-                            else
-                                *dst = d;
-                        }
+                    for (int t = 0; t < KT; t++)
+                        if (tl.live[t] && tl.head[t] == h) d += part[t];
+                    d = group_sum<G>(d);
+                    if (valid && sub == 0) {
+                        float *dst = p.grad_a + e * H + h;
+                        // a head that started in an earlier column pass keeps its partial
+                        if (h * F < c0)
+                            *dst += d;
+                        else
+                            *dst = d;
                     }
                 }
             }
@@ -99,64 +91,111 @@ __device__ __forceinline__ void dot_edges(const DotParams &p, int row, int e_beg
 }
 
 template <int VEC, int G, int KT>
-__global__ __launch_bounds__(kBlock) void spmm_bwd_dot_rows_kernel(DotParams p) {
-    const int row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-    if (row >= p.n_rows) return;
-    const int beg = p.indptr[row], end = p.indptr[row + 1];
-    if (end == beg) return;
-    if (end - beg >= p.hub_threshold) {
-        queue_hub_row(p.hub, row, end - beg);
-        return;
-    }
-    dot_edges<VEC, G, KT>(p, row, beg, end);
-}
-
-template <int VEC, int G, int KT>
-__global__ __launch_bounds__(kBlock) void spmm_bwd_dot_hub_kernel(DotParams p) {
-    if (p.hub.counters->overflow) return;
-    const int n_items = min(p.hub.counters->n_items, p.hub.max_items);
-    const int wave = threadIdx.x / kWave;
-    constexpr int kPerWave = kHubChunk / kWavesPerBlock;
-    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
-        const int4 it = p.hub.items[item];
-        const int beg = p.indptr[it.x] + it.y * kHubChunk;
-        const int end = min(p.indptr[it.x + 1], beg + kHubChunk);
-        const int wbeg = min(end, beg + wave * kPerWave), wend = min(end, wbeg + kPerWave);
-        if (wend > wbeg) dot_edges<VEC, G, KT>(p, it.x, wbeg, wend);
+__device__ __forceinline__ void load_grad_tile(float (&gt)[KT][VEC], const DotParams &p,
+                                               const TileLanes<VEC, G, KT, W_EDGEHEAD> &tl,
+                                               int row) {
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        RowLoad<VEC, float>::ld(p.grad_out + (size_t)row * p.sp.L + tl.off[t], gt[t]);
+        if (!tl.live[t])
+#pragma unroll
+            for (int i = 0; i < VEC; i++) gt[t][i] = 0.0f;
     }
 }
 
+// Short rows: a wave walks kRowsPerWave consecutive rows through a sliding edge window.
 template <int VEC, int G, int KT>
-static int dot_launch(const DotParams &p, bool with_hub, hipStream_t stream) {
-    if (with_hub) {
-        zero_hub_counters_kernel<<<1, kWave, 0, stream>>>(p.hub.counters);
-        YITU_LAUNCH_CHECK();
+__global__ __launch_bounds__(kBlock) void dot_rows_kernel(DotParams p) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        if (end == beg || end - beg >= p.sp.plan.threshold) continue;
+        for (int c0 = 0; c0 < p.sp.L; c0 += G * VEC * KT) {
+            const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+            float gt[KT][VEC];
+            load_grad_tile<VEC, G, KT>(gt, p, tl, r0 + i);
+            for (int b = beg; b < end; b += kWave) {
+                const int n = min(kWave, end - b);
+                if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                    load_window<W_NONE>(win, p.sp, b, limit);
+                dot_window<VEC, G, KT>(p, gt, tl, win, b - win.base, n, b, c0);
+            }
+        }
     }
-    spmm_bwd_dot_rows_kernel<VEC, G, KT>
-        <<<(int)ceil_div(p.n_rows, kWavesPerBlock), kBlock, 0, stream>>>(p);
+}
+
+// Long rows: the plan's band-ordered items, kItemsPerWave per wave.
+template <int VEC, int G, int KT>
+__global__ __launch_bounds__(kBlock) void dot_items_kernel(DotParams p) {
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int e_beg[kItemsPerWave], n_edges[kItemsPerWave], row[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            e_beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            row[j] = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            n_edges[j] = j < n_here ? end - e_beg[j] : 0;
+            if (n_edges[j] > 0) load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;
+            for (int c0 = 0; c0 < p.sp.L; c0 += G * VEC * KT) {
+                const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+                float gt[KT][VEC];
+                load_grad_tile<VEC, G, KT>(gt, p, tl, row[j]);
+                dot_window<VEC, G, KT>(p, gt, tl, win[j], 0, n_edges[j], e_beg[j], c0);
+            }
+        }
+    }
+}
+
+template <int VEC, int G, int KT>
+static int dot_launch(const DotParams &p, bool has_items, hipStream_t stream) {
+    dot_rows_kernel<VEC, G, KT>
+        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    if (with_hub) {
-        spmm_bwd_dot_hub_kernel<VEC, G, KT>
-            <<<(int)std::min<int64_t>(p.hub.max_items, 4096), kBlock, 0, stream>>>(p);
+    if (has_items) {
+        const int grid = (int)std::min<int64_t>(
+            ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+        dot_items_kernel<VEC, G, KT><<<grid, kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
     }
     return 0;
 }
 
 template <int VEC>
-static int dot_dispatch(DotParams &p, bool with_hub, hipStream_t stream) {
-    const int lanes = (p.L + VEC - 1) / VEC;
-    const int lph = p.F % VEC == 0 ? p.F / VEC : 0;
+static int dot_dispatch(DotParams &p, bool has_items, hipStream_t stream) {
+    const int lanes = (p.sp.L + VEC - 1) / VEC;
+    const int lph = p.sp.F % VEC == 0 ? p.sp.F / VEC : 0;
     p.lph = (lph > 0 && lph <= 64 && (lph & (lph - 1)) == 0) ? lph : 0;
     if constexpr (VEC == 4) {
-        if (lanes <= 16) return dot_launch<4, 16, 1>(p, with_hub, stream);
-        if (lanes <= 32) return dot_launch<4, 32, 1>(p, with_hub, stream);
-        if (lanes <= 64) return dot_launch<4, 64, 1>(p, with_hub, stream);
-        if (lanes <= 128) return dot_launch<4, 64, 2>(p, with_hub, stream);
-        return dot_launch<4, 64, 4>(p, with_hub, stream);
+        if (lanes <= 16) return dot_launch<4, 16, 1>(p, has_items, stream);
+        if (lanes <= 32) return dot_launch<4, 32, 1>(p, has_items, stream);
+        if (lanes <= 64) return dot_launch<4, 64, 1>(p, has_items, stream);
+        if (lanes <= 128) return dot_launch<4, 64, 2>(p, has_items, stream);
+        return dot_launch<4, 64, 4>(p, has_items, stream);
     } else {
-        if (lanes <= 64) return dot_launch<VEC, 64, 1>(p, with_hub, stream);
-        return dot_launch<VEC, 64, 4>(p, with_hub, stream);
+        if (lanes <= 64) return dot_launch<VEC, 64, 1>(p, has_items, stream);
+        return dot_launch<VEC, 64, 4>(p, has_items, stream);
     }
 }
 
@@ -171,8 +210,8 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
                                 const int32_t *t_indptr, const int32_t *t_rows,
                                 const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
                                 int64_t n_heads, int64_t n_features, int64_t max_degree,
-                                int64_t max_degree_t, void *workspace, size_t workspace_bytes,
-                                void *stream_) {
+                                int64_t max_degree_t, const void *plan, const void *plan_t,
+                                void *workspace, size_t workspace_bytes, void *stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
                  "negative size");
@@ -188,30 +227,31 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
 
     if (grad_a && nnz > 0 && n_dst > 0) {
         DotParams p{};
-        p.indptr = indptr;
-        p.indices = indices;
-        p.feat = features;
+        p.sp.indptr = indptr;
+        p.sp.indices = indices;
+        p.sp.feat = features;
+        p.sp.n_rows = (int)n_dst;
+        p.sp.n_src = (int)n_src;
+        p.sp.L = (int)L;
+        p.sp.F = (int)n_features;
+        p.sp.H = (int)n_heads;
+        p.sp.col_mask = 0xffffff;
         p.grad_out = grad_out;
         p.grad_a = grad_a;
-        p.n_rows = (int)n_dst;
-        p.L = (int)L;
-        p.F = (int)n_features;
-        p.H = (int)n_heads;
-        const bool with_hub =
-            nnz >= kHubThreshold && !(max_degree >= 0 && max_degree < kHubThreshold);
-        p.hub_threshold = with_hub ? kHubThreshold : 0x7fffffff;
-        if (with_hub) {
-            int rc = hub512_queue_init(p.hub, workspace, workspace_bytes, nnz);
-            if (rc) return rc;
-        }
-        int rc;
+        bool has_items = false;
+        void *rest = nullptr;
+        size_t rest_bytes = 0;
+        int rc = plan_resolve(p.sp.plan, has_items, plan, indptr, indices, n_dst, n_src, nnz,
+                              0xffffff, max_degree, workspace, workspace_bytes, &rest, &rest_bytes,
+                              stream);
+        if (rc) return rc;
         const bool al = aligned16(features) && aligned16(grad_out);
         if (n_features % 4 == 0 && al)
-            rc = dot_dispatch<4>(p, with_hub, stream);
+            rc = dot_dispatch<4>(p, has_items, stream);
         else if (n_features % 2 == 0 && al)
-            rc = dot_dispatch<2>(p, with_hub, stream);
+            rc = dot_dispatch<2>(p, has_items, stream);
         else
-            rc = dot_dispatch<1>(p, with_hub, stream);
+            rc = dot_dispatch<1>(p, has_items, stream);
         if (rc) return rc;
     }
     if (grad_x && n_src > 0) {
@@ -230,8 +270,8 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
         sp.H = (int)n_heads;
         sp.col_mask = 0x7fffffff;
         sp.alpha = 1.0f;
-        return launch_spmm(sp, W_EDGEHEAD, false, nnz, max_degree_t, workspace, workspace_bytes,
-                           stream);
+        return launch_spmm(sp, W_EDGEHEAD, false, nnz, max_degree_t, plan_t, workspace,
+                           workspace_bytes, stream);
     }
     return 0;
 }

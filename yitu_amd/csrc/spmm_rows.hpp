@@ -16,6 +16,7 @@
 //     combined in chunk order by a third kernel.
 #pragma once
 #include "common.hpp"
+#include "plan.hpp"
 
 namespace yitu {
 
@@ -27,12 +28,6 @@ enum WeightMode : int {
 
 constexpr int kHubChunk = 512;      // edges per hub work item (SDDMM / GAT / dot kernels)
 constexpr int kHubThreshold = 512;  // rows with >= this many edges go to the hub path there
-// The SpMM splits much finer: rows with >= 64 edges become items of 64 edges
-// (one wave each) that are processed in ascending order of their median source
-// id, so that at any moment the whole chip gathers from one narrow band of the
-// feature table and the hot sources of that band stay in every XCD's L2.
-constexpr int kAggChunk = 64;
-constexpr int kAggThreshold = 64;
 
 struct HubCounters {
     int n_items;
@@ -46,7 +41,6 @@ struct HubQueue {
     int4 *rows;             // {row, first_item, n_chunks, 0}
     int4 *items;            // {row, chunk, index into rows[], 0}
     float *partial;         // [n_items, L]
-    int32_t *order;         // SpMM: item ids sorted by median source id
     int max_rows;
     int max_items;
     int chunk;              // edges per item
@@ -68,9 +62,9 @@ struct SpmmParams {
     int H;
     int col_mask;
     float alpha;   // output scale
-    int hub_threshold;
     int xcd_remap;
-    HubQueue hub;
+    PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
+    float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
 };
 
 // Appends a hub row and its ceil(deg / kHubChunk) chunk items to the queue.
@@ -234,90 +228,20 @@ constexpr int kRowsPerWave = 16;  // consecutive rows handled by one wave of the
 // Row kernel: a wave walks kRowsPerWave consecutive rows. Their bounds come from
 // one coalesced indptr load, their edges from a sliding 64-edge window, so a
 // short row costs one round of feature gathers and nothing else that waits on
-// memory. Rows at or above the hub threshold are queued instead.
+// memory. Rows that the plan covers are skipped.
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
-    __shared__ int wave_rows[kWavesPerBlock], wave_items[kWavesPerBlock];
-    __shared__ int block_first_row, block_first_item;
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
     int blk = blockIdx.x;
     if (p.xcd_remap) blk = xcd_contiguous_block(blk, gridDim.x);
     const int r0 = (blk * kWavesPerBlock + wave) * kRowsPerWave;
-    const int n_here = max(0, min(kRowsPerWave, p.n_rows - r0));
-    const int my_ptr = n_here > 0 ? p.indptr[r0 + min(lane, n_here)] : 0;
+    if (r0 >= p.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.n_rows - r0);
+    const int my_ptr = p.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);  // end of this wave's edges
     const int sub = lane % G;
     const int slot = lane / G;
-
-    // ---- queue this workgroup's hub rows with ONE atomic --------------------
-    // (hundreds of thousands of same-address atomics would serialise in L2)
-    const int my_deg = __shfl_down(my_ptr, 1, kWave) - my_ptr;  // lane i: degree of row r0 + i
-    const bool my_hub = lane < n_here && my_deg >= p.hub_threshold;
-    const int my_chunks = my_hub ? (my_deg + p.hub.chunk - 1) / p.hub.chunk : 0;
-    if (p.hub.counters != nullptr) {  // block-uniform: the queue exists
-        // exclusive prefix sums over the (at most 16) row lanes
-        int pre_rows = my_hub ? 1 : 0, pre_items = my_chunks;
-#pragma unroll
-        for (int o = 1; o < kRowsPerWave; o <<= 1) {
-            const int a = __shfl_up(pre_rows, o, kWave), b = __shfl_up(pre_items, o, kWave);
-            if (lane >= o) {
-                pre_rows += a;
-                pre_items += b;
-            }
-        }
-        const int tot_rows = __shfl(pre_rows, kRowsPerWave - 1, kWave);
-        const int tot_items = __shfl(pre_items, kRowsPerWave - 1, kWave);
-        pre_rows -= my_hub ? 1 : 0;
-        pre_items -= my_chunks;
-        if (lane == 0) {
-            wave_rows[wave] = tot_rows;
-            wave_items[wave] = tot_items;
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int br = 0, bi = 0;
-            for (int w = 0; w < kWavesPerBlock; w++) {
-                br += wave_rows[w];
-                bi += wave_items[w];
-            }
-            unsigned long long old = 0;
-            if (br > 0)
-                old = atomicAdd(reinterpret_cast<unsigned long long *>(p.hub.counters),
-                                ((unsigned long long)(unsigned)br << 32) | (unsigned)bi);
-            block_first_item = (int)(old & 0xffffffffu);  // HubCounters: n_items then n_rows
-            block_first_row = (int)(old >> 32);
-        }
-        __syncthreads();
-        if (tot_rows > 0) {
-            int first_row = block_first_row, first_item = block_first_item;
-            for (int w = 0; w < wave; w++) {
-                first_row += wave_rows[w];
-                first_item += wave_items[w];
-            }
-            const bool fits = first_row + tot_rows <= p.hub.max_rows &&
-                              first_item + tot_items <= p.hub.max_items;
-            if (!fits) {
-                if (lane == 0) atomicExch(&p.hub.counters->overflow, 1);
-            } else {
-                if (my_hub)
-                    p.hub.rows[first_row + pre_rows] =
-                        make_int4(r0 + lane, first_item + pre_items, my_chunks, 0);
-                // the chunk items of each hub row, written by the whole wave
-                unsigned long long hubs = __ballot(my_hub);
-                while (hubs) {
-                    const int i = __builtin_ctzll(hubs);
-                    hubs &= hubs - 1;
-                    const int n_c = __shfl(my_chunks, i, kWave);
-                    const int it0 = first_item + __shfl(pre_items, i, kWave);
-                    const int rs = first_row + __shfl(pre_rows, i, kWave);
-                    for (int c = lane; c < n_c; c += kWave)
-                        p.hub.items[it0 + c] = make_int4(r0 + i, c, rs, 0);
-                }
-            }
-        }
-    }
-    if (n_here == 0) return;
 
     EdgeWindow win;
     win.base = -1;
@@ -330,7 +254,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
         const int beg = __shfl(my_ptr, i, kWave);
         const int end = __shfl(my_ptr, i + 1, kWave);
         const int deg = end - beg;
-        if (deg >= p.hub_threshold) continue;  // queued above; written by the hub kernels
+        if (deg >= p.plan.threshold) continue;  // a planned row: written by the item kernels
         const float sr = (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha;
         for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
             const TileLanes<VEC, G, KT, WMODE> tl(p, c0);
@@ -362,41 +286,6 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
     }
 }
 
-// Band-sort key of every queued item: the source id in the middle of its chunk,
-// reduced to 16 bits. Slots past the item count get the largest key.
-static __global__ __launch_bounds__(kBlock) void spmm_hub_keys_kernel(SpmmParams p, uint32_t *keys,
-                                                                      int32_t *vals, int shift) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= p.hub.max_items) return;
-    const int n_items = p.hub.counters->overflow ? 0 : min(p.hub.counters->n_items, p.hub.max_items);
-    uint32_t key = 0xffffu;
-    if (i < n_items) {
-        const int4 it = p.hub.items[i];
-        const int beg = p.indptr[it.x] + it.y * p.hub.chunk;
-        const int end = min(p.indptr[it.x + 1], beg + p.hub.chunk);
-        key = min(0xffffu, (uint32_t)(p.indices[(beg + end) >> 1] & p.col_mask) >> shift);
-    }
-    keys[i] = key;
-    vals[i] = i;
-}
-
-// After the sort: position -> {first edge, end edge, item id, row}, so the item
-// kernel needs one load per item to know its work.
-static __global__ __launch_bounds__(kBlock) void spmm_hub_records_kernel(SpmmParams p,
-                                                                         int4 *records) {
-    const int pos = blockIdx.x * kBlock + threadIdx.x;
-    if (pos >= p.hub.max_items) return;
-    const int n_items = p.hub.counters->overflow ? 0 : min(p.hub.counters->n_items, p.hub.max_items);
-    const int item = p.hub.order[pos];
-    int4 rec = make_int4(0, 0, 0, 0);
-    if (pos < n_items && item < n_items) {
-        const int4 it = p.hub.items[item];
-        const int beg = p.indptr[it.x] + it.y * p.hub.chunk;
-        rec = make_int4(beg, min(p.indptr[it.x + 1], beg + p.hub.chunk), item, it.x);
-    }
-    records[pos] = rec;
-}
-
 constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave
 
 // Items in band order, kItemsPerWave per wave: the records of a wave's items
@@ -404,26 +293,38 @@ constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave
 // feature gather, so the only waits per item are its own gathers. The unscaled
 // partial row goes to partial[item id]; the order only affects cache behaviour.
 template <int VEC, int G, int KT, int WMODE, typename TIN>
-__global__ __launch_bounds__(kBlock) void spmm_hub_items_kernel(SpmmParams p,
-                                                                const int4 *__restrict__ records) {
-    static_assert(kAggChunk <= kWave, "an item must fit one edge window");
+__global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
+    static_assert(kPlanChunk <= kWave, "an item must fit one edge window");
     const int lane = lane_id();
     const int sub = lane % G;
     const int slot = lane / G;
-    if (p.hub.counters->overflow) return;
-    const int n_items = min(p.hub.counters->n_items, p.hub.max_items);
-    const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
-         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+    if (p.plan.counters->overflow) return;
+    const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
+    const int4 *__restrict__ records = p.plan.records;
+    // Workgroups are dealt round-robin to the 8 XCDs; give every XCD its own
+    // contiguous eighth of the band-ordered list, so the 8 L2s hold 8 different
+    // bands instead of 8 copies of one.
+    const int n_groups = (n_items + kItemsPerWave - 1) / kItemsPerWave;  // one group per wave
+    const int share = (n_groups + 7) >> 3;
+    const int xcd = p.xcd_remap ? (blockIdx.x & 7) : 0;
+    const int waves_per_xcd = p.xcd_remap ? (gridDim.x >> 3) * kWavesPerBlock
+                                          : gridDim.x * kWavesPerBlock;
+    const int local0 = (p.xcd_remap ? (blockIdx.x >> 3) : blockIdx.x) * kWavesPerBlock +
+                       threadIdx.x / kWave;
+    const int lo = p.xcd_remap ? xcd * share : 0;
+    const int hi = p.xcd_remap ? min(n_groups, lo + share) : n_groups;
+    for (int grp = lo + local0; grp < hi; grp += waves_per_xcd) {
+        const int pos0 = grp * kItemsPerWave;
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = records[pos0 + min(lane, n_here - 1)];
         EdgeWindow win[kItemsPerWave];
-        int item_id[kItemsPerWave], n_edges[kItemsPerWave];
+        int item_id[kItemsPerWave], n_edges[kItemsPerWave], row_tag[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
             const int beg = __shfl(my_rec.x, j, kWave);
             const int end = __shfl(my_rec.y, j, kWave);
             item_id[j] = __shfl(my_rec.z, j, kWave);
+            row_tag[j] = __shfl(my_rec.w, j, kWave);
             n_edges[j] = j < n_here ? end - beg : 0;
             if (n_edges[j] > 0) load_window<WMODE>(win[j], p, beg, end);
         }
@@ -439,12 +340,22 @@ __global__ __launch_bounds__(kBlock) void spmm_hub_items_kernel(SpmmParams p,
                     for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
                 accumulate_window<VEC, G, KT, WMODE, TIN>(acc, p, win[j], 0, n_edges[j], tl);
                 fold_slots<VEC, G, KT>(acc);
+                const bool single = row_tag[j] < 0;
+                const int row = row_tag[j] & 0x7fffffff;
+                float *dst = single ? p.out + (size_t)row * p.L
+                                    : p.partial + (size_t)item_id[j] * p.L;
+                const float sr =
+                    single ? (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha : 1.0f;
                 if (slot == 0) {
 #pragma unroll
                     for (int t = 0; t < KT; t++) {
                         const int o = c0 + (t * G + sub) * VEC;
-                        if (o < p.L)
-                            store_row<VEC>(p.hub.partial + (size_t)item_id[j] * p.L + o, acc[t]);
+                        if (o < p.L) {
+                            float r[VEC];
+#pragma unroll
+                            for (int i = 0; i < VEC; i++) r[i] = acc[t][i] * sr;
+                            store_row<VEC>(dst + o, r);
+                        }
                     }
                 }
             }
@@ -457,13 +368,14 @@ __global__ __launch_bounds__(kBlock) void spmm_hub_items_kernel(SpmmParams p,
 // `lanes` threads; team g adds chunks g, g + groups, ... and the team sums are
 // then added in team order, so the result is a fixed function of the chunk count.
 template <int WMODE, int VEC>
-__global__ __launch_bounds__(kBlock) void spmm_hub_reduce_kernel(SpmmParams p) {
+__global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
     __shared__ float red[kBlock * VEC];
-    if (p.hub.counters->overflow) return;
-    const int n_hub = min(p.hub.counters->n_rows, p.hub.max_rows);
+    if (p.plan.counters->overflow) return;
+    const int n_hub = min(p.plan.counters->n_rows, p.plan.max_rows);
     const int lanes_total = p.L / VEC;  // VEC divides L (host picks VEC)
     for (int h = blockIdx.x; h < n_hub; h += gridDim.x) {
-        const int4 r = p.hub.rows[h];
+        const int4 r = p.plan.rows[h];
+        if (r.z <= 1) continue;  // single-item rows were written by the item kernel
         const float sr = (WMODE == W_DEGPROD ? p.scale_row[r.x] : 1.0f) * p.alpha;
         for (int l0 = 0; l0 < lanes_total; l0 += kBlock) {
             const int lanes = min(kBlock, lanes_total - l0);
@@ -476,7 +388,7 @@ __global__ __launch_bounds__(kBlock) void spmm_hub_reduce_kernel(SpmmParams p) {
                 for (int c = g; c < r.z; c += groups) {
                     float v[VEC];
                     RowLoad<VEC, float>::ld(
-                        p.hub.partial + (size_t)(r.y + c) * p.L + (size_t)(l0 + l) * VEC, v);
+                        p.partial + (size_t)(r.y + c) * p.L + (size_t)(l0 + l) * VEC, v);
 #pragma unroll
                     for (int i = 0; i < VEC; i++) s[i] += v[i];
                 }
@@ -507,13 +419,15 @@ static __global__ void zero_hub_counters_kernel(HubCounters *c) {
 }
 
 // Host side: carve the queue out of a caller-provided workspace.
-size_t hub_workspace_bytes(int64_t nnz, int64_t L);
 int hub512_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t nnz);
 
 // Picks the instantiation for (element type, L) and launches the 1 + 3 kernels.
-// max_degree_hint < 0 means unknown.
+// max_degree_hint < 0 means unknown; plan may be null (a temporary one is then
+// built in the workspace). p.n_src and p.col_mask must be set.
 int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max_degree_hint,
-                void *workspace, size_t workspace_bytes, hipStream_t stream);
+                const void *plan, void *workspace, size_t workspace_bytes, hipStream_t stream);
+// Workspace of launch_spmm: partial rows, plus the temporary plan when none is given.
+size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan);
 const char *last_error();
 // Zero-fill by kernel (safe to record into a captured graph, unlike a memset node).
 int fill_zero(float *p, int64_t n, hipStream_t stream);

@@ -47,7 +47,7 @@ def _size_fn(name):
 # transposed structure, cached per (indptr, indices) pair
 # --------------------------------------------------------------------------- #
 class _Transposed:
-    __slots__ = ("t_indptr", "t_rows", "t_perm", "max_degree_t", "n_src")
+    __slots__ = ("t_indptr", "t_rows", "t_perm", "max_degree_t", "n_src", "plan_t")
 
 
 _transposed = {}
@@ -76,6 +76,7 @@ def transposed(indptr, indices, n_src):
                                            stream_ptr(dev))
     check(rc, "yitu_csr_transpose")
     t.max_degree_t = _lib.max_degree(t.t_indptr)
+    t.plan_t = _lib.row_plan(t.t_indptr, t.t_rows, n_rows, 0x7FFFFFFF)
     _transposed[key] = t
     weakref.finalize(indices, _transposed.pop, key, None)
     return t
@@ -98,12 +99,14 @@ def spmm_forward(values, indptr, indices, features):
         raise RuntimeError("values must be [n_edges, n_heads]")
     out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 64 else 0
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
+    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f), c_int(1)) \
+        if plan is not None else 0
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_spmm_forward(ptr(out), ptr(values), ptr(indptr), ptr(indices),
                                           ptr(features), c_i64(n_dst), c_i64(n_src), c_i64(nnz),
-                                          c_i64(h), c_i64(f), c_i64(maxdeg), ptr(ws),
+                                          c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan), ptr(ws),
                                           c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_spmm_forward")
     return out
@@ -126,17 +129,19 @@ def spmm_backward(values, indptr, indices, features, grad_out):
     grad_x = torch.empty_like(features)
     tr = transposed(indptr, indices, n_src)
     maxdeg = _lib.max_degree(indptr)
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = 0
     if max(maxdeg, tr.max_degree_t) >= 64:
-        need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f))
+        need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_spmm_backward(ptr(grad_a), ptr(grad_x), ptr(values), ptr(indptr),
                                            ptr(indices), ptr(features), ptr(grad_out),
                                            ptr(tr.t_indptr), ptr(tr.t_rows), ptr(tr.t_perm),
                                            c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h), c_i64(f),
-                                           c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(ws),
-                                           c_size(ws.numel()), stream_ptr(dev))
+                                           c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan),
+                                           ptr(tr.plan_t), ptr(ws), c_size(ws.numel()),
+                                           stream_ptr(dev))
     check(rc, "yitu_spmm_backward")
     return [grad_a, grad_x]
 
@@ -156,14 +161,14 @@ def edge_dot(indptr, indices, dst_feat, src_feat):
         raise RuntimeError("dst_feat must be [n_dst, H, F] matching src_feat's H and F")
     out = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f)) if maxdeg >= 64 else 0
-    ws = _lib.workspace(need, dev)
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
+    ws = _lib.workspace(0, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_spmm_backward(ptr(out), ptr(None), ptr(None), ptr(indptr), ptr(indices),
                                            ptr(src_feat), ptr(dst_feat), ptr(None), ptr(None),
                                            ptr(None), c_i64(n_dst), c_i64(n_src), c_i64(nnz),
-                                           c_i64(h), c_i64(f), c_i64(maxdeg), c_i64(-1), ptr(ws),
-                                           c_size(ws.numel()), stream_ptr(dev))
+                                           c_i64(h), c_i64(f), c_i64(maxdeg), c_i64(-1), ptr(plan),
+                                           ptr(None), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_spmm_backward")
     return out
 
@@ -193,7 +198,7 @@ def sddmm_forward(indptr, indices, query, key):
     maxdeg = _lib.max_degree(indptr)
     need = 0
     if maxdeg >= 64:
-        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_sddmm_forward(ptr(attn), ptr(indptr), ptr(indices), ptr(query), ptr(key),
@@ -220,15 +225,15 @@ def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, determini
     grad_edge = torch.empty_like(attn_values) if deterministic else None
     need = 0
     if maxdeg >= 64 or (tr is not None and tr.max_degree_t >= 64):
-        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid))
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_sddmm_backward(
             ptr(grad_query), ptr(grad_key), ptr(grad_edge), ptr(indptr), ptr(indices), ptr(query),
             ptr(key), ptr(attn_values), ptr(grad_out), ptr(tr.t_indptr if tr else None),
             ptr(tr.t_perm if tr else None), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-            c_i64(n_bid), c_i64(maxdeg), c_i64(tr.max_degree_t if tr else -1), ptr(ws),
-            c_size(ws.numel()), stream_ptr(dev))
+            c_i64(n_bid), c_i64(maxdeg), c_i64(tr.max_degree_t if tr else -1),
+            ptr(tr.plan_t if tr else None), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_sddmm_backward")
     return [grad_query, grad_key]
 
@@ -344,13 +349,17 @@ def gat_forward(indptr, indices, query, key, features):
     out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
     attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
-    need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f)) if maxdeg >= 64 else 0
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
+    need = 0
+    if maxdeg >= 64:
+        need = _size_fn("yitu_gat_workspace_bytes")(c_i64(n_dst), c_i64(nnz), c_i64(h), c_i64(f),
+                                                    c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_gat_forward(ptr(out), ptr(attn), ptr(indptr), ptr(indices), ptr(query),
                                          ptr(key), ptr(features), c_i64(n_dst), c_i64(n_src),
-                                         c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(ws),
-                                         c_size(ws.numel()), stream_ptr(dev))
+                                         c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan),
+                                         ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_gat_forward")
     return [out, attn]
 
@@ -370,16 +379,18 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out):
     s1 = torch.empty_like(attn)
     s2 = torch.empty_like(attn)
     maxdeg = _lib.max_degree(indptr)
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = 0
     if max(maxdeg, tr.max_degree_t) >= 64:
-        need = _size_fn("yitu_gat_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(f))
+        need = _size_fn("yitu_gat_workspace_bytes")(c_i64(max(n_dst, n_src)), c_i64(nnz), c_i64(h),
+                                                    c_i64(f), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_gat_backward(
             ptr(grad_q), ptr(grad_k), ptr(grad_x), ptr(s1), ptr(s2), ptr(indptr), ptr(indices),
             ptr(query), ptr(key), ptr(features), ptr(attn), ptr(grad_out), ptr(tr.t_indptr),
             ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-            c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(ws), c_size(ws.numel()),
-            stream_ptr(dev))
+            c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan), ptr(tr.plan_t), ptr(ws),
+            c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_gat_backward")
     return [grad_q, grad_k, grad_x]
