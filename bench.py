@@ -27,10 +27,16 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per aggregation call measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (two runs, each scaled by the same counter's reading for a 1 GiB copy kernel);
-# the summaries live under profiles/. None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM-side bytes per call (reads + writes leaving L2) measured with two rocprofv3 --pmc
+# runs of this file, FETCH_SIZE then WRITE_SIZE, each scaled by what the same counter
+# reads for the library's 1 GiB copy kernel (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000):
+# profiles/bench_c3_spmm_gat_rocprofv3.md. Per yitu_agg_csr call for the C3 workloads,
+# per yitu_gat_forward call for C2.
+MEASURED_TRAFFIC_BYTES = {
+    "c3_spmm_f32": 21_803_805_752,
+    "c3_spmm_bf16": 10_910_454_990,
+    "c2_gat_f32": 6_556_746_400,
+}
 
 
 def _sync():
@@ -217,6 +223,28 @@ def run_gat(args, dev):
     }
 
 
+def calibration_copy(dev, n_bytes=1 << 30, reps=5):
+    """1 GiB streaming copy through the library's copy kernel: the known-size
+    launch that FETCH_SIZE / WRITE_SIZE are scaled by, and the achievable
+    read+write bandwidth of this GPU."""
+    from yitu_amd import _lib
+    a = torch.empty(n_bytes, dtype=torch.uint8, device=dev)
+    b = torch.empty(n_bytes, dtype=torch.uint8, device=dev)
+    a.zero_()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(reps + 1):
+        if i == 1:
+            e0.record()
+        rc = _lib.lib().yitu_stream_copy(_lib.ptr(b), _lib.ptr(a), _lib.c_i64(n_bytes),
+                                         _lib.stream_ptr(dev))
+        _lib.check(rc, "yitu_stream_copy")
+    e1.record()
+    _sync()
+    ms = e0.elapsed_time(e1) / reps
+    return {"bytes_read": n_bytes, "bytes_written": n_bytes, "ms": ms,
+            "GBps_read_plus_write": 2 * n_bytes / (ms * 1e-3) / 1e9}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -234,6 +262,7 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "c3_spmm_f32":
         res = run_spmm(args, dev, bf16=False)
+        res["copy_calibration"] = calibration_copy(dev)
         if not args.no_extra:
             # the other single-GPU configurations ride along as extra fields
             args.no_cpu = True

@@ -26,6 +26,11 @@ extern "C" {
 const char *yitu_last_error(void);
 int yitu_abi_version(void);
 
+/* Plain device-to-device streaming copy of n_bytes (multiple of 16): the known-
+ * size kernel used to calibrate HBM traffic counters and to measure achievable
+ * copy bandwidth. No reference counterpart. */
+int yitu_stream_copy(void *dst_device, const void *src_device, int64_t n_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Row plan (per graph, built once)                                            */
 /* ------------------------------------------------------------------------- */

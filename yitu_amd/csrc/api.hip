@@ -71,3 +71,27 @@ YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *i
                        static_cast<hipStream_t>(stream));
 }
 
+
+// Plain streaming copy (16 bytes per lane), used to calibrate the HBM traffic
+// counters and as the achievable-bandwidth reference of the benchmark.
+namespace yitu {
+__global__ __launch_bounds__(kBlock) void stream_copy_kernel(const uint4 *__restrict__ src,
+                                                             uint4 *__restrict__ dst, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
+}  // namespace yitu
+
+YITU_API int yitu_stream_copy(void *dst, const void *src, int64_t n_bytes, void *stream) {
+    YITU_REQUIRE(n_bytes >= 0 && n_bytes % 16 == 0, "size must be a multiple of 16 bytes");
+    YITU_REQUIRE(n_bytes == 0 || (dst && src && aligned16(dst) && aligned16(src)),
+                 "null or unaligned buffer");
+    if (n_bytes == 0) return 0;
+    const int64_t n = n_bytes / 16;
+    const int grid = (int)std::min<int64_t>(ceil_div(n, kBlock), 32768);
+    stream_copy_kernel<<<grid, kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
