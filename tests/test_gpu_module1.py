@@ -100,8 +100,10 @@ def test_bf16_input_fp32_accumulate(dev, dim):
     assert_close(got, want)
 
 
-def test_with_and_without_row_plan_agree_bitwise(dev):
-    """The cached row plan and the temporary one built per call give identical bits."""
+def test_with_and_without_row_plan_agree(dev):
+    """A call given no row plan builds a temporary one without slabs: its long rows are
+    cut at other places than the per-graph plan cuts them, so the two results agree to
+    rounding (and each of them is bitwise reproducible)."""
     from yitu_amd import _lib
     indptr, indices = powerlaw_graph(13, 200000, 8)
     n = indptr.numel() - 1
@@ -116,7 +118,15 @@ def test_with_and_without_row_plan_agree_bitwise(dev):
                                  _lib.c_i64(64), _lib.c_f32(1.0), _lib.c_i64(-1), _lib.ptr(None),
                                  _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
     _lib.check(rc, "yitu_agg_csr")
-    assert torch.equal(out, with_plan)
+    first = out.clone()
+    assert_close(first, with_plan)
+    rc = _lib.lib().yitu_agg_csr(_lib.ptr(out), _lib.ptr(x), 0, _lib.ptr(rp), _lib.ptr(ci),
+                                 _lib.ptr(deg), _lib.c_i64(n), _lib.c_i64(n), _lib.c_i64(ci.numel()),
+                                 _lib.c_i64(64), _lib.c_f32(1.0), _lib.c_i64(-1), _lib.ptr(None),
+                                 _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
+    _lib.check(rc, "yitu_agg_csr")
+    assert torch.equal(out, first)
+    assert torch.equal(K._aggregate(x, rp, ci, deg, 1.0), with_plan)
 
 
 def test_results_are_bitwise_reproducible(dev):
@@ -157,7 +167,11 @@ def test_linearity_and_row_block_invariance_at_scale(dev):
                                  _lib.c_i64(-1), _lib.ptr(None), _lib.ptr(ws),
                                  _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
     _lib.check(rc, "yitu_agg_csr")
-    assert torch.equal(out, y_unscaled[lo:hi])
+    # rows below 64 edges never depend on the launch they are in; longer rows are cut
+    # into items at places that depend on the plan, so they agree to rounding
+    short = (rp[lo + 1:hi + 1] - rp[lo:hi]) < 64
+    assert torch.equal(out[short], y_unscaled[lo:hi][short])
+    assert_close(out, y_unscaled[lo:hi], atol=5e-4)
 
 
 def test_rejects_cpu_tensors_and_bad_dtypes(dev):

@@ -156,13 +156,4 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-// Workgroups are dealt round-robin to the 8 XCDs (each with a private L2).
-// Mapping hardware block b to logical block (b % 8) * ceil(nb / 8) + b / 8
-// gives every XCD one contiguous range of rows, so rows that share neighbours
-// after a locality-improving vertex order also share an L2.
-__device__ __forceinline__ int xcd_contiguous_block(int b, int nb) {
-    const int per = (nb + 7) >> 3;
-    return (b & 7) * per + (b >> 3);
-}
-
 }  // namespace yitu

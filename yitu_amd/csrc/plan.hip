@@ -1,11 +1,13 @@
-// Builds the row plan on the device: queue the long rows and their 64-edge
-// items (one atomic per workgroup), key every item by its middle source id,
-// stable radix sort, write the band-ordered records.
+// Builds the row plan on the device: queue the long rows (one atomic per
+// workgroup), count the edges per source and place the slab boundaries, cut
+// every long row at the boundaries and into items of at most 64 edges, key every
+// item by its middle source id, stable radix sort, write the records.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 
 #include "../../include/yitu_hip.h"
 #include "plan.hpp"
@@ -14,122 +16,239 @@ namespace yitu {
 
 namespace {
 
-constexpr int kQueueRowsPerWave = 64;  // one row per lane
+constexpr int kBandBits = 16;  // sort key = middle source id reduced to this many bits
 
 struct BuildBuffers {
     PlanCounters *counters;
     int4 *rows;
     int4 *records;
-    int4 *items;  // {row, chunk, index into rows[], 0} in queue order
+    int *slab_bound;  // [kPlanSlabs + 1] first source id of every slab, in the plan
+    int4 *items;      // {first edge, end edge, index into rows[], row} in queue order
     uint32_t *keys_in, *keys_out;
     int32_t *vals_in, *order;
     void *sort_temp;
     size_t sort_temp_bytes;
+    uint32_t *pop;           // [n_buckets] edges per bucket of 2^bucket_shift consecutive sources
+    unsigned long long *cost;  // [n_buckets] inclusive prefix sums of popularity^0.75
+    void *scan_temp;
+    size_t scan_temp_bytes;
+    int n_buckets, bucket_shift, band_shift;
     int max_rows, max_items;
 };
 
-__global__ void plan_zero_kernel(PlanCounters *c) {
-    if (threadIdx.x == 0) {
-        c->n_items = 0;
-        c->n_rows = 0;
-        c->overflow = 0;
-        c->pad = 0;
+// Number of popularity buckets a graph of nnz edges gets (bounds the workspace
+// by the edge count whatever the number of sources).
+inline int64_t pop_buckets(int64_t nnz) { return std::max<int64_t>(4096, nnz / 4); }
+
+__global__ __launch_bounds__(kBlock) void plan_init_kernel(BuildBuffers b) {
+    const int64_t i0 = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    if (i0 == 0) {
+        b.counters->n_items = 0;
+        b.counters->n_rows = 0;
+        b.counters->overflow = 0;
+        b.counters->pad = 0;
+    }
+    if (i0 <= kPlanSlabs) b.slab_bound[i0] = i0 == 0 ? 0 : 0x7fffffff;
+    for (int64_t i = i0; i < b.n_buckets; i += stride) b.pop[i] = 0u;
+    // slots that get no item sort behind every real key
+    for (int64_t i = i0; i < b.max_items; i += stride) {
+        b.keys_in[i] = 0xffffu;
+        b.vals_in[i] = (int32_t)i;
     }
 }
 
-// Every lane owns one row. Long rows get consecutive item ids; a workgroup's
-// rows are numbered with a block-level prefix sum and ONE 64-bit atomic on the
-// two counters (hundreds of thousands of same-address atomics serialise in L2).
+// Every lane owns one row; the long rows of a workgroup are numbered with a
+// block-level prefix sum and ONE atomic (hundreds of thousands of same-address
+// atomics serialise in L2).
 __global__ __launch_bounds__(kBlock) void plan_queue_kernel(BuildBuffers b,
                                                             const int32_t *__restrict__ indptr,
                                                             int n_rows) {
-    __shared__ int wave_rows[kWavesPerBlock], wave_items[kWavesPerBlock];
-    __shared__ int block_first_row, block_first_item;
+    __shared__ int wave_rows[kWavesPerBlock];
+    __shared__ int block_first_row;
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
     const int row = blockIdx.x * kBlock + threadIdx.x;
     int deg = 0;
     if (row < n_rows) deg = indptr[row + 1] - indptr[row];
     const bool longrow = deg >= kPlanThreshold;
-    const int chunks = longrow ? (deg + kPlanChunk - 1) / kPlanChunk : 0;
-    int pre_rows = longrow ? 1 : 0, pre_items = chunks;
+    int pre = longrow ? 1 : 0;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
-        const int x = __shfl_up(pre_rows, o, kWave), y = __shfl_up(pre_items, o, kWave);
-        if (lane >= o) {
-            pre_rows += x;
-            pre_items += y;
-        }
+        const int x = __shfl_up(pre, o, kWave);
+        if (lane >= o) pre += x;
     }
-    if (lane == kWave - 1) {
-        wave_rows[wave] = pre_rows;
-        wave_items[wave] = pre_items;
-    }
-    pre_rows -= longrow ? 1 : 0;
-    pre_items -= chunks;
+    if (lane == kWave - 1) wave_rows[wave] = pre;
+    pre -= longrow ? 1 : 0;
     __syncthreads();
     if (threadIdx.x == 0) {
-        int br = 0, bi = 0;
-        for (int w = 0; w < kWavesPerBlock; w++) {
-            br += wave_rows[w];
-            bi += wave_items[w];
-        }
-        unsigned long long old = 0;
-        if (br > 0)  // PlanCounters starts with n_items (low word) then n_rows (high word)
-            old = atomicAdd(reinterpret_cast<unsigned long long *>(b.counters),
-                            ((unsigned long long)(unsigned)br << 32) | (unsigned)bi);
-        block_first_item = (int)(old & 0xffffffffu);
-        block_first_row = (int)(old >> 32);
+        int br = 0;
+        for (int w = 0; w < kWavesPerBlock; w++) br += wave_rows[w];
+        block_first_row = br > 0 ? atomicAdd(&b.counters->n_rows, br) : 0;
     }
     __syncthreads();
     if (!longrow) return;
-    int first_row = block_first_row + pre_rows, first_item = block_first_item + pre_items;
-    for (int w = 0; w < wave; w++) {
-        first_row += wave_rows[w];
-        first_item += wave_items[w];
-    }
-    if (first_row >= b.max_rows || first_item + chunks > b.max_items) {
+    int slot = block_first_row + pre;
+    for (int w = 0; w < wave; w++) slot += wave_rows[w];
+    if (slot >= b.max_rows) {
         atomicExch(&b.counters->overflow, 1);
         return;
     }
-    b.rows[first_row] = make_int4(row, first_item, chunks, 0);
-    for (int c = 0; c < chunks; c++) b.items[first_item + c] = make_int4(row, c, first_row, 0);
+    b.rows[slot] = make_int4(row, 0, 0, 0);
 }
 
-// Band key of every queued item: the source id in the middle of the item,
-// reduced to 16 bits. Slots past the item count get the largest key.
-__global__ __launch_bounds__(kBlock) void plan_keys_kernel(BuildBuffers b,
-                                                           const int32_t *__restrict__ indptr,
-                                                           const int32_t *__restrict__ indices,
-                                                           int col_mask, int shift) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= b.max_items) return;
-    const int n_items = b.counters->overflow ? 0 : min(b.counters->n_items, b.max_items);
-    uint32_t key = 0xffffu;
-    if (i < n_items) {
-        const int4 it = b.items[i];
-        const int beg = indptr[it.x] + it.y * kPlanChunk;
-        const int end = min(indptr[it.x + 1], beg + kPlanChunk);
-        key = min(0xffffu, (uint32_t)(indices[(beg + end) >> 1] & col_mask) >> shift);
+__global__ __launch_bounds__(kBlock) void plan_popularity_kernel(BuildBuffers b,
+                                                                 const int32_t *__restrict__ indices,
+                                                                 int64_t nnz, int col_mask,
+                                                                 int n_src) {
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (; i < nnz; i += stride) {
+        const int c = indices[i] & col_mask;
+        if (c < n_src) atomicAdd(&b.pop[c >> b.bucket_shift], 1u);
     }
-    b.keys_in[i] = key;
-    b.vals_in[i] = i;
 }
 
-__global__ __launch_bounds__(kBlock) void plan_records_kernel(BuildBuffers b,
-                                                              const int32_t *__restrict__ indptr) {
+// Cost of a bucket of sources: popularity^0.75 in quarter units. A source that
+// many edges read is fetched into L2 once and then hit, so what it costs grows
+// more slowly than its edge count.
+__global__ __launch_bounds__(kBlock) void plan_cost_kernel(BuildBuffers b) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= b.n_buckets) return;
+    const float r = sqrtf((float)b.pop[i]);
+    b.cost[i] = (unsigned long long)(r * sqrtf(r) * 4.0f + 0.5f);
+}
+
+// Slab k starts at the first bucket where the running cost reaches k/8 of the total.
+__global__ void plan_bounds_kernel(BuildBuffers b) {
+    const int k = threadIdx.x;
+    if (k < 1 || k >= kPlanSlabs) return;
+    const unsigned long long total = b.cost[b.n_buckets - 1];
+    const unsigned long long target = total / kPlanSlabs * k;
+    int lo = 0, hi = b.n_buckets;  // first index with cost >= target
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (b.cost[mid] < target) lo = mid + 1; else hi = mid;
+    }
+    const long long bound = ((long long)lo + 1) << b.bucket_shift;
+    b.slab_bound[k] = (int)(bound < 0x7fffffffLL ? bound : 0x7fffffffLL);
+}
+
+// One wave per long row. Lanes 0..8 find where the row's columns cross the slab
+// boundaries; lane 0 turns the crossings into at most min(8, deg / 16) segments
+// (none shorter than kPlanMinSegment), the wave then writes the items of every
+// segment: ceil(len / 64) pieces of equal size. Item ids of a row are
+// consecutive; a workgroup takes its ids with one atomic.
+__global__ __launch_bounds__(kBlock) void plan_items_kernel(BuildBuffers b,
+                                                            const int32_t *__restrict__ indptr,
+                                                            const int32_t *__restrict__ indices,
+                                                            int col_mask, int with_slabs) {
+    __shared__ int cut[kWavesPerBlock][kPlanSlabs + 1];
+    __shared__ int seg_beg[kWavesPerBlock][kPlanSlabs + 1];    // [n_seg] = end of the row
+    __shared__ int seg_first[kWavesPerBlock][kPlanSlabs + 1];  // first item of the segment, [n_seg] = total
+    __shared__ int n_seg[kWavesPerBlock];
+    __shared__ int wave_first[kWavesPerBlock];
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int slot = blockIdx.x * kWavesPerBlock + wave;
+    const int n_rows = b.counters->overflow ? 0 : min(b.counters->n_rows, b.max_rows);
+    const bool active = slot < n_rows;
+    int row = 0, beg = 0, end = 0;
+    if (active) {
+        row = b.rows[slot].x;
+        beg = indptr[row];
+        end = indptr[row + 1];
+    }
+    constexpr int NS = kPlanSlabs;
+    if (active && lane <= NS) {
+        int c = lane == 0 ? beg : end;
+        if (with_slabs && lane > 0 && lane < NS) {
+            const int bound = b.slab_bound[lane];
+            int lo = beg, hi = end;  // first edge whose column is >= bound
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if ((indices[mid] & col_mask) < bound) lo = mid + 1; else hi = mid;
+            }
+            c = lo;
+        }
+        cut[wave][lane] = c;
+    }
+    if (active && lane == 0) cut[wave][NS] = end;
+    __syncthreads();
+    if (active && lane == 0) {
+        // columns that are not sorted inside the row give crossings out of order;
+        // a running maximum keeps the pieces a partition of the row
+        const int deg = end - beg;
+        const int max_seg = max(1, min(NS, deg / kPlanMinSegment));
+        int n = 0, cur = beg, total = 0, reach = beg;
+        for (int k = 1; k <= NS; k++) {
+            reach = min(end, max(reach, cut[wave][k]));
+            const bool last = k == NS;
+            const int len = reach - cur;
+            if (last ? len > 0
+                     : (len >= kPlanMinSegment && end - reach >= kPlanMinSegment &&
+                        n < max_seg - 1)) {
+                seg_beg[wave][n] = cur;
+                seg_first[wave][n] = total;
+                total += (len + kPlanChunk - 1) / kPlanChunk;
+                cur = reach;
+                n++;
+            }
+        }
+        seg_beg[wave][n] = end;
+        seg_first[wave][n] = total;
+        n_seg[wave] = n;
+    }
+    if (!active && lane == 0) {
+        n_seg[wave] = 0;
+        seg_first[wave][0] = 0;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int sum = 0;
+        for (int w = 0; w < kWavesPerBlock; w++) {
+            wave_first[w] = sum;
+            sum += seg_first[w][n_seg[w]];
+        }
+        const int base = sum > 0 ? atomicAdd(&b.counters->n_items, sum) : 0;
+        for (int w = 0; w < kWavesPerBlock; w++) wave_first[w] += base;
+    }
+    __syncthreads();
+    if (!active) return;
+    const int n = n_seg[wave];
+    const int total = seg_first[wave][n];
+    const int first_item = wave_first[wave];
+    if (first_item + total > b.max_items) {
+        if (lane == 0) atomicExch(&b.counters->overflow, 1);
+        return;
+    }
+    if (lane == 0) b.rows[slot] = make_int4(row, first_item, total, 0);
+    for (int i = lane; i < total; i += kWave) {
+        int s = 0;
+        while (s + 1 < n && seg_first[wave][s + 1] <= i) s++;
+        const int sb = seg_beg[wave][s], se = seg_beg[wave][s + 1];
+        const int pieces = seg_first[wave][s + 1] - seg_first[wave][s];
+        const int size = (se - sb + pieces - 1) / pieces;
+        const int ib = sb + (i - seg_first[wave][s]) * size;
+        const int ie = min(se, ib + size);
+        const int mid_col = indices[(ib + ie) >> 1] & col_mask;
+        b.items[first_item + i] = make_int4(ib, ie, slot, row);
+        b.keys_in[first_item + i] =
+            min((uint32_t)mid_col >> b.band_shift, (1u << kBandBits) - 1u);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void plan_records_kernel(BuildBuffers b) {
     const int pos = blockIdx.x * kBlock + threadIdx.x;
-    if (pos >= b.max_items) return;
     const int n_items = b.counters->overflow ? 0 : min(b.counters->n_items, b.max_items);
+    if (pos >= b.max_items) return;
     int4 rec = make_int4(0, 0, 0, 0);
     if (pos < n_items) {
         const int item = b.order[pos];  // stable sort: real items precede the padding
         const int4 it = b.items[item];
-        const int row_beg = indptr[it.x], row_end = indptr[it.x + 1];
-        const int beg = row_beg + it.y * kPlanChunk;
         // a row that is a single item is finished by the item kernel itself
-        const int single = (row_end - row_beg <= kPlanChunk) ? (int)0x80000000 : 0;
-        rec = make_int4(beg, min(row_end, beg + kPlanChunk), item, it.x | single);
+        const int single = b.rows[it.z].z == 1 ? (int)0x80000000 : 0;
+        rec = make_int4(it.x, it.y, item, it.w | single);
     }
     b.records[pos] = rec;
 }
@@ -142,17 +261,31 @@ size_t sort_temp_bytes(int64_t n) {
     return bytes;
 }
 
+size_t scan_temp_bytes(int64_t n) {
+    size_t bytes = 0;
+    unsigned long long *c = nullptr;
+    (void)rocprim::inclusive_scan(nullptr, bytes, c, c, (size_t)n,
+                                  rocprim::plus<unsigned long long>());
+    return bytes;
+}
+
+constexpr size_t kHeaderBytes = 512;  // counters | slab_bound[kPlanSlabs + 1]
+
 }  // namespace
 
 size_t plan_bytes(int64_t nnz) {
-    return 256 + align_up(sizeof(int4) * (size_t)plan_max_rows(nnz), 256) +
+    return kHeaderBytes + align_up(sizeof(int4) * (size_t)plan_max_rows(nnz), 256) +
            align_up(sizeof(int4) * (size_t)plan_max_items(nnz), 256);
 }
 
 size_t plan_build_workspace_bytes(int64_t nnz) {
     const size_t items = (size_t)plan_max_items(nnz);
+    const size_t buckets = (size_t)pop_buckets(nnz);
     return align_up(sizeof(int4) * items, 256) + 4 * align_up(sizeof(int32_t) * items, 256) +
-           align_up(sort_temp_bytes((int64_t)items), 256);
+           align_up(sort_temp_bytes((int64_t)items), 256) +
+           align_up(sizeof(uint32_t) * buckets, 256) +
+           align_up(sizeof(unsigned long long) * buckets, 256) +
+           align_up(scan_temp_bytes((int64_t)buckets), 256);
 }
 
 size_t plan_temp_bytes(int64_t nnz) { return plan_bytes(nnz) + plan_build_workspace_bytes(nnz); }
@@ -161,7 +294,7 @@ PlanView plan_view(const void *plan, int64_t nnz) {
     PlanView v{};
     const char *w = static_cast<const char *>(plan);
     v.counters = reinterpret_cast<const PlanCounters *>(w);
-    w += 256;
+    w += kHeaderBytes;
     v.max_rows = (int)plan_max_rows(nnz);
     v.max_items = (int)plan_max_items(nnz);
     v.rows = reinterpret_cast<const int4 *>(w);
@@ -172,8 +305,8 @@ PlanView plan_view(const void *plan, int64_t nnz) {
 }
 
 int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_t *indices,
-               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, void *workspace,
-               size_t workspace_bytes, hipStream_t stream) {
+               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, bool with_slabs,
+               void *workspace, size_t workspace_bytes, hipStream_t stream) {
     YITU_REQUIRE(plan && plan_size >= plan_bytes(nnz), "plan buffer too small: need %zu bytes",
                  plan_bytes(nnz));
     YITU_REQUIRE(workspace && workspace_bytes >= plan_build_workspace_bytes(nnz),
@@ -181,10 +314,11 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
     YITU_REQUIRE((reinterpret_cast<uintptr_t>(plan) & 255u) == 0 &&
                      (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
                  "plan and workspace must be 256-byte aligned");
-    YITU_REQUIRE(n_rows < INT32_MAX && nnz < INT32_MAX, "size out of range");
+    YITU_REQUIRE(n_rows < INT32_MAX && n_src < INT32_MAX && nnz < INT32_MAX, "size out of range");
     const PlanView v = plan_view(plan, nnz);
     BuildBuffers b{};
     b.counters = const_cast<PlanCounters *>(v.counters);
+    b.slab_bound = reinterpret_cast<int *>(static_cast<char *>(plan) + 256);
     b.rows = const_cast<int4 *>(v.rows);
     b.records = const_cast<int4 *>(v.records);
     b.max_rows = v.max_rows;
@@ -200,24 +334,49 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
     w += 4 * arr;
     b.sort_temp = w;
     b.sort_temp_bytes = sort_temp_bytes(b.max_items);
+    w += align_up(b.sort_temp_bytes, 256);
+    const int64_t max_buckets = pop_buckets(nnz);
+    b.bucket_shift = 0;
+    while (((std::max<int64_t>(n_src, 1) - 1) >> b.bucket_shift) + 1 > max_buckets) b.bucket_shift++;
+    b.n_buckets = with_slabs ? (int)(((std::max<int64_t>(n_src, 1) - 1) >> b.bucket_shift) + 1) : 0;
+    b.pop = reinterpret_cast<uint32_t *>(w);
+    w += align_up(sizeof(uint32_t) * (size_t)max_buckets, 256);
+    b.cost = reinterpret_cast<unsigned long long *>(w);
+    w += align_up(sizeof(unsigned long long) * (size_t)max_buckets, 256);
+    b.scan_temp = w;
+    b.scan_temp_bytes = scan_temp_bytes(max_buckets);
+    b.band_shift = 0;
+    while (((std::max<int64_t>(n_src, 1) - 1) >> b.band_shift) >= ((int64_t)1 << kBandBits))
+        b.band_shift++;
 
-    plan_zero_kernel<<<1, kWave, 0, stream>>>(b.counters);
+    const int item_grid = (int)ceil_div(b.max_items, kBlock);
+    plan_init_kernel<<<std::min(item_grid, 4096), kBlock, 0, stream>>>(b);
     YITU_LAUNCH_CHECK();
     if (n_rows > 0) {
         plan_queue_kernel<<<(int)ceil_div(n_rows, kBlock), kBlock, 0, stream>>>(b, indptr,
                                                                                 (int)n_rows);
         YITU_LAUNCH_CHECK();
     }
-    int bits = 1;
-    while (((int64_t)1 << bits) < n_src) bits++;
-    const int grid = (int)ceil_div(b.max_items, kBlock);
-    plan_keys_kernel<<<grid, kBlock, 0, stream>>>(b, indptr, indices, col_mask,
-                                                  std::max(0, bits - 16));
+    if (with_slabs && nnz > 0) {
+        plan_popularity_kernel<<<(int)std::min<int64_t>(ceil_div(nnz, kBlock), 16384), kBlock, 0,
+                                 stream>>>(b, indices, nnz, col_mask, (int)n_src);
+        YITU_LAUNCH_CHECK();
+        plan_cost_kernel<<<(int)ceil_div(b.n_buckets, kBlock), kBlock, 0, stream>>>(b);
+        YITU_LAUNCH_CHECK();
+        size_t scan_bytes = b.scan_temp_bytes;
+        YITU_HIP(rocprim::inclusive_scan(b.scan_temp, scan_bytes, b.cost, b.cost,
+                                         (size_t)b.n_buckets,
+                                         rocprim::plus<unsigned long long>(), stream));
+        plan_bounds_kernel<<<1, kWave, 0, stream>>>(b);
+        YITU_LAUNCH_CHECK();
+    }
+    plan_items_kernel<<<(int)ceil_div(b.max_rows, kWavesPerBlock), kBlock, 0, stream>>>(
+        b, indptr, indices, col_mask, with_slabs && nnz > 0 ? 1 : 0);
     YITU_LAUNCH_CHECK();
     size_t temp_bytes = b.sort_temp_bytes;
     YITU_HIP(rocprim::radix_sort_pairs(b.sort_temp, temp_bytes, b.keys_in, b.keys_out, b.vals_in,
                                        b.order, (size_t)b.max_items, 0, 16, stream));
-    plan_records_kernel<<<grid, kBlock, 0, stream>>>(b, indptr);
+    plan_records_kernel<<<item_grid, kBlock, 0, stream>>>(b);
     YITU_LAUNCH_CHECK();
     return 0;
 }
@@ -242,7 +401,8 @@ int plan_resolve(PlanView &view, bool &has_items, const void *plan, const int32_
                  "workspace too small for a temporary row plan: need %zu bytes, got %zu", pb + bw,
                  workspace_bytes);
     char *w = static_cast<char *>(workspace);
-    int rc = plan_build(w, pb, indptr, indices, n_rows, n_src, nnz, col_mask, w + pb, bw, stream);
+    int rc = plan_build(w, pb, indptr, indices, n_rows, n_src, nnz, col_mask, false, w + pb, bw,
+                        stream);
     if (rc) return rc;
     view = plan_view(w, nnz);
     // the build scratch is dead once the records are written: hand it back
@@ -265,6 +425,6 @@ YITU_API int yitu_plan_build(void *plan, size_t plan_size, const int32_t *indptr
                              void *stream) {
     YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0, "negative size");
     YITU_REQUIRE(indptr && (nnz == 0 || indices), "null CSR");
-    return plan_build(plan, plan_size, indptr, indices, n_rows, n_src, nnz, col_mask, workspace,
-                      workspace_bytes, static_cast<hipStream_t>(stream));
+    return plan_build(plan, plan_size, indptr, indices, n_rows, n_src, nnz, col_mask, true,
+                      workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }

@@ -62,7 +62,6 @@ struct SpmmParams {
     int H;
     int col_mask;
     float alpha;   // output scale
-    int xcd_remap;
     PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
     float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
 };
@@ -233,9 +232,7 @@ template <int VEC, int G, int KT, int WMODE, typename TIN>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
-    int blk = blockIdx.x;
-    if (p.xcd_remap) blk = xcd_contiguous_block(blk, gridDim.x);
-    const int r0 = (blk * kWavesPerBlock + wave) * kRowsPerWave;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
     if (r0 >= p.n_rows) return;
     const int n_here = min(kRowsPerWave, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
@@ -288,79 +285,72 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
 
 constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave
 
-// Items in band order, kItemsPerWave per wave: the records of a wave's items
-// come from one load, their edge windows are all fetched before the first
-// feature gather, so the only waits per item are its own gathers. The unscaled
-// partial row goes to partial[item id]; the order only affects cache behaviour.
+// One group of up to kItemsPerWave consecutive records [pos0, pos0 + n_here):
+// the records come from one load, their edge windows are all fetched before the
+// first feature gather, so the only waits per item are its own gathers. The
+// unscaled partial row goes to partial[item id].
 template <int VEC, int G, int KT, int WMODE, typename TIN>
-__global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
-    static_assert(kPlanChunk <= kWave, "an item must fit one edge window");
+__device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, int n_here) {
     const int lane = lane_id();
     const int sub = lane % G;
     const int slot = lane / G;
-    if (p.plan.counters->overflow) return;
-    const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
-    const int4 *__restrict__ records = p.plan.records;
-    // Workgroups are dealt round-robin to the 8 XCDs; give every XCD its own
-    // contiguous eighth of the band-ordered list, so the 8 L2s hold 8 different
-    // bands instead of 8 copies of one.
-    const int n_groups = (n_items + kItemsPerWave - 1) / kItemsPerWave;  // one group per wave
-    const int share = (n_groups + 7) >> 3;
-    const int xcd = p.xcd_remap ? (blockIdx.x & 7) : 0;
-    const int waves_per_xcd = p.xcd_remap ? (gridDim.x >> 3) * kWavesPerBlock
-                                          : gridDim.x * kWavesPerBlock;
-    const int local0 = (p.xcd_remap ? (blockIdx.x >> 3) : blockIdx.x) * kWavesPerBlock +
-                       threadIdx.x / kWave;
-    const int lo = p.xcd_remap ? xcd * share : 0;
-    const int hi = p.xcd_remap ? min(n_groups, lo + share) : n_groups;
-    for (int grp = lo + local0; grp < hi; grp += waves_per_xcd) {
-        const int pos0 = grp * kItemsPerWave;
-        const int n_here = min(kItemsPerWave, n_items - pos0);
-        const int4 my_rec = records[pos0 + min(lane, n_here - 1)];
-        EdgeWindow win[kItemsPerWave];
-        int item_id[kItemsPerWave], n_edges[kItemsPerWave], row_tag[kItemsPerWave];
+    const int4 my_rec = p.plan.records[pos0 + min(lane, n_here - 1)];
+    EdgeWindow win[kItemsPerWave];
+    int item_id[kItemsPerWave], n_edges[kItemsPerWave], row_tag[kItemsPerWave];
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
-            const int beg = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item_id[j] = __shfl(my_rec.z, j, kWave);
-            row_tag[j] = __shfl(my_rec.w, j, kWave);
-            n_edges[j] = j < n_here ? end - beg : 0;
-            if (n_edges[j] > 0) load_window<WMODE>(win[j], p, beg, end);
-        }
+    for (int j = 0; j < kItemsPerWave; j++) {
+        const int beg = __shfl(my_rec.x, j, kWave);
+        const int end = __shfl(my_rec.y, j, kWave);
+        item_id[j] = __shfl(my_rec.z, j, kWave);
+        row_tag[j] = __shfl(my_rec.w, j, kWave);
+        n_edges[j] = j < n_here ? end - beg : 0;
+        if (n_edges[j] > 0) load_window<WMODE>(win[j], p, beg, end);
+    }
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
-            if (n_edges[j] <= 0) continue;
-            for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
-                const TileLanes<VEC, G, KT, WMODE> tl(p, c0);
-                float acc[KT][VEC];
+    for (int j = 0; j < kItemsPerWave; j++) {
+        if (n_edges[j] <= 0) continue;
+        for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
+            const TileLanes<VEC, G, KT, WMODE> tl(p, c0);
+            float acc[KT][VEC];
 #pragma unroll
-                for (int t = 0; t < KT; t++)
+            for (int t = 0; t < KT; t++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
-                accumulate_window<VEC, G, KT, WMODE, TIN>(acc, p, win[j], 0, n_edges[j], tl);
-                fold_slots<VEC, G, KT>(acc);
-                const bool single = row_tag[j] < 0;
-                const int row = row_tag[j] & 0x7fffffff;
-                float *dst = single ? p.out + (size_t)row * p.L
-                                    : p.partial + (size_t)item_id[j] * p.L;
-                const float sr =
-                    single ? (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha : 1.0f;
-                if (slot == 0) {
+                for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
+            accumulate_window<VEC, G, KT, WMODE, TIN>(acc, p, win[j], 0, n_edges[j], tl);
+            fold_slots<VEC, G, KT>(acc);
+            const bool single = row_tag[j] < 0;
+            const int row = row_tag[j] & 0x7fffffff;
+            float *dst = single ? p.out + (size_t)row * p.L : p.partial + (size_t)item_id[j] * p.L;
+            const float sr =
+                single ? (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha : 1.0f;
+            if (slot == 0) {
 #pragma unroll
-                    for (int t = 0; t < KT; t++) {
-                        const int o = c0 + (t * G + sub) * VEC;
-                        if (o < p.L) {
-                            float r[VEC];
+                for (int t = 0; t < KT; t++) {
+                    const int o = c0 + (t * G + sub) * VEC;
+                    if (o < p.L) {
+                        float r[VEC];
 #pragma unroll
-                            for (int i = 0; i < VEC; i++) r[i] = acc[t][i] * sr;
-                            store_row<VEC>(dst + o, r);
-                        }
+                        for (int i = 0; i < VEC; i++) r[i] = acc[t][i] * sr;
+                        store_row<VEC>(dst + o, r);
                     }
                 }
             }
         }
     }
+}
+
+// Items of the plan in band order, kItemsPerWave per wave. The order only
+// affects cache behaviour: every item writes its own row.
+template <int VEC, int G, int KT, int WMODE, typename TIN>
+__global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
+    static_assert(kPlanChunk <= kWave, "an item must fit one edge window");
+    if (p.plan.counters->overflow) return;
+    const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
+    const int n_groups = (n_items + kItemsPerWave - 1) / kItemsPerWave;
+    const int stride = gridDim.x * kWavesPerBlock;
+    for (int grp = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; grp < n_groups; grp += stride)
+        spmm_item_group<VEC, G, KT, WMODE, TIN>(p, grp * kItemsPerWave,
+                                                min(kItemsPerWave, n_items - grp * kItemsPerWave));
 }
 
 // Adds the chunk partials of every queued row and applies the row scale: the
@@ -421,7 +411,7 @@ static __global__ void zero_hub_counters_kernel(HubCounters *c) {
 // Host side: carve the queue out of a caller-provided workspace.
 int hub512_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t nnz);
 
-// Picks the instantiation for (element type, L) and launches the 1 + 3 kernels.
+// Picks the instantiation for (element type, L) and launches the row, item and reduce kernels.
 // max_degree_hint < 0 means unknown; plan may be null (a temporary one is then
 // built in the workspace). p.n_src and p.col_mask must be set.
 int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max_degree_hint,
