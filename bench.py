@@ -3,7 +3,8 @@
 
 Default workload (``c3_spmm_f32``): the large GCN SpMM of the baseline's third
 configuration -- R-MAT graph, 2^21 nodes, 63 M drawn edges (deduplicated, self
-loops added), CSR by destination, features [N,128] fp32, edge weight
+loops added), vertex ids renamed by the Rabbit-Order reorder (host library, a few
+seconds, untimed), CSR by destination, features [N,128] fp32, edge weight
 1/sqrt(d_i d_j). One step = forward aggregation of X plus backward aggregation
 of dY (the reference's backward applies the same CSR, YiTu_GNN_kernel.cu:447-461),
 both through the C ABI (yitu_agg_csr). ``value`` = edges / second with the
@@ -11,8 +12,9 @@ reference's definition: n_edges / (time of forward + backward)
 (YiTu_GNN/YiTu_H/test/bench_macro.py:371-391). Inputs are resident in HBM before
 the timed region.
 
-Prints ONE JSON line on stdout. Other workloads: ``--workload c3_spmm_bf16``,
-``c2_gat_f32``, ``c1_gcn_f32``.
+Prints ONE JSON line on stdout. Other workloads (also carried in ``extra`` of the
+default run): ``--workload c3_spmm_bf16``, ``c2_gat_f32``, ``c1_gcn_f32``,
+``c4_rgcn_f32``, ``c5_temporal_attention_f32``, ``c3_vertex_orders``.
 """
 import argparse
 import json
@@ -43,13 +45,32 @@ def _sync():
     torch.cuda.synchronize()
 
 
-def build_c3(dev, scale=21, draws=63_000_000, seed=20242):
+_c3_cache = {}
+
+
+def build_c3(dev, reorder=True, scale=21, draws=63_000_000, seed=20242):
+    """R-MAT graph of the third configuration as CSR by destination. With
+    ``reorder`` the vertex ids are renamed by the Rabbit-Order reorder of the host
+    library first (YiTu_GNN.rabbit.reorder, ccsrc/reorder/reorder.cpp:293-295), as
+    the configuration asks; the host time of that step is kept in ``reorder_s``."""
+    if reorder in _c3_cache:
+        return _c3_cache[reorder]
+    from yitu_amd import rabbit
     from yitu_amd.data import graphgen
     src, dst = graphgen.rmat(scale, draws, seed, self_loops=True, device=dev)
     n = 1 << scale
+    info = {"reorder_s": None}
+    if reorder:
+        ei = torch.stack([src, dst]).to(torch.int32).cpu()
+        t0 = time.perf_counter()
+        ei = rabbit.reorder(ei)
+        info["reorder_s"] = time.perf_counter() - t0
+        src, dst = ei[0].to(dev).long(), ei[1].to(dev).long()
+        del ei
     rp, ci = graphgen.csr_by_destination(src, dst, n)
     del src, dst
-    return n, rp, ci, graphgen.gcn_norm(rp)
+    _c3_cache[reorder] = (n, rp, ci, graphgen.gcn_norm(rp), info)
+    return _c3_cache[reorder]
 
 
 def agg_call(out, x, rp, ci, deg, plan, ws, maxdeg):
@@ -86,7 +107,7 @@ def cpu_baseline_spmm(rp, ci, deg, x, dy):
 
 def run_spmm(args, dev, bf16):
     from yitu_amd import _lib
-    n, rp, ci, deg = build_c3(dev)
+    n, rp, ci, deg, info = build_c3(dev)
     nnz = ci.numel()
     dim = 128
     g = torch.Generator(device=dev).manual_seed(20242)
@@ -137,7 +158,8 @@ def run_spmm(args, dev, bf16):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16-in/f32-acc" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": name, "graph": "R-MAT scale 21 (a,b,c,d)=(.57,.19,.19,.05), "
-                   "63M draws dedup + self loops, CSR by destination", "n_nodes": n,
+                   "63M draws dedup + self loops, vertex ids renamed by the Rabbit-Order "
+                   "reorder, CSR by destination", "reorder_host_s": info["reorder_s"], "n_nodes": n,
                    "n_edges": nnz, "max_in_degree": maxdeg, "feature_dim": dim,
                    "step": "aggregate(X) + aggregate(dY), same CSR, W = I"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -223,6 +245,225 @@ def run_gat(args, dev):
     }
 
 
+def _event_ms(fn, steps, warmup):
+    """Average time of fn() in ms over `steps` calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    _sync()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    _sync()
+    return e0.elapsed_time(e1) / steps
+
+
+def run_c1(args, dev):
+    """First configuration: GCN layer on an Erdos-Renyi graph (10^4 nodes, 10^5 drawn
+    edges + self loops), features [N,64] fp32, through the module-1 drop-in
+    (forward = aggregate(X W), backward = dX, dW). The working set (5.6 MB) sits in
+    L2: a latency / launch-bound case, reported as time and edges/s only."""
+    from yitu_amd import YiTu_GNN_kernel as K
+    from yitu_amd.data import graphgen
+    n, m, dim = 10_000, 100_000, 64
+    src, dst = graphgen.erdos_renyi(n, m, 20240, self_loops=True, device=dev)
+    rp, ci = graphgen.csr_by_destination(src, dst, n)
+    deg = graphgen.gcn_norm(rp)
+    nnz = ci.numel()
+    g = torch.Generator(device=dev).manual_seed(20240)
+    x = torch.randn(n, dim, generator=g, device=dev)
+    w = (torch.rand(dim, dim, generator=g, device=dev) - 0.5) / 4
+    dy = torch.ones(n, dim, device=dev)
+    pp, p2n = K.build_part(32, rp.cpu())
+    pp, p2n = pp.to(dev), p2n.to(dev)
+
+    def layer():
+        K.forward(x, w, rp, ci, deg, pp, p2n, 32, 32, 8)
+        K.backward(dy, x, w, rp, ci, deg, pp, p2n, 32, 32, 8)
+
+    out, dx = torch.empty(n, dim, device=dev), torch.empty(n, dim, device=dev)
+    ws = torch.empty(256, dtype=torch.uint8, device=dev)
+    maxdeg = int((rp[1:] - rp[:-1]).max().item())
+
+    def agg_only():
+        agg_call(out, x, rp, ci, deg, None, ws, maxdeg)
+        agg_call(dx, dy, rp, ci, deg, None, ws, maxdeg)
+
+    layer_ms = _event_ms(layer, max(args.steps, 50), args.warmup)
+    agg_ms = _event_ms(agg_only, max(args.steps, 50), args.warmup)
+    return {"value": nnz / (agg_ms * 1e-3), "unit": "edges/s", "ms_per_step": agg_ms, "dtype": "f32",
+            "config": {"workload": "c1_gcn_f32", "graph": "Erdos-Renyi 10^4 nodes, 10^5 draws + self "
+                       "loops", "n_edges": nnz, "feature_dim": dim,
+                       "step": "aggregate(X) + aggregate(dY) (two launches)"},
+            "layer_fwd_bwd_ms": layer_ms,
+            "note": "L2-resident and launch-bound: no roofline fraction"}
+
+
+def run_c4(args, dev):
+    """Fourth configuration: heterogeneous RGCN layer, 4 node types, 8 relations of
+    average degree 8, features 256. Forward: per-type GEMM H_t = X_t W_t on the
+    matrix cores, per-relation mean aggregation, sum over the relations of a
+    destination type. Backward: transposed aggregation, dW_t = X_t^T dH_t,
+    dX_t = dH_t W_t^T. The dominant dense kernel is the fp32 MFMA GEMM."""
+    from yitu_amd import YiTu_GNN_kernel as K, graph_ext
+    from yitu_amd.data import graphgen
+    sizes = [1 << 18, 1 << 17, 1 << 16, 1 << 15]
+    dim = 256
+    g = torch.Generator(device=dev).manual_seed(20243)
+    xs = [torch.randn(n, dim, generator=g, device=dev) for n in sizes]
+    wts = [torch.randn(dim, dim, generator=g, device=dev) * 0.02 for _ in sizes]
+    rels = []
+    for r in range(8):
+        s_t, d_t = r % 4, (r + 1 + r // 4) % 4
+        rp, ci = graphgen.bipartite_uniform(sizes[d_t], sizes[s_t], 8, 20243 + r, device=dev)
+        # the transposed structure for the backward aggregation (CSR by source)
+        rows = torch.repeat_interleave(torch.arange(sizes[d_t], device=dev),
+                                       (rp[1:] - rp[:-1]).long())
+        rp_t, ci_t = graphgen.csr_from_edges(ci.long(), rows, sizes[s_t], sizes[d_t])
+        indeg = (rp[1:] - rp[:-1]).float()
+        norm = torch.where(indeg > 0, 1.0 / indeg.clamp(min=1), torch.zeros_like(indeg))[:, None]
+        rels.append((s_t, d_t, rp, ci, rp_t, ci_t, norm))
+    n_edges = sum(int(r[3].numel()) for r in rels)
+    n_rel_dst = [sum(1 for r in rels if r[1] == t) for t in range(4)]
+    d_out = [torch.randn(n, dim, generator=g, device=dev) for n in sizes]
+
+    def gemm_fwd():
+        return [graph_ext.sgemm(x, w) for x, w in zip(xs, wts)]
+
+    def agg_fwd(hs):
+        outs = [None] * 4
+        for s_t, d_t, rp, ci, _, _, norm in rels:
+            o = K._aggregate(hs[s_t], rp, ci, None, 1.0) * norm
+            outs[d_t] = o if outs[d_t] is None else outs[d_t] + o
+        return [o / c for o, c in zip(outs, n_rel_dst)]
+
+    def agg_bwd():
+        dhs = [None] * 4
+        for s_t, d_t, _, _, rp_t, ci_t, norm in rels:
+            gsrc = K._aggregate(d_out[d_t] * (norm / n_rel_dst[d_t]), rp_t, ci_t, None, 1.0)
+            dhs[s_t] = gsrc if dhs[s_t] is None else dhs[s_t] + gsrc
+        return dhs
+
+    def gemm_bwd(dhs):
+        return ([graph_ext.sgemm(x, dh, trans_a=True) for x, dh in zip(xs, dhs)],
+                [graph_ext.sgemm(dh, w, trans_b=True) for dh, w in zip(dhs, wts)])
+
+    hs = gemm_fwd()
+    dhs = agg_bwd()
+    steps, warm = args.steps, args.warmup
+    t_gemm_f = _event_ms(gemm_fwd, steps, warm)
+    t_agg_f = _event_ms(lambda: agg_fwd(hs), steps, warm)
+    t_agg_b = _event_ms(agg_bwd, steps, warm)
+    t_gemm_b = _event_ms(lambda: gemm_bwd(dhs), steps, warm)
+    t_torch = _event_ms(lambda: [torch.mm(x, w) for x, w in zip(xs, wts)], steps, warm)
+    flops_f = sum(2 * n * dim * dim for n in sizes)
+    total = t_gemm_f + t_agg_f + t_agg_b + t_gemm_b
+    peak = 157.3  # fp32 matrix TFLOP/s, published
+    return {"value": n_edges / (total * 1e-3), "unit": "edges/s", "ms_per_step": total, "dtype": "f32",
+            "config": {"workload": "c4_rgcn_f32", "node_types": sizes, "relations": 8,
+                       "n_edges": n_edges, "feature_dim": dim},
+            "gemm_fwd_ms": t_gemm_f, "agg_fwd_ms": t_agg_f, "agg_bwd_ms": t_agg_b,
+            "gemm_bwd_ms": t_gemm_b, "torch_mm_fwd_ms": t_torch,
+            "roofline": {"bound": "mfma", "achieved": flops_f / (t_gemm_f * 1e-3) / 1e12,
+                         "peak": peak, "unit": "TFLOP/s",
+                         "frac": flops_f / (t_gemm_f * 1e-3) / 1e12 / peak, "traffic": None,
+                         "kernel": "sgemm_mfma_kernel, 4 typed GEMMs [n_t,256]x[256,256] fp32",
+                         "kernel_ms": t_gemm_f, "flops": flops_f,
+                         "bwd_achieved": 2 * flops_f / (t_gemm_b * 1e-3) / 1e12}}
+
+
+def run_c5(args, dev):
+    """Fifth configuration: temporal neighbour attention. 2^20 events over 2^17
+    nodes (Zipf 1.2 endpoints, sorted uniform times), T-CSR with reverse edges;
+    a batch of 2,048 query nodes takes its 20 most recent neighbours (host
+    sampler), then one attention layer (time encoding dim 100, node memory 172,
+    one head) runs forward + backward on the GPU."""
+    import numpy as np
+    from yitu_amd import sampler_core
+    from yitu_amd.temporal import TemporalBlock, TransfomerAttentionLayer
+    rng = np.random.default_rng(20244)
+    n_nodes, n_events, k, batch = 1 << 17, 1 << 20, 20, 2048
+    src = ((rng.zipf(1.2, n_events) - 1) % n_nodes).astype(np.int64)
+    dst = ((rng.zipf(1.2, n_events) - 1) % n_nodes).astype(np.int64)
+    ts = np.sort(rng.uniform(0, 1e6, n_events)).astype(np.float32)
+    # T-CSR: per node, its events (both directions) in time order
+    node = np.concatenate([src, dst])
+    other = np.concatenate([dst, src])
+    eid = np.concatenate([np.arange(n_events), np.arange(n_events)])
+    tt = np.concatenate([ts, ts])
+    order = np.lexsort((eid, tt, node))
+    indptr = np.zeros(n_nodes + 1, np.int64)
+    indptr[1:] = np.cumsum(np.bincount(node, minlength=n_nodes))
+    smp = sampler_core.ParallelSampler(indptr, other[order], eid[order], tt[order], 16, 1, 1, [k],
+                                       True, False, 1, 0.0)
+    ev = rng.integers(n_events * 9 // 10, n_events, batch // 2)
+    roots = np.concatenate([src[ev], dst[ev]])
+    root_ts = np.concatenate([ts[ev], ts[ev]])
+    smp.sample(roots, root_ts)  # warm-up
+    t0 = time.perf_counter()
+    for _ in range(5):
+        smp.reset()
+        smp.sample(roots, root_ts)
+    sample_ms = (time.perf_counter() - t0) * 1e3 / 5
+    tgb = smp.get_ret()[0]
+    torch.manual_seed(20244)
+    memory = torch.randn(n_nodes, 172, device=dev)
+    layer = TransfomerAttentionLayer(172, 0, 100, 1, 0.0, 0.0, 100).to(dev)
+    blk = TemporalBlock.from_sampler(tgb, memory, device=dev)
+    blk.h.requires_grad_()
+    gout = torch.randn(blk.n_dst, 100, device=dev)
+
+    def step():
+        out = layer(blk)
+        out.backward(gout)
+        blk.h.grad = None
+        layer.zero_grad(set_to_none=True)
+
+    ms = _event_ms(step, max(args.steps, 20), args.warmup)
+    return {"value": ms, "unit": "ms", "ms_per_step": ms, "dtype": "f32", "higher_is_better": False,
+            "config": {"workload": "c5_temporal_attention_f32", "n_nodes": n_nodes,
+                       "n_events": n_events, "batch": batch, "neighbours": k,
+                       "sampled_edges": blk.num_edges()},
+            "sampler_ms": sample_ms, "sampler_threads": 16,
+            "note": "45 MB working set, launch-bound: time only"}
+
+
+def run_c3_orders(args, dev):
+    """Third configuration under other vertex orders than the default run's (the
+    generator's ids passed through the Rabbit-Order reorder): the generator's own
+    ids (R-MAT puts its hot vertices at ids with few set bits, i.e. at feature rows
+    whose addresses differ by large powers of two), a random relabelling, and the
+    random relabelling passed through the reorder. fp32 aggregation, one call."""
+    from yitu_amd import YiTu_GNN_kernel as K, rabbit
+    from yitu_amd.data import graphgen
+    n, rp, ci, deg, _ = build_c3(dev, reorder=False)
+    g = torch.Generator(device=dev).manual_seed(20242)
+    x = torch.randn(n, 128, generator=g, device=dev)
+    res = {}
+    res["generator_ids_ms"] = _event_ms(lambda: K._aggregate(x, rp, ci, deg, 1.0), args.steps,
+                                        args.warmup)
+    rows = torch.repeat_interleave(torch.arange(n, device=dev), (rp[1:] - rp[:-1]).long())
+    perm = torch.randperm(n, generator=g, device=dev)
+    src_s, dst_s = perm[ci.long()], perm[rows]
+    del rows
+    rp_s, ci_s = graphgen.csr_by_destination(src_s, dst_s, n)
+    deg_s = graphgen.gcn_norm(rp_s)
+    res["random_ids_ms"] = _event_ms(lambda: K._aggregate(x, rp_s, ci_s, deg_s, 1.0), args.steps,
+                                     args.warmup)
+    ei = torch.stack([src_s, dst_s]).to(torch.int32).cpu()
+    t0 = time.perf_counter()
+    ei_r = rabbit.reorder(ei)
+    res["rabbit_reorder_host_s"] = time.perf_counter() - t0
+    ei_r = ei_r.to(dev)
+    rp_r, ci_r = graphgen.csr_by_destination(ei_r[0].long(), ei_r[1].long(), n)
+    deg_r = graphgen.gcn_norm(rp_r)
+    res["random_then_rabbit_ids_ms"] = _event_ms(lambda: K._aggregate(x, rp_r, ci_r, deg_r, 1.0), args.steps,
+                                     args.warmup)
+    res["n_edges"] = int(ci.numel())
+    return res
+
+
 def calibration_copy(dev, n_bytes=1 << 30, reps=5):
     """1 GiB streaming copy through the library's copy kernel: the known-size
     launch that FETCH_SIZE / WRITE_SIZE are scaled by, and the achievable
@@ -253,6 +494,9 @@ def main():
     ap.add_argument("--workload", default="c3_spmm_f32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="default workload only")
+    ap.add_argument("--orders", action="store_true",
+                    help="also time the third configuration under random and Rabbit-reordered "
+                         "vertex ids (adds about a minute of host-side reorder)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)")
@@ -269,11 +513,24 @@ def main():
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
                                                 "roofline") if k in r}
             res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
-                            "c2_gat_f32": slim(run_gat(args, dev))}
+                            "c2_gat_f32": slim(run_gat(args, dev)),
+                            "c1_gcn_f32": run_c1(args, dev),
+                            "c4_rgcn_f32": run_c4(args, dev),
+                            "c5_temporal_attention_f32": run_c5(args, dev)}
+            if args.orders:
+                res["extra"]["c3_vertex_orders"] = run_c3_orders(args, dev)
     elif args.workload == "c3_spmm_bf16":
         res = run_spmm(args, dev, bf16=True)
     elif args.workload == "c2_gat_f32":
         res = run_gat(args, dev)
+    elif args.workload == "c1_gcn_f32":
+        res = run_c1(args, dev)
+    elif args.workload == "c4_rgcn_f32":
+        res = run_c4(args, dev)
+    elif args.workload == "c5_temporal_attention_f32":
+        res = run_c5(args, dev)
+    elif args.workload == "c3_vertex_orders":
+        res = run_c3_orders(args, dev)
     else:
         sys.exit("unknown workload %s" % args.workload)
     print(json.dumps(res))
