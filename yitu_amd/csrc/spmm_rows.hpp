@@ -353,19 +353,83 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
                                                 min(kItemsPerWave, n_items - grp * kItemsPerWave));
 }
 
-// Adds the chunk partials of every queued row and applies the row scale: the
-// only writer of a hub row of the output. The 256 threads form `groups` teams of
-// `lanes` threads; team g adds chunks g, g + groups, ... and the team sums are
-// then added in team order, so the result is a fixed function of the chunk count.
+// Adds the item partials of every planned row with more than one item and
+// applies the row scale: the only writer of such a row of the output. The sum is
+// a fixed function of the item count (bitwise reproducible):
+//  * rows of up to kReduceWaveItems items: one wave per row. The row vector is
+//    spread over `lanes` lanes, the wave's 64 / lanes slots add items slot,
+//    slot + slots, ... and the slot sums are folded by a fixed butterfly;
+//  * longer rows: one workgroup per row, its 256 / lanes teams add items
+//    team, team + teams, ...; the team sums are then added in team order.
+// Blocks [0, gridDim.x / 2) take the first kind, the others the second.
+// s += src[c * L] for c = first, first + step, ... < n, added in that order;
+// four loads are in flight at a time.
+template <int VEC>
+__device__ __forceinline__ void sum_partials(float (&s)[VEC], const float *src, int L, int first,
+                                             int n, int step) {
+    int c = first;
+    for (; c + 3 * step < n; c += 4 * step) {
+        float v[4][VEC];
+#pragma unroll
+        for (int u = 0; u < 4; u++) RowLoad<VEC, float>::ld(src + (size_t)(c + u * step) * L, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < VEC; i++) s[i] += v[u][i];
+    }
+    for (; c < n; c += step) {
+        float v[VEC];
+        RowLoad<VEC, float>::ld(src + (size_t)c * L, v);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) s[i] += v[i];
+    }
+}
+
+constexpr int kReduceWaveItems = 32;
+
 template <int WMODE, int VEC>
 __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
     __shared__ float red[kBlock * VEC];
     if (p.plan.counters->overflow) return;
     const int n_hub = min(p.plan.counters->n_rows, p.plan.max_rows);
     const int lanes_total = p.L / VEC;  // VEC divides L (host picks VEC)
-    for (int h = blockIdx.x; h < n_hub; h += gridDim.x) {
+    const int half = gridDim.x / 2;
+    if ((int)blockIdx.x < half) {
+        const int lane = lane_id();
+        // lanes per row vector: the power of two >= lanes_total, at most 64
+        int lanes = 1;
+        while (lanes < lanes_total && lanes < kWave) lanes <<= 1;
+        const int slots = kWave / lanes;
+        const int slot = lane / lanes, sub = lane % lanes;
+        const int stride = half * kWavesPerBlock;
+        for (int h = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; h < n_hub; h += stride) {
+            const int4 r = p.plan.rows[h];
+            if (r.z <= 1 || r.z > kReduceWaveItems) continue;
+            const float sr = (WMODE == W_DEGPROD ? p.scale_row[r.x] : 1.0f) * p.alpha;
+            for (int l0 = 0; l0 < lanes_total; l0 += lanes) {
+                const bool live = l0 + sub < lanes_total;
+                float s[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; i++) s[i] = 0.0f;
+                if (live) {
+                    const float *src = p.partial + (size_t)r.y * p.L + (size_t)(l0 + sub) * VEC;
+                    sum_partials<VEC>(s, src, p.L, slot, r.z, slots);
+                }
+                for (int o = kWave / 2; o >= lanes; o >>= 1)
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) s[i] += __shfl_xor(s[i], o, kWave);
+                if (live && slot == 0) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) s[i] *= sr;
+                    store_row<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + sub) * VEC, s);
+                }
+            }
+        }
+        return;
+    }
+    for (int h = blockIdx.x - half; h < n_hub; h += gridDim.x - half) {
         const int4 r = p.plan.rows[h];
-        if (r.z <= 1) continue;  // single-item rows were written by the item kernel
+        if (r.z <= kReduceWaveItems) continue;  // short rows: the wave path; single items: done
         const float sr = (WMODE == W_DEGPROD ? p.scale_row[r.x] : 1.0f) * p.alpha;
         for (int l0 = 0; l0 < lanes_total; l0 += kBlock) {
             const int lanes = min(kBlock, lanes_total - l0);
@@ -375,13 +439,8 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
 #pragma unroll
             for (int i = 0; i < VEC; i++) s[i] = 0.0f;
             if (g < groups) {
-                for (int c = g; c < r.z; c += groups) {
-                    float v[VEC];
-                    RowLoad<VEC, float>::ld(
-                        p.partial + (size_t)(r.y + c) * p.L + (size_t)(l0 + l) * VEC, v);
-#pragma unroll
-                    for (int i = 0; i < VEC; i++) s[i] += v[i];
-                }
+                const float *src = p.partial + (size_t)r.y * p.L + (size_t)(l0 + l) * VEC;
+                sum_partials<VEC>(s, src, p.L, g, r.z, groups);
             }
             __syncthreads();
 #pragma unroll
