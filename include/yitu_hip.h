@@ -240,6 +240,22 @@ int yitu_b2gemm_backward(float *dx_device, float *dw_a_device, float *dw_b_devic
                          int64_t k, int64_t m, void *workspace_device, size_t workspace_bytes,
                          void *stream);
 
+/*
+ * C[m,n] = A[m,k] . op(B) with bf16 operands and fp32 accumulation on the matrix
+ * cores; C is fp32 or bf16 (round to nearest even). A is row-major [m, lda];
+ * trans_b: B is stored [n, ldb] (the layout of a Linear weight), else [k, ldb]
+ * (it is then transposed into the workspace, yitu_gemm_bf16_workspace_bytes).
+ * k and the leading dimensions of the K-contiguous operands must be multiples
+ * of 8. The bf16 form of the per-type / per-relation feature transform of the
+ * heterogeneous layers (fc_cuda.cu:4-75 and the nn.Linear calls of
+ * YiTu_H/test/common/model.py:25-29, 86-88, which the reference runs in fp32).
+ */
+size_t yitu_gemm_bf16_workspace_bytes(int64_t n, int64_t k, int trans_b);
+int yitu_gemm_bf16(void *c_device, int c_is_bf16, const void *a_bf16_device,
+                   const void *b_bf16_device, int64_t m, int64_t n, int64_t k, int trans_b,
+                   int64_t lda, int64_t ldb, int64_t ldc, void *workspace_device,
+                   size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */
 /* ------------------------------------------------------------------------- */

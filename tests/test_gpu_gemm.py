@@ -92,3 +92,31 @@ def test_b2gemm_against_oracle(dev):
     assert_close(dx, want_dx)
     assert_close(dwa, want_dwa, atol=1e-4 * 64)
     assert_close(dwb, want_dwb, atol=1e-4 * 64)
+
+
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 8), (7, 5, 16), (128, 256, 32), (130, 257, 40),
+                                   (1000, 100, 104), (4096, 256, 256), (300, 512, 0)])
+def test_gemm_bf16_against_double(dev, tb, out_dtype, m, n, k):
+    """bf16 operands are exact in fp32, so the product differs from the double one by the
+    fp32 accumulation only (and by one bf16 rounding when the output is bf16)."""
+    g = torch.Generator().manual_seed(m + 3 * n + 5 * k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    b = torch.randn((n, k) if tb else (k, n), generator=g).to(torch.bfloat16)
+    got = graph_ext.gemm_bf16(a.to(dev), b.to(dev), trans_b=tb, out_dtype=out_dtype)
+    want = a.double() @ (b.double().t() if tb else b.double())
+    assert got.dtype == out_dtype and got.shape == (m, n)
+    if out_dtype == torch.float32:
+        assert_close(got, want.float(), atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+    else:
+        # one bf16 rounding (relative 2^-9) on top of the fp32 accumulation error
+        assert_close(got.float(), want.float(), rtol=2.0 ** -8,
+                     atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+
+
+def test_gemm_bf16_rejects_unaligned_k(dev):
+    a = torch.zeros(4, 12, dtype=torch.bfloat16, device=dev)
+    b = torch.zeros(12, 4, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        graph_ext.gemm_bf16(a, b)

@@ -88,6 +88,21 @@ def backward(d_output, X, W, row_pointers, column_index, degrees, part_pointers,
     return [_mm(g, W, trans_b=True), _mm(X, g, trans_a=True)]
 
 
+def backward_transposed(d_output, X, W, row_pointers, column_index, degrees, part_pointers,
+                        part2Node, partSize, dimWorker, warpPerBlock):
+    """The gradient of ``forward`` for graphs that are not symmetric: dY is
+    aggregated over the TRANSPOSED structure (G = A^T.dY), then dX = G.W^T,
+    dW = X^T.G. Not in the reference, whose ``backward`` reuses the forward CSR
+    (cu:447-461) and is therefore exact for symmetric graphs only. Same
+    arguments as ``backward``; the by-source structure is built on the device on
+    first use and cached. Node ids must fit 24 bits."""
+    _check_inputs(d_output, X, W, row_pointers, column_index, degrees, part_pointers, part2Node)
+    from . import graph_ext
+    t = graph_ext.transposed(row_pointers, column_index, X.shape[0])
+    g = _aggregate(d_output, t.t_indptr, t.t_rows, degrees, 1.0)
+    return [_mm(g, W, trans_b=True), _mm(X, g, trans_a=True)]
+
+
 def forward_gin(input, weight, row_pointers, column_index, epsilon, part_pointers, part2Node,
                 partSize, dimWorker, warpPerBlock):
     """GIN: A = eps * sum_j X[j]; out = A.W (YiTu_GNN.cpp:150-172; cu:563-618). Returns [out, A]."""

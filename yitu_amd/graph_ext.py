@@ -329,6 +329,30 @@ def sgemm(a, b, trans_a=False, trans_b=False):
     return c
 
 
+def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32):
+    """a . op(b) with bf16 operands and fp32 accumulation on the matrix cores.
+    ``a`` [m, k]; ``b`` [k, n], or [n, k] with ``trans_b`` (a Linear weight)."""
+    _check(a, torch.bfloat16, "a", 2)
+    _check(b, torch.bfloat16, "b", 2)
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise RuntimeError("out_dtype must be float32 or bfloat16")
+    dev = _lib.require_device(a, b)
+    m, k = a.shape
+    n, kb = (b.size(0), b.size(1)) if trans_b else (b.size(1), b.size(0))
+    if k != kb:
+        raise RuntimeError("inner dimensions differ: %d vs %d" % (k, kb))
+    c = torch.empty((m, n), dtype=out_dtype, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_gemm_bf16_workspace_bytes")(c_i64(n), c_i64(k),
+                                                                  c_int(int(trans_b))), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gemm_bf16(ptr(c), c_int(int(out_dtype == torch.bfloat16)), ptr(a),
+                                       ptr(b), c_i64(m), c_i64(n), c_i64(k), c_int(int(trans_b)),
+                                       c_i64(a.size(1)), c_i64(b.size(1)), c_i64(n), ptr(ws),
+                                       c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_gemm_bf16")
+    return c
+
+
 # --------------------------------------------------------------------------- #
 # fused GAT attention (extension: the composition sddmm_forward -> spmm_forward)
 # --------------------------------------------------------------------------- #
