@@ -158,14 +158,14 @@ YITU_API int yitu_sddmm_forward(float *attn, const int32_t *indptr, const int32_
     return sddmm_fwd_dispatch(p, with_hub, static_cast<hipStream_t>(stream));
 }
 
-YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad_edge,
-                                 const int32_t *indptr, const int32_t *indices, const float *query,
-                                 const float *key, const float *attn, const float *grad_out,
-                                 const int32_t *t_indptr, const int32_t *t_perm, int64_t n_dst,
-                                 int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                 int64_t max_degree, int64_t max_degree_t, const void *plan_t,
-                                 void *workspace, size_t workspace_bytes, void *stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+namespace yitu {
+int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, const int32_t *indptr,
+                       const int32_t *indices, const float *query, const float *key,
+                       const float *attn, const float *grad_out, const int32_t *t_indptr,
+                       const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
+                       int64_t n_heads, int64_t n_bid, int64_t max_degree, int64_t max_degree_t,
+                       const void *plan_t, void *workspace, size_t workspace_bytes, int skip_below,
+                       hipStream_t stream) {
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
     if (n_heads == 0) return 0;
@@ -178,7 +178,7 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
         rc = fill_zero(grad_key, n_src * n_heads, stream);
         if (rc) return rc;
     }
-    if (n_dst > 0) {
+    if (n_dst > 0 && skip_below != INT32_MAX) {  // INT32_MAX: only the grad_key gather is wanted
         SddmmParams p{};
         p.indptr = indptr;
         p.indices = indices;
@@ -192,6 +192,7 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
         p.n_dst = (int)n_dst;
         p.H = (int)n_heads;
         p.n_bid = (int)n_bid;
+        p.skip_below = skip_below;
         bool with_hub;
         rc = sddmm_setup(p, nnz, max_degree, workspace, workspace_bytes, with_hub);
         if (rc) return rc;
@@ -217,4 +218,18 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
                            workspace_bytes, stream);
     }
     return 0;
+}
+}  // namespace yitu
+
+YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad_edge,
+                                 const int32_t *indptr, const int32_t *indices, const float *query,
+                                 const float *key, const float *attn, const float *grad_out,
+                                 const int32_t *t_indptr, const int32_t *t_perm, int64_t n_dst,
+                                 int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
+                                 int64_t max_degree, int64_t max_degree_t, const void *plan_t,
+                                 void *workspace, size_t workspace_bytes, void *stream_) {
+    return sddmm_backward_run(grad_query, grad_key, grad_edge, indptr, indices, query, key, attn,
+                              grad_out, t_indptr, t_perm, n_dst, n_src, nnz, n_heads, n_bid,
+                              max_degree, max_degree_t, plan_t, workspace, workspace_bytes, 0,
+                              static_cast<hipStream_t>(stream_));
 }

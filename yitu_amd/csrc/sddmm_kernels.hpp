@@ -37,6 +37,7 @@ struct SddmmParams {
     int H;
     int n_bid;
     int hub_threshold;
+    int skip_below;  // bwd: rows with fewer edges were handled by another kernel
     HubQueue hub;   // hub.partial = per-item statistics [item][n_bid][H][3]
     float *rowstat; // [hub row][n_bid][H][3]
 };
@@ -287,6 +288,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_bwd_rows_kernel(SddmmParams p) {
     const int row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
     if (row >= p.n_dst) return;
     const int beg = p.indptr[row], end = p.indptr[row + 1];
+    if (end - beg < p.skip_below) return;
     const int lane = lane_id(), hl = lane % HP;
     const bool hub = end - beg >= p.hub_threshold;
     if (hub) queue_hub_row(p.hub, row, end - beg);
@@ -394,5 +396,15 @@ __global__ __launch_bounds__(kBlock) void sddmm_bwd_hub_apply_kernel(SddmmParams
         }
     }
 }
+
+// The body of yitu_sddmm_backward; rows with fewer than skip_below edges are
+// left alone (the fused GAT backward has already written their results).
+int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, const int32_t *indptr,
+                       const int32_t *indices, const float *query, const float *key,
+                       const float *attn, const float *grad_out, const int32_t *t_indptr,
+                       const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
+                       int64_t n_heads, int64_t n_bid, int64_t max_degree, int64_t max_degree_t,
+                       const void *plan_t, void *workspace, size_t workspace_bytes, int skip_below,
+                       hipStream_t stream);
 
 }  // namespace yitu

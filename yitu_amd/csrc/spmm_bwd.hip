@@ -14,6 +14,7 @@ struct DotParams {
     const float *grad_out;  // [n_dst, L]
     float *grad_a;          // [nnz, H]
     int lph;  // lanes per head (F / VEC) when that is a power of two <= G, else 0
+    int long_rows_only;  // the rows below the plan threshold were handled by another kernel
 };
 
 // Dot products of the row's grad_out tile `gt` with the n edges in window lanes
@@ -170,9 +171,11 @@ __global__ __launch_bounds__(kBlock) void dot_items_kernel(DotParams p) {
 
 template <int VEC, int G, int KT>
 static int dot_launch(const DotParams &p, bool has_items, hipStream_t stream) {
-    dot_rows_kernel<VEC, G, KT>
-        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
+    if (!p.long_rows_only) {
+        dot_rows_kernel<VEC, G, KT>
+            <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+    }
     if (has_items) {
         const int grid = (int)std::min<int64_t>(
             ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
@@ -199,20 +202,16 @@ static int dot_dispatch(DotParams &p, bool has_items, hipStream_t stream) {
     }
 }
 
-}  // namespace yitu
 
-using namespace yitu;
-#define YITU_API extern "C" __attribute__((visibility("default")))
-
-YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *values,
-                                const int32_t *indptr, const int32_t *indices,
-                                const float *features, const float *grad_out,
-                                const int32_t *t_indptr, const int32_t *t_rows,
-                                const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
-                                int64_t n_heads, int64_t n_features, int64_t max_degree,
-                                int64_t max_degree_t, const void *plan, const void *plan_t,
-                                void *workspace, size_t workspace_bytes, void *stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+// The body of yitu_spmm_backward. With long_rows_only the per-edge dot skips
+// the rows below the plan threshold (the fused GAT backward has done them).
+int spmm_backward_run(float *grad_a, float *grad_x, const float *values, const int32_t *indptr,
+                      const int32_t *indices, const float *features, const float *grad_out,
+                      const int32_t *t_indptr, const int32_t *t_rows, const int32_t *t_perm,
+                      int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                      int64_t n_features, int64_t max_degree, int64_t max_degree_t,
+                      const void *plan, const void *plan_t, void *workspace,
+                      size_t workspace_bytes, bool long_rows_only, hipStream_t stream) {
     YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
                  "negative size");
     const int64_t L = n_heads * n_features;
@@ -238,6 +237,7 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
         p.sp.col_mask = 0xffffff;
         p.grad_out = grad_out;
         p.grad_a = grad_a;
+        p.long_rows_only = long_rows_only ? 1 : 0;
         bool has_items = false;
         void *rest = nullptr;
         size_t rest_bytes = 0;
@@ -274,4 +274,23 @@ YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *value
                            workspace_bytes, stream);
     }
     return 0;
+}
+
+}  // namespace yitu
+
+using namespace yitu;
+#define YITU_API extern "C" __attribute__((visibility("default")))
+
+YITU_API int yitu_spmm_backward(float *grad_a, float *grad_x, const float *values,
+                                const int32_t *indptr, const int32_t *indices,
+                                const float *features, const float *grad_out,
+                                const int32_t *t_indptr, const int32_t *t_rows,
+                                const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
+                                int64_t n_heads, int64_t n_features, int64_t max_degree,
+                                int64_t max_degree_t, const void *plan, const void *plan_t,
+                                void *workspace, size_t workspace_bytes, void *stream_) {
+    return spmm_backward_run(grad_a, grad_x, values, indptr, indices, features, grad_out, t_indptr,
+                             t_rows, t_perm, n_dst, n_src, nnz, n_heads, n_features, max_degree,
+                             max_degree_t, plan, plan_t, workspace, workspace_bytes, false,
+                             static_cast<hipStream_t>(stream_));
 }
