@@ -261,6 +261,20 @@ int yitu_gemm_bf16(void *c_device, int c_is_bf16, const void *a_bf16_device,
 /* ------------------------------------------------------------------------- */
 
 /*
+ * Edge list -> canonical CSR on the device: rows ascending, columns ascending
+ * inside a row, duplicate edges merged, int32 -- the form the reference gets
+ * from scipy's coo_matrix(...).tocsr() (YiTu_GNN/data/dataset.py:116-129).
+ * indices_device must hold n_edges entries; the number of distinct edges is
+ * written to *nnz_device (a device int64; -1 if an id is out of range).
+ * Workspace 256-byte aligned.
+ */
+size_t yitu_coo_to_csr_workspace_bytes(int64_t n_edges, int64_t n_rows);
+int yitu_coo_to_csr(int32_t *indptr_device, int32_t *indices_device, long long *nnz_device,
+                    const int32_t *rows_device, const int32_t *cols_device, int64_t n_edges,
+                    int64_t n_rows, int64_t n_cols, void *workspace_device, size_t workspace_bytes,
+                    void *stream);
+
+/*
  * By-source (transposed) view of a CSR, built once per graph on the device.
  * The reference has no such step: its backward kernels scatter with atomics
  * (spmm_cuda.cu:33-38, sddmm_cuda.cu:59-63); this turns those scatters into

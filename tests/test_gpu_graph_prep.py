@@ -1,0 +1,63 @@
+"""Device-side edge list -> canonical CSR (yitu_coo_to_csr) against scipy's
+coo_matrix(...).tocsr(), the routine the reference's dataset loader uses
+(YiTu_GNN/data/dataset.py:116-129). Integer work: bit-exact."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+
+from yitu_amd.data import csr, graphgen
+
+pytestmark = pytest.mark.gpu
+
+
+def _scipy_csr(rows, cols, n_rows, n_cols):
+    m = sp.coo_matrix((np.ones(rows.size, np.float32), (rows, cols)), shape=(n_rows, n_cols)).tocsr()
+    m.sum_duplicates()
+    m.sort_indices()
+    return m.indptr.astype(np.int32), m.indices.astype(np.int32)
+
+
+@pytest.mark.parametrize("n_rows,n_cols,n_edges,seed", [
+    (1, 1, 1, 0), (10, 10, 0, 1), (100, 100, 1000, 2), (257, 33, 5000, 3), (33, 4000, 5000, 4),
+    (5000, 5000, 200000, 5), (3, 3, 10000, 6)])
+def test_matches_scipy(dev, n_rows, n_cols, n_edges, seed):
+    rng = np.random.default_rng(seed)
+    rows = rng.integers(0, n_rows, n_edges)
+    cols = rng.integers(0, n_cols, n_edges)
+    indptr, indices = csr.coo_to_csr(torch.from_numpy(rows).to(dev), torch.from_numpy(cols).to(dev),
+                                     n_rows, n_cols)
+    want_ptr, want_idx = _scipy_csr(rows, cols, n_rows, n_cols)
+    assert indptr.dtype == torch.int32 and indices.dtype == torch.int32
+    assert np.array_equal(indptr.cpu().numpy(), want_ptr)
+    assert np.array_equal(indices.cpu().numpy(), want_idx)
+
+
+def test_power_law_graph_matches_the_host_build(dev):
+    """2^18 nodes, 4 M draws with many duplicates: same bits as the torch build."""
+    src, dst = graphgen.rmat(18, 4_000_000, 9, self_loops=True, device=dev)
+    want_ptr, want_idx = graphgen.csr_by_destination(src, dst, 1 << 18)
+    indptr, indices = csr.coo_to_csr(dst, src, 1 << 18)
+    assert torch.equal(indptr, want_ptr) and torch.equal(indices, want_idx)
+
+
+def test_out_of_range_id_is_an_error(dev):
+    rows = torch.tensor([0, 1, 5], device=dev)
+    cols = torch.tensor([0, 1, 2], device=dev)
+    with pytest.raises(RuntimeError, match="outside"):
+        csr.coo_to_csr(rows, cols, 4, 4)
+    with pytest.raises(RuntimeError, match="outside"):
+        csr.coo_to_csr(cols, torch.tensor([0, -1, 2], device=dev), 4, 4)
+
+
+def test_common_dataset_builds_its_csr_on_the_device(dev):
+    from yitu_amd.data.dataset import CommonDataset
+    rng = np.random.default_rng(0)
+    ei = rng.integers(0, 500, (2, 6000))
+    ds = CommonDataset(None, 8, 3, edge_index=ei, num_nodes=500, device=dev)
+    want_ptr, want_idx = _scipy_csr(ei[0], ei[1], 500, 500)
+    assert not ds.row_pointers.is_cuda and ds.row_pointers.dtype == torch.int32
+    assert np.array_equal(ds.row_pointers.numpy(), want_ptr)
+    assert np.array_equal(ds.column_index.numpy(), want_idx)
+    assert torch.allclose(ds.degrees.cpu(), torch.sqrt(torch.clamp(
+        torch.from_numpy(np.diff(want_ptr)).float(), min=1.0)))

@@ -1,14 +1,16 @@
-// One-time integer graph preparation on the device: the transposed (by-source)
-// view of a CSR with the edge permutation that links the two orders. The
-// backward kernels use it to turn scatter-adds into gathers.
+// One-time integer graph preparation on the device: edge list -> canonical CSR,
+// and the transposed (by-source) view of a CSR with the edge permutation that
+// links the two orders. The backward kernels use the latter to turn
+// scatter-adds into gathers.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_select.hpp>
 
 #include "../../include/yitu_hip.h"
-#include "common.hpp"
+#include "spmm_rows.hpp"
 
 namespace yitu {
 
@@ -52,6 +54,64 @@ __global__ __launch_bounds__(kBlock) void transpose_rows_kernel(const int32_t *_
             hi = mid;
     }
     t_rows[j] = lo;
+}
+
+
+// ---- edge list -> canonical CSR ---------------------------------------------------
+__global__ __launch_bounds__(kBlock) void coo_keys_kernel(const int32_t *__restrict__ rows,
+                                                          const int32_t *__restrict__ cols,
+                                                          unsigned long long *__restrict__ keys,
+                                                          int64_t n_edges, int32_t n_rows,
+                                                          int32_t n_cols, int *__restrict__ bad) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_edges) return;
+    const int32_t r = rows[i], c = cols[i];
+    if (r < 0 || r >= n_rows || c < 0 || c >= n_cols) {
+        atomicExch(bad, 1);
+        keys[i] = ~0ull;  // sorts last; the count below excludes it
+    } else {
+        keys[i] = ((unsigned long long)(uint32_t)r << 32) | (uint32_t)c;
+    }
+}
+
+// unique sorted keys -> indices; indptr[r] = first position whose key is >= (r, 0)
+__global__ __launch_bounds__(kBlock) void coo_finish_kernel(
+    const unsigned long long *__restrict__ uniq, const size_t *__restrict__ n_unique,
+    const int *__restrict__ bad, int32_t *__restrict__ indptr, int32_t *__restrict__ indices,
+    long long *__restrict__ nnz_out, int32_t n_rows, int64_t n_edges) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    // an out-of-range edge leaves one ~0 key at the end of the unique list
+    const int64_t nnz = (int64_t)*n_unique - (*bad ? 1 : 0);
+    if (i == 0) *nnz_out = *bad ? -1 : nnz;
+    if (i < nnz) indices[i] = (int32_t)(uniq[i] & 0xffffffffull);
+    if (i <= n_rows) {
+        const unsigned long long first = (unsigned long long)i << 32;
+        int64_t lo = 0, hi = nnz;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (uniq[mid] < first) lo = mid + 1; else hi = mid;
+        }
+        indptr[i] = (int32_t)lo;
+    }
+}
+
+static int coo_key_bits(int64_t n_rows) {
+    int b = 1;
+    while (((int64_t)1 << b) < n_rows) b++;
+    return 32 + b;
+}
+
+struct CooTemp {
+    size_t sort_bytes, unique_bytes;
+};
+static CooTemp coo_temp(int64_t n_edges, int bits) {
+    CooTemp t{};
+    unsigned long long *k = nullptr;
+    size_t *cnt = nullptr;
+    (void)bits;  // all 64 bits are sorted: an out-of-range edge carries the ~0 key
+    (void)rocprim::radix_sort_keys(nullptr, t.sort_bytes, k, k, (size_t)n_edges, 0, 64);
+    (void)rocprim::unique(nullptr, t.unique_bytes, k, k, cnt, (size_t)n_edges);
+    return t;
 }
 
 static int key_bits(int64_t n_cols) {
@@ -118,6 +178,58 @@ YITU_API int yitu_csr_transpose(int32_t *t_indptr, int32_t *t_rows, int32_t *t_p
     YITU_LAUNCH_CHECK();
     transpose_rows_kernel<<<grid, kBlock, 0, stream>>>(indptr, t_perm, t_rows, nnz,
                                                        (int32_t)n_rows);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+YITU_API size_t yitu_coo_to_csr_workspace_bytes(int64_t n_edges, int64_t n_rows) {
+    if (n_edges <= 0) return 256;
+    const CooTemp t = coo_temp(n_edges, coo_key_bits(n_rows));
+    return 256 + 2 * align_up(sizeof(unsigned long long) * (size_t)n_edges, 256) +
+           align_up(std::max(t.sort_bytes, t.unique_bytes), 256);
+}
+
+YITU_API int yitu_coo_to_csr(int32_t *indptr, int32_t *indices, long long *nnz_out,
+                             const int32_t *rows, const int32_t *cols, int64_t n_edges,
+                             int64_t n_rows, int64_t n_cols, void *workspace,
+                             size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_edges >= 0 && n_rows >= 0 && n_cols >= 0, "negative size");
+    YITU_REQUIRE(n_rows < INT32_MAX && n_cols < INT32_MAX && n_edges < INT32_MAX,
+                 "size out of range");
+    YITU_REQUIRE(indptr && nnz_out, "null output");
+    YITU_REQUIRE(n_edges == 0 || (indices && rows && cols), "null edge array");
+    YITU_REQUIRE(workspace && workspace_bytes >= yitu_coo_to_csr_workspace_bytes(n_edges, n_rows) &&
+                     (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
+                 "workspace too small or not 256-byte aligned: need %zu bytes",
+                 yitu_coo_to_csr_workspace_bytes(n_edges, n_rows));
+    char *w = static_cast<char *>(workspace);
+    size_t *n_unique = reinterpret_cast<size_t *>(w);
+    int *bad = reinterpret_cast<int *>(w + 64);
+    w += 256;
+    const size_t arr = align_up(sizeof(unsigned long long) * (size_t)n_edges, 256);
+    unsigned long long *keys = reinterpret_cast<unsigned long long *>(w);
+    unsigned long long *sorted = reinterpret_cast<unsigned long long *>(w + arr);
+    void *temp = w + 2 * arr;
+    int rc = fill_zero(reinterpret_cast<float *>(workspace), 64, stream);  // count and flag
+    if (rc) return rc;
+    const int grid = (int)ceil_div(std::max<int64_t>(std::max(n_edges, n_rows + 1), 1), kBlock);
+    if (n_edges > 0) {
+        const int bits = coo_key_bits(n_rows);
+        const CooTemp t = coo_temp(n_edges, bits);
+        coo_keys_kernel<<<(int)ceil_div(n_edges, kBlock), kBlock, 0, stream>>>(
+            rows, cols, keys, n_edges, (int32_t)n_rows, (int32_t)n_cols, bad);
+        YITU_LAUNCH_CHECK();
+        size_t bytes = t.sort_bytes;
+        // all 64 bits when an out-of-range edge may carry the ~0 key
+        YITU_HIP(rocprim::radix_sort_keys(temp, bytes, keys, sorted, (size_t)n_edges, 0, 64, stream));
+        bytes = t.unique_bytes;
+        YITU_HIP(rocprim::unique(temp, bytes, sorted, keys, n_unique, (size_t)n_edges,
+                                 rocprim::equal_to<unsigned long long>(), stream));
+    }
+    // after unique, `keys` holds the distinct (row, col) pairs in ascending order
+    coo_finish_kernel<<<grid, kBlock, 0, stream>>>(keys, n_unique, bad, indptr, indices, nnz_out,
+                                                   (int32_t)n_rows, n_edges);
     YITU_LAUNCH_CHECK();
     return 0;
 }

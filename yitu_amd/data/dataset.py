@@ -63,7 +63,14 @@ class CommonDataset(torch.nn.Module):
     def _build_csr(self):
         src = torch.as_tensor(self.edge_index[0], dtype=torch.int64)
         dst = torch.as_tensor(self.edge_index[1], dtype=torch.int64)
-        indptr, indices = graphgen.csr_from_edges(src, dst, self.num_nodes)
+        if self.device.type == "cuda":
+            # sort + merge on the device, then back to the host tensors the callers expect
+            from . import csr
+            indptr, indices = csr.coo_to_csr(src.to(self.device), dst.to(self.device),
+                                             self.num_nodes)
+            indptr, indices = indptr.cpu(), indices.cpu()
+        else:
+            indptr, indices = graphgen.csr_from_edges(src, dst, self.num_nodes)
         self.row_pointers = indptr  # CPU int32, as torch.IntTensor in the reference
         self.column_index = indices
         deg = (indptr[1:] - indptr[:-1]).to(torch.float32).clamp_(min=1.0)
