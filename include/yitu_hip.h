@@ -133,13 +133,15 @@ int yitu_spmm_backward(float *grad_a_device, float *grad_x_device, const float *
  * query [n_bid,n_dst,H], key [n_src,H], attn [nnz,H] (every entry is written).
  * The softmax subtracts the running maximum; the reference does not
  * (sddmm_cuda.cu:15-21) and overflows for logits above ~88.
+ * plan_device: row plan of the CSR (yitu_plan_build with col_mask 0xffffff), or NULL.
  */
-size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid, int with_plan);
+size_t yitu_sddmm_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads, int64_t n_bid,
+                                  int with_plan);
 int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
                        const int32_t *indices_device, const float *query_device,
                        const float *key_device, int64_t n_dst, int64_t n_src, int64_t nnz,
-                       int64_t n_heads, int64_t n_bid, int64_t max_degree, void *workspace_device,
-                       size_t workspace_bytes, void *stream);
+                       int64_t n_heads, int64_t n_bid, int64_t max_degree, const void *plan_device,
+                       void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
  * sddmm_backward (entry.cpp:118-134; sddmm_cuda.cu:36-67,91-118):
@@ -151,7 +153,8 @@ int yitu_sddmm_forward(float *attn_device, const int32_t *indptr_device,
  *   scratch: gv is stored per edge and summed by a gather over the transposed
  *   structure (bitwise reproducible).
  * max_degree / max_degree_t: widest row of the CSR / of its transpose, or -1.
- * plan_t_device: row plan of the transposed structure (gather form only), or NULL.
+ * plan_device / plan_t_device: row plans of the CSR and of the transposed structure
+ * (gather form only), or NULL.
  */
 int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float *grad_edge_device,
                         const int32_t *indptr_device, const int32_t *indices_device,
@@ -159,8 +162,9 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
                         const float *attn_device, const float *grad_out_device,
                         const int32_t *t_indptr_device, const int32_t *t_perm_device,
                         int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                        int64_t max_degree, int64_t max_degree_t, const void *plan_t_device,
-                        void *workspace_device, size_t workspace_bytes, void *stream);
+                        int64_t max_degree, int64_t max_degree_t, const void *plan_device,
+                        const void *plan_t_device, void *workspace_device, size_t workspace_bytes,
+                        void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Fused GAT attention (composition of the two ops above in one pass)          */

@@ -46,10 +46,20 @@ __device__ __forceinline__ MaxSum gat_stats_window(const GatParams &p, const Edg
     const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
     const int H = p.sp.H;
     MaxSum a = ms_init();
-    for (int k0 = 0; k0 < n; k0 += eps) {
-        const int k = k0 + esub;
-        const int col = __shfl(win.col, first + min(k, n - 1), kWave);
-        if (k < n && hl < H) a = ms_push(a, leaky(qv + p.key[(size_t)col * H + hl]));
+    // four steps of key gathers in flight before the first is used
+    for (int k0 = 0; k0 < n; k0 += 4 * eps) {
+        float kv[4];
+        bool ok[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+            ok[u] = k < n && hl < H;
+            kv[u] = ok[u] ? p.key[(size_t)col * H + hl] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (ok[u]) a = ms_push(a, leaky(qv + kv[u]));
     }
     return a;
 }
@@ -190,19 +200,30 @@ __global__ __launch_bounds__(kBlock) void gat_item_stats_kernel(GatParams p) {
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        // all windows and query values first, so the items' key gathers do not
+        // each wait behind their own index load
+        EdgeWindow win[kItemsPerWave];
+        int n[kItemsPerWave], item[kItemsPerWave];
+        float qv[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            if (j >= n_here) break;
             const int beg = __shfl(my_rec.x, j, kWave), end = __shfl(my_rec.y, j, kWave);
-            const int item = __shfl(my_rec.z, j, kWave);
+            item[j] = __shfl(my_rec.z, j, kWave);
             const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
-            EdgeWindow win;
-            load_window<W_NONE>(win, p.sp, beg, end);
-            const float qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
-            MaxSum a = ms_wave_rt(gat_stats_window(p, win, 0, end - beg, qv), p.HP);
+            n[j] = j < n_here ? end - beg : 0;
+            qv[j] = 0.0f;
+            if (n[j] > 0) {
+                load_window<W_NONE>(win[j], p.sp, beg, end);
+                if (hl < H) qv[j] = p.query[(size_t)row * H + hl];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n[j] <= 0) continue;
+            MaxSum a = ms_wave_rt(gat_stats_window(p, win[j], 0, n[j], qv[j]), p.HP);
             if (lane < p.HP && lane < H) {
-                p.item_stats[((size_t)item * H + lane) * 2] = a.m;
-                p.item_stats[((size_t)item * H + lane) * 2 + 1] = a.s;
+                p.item_stats[((size_t)item[j] * H + lane) * 2] = a.m;
+                p.item_stats[((size_t)item[j] * H + lane) * 2 + 1] = a.s;
             }
         }
     }
@@ -317,6 +338,7 @@ struct GatBwdParams {
     float *grad_a;      // [nnz, H] d_attn of the planned rows' edges
     float *item_sums;   // [plan item id][H][3]: (S, A1, A2) over the item's edges
     float *row_sum;     // [n_dst][H]: S of every planned row
+    int HP;             // heads rounded up to a power of two (item sums / combine lane layout)
 };
 
 // d_attn of the n (<= 64) edges in window lanes [first, first + n) against the
@@ -494,25 +516,27 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_combine_kernel(GatBwdParams p)
     if (p.sp.plan.counters->overflow) return;
     const int n_rows = min(p.sp.plan.counters->n_rows, p.sp.plan.max_rows);
     const int lane = lane_id();
-    const int H = p.sp.H;  // a power of two <= 8 here
-    const int h = lane % H, c0 = lane / H, step = kWave / H;
+    const int H = p.sp.H;
+    const int h = lane & (p.HP - 1), c0 = lane / p.HP, step = kWave / p.HP;
     const int n_waves = gridDim.x * kWavesPerBlock;
     for (int slot = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; slot < n_rows;
          slot += n_waves) {
         const int4 r = p.sp.plan.rows[slot];
         float s = 0.0f, a1 = 0.0f, a2 = 0.0f;
-        for (int c = c0; c < r.z; c += step) {
-            const float *st = p.item_sums + ((size_t)(r.y + c) * H + h) * 3;
-            s += st[0];
-            a1 += st[1];
-            a2 += st[2];
+        if (h < H) {
+            for (int c = c0; c < r.z; c += step) {
+                const float *st = p.item_sums + ((size_t)(r.y + c) * H + h) * 3;
+                s += st[0];
+                a1 += st[1];
+                a2 += st[2];
+            }
         }
-        for (int o = kWave / 2; o >= H; o >>= 1) {
+        for (int o = kWave / 2; o >= p.HP; o >>= 1) {
             s += __shfl_xor(s, o, kWave);
             a1 += __shfl_xor(a1, o, kWave);
             a2 += __shfl_xor(a2, o, kWave);
         }
-        if (lane < H) {
+        if (lane < p.HP && h < H) {
             p.row_sum[(size_t)r.x * H + h] = s;
             p.grad_q[(size_t)r.x * H + h] = a1 - s * a2;
         }
@@ -525,20 +549,286 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_apply_kernel(GatBwdParams p) {
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int lane = lane_id();
     const int H = p.sp.H;
+    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; pos < n_items;
-         pos += n_waves) {
-        const int4 rec = p.sp.plan.records[pos];
-        const int row = rec.w & 0x7fffffff;
-        const int total = (rec.y - rec.x) * H;
-        for (int idx = lane; idx < total; idx += kWave) {
-            const int k = idx / H, h = idx % H;
-            const size_t e = (size_t)(rec.x + k);
-            const int c = p.sp.indices[e] & p.sp.col_mask;
-            const float a = p.attn[e * H + h];
-            const float sl = p.query[(size_t)row * H + h] + p.key[(size_t)c * H + h] < 0.0f
-                                 ? kSlope : 1.0f;
-            p.grad_e[e * H + h] = a * (p.grad_a[e * H + h] - p.row_sum[(size_t)row * H + h]) * sl;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int beg[kItemsPerWave], n[kItemsPerWave];
+        float qv[kItemsPerWave], S[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            n[j] = j < n_here ? end - beg[j] : 0;
+            qv[j] = S[j] = 0.0f;
+            if (n[j] > 0) {
+                load_window<W_NONE>(win[j], p.sp, beg[j], end);
+                if (hl < H) {
+                    qv[j] = p.query[(size_t)row * H + hl];
+                    S[j] = p.row_sum[(size_t)row * H + hl];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            for (int k0 = 0; k0 < n[j]; k0 += 4 * eps) {
+                float a[4], g[4], kv[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int k = k0 + u * eps + esub;
+                    const int col = __shfl(win[j].col, min(k, n[j] - 1), kWave);
+                    a[u] = g[u] = kv[u] = 0.0f;
+                    if (k < n[j] && hl < H) {
+                        const size_t e = (size_t)(beg[j] + k) * H + hl;
+                        a[u] = p.attn[e];
+                        g[u] = p.grad_a[e];
+                        kv[u] = p.key[(size_t)col * H + hl];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int k = k0 + u * eps + esub;
+                    if (k < n[j] && hl < H)
+                        p.grad_e[(size_t)(beg[j] + k) * H + hl] =
+                            a[u] * (g[u] - S[j]) * (qv[j] + kv[u] < 0.0f ? kSlope : 1.0f);
+                }
+            }
+        }
+    }
+}
+
+// ---- attention only (the stand-alone SDDMM + LeakyReLU + edge softmax, one
+// query block): the statistics / write halves of the fused kernels above, and
+// the softmax backward over (edge, head) lanes. --------------------------------
+
+// Probabilities of the n edges in window lanes [first, first + n) (CSR edges e0 ...).
+__device__ __forceinline__ void attn_write_window(const GatParams &p, const EdgeWindow &win,
+                                                  int first, int n, int e0, float qv, float m,
+                                                  float inv) {
+    const int lane = lane_id();
+    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int H = p.sp.H;
+    for (int k0 = 0; k0 < n; k0 += 4 * eps) {
+        float kv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+            kv[u] = (k < n && hl < H) ? p.key[(size_t)col * H + hl] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            if (k < n && hl < H)
+                p.attn[(size_t)(e0 + k) * H + hl] = expf(leaky(qv + kv[u]) - m) * inv;
+        }
+    }
+}
+
+// Short rows: kRowsPerWave rows per wave through the sliding edge window.
+__global__ __launch_bounds__(kBlock) void attn_rows_kernel(GatParams p) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int hl = lane & (p.HP - 1);
+    const int H = p.sp.H;
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int n = end - beg;
+        if (n == 0 || n >= p.sp.plan.threshold) continue;
+        if (win.base < 0 || beg < win.base || end > win.base + kWave)
+            load_window<W_NONE>(win, p.sp, beg, limit);
+        const float qv = hl < H ? p.query[(size_t)(r0 + i) * H + hl] : 0.0f;
+        const MaxSum a = ms_wave_rt(gat_stats_window(p, win, beg - win.base, n, qv), p.HP);
+        attn_write_window(p, win, beg - win.base, n, beg, qv, a.m, 1.0f / a.s);
+    }
+}
+
+// Planned rows, step 3 (after gat_item_stats_kernel and gat_row_combine_kernel).
+__global__ __launch_bounds__(kBlock) void attn_item_write_kernel(GatParams p) {
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int hl = lane & (p.HP - 1);
+    const int H = p.sp.H;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int beg[kItemsPerWave], n[kItemsPerWave];
+        float qv[kItemsPerWave], m[kItemsPerWave], inv[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            n[j] = j < n_here ? end - beg[j] : 0;
+            qv[j] = m[j] = inv[j] = 0.0f;
+            if (n[j] > 0) {
+                load_window<W_NONE>(win[j], p.sp, beg[j], end);
+                if (hl < H) {
+                    qv[j] = p.query[(size_t)row * H + hl];
+                    m[j] = p.row_stats[((size_t)row * H + hl) * 2];
+                    inv[j] = p.row_stats[((size_t)row * H + hl) * 2 + 1];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++)
+            if (n[j] > 0) attn_write_window(p, win[j], 0, n[j], beg[j], qv[j], m[j], inv[j]);
+    }
+}
+
+// Softmax + LeakyReLU backward sums of the n edges in window lanes [first, ...):
+// S = sum a g, A1 = sum a g s, A2 = sum a s for this lane's head (lane % HP),
+// g = grad_a (the gradient that arrives at attn). Not yet reduced over lanes.
+__device__ __forceinline__ void attn_bwd_sums_window(const GatBwdParams &p, const EdgeWindow &win,
+                                                     int first, int n, int e0, float qv, float &S,
+                                                     float &A1, float &A2) {
+    const int lane = lane_id();
+    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int H = p.sp.H;
+    for (int k0 = 0; k0 < n; k0 += 4 * eps) {
+        float a[4], g[4], kv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+            a[u] = g[u] = kv[u] = 0.0f;  // a = 0 makes a lane past the range add nothing
+            if (k < n && hl < H) {
+                const size_t e = (size_t)(e0 + k) * H + hl;
+                a[u] = p.attn[e];
+                g[u] = p.grad_a[e];
+                kv[u] = p.key[(size_t)col * H + hl];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const float sl = qv + kv[u] < 0.0f ? kSlope : 1.0f;
+            S += a[u] * g[u];
+            A1 += a[u] * g[u] * sl;
+            A2 += a[u] * sl;
+        }
+    }
+}
+
+__device__ __forceinline__ void attn_bwd_reduce(float &S, float &A1, float &A2, int hp) {
+    for (int o = kWave / 2; o >= hp; o >>= 1) {
+        S += __shfl_xor(S, o, kWave);
+        A1 += __shfl_xor(A1, o, kWave);
+        A2 += __shfl_xor(A2, o, kWave);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int H = p.sp.H;
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int row = r0 + i;
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int n = end - beg;
+        if (n >= p.sp.plan.threshold) continue;
+        if (n == 0) {
+            if (lane < p.HP && hl < H) p.grad_q[(size_t)row * H + hl] = 0.0f;
+            continue;
+        }
+        if (win.base < 0 || beg < win.base || end > win.base + kWave)
+            load_window<W_NONE>(win, p.sp, beg, limit);
+        const int first = beg - win.base;
+        const float qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
+        float S = 0.0f, A1 = 0.0f, A2 = 0.0f;
+        attn_bwd_sums_window(p, win, first, n, beg, qv, S, A1, A2);
+        attn_bwd_reduce(S, A1, A2, p.HP);
+        if (lane < p.HP && hl < H) p.grad_q[(size_t)row * H + hl] = A1 - S * A2;
+        for (int k0 = 0; k0 < n; k0 += 4 * eps) {
+            float a[4], g[4], kv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int k = k0 + u * eps + esub;
+                const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+                a[u] = g[u] = kv[u] = 0.0f;
+                if (k < n && hl < H) {
+                    const size_t e = (size_t)(beg + k) * H + hl;
+                    a[u] = p.attn[e];
+                    g[u] = p.grad_a[e];
+                    kv[u] = p.key[(size_t)col * H + hl];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int k = k0 + u * eps + esub;
+                if (k < n && hl < H)
+                    p.grad_e[(size_t)(beg + k) * H + hl] =
+                        a[u] * (g[u] - S) * (qv + kv[u] < 0.0f ? kSlope : 1.0f);
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams p) {
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int hl = lane & (p.HP - 1);
+    const int H = p.sp.H;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int beg[kItemsPerWave], n[kItemsPerWave], item[kItemsPerWave];
+        float qv[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            item[j] = __shfl(my_rec.z, j, kWave);
+            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            n[j] = j < n_here ? end - beg[j] : 0;
+            qv[j] = 0.0f;
+            if (n[j] > 0) {
+                load_window<W_NONE>(win[j], p.sp, beg[j], end);
+                if (hl < H) qv[j] = p.query[(size_t)row * H + hl];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n[j] <= 0) continue;
+            float S = 0.0f, A1 = 0.0f, A2 = 0.0f;
+            attn_bwd_sums_window(p, win[j], 0, n[j], beg[j], qv[j], S, A1, A2);
+            attn_bwd_reduce(S, A1, A2, p.HP);
+            if (lane < p.HP && hl < H) {
+                float *st = p.item_sums + ((size_t)item[j] * H + hl) * 3;
+                st[0] = S;
+                st[1] = A1;
+                st[2] = A2;
+            }
         }
     }
 }
@@ -571,7 +861,8 @@ static int gat_bwd_items_launch(const GatBwdParams &p, hipStream_t stream) {
                                                     1 << 15),
                              kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    gat_bwd_apply_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items, kWavesPerBlock),
+    gat_bwd_apply_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
+                                                           kWavesPerBlock * kItemsPerWave),
                                                   1 << 16),
                            kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
@@ -609,6 +900,115 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
     return 0;
 }
 
+// ---- attention only: host side ---------------------------------------------------
+size_t attn_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t H) {
+    return align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * H), 256) +
+           align_up(sizeof(float) * 2 * (size_t)(n_dst * H), 256);
+}
+
+int attn_forward_run(float *attn, const int32_t *indptr, const int32_t *indices,
+                     const float *query, const float *key, int64_t n_dst, int64_t n_src,
+                     int64_t nnz, int64_t n_heads, int64_t max_degree, const void *plan,
+                     void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    GatParams p{};
+    p.sp.indptr = indptr;
+    p.sp.indices = indices;
+    p.sp.n_rows = (int)n_dst;
+    p.sp.n_src = (int)n_src;
+    p.sp.H = (int)n_heads;
+    p.sp.L = p.sp.F = (int)n_heads;
+    p.sp.col_mask = kColMask;
+    p.query = query;
+    p.key = key;
+    p.attn = attn;
+    p.HP = 1;
+    while (p.HP < p.sp.H) p.HP <<= 1;
+    bool has_items = false;
+    void *rest = nullptr;
+    size_t rest_bytes = 0;
+    int rc = plan_resolve(p.sp.plan, has_items, plan, indptr, indices, n_dst, n_src, nnz, kColMask,
+                          max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
+    if (rc) return rc;
+    if (!has_items) p.sp.plan.threshold = 0x7fffffff;
+    attn_rows_kernel<<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    if (!has_items) return 0;
+    const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);
+    YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes", need);
+    char *w = static_cast<char *>(rest);
+    p.item_stats = reinterpret_cast<float *>(w);
+    w += align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * n_heads), 256);
+    p.row_stats = reinterpret_cast<float *>(w);
+    const int item_grid = (int)std::min<int64_t>(
+        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+    gat_item_stats_kernel<<<item_grid, kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    gat_row_combine_kernel<<<(int)std::min<int64_t>(
+                                 ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15),
+                             kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    attn_item_write_kernel<<<item_grid, kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+// grad_query and the per-edge logit gradient grad_edge [nnz, H]; the caller sums
+// grad_edge into grad_key over the transposed structure.
+int attn_backward_run(float *grad_query, float *grad_edge, const int32_t *indptr,
+                      const int32_t *indices, const float *query, const float *key,
+                      const float *attn, const float *grad_attn, int64_t n_dst, int64_t n_src,
+                      int64_t nnz, int64_t n_heads, int64_t max_degree, const void *plan,
+                      void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    GatBwdParams p{};
+    p.sp.indptr = indptr;
+    p.sp.indices = indices;
+    p.sp.n_rows = (int)n_dst;
+    p.sp.n_src = (int)n_src;
+    p.sp.H = (int)n_heads;
+    p.sp.L = p.sp.F = (int)n_heads;
+    p.sp.col_mask = kColMask;
+    p.query = query;
+    p.key = key;
+    p.attn = attn;
+    p.grad_a = const_cast<float *>(grad_attn);
+    p.grad_q = grad_query;
+    p.grad_e = grad_edge;
+    p.HP = 1;
+    while (p.HP < p.sp.H) p.HP <<= 1;
+    bool has_items = false;
+    void *rest = nullptr;
+    size_t rest_bytes = 0;
+    int rc = plan_resolve(p.sp.plan, has_items, plan, indptr, indices, n_dst, n_src, nnz, kColMask,
+                          max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
+    if (rc) return rc;
+    if (!has_items) p.sp.plan.threshold = 0x7fffffff;
+    attn_bwd_rows_kernel<<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0,
+                           stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    if (!has_items) return 0;
+    const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);
+    YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes", need);
+    char *w = static_cast<char *>(rest);
+    p.item_sums = reinterpret_cast<float *>(w);
+    w += align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * n_heads), 256);
+    p.row_sum = reinterpret_cast<float *>(w);
+    attn_bwd_item_sums_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
+                                                                kWavesPerBlock * kItemsPerWave),
+                                                       1 << 16),
+                                kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    gat_bwd_combine_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock),
+                                                    1 << 15),
+                             kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    gat_bwd_apply_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
+                                                           kWavesPerBlock * kItemsPerWave),
+                                                  1 << 16),
+                           kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
 }  // namespace yitu
 
 using namespace yitu;
@@ -619,7 +1019,7 @@ YITU_API size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_h
     const int64_t L = n_heads * n_features;
     size_t b = gat_own_bytes(n_dst, nnz, n_heads, L) + (with_plans ? 0 : plan_temp_bytes(nnz));
     b = std::max(b, (size_t)yitu_spmm_workspace_bytes(nnz, L, with_plans));
-    b = std::max(b, (size_t)yitu_sddmm_workspace_bytes(nnz, n_heads, 1, with_plans));
+    b = std::max(b, (size_t)yitu_sddmm_workspace_bytes(n_dst, nnz, n_heads, 1, with_plans));
     return b + 256;
 }
 
@@ -644,7 +1044,7 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
         // shapes outside the fused kernel's vector layout: the two-op composition
         YITU_REQUIRE(attn, "this shape needs the attn buffer (unfused path)");
         int rc = yitu_sddmm_forward(attn, indptr, indices, query, key, n_dst, n_src, nnz, n_heads,
-                                    1, max_degree, workspace, workspace_bytes, stream_);
+                                    1, max_degree, plan, workspace, workspace_bytes, stream_);
         if (rc) return rc;
         return yitu_spmm_forward(out, attn, indptr, indices, features, n_dst, n_src, nnz, n_heads,
                                  n_features, max_degree, plan, workspace, workspace_bytes,
@@ -733,6 +1133,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         p.grad_q = grad_query;
         p.grad_e = grad_edge_scratch;
         p.grad_a = grad_attn_scratch;
+        p.HP = (int)n_heads;  // a power of two here
         bool has_items = false;
         void *rest = nullptr;
         size_t rest_bytes = 0;
@@ -762,7 +1163,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         // every row has been handled above, so the softmax backward kernels skip all rows
         return sddmm_backward_run(grad_query, grad_key, grad_edge_scratch, indptr, indices, query,
                                   key, attn, grad_attn_scratch, t_indptr, t_perm, n_dst, n_src, nnz,
-                                  n_heads, 1, max_degree, max_degree_t, plan_t, workspace,
+                                  n_heads, 1, max_degree, max_degree_t, plan, plan_t, workspace,
                                   workspace_bytes, INT32_MAX, stream);
     }
     // d attn = <grad_out[row], x[col]> per edge and head; grad_x = attn-weighted
@@ -775,6 +1176,6 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
     // softmax + LeakyReLU backward; grad_key gathered over the transposed structure
     return sddmm_backward_run(grad_query, grad_key, grad_edge_scratch, indptr, indices, query, key,
                               attn, grad_attn_scratch, t_indptr, t_perm, n_dst, n_src, nnz, n_heads,
-                              1, max_degree, max_degree_t, plan_t, workspace, workspace_bytes, 0,
-                              stream);
+                              1, max_degree, max_degree_t, plan, plan_t, workspace, workspace_bytes,
+                              0, stream);
 }

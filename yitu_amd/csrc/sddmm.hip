@@ -114,11 +114,15 @@ static int sddmm_bwd_dispatch(const SddmmParams &p, bool with_hub, hipStream_t s
 using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
-YITU_API size_t yitu_sddmm_workspace_bytes(int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                           int with_plan) {
+YITU_API size_t yitu_sddmm_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads,
+                                           int64_t n_bid, int with_plan) {
     // the backward's gather pass reuses the buffer as SpMM workspace
-    return std::max(sddmm_ws_bytes(nnz, n_heads, n_bid),
-                    spmm_workspace_bytes(nnz, n_heads, with_plan != 0));
+    size_t b = std::max(sddmm_ws_bytes(nnz, n_heads, n_bid),
+                        spmm_workspace_bytes(nnz, n_heads, with_plan != 0));
+    if (n_bid == 1)
+        b = std::max(b, attn_workspace_bytes(n_dst, nnz, n_heads) +
+                            (with_plan ? 0 : plan_temp_bytes(nnz)));
+    return b;
 }
 
 static int sddmm_check(const int32_t *indptr, const int32_t *indices, const float *query,
@@ -137,12 +141,16 @@ static int sddmm_check(const int32_t *indptr, const int32_t *indices, const floa
 YITU_API int yitu_sddmm_forward(float *attn, const int32_t *indptr, const int32_t *indices,
                                 const float *query, const float *key, int64_t n_dst,
                                 int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                int64_t max_degree, void *workspace, size_t workspace_bytes,
-                                void *stream) {
+                                int64_t max_degree, const void *plan, void *workspace,
+                                size_t workspace_bytes, void *stream) {
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
     if (n_dst == 0 || nnz == 0 || n_heads == 0) return 0;
     YITU_REQUIRE(attn, "null output");
+    if (n_bid == 1 && n_heads <= 64)
+        return attn_forward_run(attn, indptr, indices, query, key, n_dst, n_src, nnz, n_heads,
+                                max_degree, plan, workspace, workspace_bytes,
+                                static_cast<hipStream_t>(stream));
     SddmmParams p{};
     p.indptr = indptr;
     p.indices = indices;
@@ -164,8 +172,8 @@ int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, con
                        const float *attn, const float *grad_out, const int32_t *t_indptr,
                        const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
                        int64_t n_heads, int64_t n_bid, int64_t max_degree, int64_t max_degree_t,
-                       const void *plan_t, void *workspace, size_t workspace_bytes, int skip_below,
-                       hipStream_t stream) {
+                       const void *plan, const void *plan_t, void *workspace,
+                       size_t workspace_bytes, int skip_below, hipStream_t stream) {
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
     if (n_heads == 0) return 0;
@@ -178,7 +186,13 @@ int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, con
         rc = fill_zero(grad_key, n_src * n_heads, stream);
         if (rc) return rc;
     }
-    if (n_dst > 0 && skip_below != INT32_MAX) {  // INT32_MAX: only the grad_key gather is wanted
+    if (n_dst > 0 && nnz > 0 && skip_below == 0 && gather && n_bid == 1 && n_heads <= 64) {
+        // one query block: windowed row kernel + row-plan items
+        rc = attn_backward_run(grad_query, grad_edge, indptr, indices, query, key, attn, grad_out,
+                               n_dst, n_src, nnz, n_heads, max_degree, plan, workspace,
+                               workspace_bytes, stream);
+        if (rc) return rc;
+    } else if (n_dst > 0 && skip_below != INT32_MAX) {  // INT32_MAX: only the grad_key gather
         SddmmParams p{};
         p.indptr = indptr;
         p.indices = indices;
@@ -226,10 +240,11 @@ YITU_API int yitu_sddmm_backward(float *grad_query, float *grad_key, float *grad
                                  const float *key, const float *attn, const float *grad_out,
                                  const int32_t *t_indptr, const int32_t *t_perm, int64_t n_dst,
                                  int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_bid,
-                                 int64_t max_degree, int64_t max_degree_t, const void *plan_t,
-                                 void *workspace, size_t workspace_bytes, void *stream_) {
+                                 int64_t max_degree, int64_t max_degree_t, const void *plan,
+                                 const void *plan_t, void *workspace, size_t workspace_bytes,
+                                 void *stream_) {
     return sddmm_backward_run(grad_query, grad_key, grad_edge, indptr, indices, query, key, attn,
                               grad_out, t_indptr, t_perm, n_dst, n_src, nnz, n_heads, n_bid,
-                              max_degree, max_degree_t, plan_t, workspace, workspace_bytes, 0,
-                              static_cast<hipStream_t>(stream_));
+                              max_degree, max_degree_t, plan, plan_t, workspace, workspace_bytes,
+                              0, static_cast<hipStream_t>(stream_));
 }

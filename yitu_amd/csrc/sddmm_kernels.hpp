@@ -397,6 +397,18 @@ __global__ __launch_bounds__(kBlock) void sddmm_bwd_hub_apply_kernel(SddmmParams
     }
 }
 
+// One query block (n_bid = 1): windowed row kernels + row-plan items (gat.hip).
+size_t attn_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t H);
+int attn_forward_run(float *attn, const int32_t *indptr, const int32_t *indices,
+                     const float *query, const float *key, int64_t n_dst, int64_t n_src,
+                     int64_t nnz, int64_t n_heads, int64_t max_degree, const void *plan,
+                     void *workspace, size_t workspace_bytes, hipStream_t stream);
+int attn_backward_run(float *grad_query, float *grad_edge, const int32_t *indptr,
+                      const int32_t *indices, const float *query, const float *key,
+                      const float *attn, const float *grad_attn, int64_t n_dst, int64_t n_src,
+                      int64_t nnz, int64_t n_heads, int64_t max_degree, const void *plan,
+                      void *workspace, size_t workspace_bytes, hipStream_t stream);
+
 // The body of yitu_sddmm_backward; rows with fewer than skip_below edges are
 // left alone (the fused GAT backward has already written their results).
 int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, const int32_t *indptr,
@@ -404,7 +416,7 @@ int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, con
                        const float *attn, const float *grad_out, const int32_t *t_indptr,
                        const int32_t *t_perm, int64_t n_dst, int64_t n_src, int64_t nnz,
                        int64_t n_heads, int64_t n_bid, int64_t max_degree, int64_t max_degree_t,
-                       const void *plan_t, void *workspace, size_t workspace_bytes, int skip_below,
-                       hipStream_t stream);
+                       const void *plan, const void *plan_t, void *workspace,
+                       size_t workspace_bytes, int skip_below, hipStream_t stream);
 
 }  // namespace yitu

@@ -196,15 +196,17 @@ def sddmm_forward(indptr, indices, query, key):
     dev = _lib.require_device(indptr, indices, query, key)
     attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
     maxdeg = _lib.max_degree(indptr)
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK) if n_bid == 1 else None
     need = 0
     if maxdeg >= 64:
-        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid), c_int(1))
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(n_dst), c_i64(nnz), c_i64(h),
+                                                      c_i64(n_bid), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_sddmm_forward(ptr(attn), ptr(indptr), ptr(indices), ptr(query), ptr(key),
                                            c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-                                           c_i64(n_bid), c_i64(maxdeg), ptr(ws), c_size(ws.numel()),
-                                           stream_ptr(dev))
+                                           c_i64(n_bid), c_i64(maxdeg), ptr(plan), ptr(ws),
+                                           c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_sddmm_forward")
     return attn
 
@@ -223,16 +225,18 @@ def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, determini
     maxdeg = _lib.max_degree(indptr)
     tr = transposed(indptr, indices, n_src) if deterministic else None
     grad_edge = torch.empty_like(attn_values) if deterministic else None
+    plan = _lib.row_plan(indptr, indices, n_src, COL_MASK) if n_bid == 1 and deterministic else None
     need = 0
     if maxdeg >= 64 or (tr is not None and tr.max_degree_t >= 64):
-        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(nnz), c_i64(h), c_i64(n_bid), c_int(1))
+        need = _size_fn("yitu_sddmm_workspace_bytes")(c_i64(n_dst), c_i64(nnz), c_i64(h),
+                                                      c_i64(n_bid), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_sddmm_backward(
             ptr(grad_query), ptr(grad_key), ptr(grad_edge), ptr(indptr), ptr(indices), ptr(query),
             ptr(key), ptr(attn_values), ptr(grad_out), ptr(tr.t_indptr if tr else None),
             ptr(tr.t_perm if tr else None), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-            c_i64(n_bid), c_i64(maxdeg), c_i64(tr.max_degree_t if tr else -1),
+            c_i64(n_bid), c_i64(maxdeg), c_i64(tr.max_degree_t if tr else -1), ptr(plan),
             ptr(tr.plan_t if tr else None), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_sddmm_backward")
     return [grad_query, grad_key]
