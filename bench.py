@@ -222,6 +222,14 @@ def run_gat(args, dev):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     fwd_ms = sum(a.elapsed_time(b) for a, b in ev["fwd"]) / args.steps
     bwd_ms = sum(a.elapsed_time(b) for a, b in ev["bwd"]) / args.steps
+    # the stand-alone SDDMM + LeakyReLU + edge softmax of the same graph (one query block)
+    q1 = q.unsqueeze(0).contiguous()
+    attn_sa = graph_ext.sddmm_forward(rp, ci, q1, k)
+    ga = torch.randn(nnz, h, generator=g, device=dev)
+    sd_fwd_ms = _event_ms(lambda: graph_ext.sddmm_forward(rp, ci, q1, k), args.steps, args.warmup)
+    sd_bwd_ms = _event_ms(lambda: graph_ext.sddmm_backward(rp, ci, q1, k, attn_sa, ga), args.steps,
+                          args.warmup)
+    alg_sd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h
     alg_fwd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h + 8 * n * h * f
     alg_bwd = (2 * 4 * n * h * f + 4 * nnz * h + 8 * nnz + 8 * (n + 1) + 4 * nnz
                + 4 * n * h * f + 8 * n * h)
@@ -233,6 +241,11 @@ def run_gat(args, dev):
         "config": {"workload": "c2_gat_f32", "graph": "R-MAT scale 18, 13M draws dedup, CSR by "
                    "destination", "n_nodes": n, "n_edges": nnz, "heads": h, "head_dim": f},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "sddmm": {"fwd_ms": sd_fwd_ms, "bwd_ms": sd_bwd_ms,
+                  "edges_per_s_fwd_bwd": nnz / ((sd_fwd_ms + sd_bwd_ms) * 1e-3),
+                  "fwd_algorithmic_bytes": alg_sd,
+                  "fwd_GBps": alg_sd / (sd_fwd_ms * 1e-3) / 1e9,
+                  "fwd_hbm_frac": alg_sd / (sd_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "achieved": alg_fwd / (fwd_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -530,7 +543,8 @@ def main():
             # the other single-GPU configurations ride along as extra fields
             args.no_cpu = True
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
-                                                "roofline") if k in r}
+                                                "roofline", "fwd_ms", "bwd_ms", "sddmm")
+                              if k in r}
             res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
                             "c2_gat_f32": slim(run_gat(args, dev)),
                             "c1_gcn_f32": run_c1(args, dev),
