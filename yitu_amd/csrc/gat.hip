@@ -343,7 +343,9 @@ struct GatBwdParams {
 
 // d_attn of the n (<= 64) edges in window lanes [first, first + n) against the
 // row's grad_out tile, left in `keep` in the (edge, head) layout: lane (h, sub)
-// gets edge j * LPH + sub in keep[j]. Four gathers are in flight at a time.
+// gets edge j * LPH + sub in keep[j]. kDotUnroll gathers are in flight at a time.
+constexpr int kDotUnroll = 4;  // gathers in flight per wave in the backward dots (LPH >= 8)
+
 template <int LPH>
 __device__ __forceinline__ void gat_bwd_dots(const GatBwdParams &p, const EdgeWindow &win,
                                              int first, int n, const float (&gt)[4],
@@ -356,10 +358,10 @@ __device__ __forceinline__ void gat_bwd_dots(const GatBwdParams &p, const EdgeWi
 #pragma unroll
     for (int j = 0; j < NS; j++) {
         keep[j] = 0.0f;
-        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += 4) {
-            float v[4][4];
+        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += kDotUnroll) {
+            float v[kDotUnroll][4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < kDotUnroll; u++) {
                 const int k = j * LPH + kk + u;
                 if (k < n) {  // wave-uniform
                     const int c = __builtin_amdgcn_readlane(win.col, first + k);
@@ -367,7 +369,7 @@ __device__ __forceinline__ void gat_bwd_dots(const GatBwdParams &p, const EdgeWi
                 }
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < kDotUnroll; u++) {
                 const int k = j * LPH + kk + u;
                 if (k < n) {
                     float d = gt[0] * v[u][0] + gt[1] * v[u][1] + gt[2] * v[u][2] + gt[3] * v[u][3];

@@ -1,6 +1,8 @@
 // Kernels of the SDDMM(u_add_v) + LeakyReLU(0.2) + per-destination edge softmax,
 // forward and backward, for packed indices (bid << 24 | col) and up to 16 query
-// blocks. Shared by the stand-alone op and the fused GAT forward.
+// blocks. With one query block the op runs on the windowed / row-plan kernels of
+// gat.hip instead; these kernels serve stitched multi-block graphs and the
+// atomic form of the backward.
 //
 // Mapping (wave64): one wave per destination row; a step covers 64 / HP edges
 // with HP lanes (the head count rounded up to a power of two) per edge, so the
@@ -17,6 +19,58 @@
 #include "spmm_rows.hpp"
 
 namespace yitu {
+
+// ---- queue of long rows for the multi-block kernels (rows of 512+ edges are
+// spread over workgroups of 512-edge chunks) -----------------------------------
+constexpr int kHubChunk = 512;      // edges per hub work item
+constexpr int kHubThreshold = 512;  // rows with >= this many edges go to the chunk kernels
+
+struct HubCounters {
+    int n_items;
+    int n_rows;
+    int overflow;  // set when the queue capacity was exceeded; the hub kernels then do nothing
+    int pad;
+};
+
+struct HubQueue {
+    HubCounters *counters;  // zeroed before the row kernel
+    int4 *rows;             // {row, first_item, n_chunks, 0}
+    int4 *items;            // {row, chunk, index into rows[], 0}
+    float *partial;         // [n_items, L]
+    int max_rows;
+    int max_items;
+    int chunk;              // edges per item
+};
+
+// Appends a hub row and its ceil(deg / kHubChunk) chunk items to the queue.
+// Called by all lanes of the wave that owns the row.
+__device__ __forceinline__ void queue_hub_row(const HubQueue &q, int row, int deg) {
+    const int lane = lane_id();
+    const int n_chunks = (deg + q.chunk - 1) / q.chunk;
+    int first = 0, slot_r = 0;
+    if (lane == 0) {
+        first = atomicAdd(&q.counters->n_items, n_chunks);
+        slot_r = atomicAdd(&q.counters->n_rows, 1);
+    }
+    first = __shfl(first, 0, kWave);
+    slot_r = __shfl(slot_r, 0, kWave);
+    if (slot_r < q.max_rows && first + n_chunks <= q.max_items) {
+        if (lane == 0) q.rows[slot_r] = make_int4(row, first, n_chunks, 0);
+        for (int c = lane; c < n_chunks; c += kWave)
+            q.items[first + c] = make_int4(row, c, slot_r, 0);
+    } else if (lane == 0) {
+        atomicExch(&q.counters->overflow, 1);
+    }
+}
+
+static __global__ void zero_hub_counters_kernel(HubCounters *c) {
+    if (threadIdx.x == 0) {
+        c->n_items = 0;
+        c->n_rows = 0;
+        c->overflow = 0;
+        c->pad = 0;
+    }
+}
 
 constexpr float kSlope = 0.2f;  // LeakyReLU slope fixed by the reference (sddmm_cuda.cu:22)
 constexpr int kColMask = 0xffffff;

@@ -35,29 +35,6 @@ size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan) {
     return b + 256;
 }
 
-// Queue of (row, 512-edge chunk) items without partial rows, for kernels whose
-// per-edge results need no cross-chunk reduction (the per-edge dot products).
-int hub512_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t nnz) {
-    const int64_t rows = nnz / kHubThreshold + 1, items = nnz / kHubChunk + rows + 1;
-    const size_t need = 256 + align_up(sizeof(int4) * (size_t)rows, 256) +
-                        align_up(sizeof(int4) * (size_t)items, 256);
-    YITU_REQUIRE(workspace != nullptr && workspace_bytes >= need,
-                 "workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
-    YITU_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
-                 "workspace must be 256-byte aligned");
-    char *w = static_cast<char *>(workspace);
-    q = HubQueue{};
-    q.counters = reinterpret_cast<HubCounters *>(w);
-    w += 256;
-    q.max_rows = (int)rows;
-    q.max_items = (int)items;
-    q.chunk = kHubChunk;
-    q.rows = reinterpret_cast<int4 *>(w);
-    w += align_up(sizeof(int4) * (size_t)rows, 256);
-    q.items = reinterpret_cast<int4 *>(w);
-    return 0;
-}
-
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 static int launch_variant(const SpmmParams &p, bool has_items, hipStream_t stream) {
     const int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave);

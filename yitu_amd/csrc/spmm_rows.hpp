@@ -3,17 +3,19 @@
 // transposed pass of its backward, and the aggregate step of the fused GAT).
 //
 // Mapping (wave64):
-//   * one wave owns one output row; the row vector of L = H*F floats is laid
-//     across G lanes x VEC elements x KT tiles, so one wave-wide load
-//     instruction fetches 64/G ("slots") neighbour rows at once;
-//   * column ids (and per-edge scalars) of up to 64 edges are fetched with one
-//     coalesced load, then broadcast lane-to-lane, so the feature gathers of
-//     one batch are independent and UNROLL of them are in flight per wave;
-//   * slots are folded with a fixed butterfly and the row is written once:
-//     no atomics, bitwise reproducible.
-//   * rows with at least hub_threshold edges are not processed here but queued
-//     (row, chunk) for the workgroup-per-chunk kernel, whose partial sums are
-//     combined in chunk order by a third kernel.
+//   * the row vector of L = H*F floats is laid across G lanes x VEC elements x
+//     KT tiles, so one wave-wide load instruction fetches 64/G ("slots")
+//     neighbour rows at once;
+//   * column ids (and per-edge scalars) of 64 consecutive CSR edges are fetched
+//     with one coalesced load (an "edge window"), then broadcast lane-to-lane, so
+//     the feature gathers of one round are independent and UNROLL of them are
+//     in flight per wave;
+//   * slots are folded with a fixed butterfly and a row is written once:
+//     no atomics, bitwise reproducible;
+//   * rows below the plan threshold (64 edges): a wave walks 16 consecutive rows
+//     through a sliding window; longer rows: the row plan's items of at most 64
+//     edges in band order, four per wave, whose partial rows a third kernel adds
+//     in a fixed order.
 #pragma once
 #include "common.hpp"
 #include "plan.hpp"
@@ -24,26 +26,6 @@ enum WeightMode : int {
     W_NONE = 0,      // w = 1
     W_DEGPROD = 1,   // w = s_row * s_col            (module-1 GCN norm)
     W_EDGEHEAD = 2,  // w = values[edge, head]       (module-2 SpMM)
-};
-
-constexpr int kHubChunk = 512;      // edges per hub work item (SDDMM / GAT / dot kernels)
-constexpr int kHubThreshold = 512;  // rows with >= this many edges go to the hub path there
-
-struct HubCounters {
-    int n_items;
-    int n_rows;
-    int overflow;  // set when the queue capacity was exceeded; the hub kernels then do nothing
-    int pad;
-};
-
-struct HubQueue {
-    HubCounters *counters;  // zeroed before the row kernel
-    int4 *rows;             // {row, first_item, n_chunks, 0}
-    int4 *items;            // {row, chunk, index into rows[], 0}
-    float *partial;         // [n_items, L]
-    int max_rows;
-    int max_items;
-    int chunk;              // edges per item
 };
 
 struct SpmmParams {
@@ -65,27 +47,6 @@ struct SpmmParams {
     PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
     float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
 };
-
-// Appends a hub row and its ceil(deg / kHubChunk) chunk items to the queue.
-// Called by all lanes of the wave that owns the row.
-__device__ __forceinline__ void queue_hub_row(const HubQueue &q, int row, int deg) {
-    const int lane = lane_id();
-    const int n_chunks = (deg + q.chunk - 1) / q.chunk;
-    int first = 0, slot_r = 0;
-    if (lane == 0) {
-        first = atomicAdd(&q.counters->n_items, n_chunks);
-        slot_r = atomicAdd(&q.counters->n_rows, 1);
-    }
-    first = __shfl(first, 0, kWave);
-    slot_r = __shfl(slot_r, 0, kWave);
-    if (slot_r < q.max_rows && first + n_chunks <= q.max_items) {
-        if (lane == 0) q.rows[slot_r] = make_int4(row, first, n_chunks, 0);
-        for (int c = lane; c < n_chunks; c += kWave)
-            q.items[first + c] = make_int4(row, c, slot_r, 0);
-    } else if (lane == 0) {
-        atomicExch(&q.counters->overflow, 1);
-    }
-}
 
 // A window is up to 64 consecutive CSR edges held one per lane: column id,
 // per-edge scalar weight (W_NONE / W_DEGPROD) or the row of `values` to read
@@ -457,18 +418,6 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
         }
     }
 }
-
-static __global__ void zero_hub_counters_kernel(HubCounters *c) {
-    if (threadIdx.x == 0) {
-        c->n_items = 0;
-        c->n_rows = 0;
-        c->overflow = 0;
-        c->pad = 0;
-    }
-}
-
-// Host side: carve the queue out of a caller-provided workspace.
-int hub512_queue_init(HubQueue &q, void *workspace, size_t workspace_bytes, int64_t nnz);
 
 // Picks the instantiation for (element type, L) and launches the row, item and reduce kernels.
 // max_degree_hint < 0 means unknown; plan may be null (a temporary one is then
