@@ -19,7 +19,7 @@ from yitu_amd import _lib
 pytestmark = pytest.mark.gpu
 
 CHUNK = 64
-SLABS = 8
+SLABS = 4
 
 
 def read_plan(plan, nnz):

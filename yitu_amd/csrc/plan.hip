@@ -134,8 +134,8 @@ __global__ void plan_bounds_kernel(BuildBuffers b) {
     b.slab_bound[k] = (int)(bound < 0x7fffffffLL ? bound : 0x7fffffffLL);
 }
 
-// One wave per long row. Lanes 0..8 find where the row's columns cross the slab
-// boundaries; lane 0 turns the crossings into at most min(8, deg / 16) segments
+// One wave per long row. Lanes 0..4 find where the row's columns cross the slab
+// boundaries; lane 0 turns the crossings into at most min(4, deg / 16) segments
 // (none shorter than kPlanMinSegment), the wave then writes the items of every
 // segment: ceil(len / 64) pieces of equal size. Item ids of a row are
 // consecutive; a workgroup takes its ids with one atomic.

@@ -8,12 +8,14 @@
 // speed. Short rows are not in the plan; a wave of the row kernels walks 16 of
 // them in a row.
 //
-// Slabs: the source ids are cut into 8 contiguous ranges and a long row is cut
+// Slabs: the source ids are cut into 4 contiguous ranges and a long row is cut
 // where its (sorted) columns cross a range boundary (at most deg / 16 pieces,
 // none shorter than 16 edges), so most items gather from one range only. With
 // items that straddle the whole id space, the band that the chip reads at one
 // moment is polluted by the far ends of every item; with the cuts it is not
-// (measured on a 2^21-node R-MAT graph: 7 % less time for the fp32 SpMM).
+// (measured on a 2^21-node R-MAT graph: 3 to 7 % less time for the fp32 SpMM;
+// 8 and 16 ranges cut the rows into smaller items and cost the bf16 path more
+// than they gain).
 // Boundaries are placed so that the ranges have equal sums of popularity^0.75
 // over their sources: a hot source is fetched into L2 once and then hit, so its
 // cost grows more slowly than its edge count, and equal-cost ranges keep the
@@ -31,7 +33,7 @@ namespace yitu {
 
 constexpr int kPlanChunk = 64;      // edges per item = one edge window of a wave
 constexpr int kPlanThreshold = 64;  // rows with at least this many edges are planned
-constexpr int kPlanSlabs = 8;       // source ranges at whose boundaries long rows are cut
+constexpr int kPlanSlabs = 4;       // source ranges at whose boundaries long rows are cut
 constexpr int kPlanMinSegment = 16; // a row of deg edges is cut into at most deg / 16 pieces,
                                     // none shorter than this
 
@@ -53,7 +55,7 @@ struct PlanView {
 };
 
 inline int64_t plan_max_rows(int64_t nnz) { return nnz / kPlanThreshold + 1; }
-// A row of deg >= 64 edges gives at most deg / 64 + min(8, deg / 16) items.
+// A row of deg >= 64 edges gives at most deg / 64 + min(4, deg / 16) items.
 inline int64_t plan_max_items(int64_t nnz) {
     return nnz / kPlanChunk + nnz / kPlanMinSegment + plan_max_rows(nnz) + 1;
 }
