@@ -72,8 +72,33 @@ static int dispatch_shape(const SpmmParams &p, bool with_hub, hipStream_t stream
     }
 }
 
+// Unweighted fp32 rows of 1, 2 or 4 floats: one lane per edge.
+template <int VEC>
+static int launch_tiny(const SpmmParams &p, bool has_items, hipStream_t stream) {
+    tiny_rows_kernel<VEC>
+        <<<(int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    if (has_items) {
+        const int item_grid = (int)std::min<int64_t>(
+            ceil_div(p.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+        tiny_items_kernel<VEC><<<item_grid, kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        spmm_reduce_kernel<W_NONE, VEC>
+            <<<(int)std::min<int64_t>(p.plan.max_rows, 1 << 16), kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 template <int WMODE>
 static int dispatch_type(const SpmmParams &p, bool bf16_in, bool with_hub, hipStream_t stream) {
+    if constexpr (WMODE == W_NONE) {
+        if (!bf16_in && aligned16(p.feat) && aligned16(p.out)) {
+            if (p.L == 4) return launch_tiny<4>(p, with_hub, stream);
+            if (p.L == 2) return launch_tiny<2>(p, with_hub, stream);
+            if (p.L == 1) return launch_tiny<1>(p, with_hub, stream);
+        }
+    }
     // a lane's VEC elements must stay inside one head and one aligned vector
     const int unit = WMODE == W_EDGEHEAD ? p.F : p.L;
     if constexpr (WMODE != W_EDGEHEAD) {

@@ -422,6 +422,118 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
     }
 }
 
+
+// ---- rows of at most 4 floats (one 16-byte vector or less) ------------------------
+// The generic mapping would leave 15 of 16 lanes of a slot idle. Here a lane owns
+// an EDGE: the window's 64 column ids and the 64 gathered vectors come from two
+// load instructions, and every row that lies inside the window is then a masked
+// full-wave butterfly sum: no further memory round trip per row. Unweighted sums
+// only (the grad_key gather of the attention backward).
+template <int VEC>
+struct TinyWindow {
+    int base;  // CSR position of lane 0; -1 = nothing loaded
+    float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ void load_tiny_window(TinyWindow<VEC> &w, const SpmmParams &p, int base,
+                                                 int limit) {
+    const int e = min(base + lane_id(), limit - 1);
+    const int c = p.indices[e] & p.col_mask;
+    w.base = base;
+    RowLoad<VEC, float>::ld(static_cast<const float *>(p.feat) + (size_t)c * VEC, w.v);
+}
+
+// sum of the window lanes [first, first + n) in every lane
+template <int VEC>
+__device__ __forceinline__ void tiny_sum(float (&acc)[VEC], const TinyWindow<VEC> &w, int first,
+                                         int n) {
+    const int lane = lane_id();
+    const bool in = lane >= first && lane < first + n;
+    float t[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++) t[i] = in ? w.v[i] : 0.0f;
+#pragma unroll
+    for (int o = kWave / 2; o >= 1; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < VEC; i++) t[i] += __shfl_xor(t[i], o, kWave);
+#pragma unroll
+    for (int i = 0; i < VEC; i++) acc[i] += t[i];
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.n_rows - r0);
+    const int my_ptr = p.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    TinyWindow<VEC> win;
+    win.base = -1;
+#pragma unroll
+    for (int i = 0; i < VEC; i++) win.v[i] = 0.0f;
+    for (int i = 0; i < n_here; i++) {
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        if (end - beg >= p.plan.threshold) continue;  // a planned row: the item kernel
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) acc[k] = 0.0f;
+        for (int b = beg; b < end; b += kWave) {
+            const int n = min(kWave, end - b);
+            if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                load_tiny_window<VEC>(win, p, b, limit);
+            tiny_sum<VEC>(acc, win, b - win.base, n);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc[k] *= p.alpha;
+            store_row<VEC>(p.out + (size_t)(r0 + i) * VEC, acc);
+        }
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void tiny_items_kernel(SpmmParams p) {
+    const int lane = lane_id();
+    if (p.plan.counters->overflow) return;
+    const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.plan.records[pos0 + min(lane, n_here - 1)];
+        TinyWindow<VEC> win[kItemsPerWave];
+        int n[kItemsPerWave], item[kItemsPerWave], tag[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            const int beg = __shfl(my_rec.x, j, kWave), end = __shfl(my_rec.y, j, kWave);
+            item[j] = __shfl(my_rec.z, j, kWave);
+            tag[j] = __shfl(my_rec.w, j, kWave);
+            n[j] = j < n_here ? end - beg : 0;
+            if (n[j] > 0) load_tiny_window<VEC>(win[j], p, beg, end);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n[j] <= 0) continue;
+            float acc[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc[k] = 0.0f;
+            tiny_sum<VEC>(acc, win[j], 0, n[j]);
+            if (lane == 0) {
+                const bool single = tag[j] < 0;
+                if (single) {
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) acc[k] *= p.alpha;
+                }
+                store_row<VEC>(single ? p.out + (size_t)(tag[j] & 0x7fffffff) * VEC
+                                      : p.partial + (size_t)item[j] * VEC,
+                               acc);
+            }
+        }
+    }
+}
+
 // Picks the instantiation for (element type, L) and launches the row, item and reduce kernels.
 // max_degree_hint < 0 means unknown; plan may be null (a temporary one is then
 // built in the workspace). p.n_src and p.col_mask must be set.
