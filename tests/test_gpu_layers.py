@@ -81,3 +81,60 @@ def test_hetero_conv_mean_over_relations(dev):
     b1 = conv.convs["r1"](hgraph[rels[1]], norms[str(rels[1])], (xs["b"], xs["b"]))
     assert_close(out["b"], (b0 + b1) / 2)
     assert out["a"].shape == (50, 8)
+
+
+def test_two_layer_gcn_training_matches_dense_autograd(dev):
+    """Twenty SGD steps of a 2-layer GCN built from the module-1 conv (forward and the
+    reference-semantics backward through the C ABI) follow the same loss curve as a dense
+    autograd model. The graph is symmetric, where aggregating dY with the forward CSR
+    (the reference's backward, YiTu_GNN_kernel.cu:447-461) is the true gradient."""
+    import types
+
+    import torch.nn.functional as F_
+    from yitu_amd import YiTu_GNN_kernel as K
+    from yitu_amd.data import graphgen
+    from yitu_amd.nn.GCNConv import GCNConv
+
+    n, fin, hid, ncls = 600, 32, 16, 5
+    g = torch.Generator().manual_seed(11)
+    src = torch.randint(0, n, (4000,), generator=g)
+    dst = torch.randint(0, n, (4000,), generator=g)
+    loops = torch.arange(n)
+    rows = torch.cat([src, dst, loops])  # both directions: symmetric
+    cols = torch.cat([dst, src, loops])
+    indptr, indices = graphgen.csr_from_edges(rows, cols, n)
+    s = graphgen.gcn_norm(indptr)
+    pp, p2n = K.build_part(32, indptr)
+    info = types.SimpleNamespace(row_pointers=indptr.to(dev), column_index=indices.to(dev),
+                                 degrees=s.to(dev), partPtr=pp.to(dev), part2Node=p2n.to(dev),
+                                 partSize=32, dimWorker=32, warpPerBlock=8)
+    dense = torch.zeros(n, n)
+    r = torch.repeat_interleave(torch.arange(n), (indptr[1:] - indptr[:-1]).long())
+    dense[r, indices.long()] = s[r] * s[indices.long()]
+    dense = dense.to(dev)
+    x = torch.randn(n, fin, generator=g).to(dev)
+    teacher = torch.randn(fin, ncls, generator=g).to(dev)
+    y = (dense @ (x @ teacher)).argmax(1)  # labels a GCN can fit
+
+    torch.manual_seed(3)
+    c1, c2 = GCNConv(fin, hid).to(dev), GCNConv(hid, ncls).to(dev)
+    w1 = c1.weights.detach().clone().requires_grad_()
+    w2 = c2.weights.detach().clone().requires_grad_()
+    opt_a = torch.optim.SGD(list(c1.parameters()) + list(c2.parameters()), lr=0.5)
+    opt_b = torch.optim.SGD([w1, w2], lr=0.5)
+    losses_a, losses_b = [], []
+    for _ in range(20):
+        opt_a.zero_grad()
+        la = F_.nll_loss(F_.log_softmax(c2(torch.relu(c1(x, info)), info), dim=1), y)
+        la.backward()
+        opt_a.step()
+        opt_b.zero_grad()
+        lb = F_.nll_loss(F_.log_softmax(dense @ (torch.relu(dense @ (x @ w1)) @ w2), dim=1), y)
+        lb.backward()
+        opt_b.step()
+        losses_a.append(la.item())
+        losses_b.append(lb.item())
+    assert losses_a[-1] < losses_a[0] - 0.01          # it learns
+    assert np.allclose(losses_a, losses_b, rtol=2e-4, atol=2e-5), (losses_a, losses_b)
+    assert_close(c1.weights, w1, rtol=1e-3, atol=1e-4)
+    assert_close(c2.weights, w2, rtol=1e-3, atol=1e-4)
