@@ -439,6 +439,20 @@ def run_c5(args, dev):
         smp.sample(roots, root_ts)
     sample_ms = (time.perf_counter() - t0) * 1e3 / 5
     tgb = smp.get_ret()[0]
+    # the same sampling with the T-CSR and the cursors resident on the GPU
+    gsmp = sampler_core.GpuParallelSampler(indptr, other[order], eid[order], tt[order], 16, 1, 1,
+                                           [k], True, False, 1, 0.0, device=dev)
+    d_roots = torch.as_tensor(roots, dtype=torch.int32, device=dev)
+    d_root_ts = torch.as_tensor(root_ts, dtype=torch.float32, device=dev)
+
+    def gpu_sample():
+        gsmp.reset()
+        gsmp.sample(d_roots, d_root_ts)
+
+    gpu_sample_ms = _event_ms(gpu_sample, 20, 3)
+    dblk = gsmp.get_ret()[0].cpu_block()
+    assert all(np.array_equal(getattr(dblk, f)(), getattr(tgb, f)())
+               for f in ("row", "col", "eid", "ts", "dts", "nodes")), "device sampler differs"
     torch.manual_seed(20244)
     memory = torch.randn(n_nodes, 172, device=dev)
     layer = TransfomerAttentionLayer(172, 0, 100, 1, 0.0, 0.0, 100).to(dev)
@@ -459,7 +473,7 @@ def run_c5(args, dev):
             "config": {"workload": "c5_temporal_attention_f32", "n_nodes": n_nodes,
                        "n_events": n_events, "batch": batch, "neighbours": k,
                        "sampled_edges": blk.num_edges()},
-            "sampler_ms": sample_ms, "sampler_threads": 16,
+            "sampler_ms": sample_ms, "sampler_threads": 16, "gpu_sampler_ms": gpu_sample_ms,
             "note": "45 MB working set, launch-bound: time only"}
 
 

@@ -261,6 +261,34 @@ int yitu_gemm_bf16(void *c_device, int c_is_bf16, const void *a_bf16_device,
                    size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Temporal most-recent-neighbour sampling on the device                       */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * One layer of sampler_core.ParallelSampler.sample in its recent = True mode
+ * (YiTu_GNN/YiTu_T/sampler_core.cpp:103-127, 153-199, 295-305) with the T-CSR
+ * (indptr [n_nodes+1], indices / eid [E] int32, ts [E] float32 ascending per
+ * node) and the per-node cursors [n_nodes] in device memory. cursor is state:
+ * yitu_tsample_reset sets it to indptr[0..n_nodes) (ParallelSampler.reset),
+ * every call advances it. Outputs (device): row, col, eid_out with room for
+ * n_roots * fan entries; ts_out, dts_out, nodes_out with room for
+ * n_roots * (fan + 1); *n_edges_out (device int64) = number of sampled edges,
+ * or -1 if a root id is out of range. Same bits as yitu_sampler_sample of the
+ * host library.
+ */
+int yitu_tsample_reset(int32_t *cursor_device, const int32_t *indptr_device, int64_t n_nodes,
+                       void *stream);
+size_t yitu_tsample_workspace_bytes(int64_t n_roots);
+int yitu_tsample_recent(int32_t *row_device, int32_t *col_device, int32_t *eid_out_device,
+                        float *ts_out_device, float *dts_out_device, int32_t *nodes_out_device,
+                        long long *n_edges_device, int32_t *cursor_device,
+                        const int32_t *indptr_device, const int32_t *indices_device,
+                        const int32_t *eid_device, const float *ts_device, int64_t n_nodes,
+                        const int32_t *roots_device, const float *root_ts_device, int64_t n_roots,
+                        int fan, int prop_time, void *workspace_device, size_t workspace_bytes,
+                        void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */
 /* ------------------------------------------------------------------------- */
 

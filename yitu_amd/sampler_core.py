@@ -114,3 +114,114 @@ class ParallelSampler:
 
     def get_ret(self):
         return list(self._ret)
+
+
+class DeviceTemporalGraphBlock:
+    """A sampled block whose arrays are torch tensors on the GPU; the accessors
+    mirror TemporalGraphBlock (``.cpu_block()`` converts to the numpy form)."""
+
+    def __init__(self, row, col, eid, ts, dts, nodes, dim_in, dim_out):
+        self._a = (row, col, eid, ts, dts, nodes)
+        self._dim_in, self._dim_out = int(dim_in), int(dim_out)
+
+    def row(self):
+        return self._a[0]
+
+    def col(self):
+        return self._a[1]
+
+    def eid(self):
+        return self._a[2]
+
+    def ts(self):
+        return self._a[3]
+
+    def dts(self):
+        return self._a[4]
+
+    def nodes(self):
+        return self._a[5]
+
+    def dim_in(self):
+        return self._dim_in
+
+    def dim_out(self):
+        return self._dim_out
+
+    def cpu_block(self):
+        return TemporalGraphBlock(*[t.cpu().numpy() for t in self._a], self._dim_in, self._dim_out)
+
+
+class GpuParallelSampler:
+    """ParallelSampler (recent = True, one snapshot) with the T-CSR and the cursors
+    in device memory (yitu_tsample_recent): same constructor arguments, same
+    results bit for bit, blocks returned as DeviceTemporalGraphBlock."""
+
+    def __init__(self, indptr, indices, eid, ts, num_thread_per_worker, num_workers, num_layers,
+                 num_neighbors, recent, prop_time, num_history, window_duration, device="cuda"):
+        import torch
+        if not recent:
+            raise NotImplementedError("only recent=True (most-recent-k neighbours) is built")
+        if num_history != 1 or abs(window_duration) > 1e-7:
+            raise NotImplementedError("only num_history=1, window_duration=0 is built")
+        if len(num_neighbors) < num_layers:
+            raise ValueError("num_neighbors needs one entry per layer")
+        self._dev = torch.device(device)
+        to = lambda a, dt: torch.as_tensor(np.ascontiguousarray(a, dtype=dt)).to(self._dev)
+        self._indptr = to(indptr, np.int32)
+        self._indices = to(indices, np.int32)
+        self._eid = to(eid, np.int32)
+        self._ts = to(ts, np.float32)
+        self._n_nodes = self._indptr.numel() - 1
+        self._fan = [int(x) for x in num_neighbors[:num_layers]]
+        self._prop_time = bool(prop_time)
+        self._cursor = torch.empty(max(self._n_nodes, 1), dtype=torch.int32, device=self._dev)
+        self._ret = []
+        self.reset()
+
+    def reset(self):
+        from . import _lib
+        rc = _lib.lib().yitu_tsample_reset(_lib.ptr(self._cursor), _lib.ptr(self._indptr),
+                                           _lib.c_i64(self._n_nodes), _lib.stream_ptr(self._dev))
+        _lib.check(rc, "yitu_tsample_reset")
+
+    def _layer(self, roots, root_ts, fan):
+        import torch
+        from . import _lib
+        n = roots.numel()
+        i32 = lambda m: torch.empty(max(m, 1), dtype=torch.int32, device=self._dev)
+        f32 = lambda m: torch.empty(max(m, 1), dtype=torch.float32, device=self._dev)
+        row, col, eid = i32(n * fan), i32(n * fan), i32(n * fan)
+        ts, dts, nodes = f32(n * (fan + 1)), f32(n * (fan + 1)), i32(n * (fan + 1))
+        count = torch.empty(1, dtype=torch.int64, device=self._dev)
+        ws = _lib.workspace(_lib.size_fn("yitu_tsample_workspace_bytes")(_lib.c_i64(n)), self._dev)
+        with torch.cuda.device(self._dev):
+            rc = _lib.lib().yitu_tsample_recent(
+                _lib.ptr(row), _lib.ptr(col), _lib.ptr(eid), _lib.ptr(ts), _lib.ptr(dts),
+                _lib.ptr(nodes), _lib.ptr(count), _lib.ptr(self._cursor), _lib.ptr(self._indptr),
+                _lib.ptr(self._indices), _lib.ptr(self._eid), _lib.ptr(self._ts),
+                _lib.c_i64(self._n_nodes), _lib.ptr(roots), _lib.ptr(root_ts), _lib.c_i64(n),
+                _lib.c_int(fan), _lib.c_int(int(self._prop_time)), _lib.ptr(ws),
+                _lib.c_size(ws.numel()), _lib.stream_ptr(self._dev))
+        _lib.check(rc, "yitu_tsample_recent")
+        m = int(count.item())
+        if m < 0:
+            raise RuntimeError("sample failed: a root node id is out of range")
+        return DeviceTemporalGraphBlock(row[:m], col[:m], eid[:m], ts[:n + m], dts[:n + m],
+                                        nodes[:n + m], n + m, n)
+
+    def sample(self, root_nodes, root_ts):
+        import torch
+        roots = torch.as_tensor(root_nodes).to(self._dev, torch.int32).contiguous()
+        ts = torch.as_tensor(root_ts).to(self._dev, torch.float32).contiguous()
+        if roots.shape != ts.shape or roots.dim() != 1:
+            raise ValueError("root_nodes and root_ts must be 1-D and equally long")
+        self._ret = []
+        for fan in self._fan:
+            blk = self._layer(roots, ts, fan)
+            self._ret.append(blk)
+            # the next layer expands every node of this block (roots and neighbours)
+            roots, ts = blk.nodes(), blk.ts()
+
+    def get_ret(self):
+        return list(self._ret)

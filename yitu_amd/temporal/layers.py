@@ -67,6 +67,27 @@ class TemporalBlock:
             h = memory[ids].to(device)
         return TemporalBlock(tgb.row(), n_dst, tgb.dts()[n_dst:], h=h, device=device)
 
+    @staticmethod
+    def from_device_block(dtgb, memory):
+        """The same from a DeviceTemporalGraphBlock (GpuParallelSampler): nothing
+        leaves the GPU. ``memory`` is the [num_nodes, dim] feature table on it."""
+        b = TemporalBlock.__new__(TemporalBlock)
+        dev = memory.device
+        n_dst = dtgb.dim_out()
+        row = dtgb.row().to(torch.int64)
+        indptr = torch.zeros(n_dst + 1, dtype=torch.int64, device=dev)
+        indptr[1:] = torch.cumsum(torch.bincount(row, minlength=n_dst), 0)
+        b.n_dst = int(n_dst)
+        b.n_edges = int(row.numel())
+        b.row = row
+        b.blk = xblock.Block([n_dst, b.n_edges],
+                             [indptr.to(torch.int32),
+                              torch.arange(b.n_edges, dtype=torch.int32, device=dev)])
+        b.dt = dtgb.dts()[n_dst:]
+        b.h = memory[dtgb.nodes().to(torch.int64)]
+        b.f = None
+        return b
+
     def num_edges(self):
         return self.n_edges
 
