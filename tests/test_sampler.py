@@ -162,3 +162,34 @@ def test_against_compiled_reference_live(seed):
         for f in FIELDS:
             assert np.array_equal(getattr(g, f)(), np.asarray(getattr(w, f)())), (seed, b, f)
         assert (g.dim_in(), g.dim_out()) == (w.dim_in(), w.dim_out())
+
+
+@pytest.mark.parametrize("add_reverse", [True, False])
+def test_build_tcsr_equals_per_node_lists_sorted_by_time(add_reverse):
+    """gen_graph.py:40-95 restated with Python lists and a stable sort, on a stream whose
+    timestamps repeat (ties keep stream order) and arrive unsorted."""
+    import torch
+    from yitu_amd.temporal import build_tcsr
+    rng = np.random.default_rng(3)
+    n, m = 40, 600
+    src, dst = rng.integers(0, n, m), rng.integers(0, n, m)
+    ts = rng.integers(0, 50, m).astype(np.float32)
+    lists = [[] for _ in range(n)]
+    for e in range(m):
+        lists[src[e]].append((ts[e], dst[e], e))
+        if add_reverse:
+            lists[dst[e]].append((ts[e], src[e], e))
+    indptr, indices, eid, tt = [0], [], [], []
+    for l in lists:
+        for t, d, e in sorted(l, key=lambda x: x[0]):  # stable
+            indices.append(d), eid.append(e), tt.append(t)
+        indptr.append(len(indices))
+    got = build_tcsr(torch.from_numpy(src), torch.from_numpy(dst), torch.from_numpy(ts), n,
+                     add_reverse)
+    assert [g.dtype for g in got] == [torch.int32, torch.int32, torch.int32, torch.float32]
+    assert np.array_equal(got[0].numpy(), indptr) and np.array_equal(got[1].numpy(), indices)
+    assert np.array_equal(got[2].numpy(), eid) and np.array_equal(got[3].numpy(), tt)
+    # and it is a valid input of the sampler
+    s = sampler_core.ParallelSampler(*[g.numpy() for g in got], 1, 1, 1, [5], True, False, 1, 0.0)
+    s.sample(src[-20:], np.full(20, 60.0, np.float32))
+    assert s.get_ret()[0].dim_out() == 20
