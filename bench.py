@@ -316,12 +316,20 @@ def run_c1(args, dev):
 def run_c4(args, dev):
     """Fourth configuration: heterogeneous RGCN layer, 4 node types, 8 relations of
     average degree 8, features 256. Forward: per-type GEMM H_t = X_t W_t on the
-    matrix cores, per-relation mean aggregation, sum over the relations of a
-    destination type. Backward: transposed aggregation, dW_t = X_t^T dH_t,
-    dX_t = dH_t W_t^T. The dominant dense kernel is the fp32 MFMA GEMM."""
+    matrix cores, written into one buffer; per-relation mean aggregation and the
+    sum over the relations of a destination type as ONE edge-weighted SpMM over the
+    stacked CSR (xgnn_h.block.stack_blocks). Backward: the same over the transposed
+    structure, dW_t = X_t^T dH_t, dX_t = dH_t W_t^T. The dominant dense kernel is
+    the fp32 MFMA GEMM. The relation-by-relation composition (one aggregation
+    launch per relation plus elementwise scale / add passes) is timed beside it."""
     from yitu_amd import YiTu_GNN_kernel as K, graph_ext
     from yitu_amd.data import graphgen
+    from yitu_amd.xgnn_h import block as xblock
     sizes = [1 << 18, 1 << 17, 1 << 16, 1 << 15]
+    off = [0]
+    for n in sizes:
+        off.append(off[-1] + n)
+    n_all = off[-1]
     dim = 256
     g = torch.Generator(device=dev).manual_seed(20243)
     xs = [torch.randn(n, dim, generator=g, device=dev) for n in sizes]
@@ -330,45 +338,56 @@ def run_c4(args, dev):
     for r in range(8):
         s_t, d_t = r % 4, (r + 1 + r // 4) % 4
         rp, ci = graphgen.bipartite_uniform(sizes[d_t], sizes[s_t], 8, 20243 + r, device=dev)
-        # the transposed structure for the backward aggregation (CSR by source)
-        rows = torch.repeat_interleave(torch.arange(sizes[d_t], device=dev),
-                                       (rp[1:] - rp[:-1]).long())
-        rp_t, ci_t = graphgen.csr_from_edges(ci.long(), rows, sizes[s_t], sizes[d_t])
         indeg = (rp[1:] - rp[:-1]).float()
         norm = torch.where(indeg > 0, 1.0 / indeg.clamp(min=1), torch.zeros_like(indeg))[:, None]
-        rels.append((s_t, d_t, rp, ci, rp_t, ci_t, norm))
+        rels.append((s_t, d_t, rp, ci, norm))
     n_edges = sum(int(r[3].numel()) for r in rels)
     n_rel_dst = [sum(1 for r in rels if r[1] == t) for t in range(4)]
-    d_out = [torch.randn(n, dim, generator=g, device=dev) for n in sizes]
+    stacked, values = xblock.stack_blocks(
+        [xblock.Block([sizes[d], sizes[s]], [rp, ci]) for s, d, rp, ci, _ in rels],
+        [off[d] for _, d, _, _, _ in rels], [off[s] for s, _, _, _, _ in rels], n_all, n_all,
+        [norm / n_rel_dst[d] for _, d, _, _, norm in rels])
+    indptr, indices = stacked.adj_sparse
+    h_all = torch.empty(n_all, dim, device=dev)
+    d_out = torch.randn(n_all, dim, generator=g, device=dev)
 
     def gemm_fwd():
-        return [graph_ext.sgemm(x, w) for x, w in zip(xs, wts)]
+        for t in range(4):
+            graph_ext.sgemm(xs[t], wts[t], out=h_all[off[t]:off[t + 1]])
 
-    def agg_fwd(hs):
+    def agg_fwd():
+        return graph_ext.spmm_forward(values, indptr, indices, h_all.view(n_all, 1, dim))
+
+    def agg_bwd():
+        return graph_ext.spmm_backward(values, indptr, indices, h_all.view(n_all, 1, dim),
+                                       d_out.view(n_all, 1, dim), need_grad_a=False)[1]
+
+    def gemm_bwd(dh):
+        dh = dh.view(n_all, dim)
+        parts = [dh[off[t]:off[t + 1]] for t in range(4)]
+        return ([graph_ext.sgemm(x, p, trans_a=True) for x, p in zip(xs, parts)],
+                [graph_ext.sgemm(p, w, trans_b=True) for p, w in zip(parts, wts)])
+
+    def agg_fwd_by_relation(hs):
         outs = [None] * 4
-        for s_t, d_t, rp, ci, _, _, norm in rels:
+        for s_t, d_t, rp, ci, norm in rels:
             o = K._aggregate(hs[s_t], rp, ci, None, 1.0) * norm
             outs[d_t] = o if outs[d_t] is None else outs[d_t] + o
         return [o / c for o, c in zip(outs, n_rel_dst)]
 
-    def agg_bwd():
-        dhs = [None] * 4
-        for s_t, d_t, _, _, rp_t, ci_t, norm in rels:
-            gsrc = K._aggregate(d_out[d_t] * (norm / n_rel_dst[d_t]), rp_t, ci_t, None, 1.0)
-            dhs[s_t] = gsrc if dhs[s_t] is None else dhs[s_t] + gsrc
-        return dhs
-
-    def gemm_bwd(dhs):
-        return ([graph_ext.sgemm(x, dh, trans_a=True) for x, dh in zip(xs, dhs)],
-                [graph_ext.sgemm(dh, w, trans_b=True) for dh, w in zip(dhs, wts)])
-
-    hs = gemm_fwd()
-    dhs = agg_bwd()
+    gemm_fwd()
+    hs = [h_all[off[t]:off[t + 1]] for t in range(4)]
+    by_rel = torch.cat(agg_fwd_by_relation(hs))
+    one = agg_fwd().view(n_all, dim)
+    if not torch.allclose(one, by_rel, rtol=1e-5, atol=1e-4):
+        raise RuntimeError("stacked aggregation differs from the per-relation composition")
+    dh = agg_bwd()
     steps, warm = args.steps, args.warmup
     t_gemm_f = _event_ms(gemm_fwd, steps, warm)
-    t_agg_f = _event_ms(lambda: agg_fwd(hs), steps, warm)
+    t_agg_f = _event_ms(agg_fwd, steps, warm)
     t_agg_b = _event_ms(agg_bwd, steps, warm)
-    t_gemm_b = _event_ms(lambda: gemm_bwd(dhs), steps, warm)
+    t_gemm_b = _event_ms(lambda: gemm_bwd(dh), steps, warm)
+    t_agg_rel = _event_ms(lambda: agg_fwd_by_relation(hs), steps, warm)
     t_torch = _event_ms(lambda: [torch.mm(x, w) for x, w in zip(xs, wts)], steps, warm)
     flops_f = sum(2 * n * dim * dim for n in sizes)
     total = t_gemm_f + t_agg_f + t_agg_b + t_gemm_b
@@ -382,16 +401,21 @@ def run_c4(args, dev):
 
     hs16 = gemm16()
     t_gemm16 = _event_ms(gemm16, steps, warm)
-    t_agg16 = _event_ms(lambda: agg_fwd(hs16), steps, warm)
+    t_agg16 = _event_ms(lambda: agg_fwd_by_relation(hs16), steps, warm)
     t_torch16 = _event_ms(lambda: [torch.mm(x, w) for x, w in zip(xs16, wts16)], steps, warm)
     bytes16 = sum(2 * n * dim * 2 + 2 * dim * dim for n in sizes)
+    gather = n_edges * dim * 4
     peak = 157.3  # fp32 matrix TFLOP/s, published
     return {"value": n_edges / (total * 1e-3), "unit": "edges/s", "ms_per_step": total, "dtype": "f32",
             "config": {"workload": "c4_rgcn_f32", "node_types": sizes, "relations": 8,
-                       "n_edges": n_edges, "feature_dim": dim},
+                       "n_edges": n_edges, "feature_dim": dim,
+                       "aggregation": "one edge-weighted SpMM over the stacked relations"},
             "gemm_fwd_ms": t_gemm_f, "agg_fwd_ms": t_agg_f, "agg_bwd_ms": t_agg_b,
             "gemm_bwd_ms": t_gemm_b, "torch_mm_fwd_ms": t_torch,
-            "bf16": {"gemm_fwd_ms": t_gemm16, "agg_fwd_ms": t_agg16, "torch_mm_fwd_ms": t_torch16,
+            "agg_fwd_by_relation_ms": t_agg_rel,
+            "agg_gather_GBps": gather / (t_agg_f * 1e-3) / 1e9,
+            "bf16": {"gemm_fwd_ms": t_gemm16, "agg_fwd_by_relation_ms": t_agg16,
+                     "torch_mm_fwd_ms": t_torch16,
                      "gemm_TFLOPs": flops_f / (t_gemm16 * 1e-3) / 1e12,
                      "gemm_GBps": bytes16 / (t_gemm16 * 1e-3) / 1e9,
                      "gemm_hbm_frac": bytes16 / (t_gemm16 * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -138,3 +138,54 @@ def test_two_layer_gcn_training_matches_dense_autograd(dev):
     assert np.allclose(losses_a, losses_b, rtol=2e-4, atol=2e-5), (losses_a, losses_b)
     assert_close(c1.weights, w1, rtol=1e-3, atol=1e-4)
     assert_close(c2.weights, w2, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("per_relation", [True, False])
+def test_stacked_hetero_gcn_equals_per_relation_convs(dev, per_relation):
+    """One stacked edge-weighted SpMM == HeteroGraphConv over GCNLayers (model.py:137-171):
+    outputs, input gradients and weight gradients, with weights per edge type or shared
+    per source node type."""
+    torch.manual_seed(4)
+    sizes = {"a": 90, "b": 130, "c": 40}
+    rels = [("a", "r0", "b"), ("b", "r1", "b"), ("b", "r2", "a"), ("c", "r3", "a"),
+            ("a", "r4", "c")]
+    fin, fout = 20, 12
+    hgraph, norms = {}, {}
+    for i, (s, e, d) in enumerate(rels):
+        ip, ix = random_csr(sizes[d], sizes[s], 0.08, 30 + i, empty_rows=(i,))
+        blk = xblock.Block([sizes[d], sizes[s]], [ip, ix]).to(dev)
+        hgraph[(s, e, d)] = blk
+        norms[str((s, e, d))] = layers.right_norm(blk)
+    stacked = layers.StackedHeteroGCN(sizes, rels, fin, fout, per_relation=per_relation).to(dev)
+    stacked.stack(hgraph, norms)
+    conv = layers.HeteroGraphConv({e: layers.GCNLayer(fin, fout) for _, e, _ in rels}).to(dev)
+    with torch.no_grad():
+        for s, e, _ in rels:
+            src = stacked.fcs[e if per_relation else s]
+            conv.convs[e].fc.weight.copy_(src.weight)
+            conv.convs[e].fc.bias.copy_(src.bias)
+    xs = {t: torch.randn(n, fin, device=dev, requires_grad=True) for t, n in sizes.items()}
+    ws = {t: torch.randn(n, fout, device=dev) for t, n in sizes.items()}
+
+    out = stacked(xs)
+    sum((out[t] * ws[t]).sum() for t in out).backward()
+    got_x = {t: xs[t].grad.clone() for t in xs}
+    got_w = {k: (fc.weight.grad.clone(), fc.bias.grad.clone()) for k, fc in stacked.fcs.items()}
+    for t in xs:
+        xs[t].grad = None
+
+    want = conv(hgraph, xs, norms)
+    sum((want[t] * ws[t]).sum() for t in want).backward()
+    assert set(out) == set(want)
+    for t in want:
+        assert_close(out[t], want[t], rtol=1e-5, atol=1e-4)
+    for t in xs:
+        assert_close(got_x[t], xs[t].grad, rtol=1e-5, atol=1e-4)
+    for k, (gw, gb) in got_w.items():
+        if per_relation:
+            ref_w, ref_b = conv.convs[k].fc.weight.grad, conv.convs[k].fc.bias.grad
+        else:  # shared per source type: the sum over the relations that leave it
+            ref_w = sum(conv.convs[e].fc.weight.grad for s, e, _ in rels if s == k)
+            ref_b = sum(conv.convs[e].fc.bias.grad for s, e, _ in rels if s == k)
+        assert_close(gw, ref_w, rtol=1e-5, atol=1e-4)
+        assert_close(gb, ref_b, rtol=1e-5, atol=1e-4)

@@ -159,3 +159,39 @@ def test_b2gemm_equals_two_linears():
     assert_close(dx, x.grad.float())
     assert_close(dwa, fc1.weight.grad.float())
     assert_close(dwb, fc2.weight.grad.float())
+
+
+def test_stack_blocks_places_every_block_in_the_union_matrix():
+    """stack_blocks against a dense construction: block b lands at (row_offsets[b],
+    col_offsets[b]) with its row scales as edge weights; inside a row the edges keep
+    block order, then the block's own order."""
+    rng = np.random.default_rng(5)
+    shapes = [(7, 9), (7, 4), (5, 9), (3, 6)]       # (n_dst, n_src) per block
+    row_off, col_off = [0, 0, 7, 12], [0, 9, 4, 13]  # overlapping row ranges (0 and 1), shared columns
+    n_rows, n_cols = 15, 19
+    blocks, scales, dense = [], [], np.zeros((n_rows, n_cols))
+    for b, (nd, ns) in enumerate(shapes):
+        ip, ix = random_csr(nd, ns, 0.4, 50 + b, empty_rows=(b,))
+        sc = torch.tensor(rng.uniform(0.5, 2.0, nd), dtype=torch.float32)
+        blocks.append(xblock.Block([nd, ns], [ip, ix]))
+        scales.append(sc)
+        for r in range(nd):
+            for i in range(int(ip[r]), int(ip[r + 1])):
+                dense[row_off[b] + r, col_off[b] + int(ix[i])] += float(sc[r])
+    blk, values = xblock.stack_blocks(blocks, row_off, col_off, n_rows, n_cols, scales)
+    indptr, indices = blk.adj_sparse
+    assert indptr.dtype == torch.int32 and indices.dtype == torch.int32
+    assert blk.size == [n_rows, n_cols] and values.shape == (indices.numel(), 1)
+    assert indices.numel() == sum(b.adj_sparse[1].numel() for b in blocks)
+    got = np.zeros((n_rows, n_cols))
+    for r in range(n_rows):
+        for i in range(int(indptr[r]), int(indptr[r + 1])):
+            got[r, int(indices[i])] += float(values[i, 0])
+    assert np.allclose(got, dense, atol=1e-6)
+    # row 2 of the union: block 0's edges first, then block 1's, each in its own order
+    want = [int(c) for c in blocks[0].adj_sparse[1][blocks[0].adj_sparse[0][2]:blocks[0].adj_sparse[0][3]]]
+    want += [9 + int(c) for c in blocks[1].adj_sparse[1][blocks[1].adj_sparse[0][2]:blocks[1].adj_sparse[0][3]]]
+    assert indices[indptr[2]:indptr[3]].tolist() == want
+    # no scales: unit weights
+    _, ones = xblock.stack_blocks(blocks, row_off, col_off, n_rows, n_cols)
+    assert torch.equal(ones, torch.ones_like(values))

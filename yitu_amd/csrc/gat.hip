@@ -14,6 +14,11 @@
 // Rows of 64 or more edges take the row plan's band-ordered 64-edge items:
 // item statistics, per-row merge, item apply (attn + partial rows), and the SpMM
 // reduce kernel, which adds a row's partials in a fixed order.
+//
+// Backward: one pass over the by-source structure gathers grad_out[row] once per
+// edge and produces both d_attn (dot with the source's own row) and grad_x
+// (attn-weighted sum); the softmax + LeakyReLU backward and the grad_key sum
+// then work on [nnz, H] edge arrays only.
 #include "../../include/yitu_hip.h"
 #include "sddmm_kernels.hpp"
 
@@ -317,202 +322,26 @@ __global__ __launch_bounds__(kBlock) void gat_item_apply_kernel(GatParams p) {
     }
 }
 
-// ---- backward, short rows -------------------------------------------------------
-// For a row of fewer than 64 edges the whole backward of the attention fits one
-// wave and one edge window: the per-edge dot d_attn = <grad_out[row,h,:], x[col,h,:]>
-// (the only gather), the three row sums of the softmax + LeakyReLU backward
+// ---- backward of the softmax + LeakyReLU ----------------------------------------
+// Given d_attn per edge and head, the three row sums
 //   S = sum a d_attn,  A1 = sum a d_attn s,  A2 = sum a s   (s = LeakyReLU slope)
-// the per-edge logit gradient a (d_attn - S) s and grad_q = A1 - S A2. Lane
-// layout: the 256-float row is spread over the 64 lanes (4 floats each), so a
-// head owns LPH = F / 4 consecutive lanes and the dot of one edge is reduced
-// inside that group; every lane of the group accumulates the head's sums, and
-// lane (k % LPH) of the group keeps d_attn of edge k in register k / LPH, which is
-// the (edge, head) layout the second pass needs. d_attn never goes to memory.
+// give the per-edge logit gradient a (d_attn - S) s and grad_q = A1 - S A2.
 struct GatBwdParams {
-    SpmmParams sp;  // indptr, indices, feat = x [n_src, L], n_rows, L, F, H, col_mask, plan
-    const float *grad_out;  // [n_dst, L]
+    SpmmParams sp;  // indptr, indices, n_rows, H, col_mask, plan
+    const float *grad_out;  // unused by the attention-only kernels
     const float *query, *key, *attn;
     float *grad_q;  // [n_dst, H]
     float *grad_e;  // [nnz, H] per-edge logit gradient
     // planned rows (three kernels: item sums, row combine, item apply)
-    float *grad_a;      // [nnz, H] d_attn of the planned rows' edges
+    float *grad_a;      // [nnz, H] d_attn (input)
     float *item_sums;   // [plan item id][H][3]: (S, A1, A2) over the item's edges
     float *row_sum;     // [n_dst][H]: S of every planned row
     int HP;             // heads rounded up to a power of two (item sums / combine lane layout)
 };
 
-// d_attn of the n (<= 64) edges in window lanes [first, first + n) against the
-// row's grad_out tile, left in `keep` in the (edge, head) layout: lane (h, sub)
-// gets edge j * LPH + sub in keep[j]. kDotUnroll gathers are in flight at a time.
-constexpr int kDotUnroll = 4;  // gathers in flight per wave in the backward dots (LPH >= 8)
+constexpr int kDotUnroll = 4;  // gathers in flight per wave in the backward dots
 
-template <int LPH>
-__device__ __forceinline__ void gat_bwd_dots(const GatBwdParams &p, const EdgeWindow &win,
-                                             int first, int n, const float (&gt)[4],
-                                             float (&keep)[kWave / LPH]) {
-    constexpr int NS = kWave / LPH;
-    const int lane = lane_id();
-    const int sub = lane % LPH;
-    const int L = p.sp.L;
-    const float *__restrict__ x = static_cast<const float *>(p.sp.feat);
-#pragma unroll
-    for (int j = 0; j < NS; j++) {
-        keep[j] = 0.0f;
-        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += kDotUnroll) {
-            float v[kDotUnroll][4];
-#pragma unroll
-            for (int u = 0; u < kDotUnroll; u++) {
-                const int k = j * LPH + kk + u;
-                if (k < n) {  // wave-uniform
-                    const int c = __builtin_amdgcn_readlane(win.col, first + k);
-                    RowLoad<4, float>::ld(x + (size_t)c * L + lane * 4, v[u]);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kDotUnroll; u++) {
-                const int k = j * LPH + kk + u;
-                if (k < n) {
-                    float d = gt[0] * v[u][0] + gt[1] * v[u][1] + gt[2] * v[u][2] + gt[3] * v[u][3];
-#pragma unroll
-                    for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
-                    if (sub == kk + u) keep[j] = d;
-                }
-            }
-        }
-    }
-}
-
-// In the (edge, head) layout: attention a and LeakyReLU slope sl of this lane's
-// edges, and the head's sums S = sum a d, A1 = sum a d sl, A2 = sum a sl over the
-// n edges (identical in all lanes of the head afterwards).
-template <int LPH>
-__device__ __forceinline__ void gat_bwd_sums(const GatBwdParams &p, const EdgeWindow &win,
-                                             int first, int n, int beg, float qh,
-                                             const float (&keep)[kWave / LPH],
-                                             float (&a)[kWave / LPH], float (&sl)[kWave / LPH],
-                                             float &S, float &A1, float &A2) {
-    constexpr int NS = kWave / LPH;
-    const int lane = lane_id();
-    const int h = lane / LPH, sub = lane % LPH;
-    const int H = p.sp.H;
-    S = A1 = A2 = 0.0f;
-#pragma unroll
-    for (int j = 0; j < NS; j++) {
-        const int k = j * LPH + sub;
-        const int c = __shfl(win.col, first + min(k, n - 1), kWave);
-        a[j] = 0.0f;
-        sl[j] = 1.0f;
-        if (k < n) {
-            a[j] = p.attn[(size_t)(beg + k) * H + h];
-            sl[j] = qh + p.key[(size_t)c * H + h] < 0.0f ? kSlope : 1.0f;
-        }
-        S += a[j] * keep[j];
-        A1 += a[j] * keep[j] * sl[j];
-        A2 += a[j] * sl[j];
-    }
-#pragma unroll
-    for (int o = LPH >> 1; o >= 1; o >>= 1) {
-        S += __shfl_xor(S, o, kWave);
-        A1 += __shfl_xor(A1, o, kWave);
-        A2 += __shfl_xor(A2, o, kWave);
-    }
-}
-
-template <int LPH>
-__global__ __launch_bounds__(kBlock) void gat_bwd_rows_kernel(GatBwdParams p) {
-    constexpr int NS = kWave / LPH;  // = number of heads; registers of kept d_attn per lane
-    const int lane = lane_id();
-    const int h = lane / LPH, sub = lane % LPH;
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
-    if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
-    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
-    const int L = p.sp.L, H = p.sp.H;
-    EdgeWindow win;
-    win.base = -1;
-    win.col = 0;
-    win.w = 0.0f;
-    win.vrow = 0;
-    for (int i = 0; i < n_here; i++) {
-        const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
-        const int n = end - beg;
-        if (n >= p.sp.plan.threshold) continue;  // a planned row: the item kernels
-        if (n == 0) {
-            if (sub == 0) p.grad_q[(size_t)row * H + h] = 0.0f;
-            continue;
-        }
-        if (win.base < 0 || beg < win.base || end > win.base + kWave)
-            load_window<W_NONE>(win, p.sp, beg, limit);
-        const int first = beg - win.base;
-        float gt[4];
-        RowLoad<4, float>::ld(p.grad_out + (size_t)row * L + lane * 4, gt);
-        const float qh = p.query[(size_t)row * H + h];
-        float keep[NS], a[NS], sl[NS], S, A1, A2;
-        gat_bwd_dots<LPH>(p, win, first, n, gt, keep);
-        gat_bwd_sums<LPH>(p, win, first, n, beg, qh, keep, a, sl, S, A1, A2);
-        if (sub == 0) p.grad_q[(size_t)row * H + h] = A1 - S * A2;
-#pragma unroll
-        for (int j = 0; j < NS; j++) {
-            const int k = j * LPH + sub;
-            if (k < n) p.grad_e[(size_t)(beg + k) * H + h] = a[j] * (keep[j] - S) * sl[j];
-        }
-    }
-}
-
-// Planned rows, step 1: per item (<= 64 edges, band order, kItemsPerWave per
-// wave) the dots, written to grad_a in the (edge, head) layout, and the item's
-// partial (S, A1, A2).
-template <int LPH>
-__global__ __launch_bounds__(kBlock) void gat_bwd_items_kernel(GatBwdParams p) {
-    constexpr int NS = kWave / LPH;
-    const int lane = lane_id();
-    const int h = lane / LPH, sub = lane % LPH;
-    if (p.sp.plan.counters->overflow) return;
-    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
-    const int n_waves = gridDim.x * kWavesPerBlock;
-    const int L = p.sp.L, H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
-         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
-        const int n_here = min(kItemsPerWave, n_items - pos0);
-        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
-        EdgeWindow win[kItemsPerWave];
-        int e_beg[kItemsPerWave], n_edges[kItemsPerWave], row[kItemsPerWave], item[kItemsPerWave];
-#pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
-            e_beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item[j] = __shfl(my_rec.z, j, kWave);
-            row[j] = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
-            n_edges[j] = j < n_here ? end - e_beg[j] : 0;
-            if (n_edges[j] > 0) load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
-        }
-#pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
-            if (n_edges[j] <= 0) continue;
-            float gt[4];
-            RowLoad<4, float>::ld(p.grad_out + (size_t)row[j] * L + lane * 4, gt);
-            const float qh = p.query[(size_t)row[j] * H + h];
-            float keep[NS], a[NS], sl[NS], S, A1, A2;
-            gat_bwd_dots<LPH>(p, win[j], 0, n_edges[j], gt, keep);
-            gat_bwd_sums<LPH>(p, win[j], 0, n_edges[j], e_beg[j], qh, keep, a, sl, S, A1, A2);
-#pragma unroll
-            for (int i = 0; i < NS; i++) {
-                const int k = i * LPH + sub;
-                if (k < n_edges[j]) p.grad_a[(size_t)(e_beg[j] + k) * H + h] = keep[i];
-            }
-            if (sub == 0) {
-                float *st = p.item_sums + ((size_t)item[j] * H + h) * 3;
-                st[0] = S;
-                st[1] = A1;
-                st[2] = A2;
-            }
-        }
-    }
-}
-
-// Step 2: one wave per planned row adds its items' sums (lane = (item slot, head),
+// One wave per planned row adds its items' sums (lane = (item slot, head),
 // fixed butterfly), writes S of the row and grad_q = A1 - S A2.
 __global__ __launch_bounds__(kBlock) void gat_bwd_combine_kernel(GatBwdParams p) {
     if (p.sp.plan.counters->overflow) return;
@@ -545,7 +374,7 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_combine_kernel(GatBwdParams p)
     }
 }
 
-// Step 3: per-edge logit gradient of the planned rows' edges, (edge, head) per lane.
+// Per-edge logit gradient of the planned rows' edges, (edge, head) per lane.
 __global__ __launch_bounds__(kBlock) void gat_bwd_apply_kernel(GatBwdParams p) {
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
@@ -835,40 +664,156 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams
     }
 }
 
-static int gat_bwd_rows_launch(const GatBwdParams &p, hipStream_t stream) {
-    const int grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave);
-    switch (p.sp.F / 4) {
-        case 8: gat_bwd_rows_kernel<8><<<grid, kBlock, 0, stream>>>(p); break;
-        case 16: gat_bwd_rows_kernel<16><<<grid, kBlock, 0, stream>>>(p); break;
-        case 32: gat_bwd_rows_kernel<32><<<grid, kBlock, 0, stream>>>(p); break;
-        case 64: gat_bwd_rows_kernel<64><<<grid, kBlock, 0, stream>>>(p); break;
-        default: set_error("gat_bwd_rows: unsupported head width %d", p.sp.F); return -1;
+// ---- backward over the transposed structure: one gather for two results ----------
+// Walking the edges by source c, the source's own row x[c] is local and the
+// gathered row is grad_out[row_e]. That single gather gives both
+//   d_attn[e,h]   = <grad_out[row_e,h,:], x[c,h,:]>          (written in CSR order)
+//   grad_x[c,h,:] = sum_e attn[e,h] grad_out[row_e,h,:]
+// so the backward needs one pass over the 1 KB rows instead of two. Lane layout
+// as above: 4 floats per lane, a head owns LPH lanes, the dot of edge k is kept
+// by lane (k % LPH) of each head and stored through the edge permutation.
+struct GatSrcParams {
+    SpmmParams sp;   // indptr / indices / eperm = by-source structure, values = attn,
+                     // feat = grad_out, out = grad_x, plan = its row plan, partial
+    const float *x;  // [n_src, L]
+    float *grad_a;   // [nnz, H], CSR order
+};
+
+template <int LPH>
+__device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const EdgeWindow &win,
+                                               int first, int n, const float (&xt)[4],
+                                               float (&acc)[4]) {
+    constexpr int NS = kWave / LPH;
+    const int lane = lane_id();
+    const int h = lane / LPH, sub = lane % LPH;
+    const int L = p.sp.L, H = p.sp.H;
+    const float *__restrict__ g = static_cast<const float *>(p.sp.feat);
+#pragma unroll
+    for (int j = 0; j < NS; j++) {
+        if (j * LPH >= n) break;  // wave-uniform
+        float keep = 0.0f;
+        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += kDotUnroll) {
+            float v[kDotUnroll][4], a[kDotUnroll];
+#pragma unroll
+            for (int u = 0; u < kDotUnroll; u++) {
+                const int k = j * LPH + kk + u;
+                if (k < n) {  // wave-uniform
+                    const int r = __builtin_amdgcn_readlane(win.col, first + k);
+                    const int vr = __builtin_amdgcn_readlane(win.vrow, first + k);
+                    RowLoad<4, float>::ld(g + (size_t)r * L + lane * 4, v[u]);
+                    a[u] = p.sp.values[(size_t)vr * H + h];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kDotUnroll; u++) {
+                const int k = j * LPH + kk + u;
+                if (k < n) {
+                    float d = xt[0] * v[u][0] + xt[1] * v[u][1] + xt[2] * v[u][2] + xt[3] * v[u][3];
+#pragma unroll
+                    for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                    if (sub == kk + u) keep = d;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[i] += a[u] * v[u][i];
+                }
+            }
+        }
+        const int k = j * LPH + sub;
+        const int vr = __shfl(win.vrow, first + min(k, n - 1), kWave);
+        if (k < n) p.grad_a[(size_t)vr * H + h] = keep;
     }
+}
+
+template <int LPH>
+__global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int L = p.sp.L;
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int row = r0 + i;
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
+        float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (end > beg) RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
+        for (int b = beg; b < end; b += kWave) {
+            const int n = min(kWave, end - b);
+            if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                load_window<W_EDGEHEAD>(win, p.sp, b, limit);
+            gat_src_window<LPH>(p, win, b - win.base, n, xt, acc);
+        }
+        store_row<4>(p.sp.out + (size_t)row * L + lane * 4, acc);
+    }
+}
+
+template <int LPH>
+__global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int L = p.sp.L;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int n_edges[kItemsPerWave], tag[kItemsPerWave], item[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            const int beg = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            item[j] = __shfl(my_rec.z, j, kWave);
+            tag[j] = __shfl(my_rec.w, j, kWave);
+            n_edges[j] = j < n_here ? end - beg : 0;
+            if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;
+            const int row = tag[j] & 0x7fffffff;
+            float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
+            gat_src_window<LPH>(p, win[j], 0, n_edges[j], xt, acc);
+            float *dst = tag[j] < 0 ? p.sp.out + (size_t)row * L : p.sp.partial + (size_t)item[j] * L;
+            store_row<4>(dst + lane * 4, acc);
+        }
+    }
+}
+
+template <int LPH>
+static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, hipStream_t stream) {
+    gat_src_rows_kernel<LPH>
+        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    if (!has_items) return 0;
+    gat_src_items_kernel<LPH><<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
+                                                                kWavesPerBlock * kItemsPerWave),
+                                                       1 << 16),
+                                kBlock, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    spmm_reduce_kernel<W_NONE, 4>
+        <<<(int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16), kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
     return 0;
 }
 
-static int gat_bwd_items_launch(const GatBwdParams &p, hipStream_t stream) {
-    const int grid = (int)std::min<int64_t>(
-        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+static int gat_src_launch(const GatSrcParams &p, bool has_items, hipStream_t stream) {
     switch (p.sp.F / 4) {
-        case 8: gat_bwd_items_kernel<8><<<grid, kBlock, 0, stream>>>(p); break;
-        case 16: gat_bwd_items_kernel<16><<<grid, kBlock, 0, stream>>>(p); break;
-        case 32: gat_bwd_items_kernel<32><<<grid, kBlock, 0, stream>>>(p); break;
-        case 64: gat_bwd_items_kernel<64><<<grid, kBlock, 0, stream>>>(p); break;
-        default: set_error("gat_bwd_items: unsupported head width %d", p.sp.F); return -1;
+        case 8: return gat_src_launch_lph<8>(p, has_items, stream);
+        case 16: return gat_src_launch_lph<16>(p, has_items, stream);
+        case 32: return gat_src_launch_lph<32>(p, has_items, stream);
+        case 64: return gat_src_launch_lph<64>(p, has_items, stream);
     }
-    YITU_LAUNCH_CHECK();
-    gat_bwd_combine_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock),
-                                                    1 << 15),
-                             kBlock, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
-    gat_bwd_apply_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
-                                                           kWavesPerBlock * kItemsPerWave),
-                                                  1 << 16),
-                           kBlock, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
-    return 0;
+    set_error("gat backward: unsupported head width %d", p.sp.F);
+    return -1;
 }
 
 // ---- host side ----------------------------------------------------------------
@@ -1109,64 +1054,51 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
     YITU_REQUIRE(t_indptr && (nnz == 0 || (t_rows && t_perm)),
                  "gat_backward needs the transposed structure (yitu_csr_transpose)");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // Rows of 256 floats with a power-of-two head width: the rows below the plan
-    // threshold take the single-wave fused kernel, and the general kernels that
-    // follow skip them.
+    // Rows of 256 floats with a power-of-two head width: one pass over the
+    // transposed structure gives d_attn and grad_features from a single gather.
     const int64_t L = n_heads * n_features;
     const int lph = (int)(n_features / 4);
-    const bool fused_rows = L == 256 && n_features % 4 == 0 && lph >= 8 && (lph & (lph - 1)) == 0 &&
+    const bool one_gather = L == 256 && n_features % 4 == 0 && lph >= 8 && (lph & (lph - 1)) == 0 &&
                             n_dst > 0 && nnz > 0 && n_dst < INT32_MAX && n_src <= (1 << 24) &&
-                            aligned16(features) && aligned16(grad_out);
-    if (fused_rows) {
-        GatBwdParams p{};
-        p.sp.indptr = indptr;
-        p.sp.indices = indices;
-        p.sp.feat = features;
-        p.sp.n_rows = (int)n_dst;
-        p.sp.n_src = (int)n_src;
+                            aligned16(features) && aligned16(grad_out) &&
+                            aligned16(grad_features);
+    if (one_gather) {
+        GatSrcParams p{};
+        p.sp.indptr = t_indptr;
+        p.sp.indices = t_rows;
+        p.sp.eperm = t_perm;
+        p.sp.values = attn;
+        p.sp.feat = grad_out;
+        p.sp.out = grad_features;
+        p.sp.n_rows = (int)n_src;
+        p.sp.n_src = (int)n_dst;
         p.sp.L = (int)L;
         p.sp.F = (int)n_features;
         p.sp.H = (int)n_heads;
-        p.sp.col_mask = kColMask;
-        p.grad_out = grad_out;
-        p.query = query;
-        p.key = key;
-        p.attn = attn;
-        p.grad_q = grad_query;
-        p.grad_e = grad_edge_scratch;
+        p.sp.col_mask = 0x7fffffff;
+        p.sp.alpha = 1.0f;
+        p.x = features;
         p.grad_a = grad_attn_scratch;
-        p.HP = (int)n_heads;  // a power of two here
         bool has_items = false;
         void *rest = nullptr;
         size_t rest_bytes = 0;
-        int rc = plan_resolve(p.sp.plan, has_items, plan, indptr, indices, n_dst, n_src, nnz,
-                              kColMask, max_degree, workspace, workspace_bytes, &rest, &rest_bytes,
-                              stream);
-        if (rc) return rc;
-        if (!has_items) p.sp.plan.threshold = kPlanThreshold;  // rows of 64+ edges cannot exist
-        rc = gat_bwd_rows_launch(p, stream);
+        int rc = plan_resolve(p.sp.plan, has_items, plan_t, t_indptr, t_rows, n_src, n_dst, nnz,
+                              0x7fffffff, max_degree_t, workspace, workspace_bytes, &rest,
+                              &rest_bytes, stream);
         if (rc) return rc;
         if (has_items) {
-            const size_t sums = align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * n_heads), 256);
-            const size_t need = sums + sizeof(float) * (size_t)(n_dst * n_heads);
-            YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes", need);
-            p.item_sums = static_cast<float *>(rest);
-            p.row_sum = reinterpret_cast<float *>(static_cast<char *>(rest) + sums);
-            rc = gat_bwd_items_launch(p, stream);
-            if (rc) return rc;
+            const size_t need = sizeof(float) * (size_t)p.sp.plan.max_items * (size_t)L;
+            YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes",
+                         need);
+            p.sp.partial = static_cast<float *>(rest);
         }
-        // grad_x = attn-weighted gather of grad_out over the transposed structure
-        rc = spmm_backward_run(nullptr, grad_features, attn, indptr, indices, features, grad_out,
-                               t_indptr, t_rows, t_perm, n_dst, n_src, nnz, n_heads, n_features,
-                               max_degree, max_degree_t, plan, plan_t, workspace, workspace_bytes,
-                               false, stream);
+        rc = gat_src_launch(p, has_items, stream);
         if (rc) return rc;
-        // grad_key: the per-edge logit gradients gathered over the transposed structure;
-        // every row has been handled above, so the softmax backward kernels skip all rows
+        // softmax + LeakyReLU backward from d_attn; grad_key over the transposed structure
         return sddmm_backward_run(grad_query, grad_key, grad_edge_scratch, indptr, indices, query,
                                   key, attn, grad_attn_scratch, t_indptr, t_perm, n_dst, n_src, nnz,
                                   n_heads, 1, max_degree, max_degree_t, plan, plan_t, workspace,
-                                  workspace_bytes, INT32_MAX, stream);
+                                  workspace_bytes, 0, stream);
     }
     // d attn = <grad_out[row], x[col]> per edge and head; grad_x = attn-weighted
     // gather of grad_out over the transposed structure

@@ -112,8 +112,10 @@ def spmm_forward(values, indptr, indices, features):
     return out
 
 
-def spmm_backward(values, indptr, indices, features, grad_out):
-    """Returns [grad_a [E,H], grad_x [Ns,H,F]] (entry.cpp:92-104)."""
+def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
+                  need_grad_x=True):
+    """Returns [grad_a [E,H], grad_x [Ns,H,F]] (entry.cpp:92-104). A gradient
+    that the caller does not need is skipped and returned as None."""
     _check(values, torch.float32, "values", 2)
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
@@ -125,8 +127,10 @@ def spmm_backward(values, indptr, indices, features, grad_out):
     nnz = indices.numel()
     if grad_out.shape[0] != n_dst or grad_out.shape[1] != h or grad_out.shape[2] != f:
         raise RuntimeError("grad_out must be [n_dst, n_heads, n_features]")
-    grad_a = torch.empty_like(values)
-    grad_x = torch.empty_like(features)
+    if not (need_grad_a or need_grad_x):
+        return [None, None]
+    grad_a = torch.empty_like(values) if need_grad_a else None
+    grad_x = torch.empty_like(features) if need_grad_x else None
     tr = transposed(indptr, indices, n_src)
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
@@ -312,8 +316,9 @@ def b2gemm_backward(x, w_a, w_b, grad_a, grad_b):
     return [dx, dw_a, dw_b]
 
 
-def sgemm(a, b, trans_a=False, trans_b=False):
-    """op(a) . op(b) in fp32 on the matrix cores; a, b contiguous 2-D."""
+def sgemm(a, b, trans_a=False, trans_b=False, out=None):
+    """op(a) . op(b) in fp32 on the matrix cores; a, b contiguous 2-D. ``out``:
+    a contiguous [m, n] tensor (e.g. a row slice of a larger buffer) to write."""
     _check(a, torch.float32, "a", 2)
     _check(b, torch.float32, "b", 2)
     dev = _lib.require_device(a, b)
@@ -321,7 +326,13 @@ def sgemm(a, b, trans_a=False, trans_b=False):
     kb, n = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
     if k != kb:
         raise RuntimeError("inner dimensions differ: %d vs %d" % (k, kb))
-    c = torch.empty((m, n), dtype=torch.float32, device=dev)
+    if out is None:
+        c = torch.empty((m, n), dtype=torch.float32, device=dev)
+    else:
+        _check(out, torch.float32, "out", 2)
+        if tuple(out.shape) != (m, n) or out.device != dev:
+            raise RuntimeError("out must be [%d, %d] on the operands' device" % (m, n))
+        c = out
     ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(c_i64(m), c_i64(n), c_i64(k),
                                                                c_i64(1)), dev)
     with torch.cuda.device(dev):

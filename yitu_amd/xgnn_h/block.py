@@ -68,3 +68,42 @@ def stitch_csr(block_list: List[Block]):
     new_indptr[1:] = torch.cumsum(counts, 0)
     n_cols = sum(blk.size[1] for blk in block_list)
     return Block(size=[n_rows, n_cols], adj=[new_indptr.to(torch.int32), new_indices])
+
+
+def stack_blocks(block_list: List[Block], row_offsets: List[int], col_offsets: List[int],
+                 n_rows: int, n_cols: int, row_scales: List[torch.Tensor] = None):
+    """Places blocks in one [n_rows, n_cols] CSR over a union node space: block
+    ``b`` occupies rows ``row_offsets[b] + r`` and columns ``col_offsets[b] + c``.
+    Where ``stitch_csr`` (block.py:36-67) joins blocks of one destination set side
+    by side for one launch, this also stacks different destination sets, so that
+    a whole heterogeneous layer (per-relation aggregate, sum over the relations
+    of a destination type) is a single edge-weighted SpMM.
+
+    Returns ``(Block, values [E, 1])``; ``values[e] = row_scales[b][r]`` of the
+    block and row the edge came from (1 when no scales are given). Inside a row,
+    edges are ordered by block, then in the block's own order; columns are plain
+    ids (no block tag), so ``n_cols`` is limited to 2^24 like any packed CSR.
+    """
+    assert len(block_list) == len(row_offsets) == len(col_offsets) and len(block_list) > 0
+    assert n_cols <= 2 ** 24
+    dev = block_list[0].adj_sparse[0].device
+    rows, cols, vals, blk_of = [], [], [], []
+    for bid, blk in enumerate(block_list):
+        indptr, indices = blk.adj_sparse
+        assert row_offsets[bid] + blk.size[0] <= n_rows and col_offsets[bid] + blk.size[1] <= n_cols
+        deg = (indptr[1:] - indptr[:-1]).to(torch.int64)
+        r = torch.repeat_interleave(torch.arange(blk.size[0], device=dev), deg)
+        rows.append(r + row_offsets[bid])
+        cols.append((indices.to(torch.int64) & 0xFFFFFF) + col_offsets[bid])
+        if row_scales is not None:
+            vals.append(row_scales[bid].reshape(-1).to(torch.float32)[r])
+        else:
+            vals.append(torch.ones(r.numel(), dtype=torch.float32, device=dev))
+        blk_of.append(torch.full((r.numel(),), bid, dtype=torch.int64, device=dev))
+    rows, cols, vals, blk_of = torch.cat(rows), torch.cat(cols), torch.cat(vals), torch.cat(blk_of)
+    order = torch.argsort(rows * len(block_list) + blk_of, stable=True)
+    new_indptr = torch.zeros(n_rows + 1, dtype=torch.int64, device=dev)
+    new_indptr[1:] = torch.cumsum(torch.bincount(rows, minlength=n_rows), 0)
+    return (Block(size=[n_rows, n_cols],
+                  adj=[new_indptr.to(torch.int32), cols[order].to(torch.int32)]),
+            vals[order].unsqueeze(-1).contiguous())

@@ -93,3 +93,111 @@ class HeteroGraphConv(nn.Module):
         for dty, res in outputs.items():
             outputs[dty] = res / counts[dty]
         return outputs
+
+
+class _TypedLinear(torch.autograd.Function):
+    """y[off_i : off_i + n_i] = x_i . W_i^T (+ b_i) for every (x_i, W_i, b_i), all
+    written into one [sum n_i, out] buffer by the MFMA GEMM: the layout the
+    stacked aggregation reads, produced without a concatenation pass."""
+
+    @staticmethod
+    def forward(ctx, n_parts, *args):
+        from .. import graph_ext
+        xs, ws, bs = args[:n_parts], args[n_parts:2 * n_parts], args[2 * n_parts:]
+        total = sum(x.size(0) for x in xs)
+        y = torch.empty((total, ws[0].size(0)), dtype=torch.float32, device=xs[0].device)
+        off = 0
+        for x, w, b in zip(xs, ws, bs):
+            part = y[off:off + x.size(0)]
+            graph_ext.sgemm(x.contiguous(), w.contiguous(), trans_b=True, out=part)
+            if b is not None:
+                part += b
+            off += x.size(0)
+        ctx.n_parts = n_parts
+        ctx.has_bias = [b is not None for b in bs]
+        ctx.save_for_backward(*xs, *ws)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        from .. import graph_ext
+        n = ctx.n_parts
+        xs, ws = ctx.saved_tensors[:n], ctx.saved_tensors[n:]
+        grad_y = grad_y.contiguous()
+        gx, gw, gb = [], [], []
+        off = 0
+        for i, (x, w) in enumerate(zip(xs, ws)):
+            g = grad_y[off:off + x.size(0)]
+            gx.append(graph_ext.sgemm(g, w.contiguous()) if ctx.needs_input_grad[1 + i] else None)
+            gw.append(graph_ext.sgemm(g, x.contiguous(), trans_a=True)
+                      if ctx.needs_input_grad[1 + n + i] else None)
+            gb.append(g.sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None)
+            off += x.size(0)
+        return (None, *gx, *gw, *gb)
+
+
+class StackedHeteroGCN(nn.Module):
+    """``HeteroGraphConv`` over ``GCNLayer``s (model.py:137-171 with :7-30) as one
+    launch: the transformed features of all source sets sit in one buffer, the
+    relations are stacked into one CSR whose edge weights carry
+    ``norm[row] / (relations reaching the destination type)``, and a single
+    edge-weighted SpMM gives every destination type's output.
+
+    ``ntypes``: {node type: count}; ``relations``: [(src type, edge type, dst
+    type)]. ``per_relation=True`` keeps one Linear per edge type like the
+    reference's model; ``False`` shares one Linear per source node type (each
+    type's features are then transformed once, whatever the number of relations
+    leaving it). Parameters: ``fcs[edge type or node type]`` = ``nn.Linear``.
+    """
+
+    def __init__(self, ntypes: dict, relations: list, in_features: int, out_features: int,
+                 per_relation: bool = True, bias: bool = True):
+        super().__init__()
+        self.ntypes = dict(ntypes)
+        self.relations = [tuple(r) for r in relations]
+        self.per_relation = per_relation
+        # the feature buffer: one segment per relation (its source type's rows) or per type
+        self.segments = ([(ety, sty) for sty, ety, _ in self.relations] if per_relation
+                         else [(nty, nty) for nty in self.ntypes])
+        self.fcs = nn.ModuleDict({name: nn.Linear(in_features, out_features, bias=bias)
+                                  for name, _ in self.segments})
+        self.col_offset, off = {}, 0
+        for name, nty in self.segments:
+            self.col_offset[name] = off
+            off += self.ntypes[nty]
+        self.n_cols = off
+        self.row_offset, off = {}, 0
+        for nty in self.ntypes:
+            self.row_offset[nty] = off
+            off += self.ntypes[nty]
+        self.n_rows = off
+        self._stacked = None
+
+    def stack(self, hgraph: dict, norms: dict = None):
+        """Builds (once per graph) the stacked CSR and its edge weights from
+        ``hgraph`` {(src type, edge type, dst type): Block}; ``norms`` as in
+        ``HeteroGraphConv`` ({str(key): [n_dst, 1]}), default 1 / in-degree."""
+        reach = {}
+        for _, _, dty in self.relations:
+            reach[dty] = reach.get(dty, 0) + 1
+        blocks, rows, cols, scales = [], [], [], []
+        for sty, ety, dty in self.relations:
+            blk = hgraph[(sty, ety, dty)]
+            norm = norms[str((sty, ety, dty))] if norms else right_norm(blk)
+            blocks.append(blk)
+            rows.append(self.row_offset[dty])
+            cols.append(self.col_offset[ety if self.per_relation else sty])
+            scales.append(norm.reshape(-1) / reach[dty])
+        self._stacked = block.stack_blocks(blocks, rows, cols, self.n_rows, self.n_cols, scales)
+        return self._stacked
+
+    def forward(self, xs: dict, stacked=None):
+        blk, values = stacked if stacked is not None else self._stacked
+        parts = [xs[nty] for _, nty in self.segments]
+        fcs = [self.fcs[name] for name, _ in self.segments]
+        h = _TypedLinear.apply(len(parts), *parts, *[fc.weight for fc in fcs],
+                               *[fc.bias for fc in fcs])
+        out = sparse.gspmm(blk, values, h.unsqueeze(1)).squeeze(1)
+        reached = {dty for _, _, dty in self.relations}
+        return {nty: out[self.row_offset[nty]:self.row_offset[nty] + n]
+                for nty, n in self.ntypes.items() if nty in reached}

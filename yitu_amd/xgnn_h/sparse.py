@@ -25,7 +25,10 @@ class GSPMMFunction(autograd.Function):
         grad_out = grad_out.contiguous()
         assert len(ctx.needs_input_grad) == 3
         assert ctx.needs_input_grad[0] is False
-        grad_a, grad_x = graph_ext.spmm_backward(values, indptr, indices, x, grad_out)
+        # a gradient nobody asked for (constant edge weights) is not computed
+        grad_a, grad_x = graph_ext.spmm_backward(values, indptr, indices, x, grad_out,
+                                                 need_grad_a=ctx.needs_input_grad[1],
+                                                 need_grad_x=ctx.needs_input_grad[2])
         return None, grad_a, grad_x
 
 
