@@ -1,0 +1,97 @@
+"""Evaluates a dataflow graph on real arguments (the role of
+xgnn_h/executor.py). Lowered nodes run on the HIP ops; ``call`` nodes replay
+the recorded torch function; message-passing nodes that were not lowered are
+computed from their definitions (the reference raises on those,
+executor.py:145-146), which is what the parity tests compare a lowered graph
+against."""
+import torch
+from torch.nn import functional as F
+
+from . import block, bundle, ir, mp, sparse
+
+
+def _fill(template, values):
+    if isinstance(template, ir.Slot):
+        return values[template.key]
+    if isinstance(template, (list, tuple)):
+        return type(template)(_fill(t, values) for t in template)
+    if isinstance(template, dict):
+        return {k: _fill(t, values) for k, t in template.items()}
+    return template
+
+
+class Executor:
+    def __init__(self):
+        self._is_training = None
+
+    def eval(self):
+        self._is_training = False
+
+    def train(self):
+        self._is_training = True
+
+    # -- arguments by name -------------------------------------------------
+    @staticmethod
+    def _lookup(name: str, kwargs: dict):
+        head, _, rest = name.partition(".")
+        value = kwargs[head]
+        if not rest:
+            return value.blk if isinstance(value, mp.Graph) else value
+        if isinstance(value, mp.HeteroGraph):
+            sty, ety, dty = value.idx2rel[int(rest)]
+            return value.hetero_graph[sty, ety, dty].blk
+        if isinstance(value, dict):
+            return value[rest]
+        return value[int(rest)]
+
+    # -- one node ------------------------------------------------------------
+    def _eval(self, node: ir.Node, v: dict, kwargs: dict):
+        op = node.op
+        if op in ("input", "graph"):
+            return self._lookup(node.name, kwargs)
+        if op == "call":
+            return node.attrs["fn"](*_fill(node.attrs["args"], v), **_fill(node.attrs["kwargs"], v))
+        if op == "linear":
+            return F.linear(v["x"], node.attrs["weight"], node.attrs["bias"])
+        if op == "dropout":
+            if self._is_training is None:
+                raise RuntimeError("call train() or eval() on the executor first")
+            return F.dropout(v["x"], p=node.attrs["p"], training=self._is_training)
+        if op == "spmm":
+            return sparse.gspmm(v["g"], v.get("e"), v["x"])
+        if op == "sddmm":
+            return sparse.fused_gsddmm(v["g"], v["q"], v["k"])
+        if op == "gat":
+            return sparse.fused_gat(v["g"], v["q"], v["k"], v["x"])
+        if op == "bundle":
+            w_a, w_b = node.attrs["weights"]
+            b_a, b_b = node.attrs["biases"]
+            y_a, y_b = bundle.GEMMBundleFunction.apply(v["x"], w_a, w_b, b_a, b_b)
+            # the bundled GEMM leaves the biases out (bundle.py:8-14): add them here
+            return (y_a if b_a is None else y_a + b_a, y_b if b_b is None else y_b + b_b)
+        if op == "select":
+            return v["x"][node.attrs["index"]]
+        if op in ("concat", "stack"):
+            parts = [v[str(i)] for i in range(len(node.inputs))]
+            return torch.cat(parts, dim=0) if op == "concat" else torch.stack(parts, dim=0)
+        if op == "edge_values":
+            scales = torch.stack([v[str(i)].reshape(-1) for i in range(len(node.inputs) - 1)])
+            rows, _, bids = mp.edge_endpoints(v["g"])
+            return scales[bids, rows].unsqueeze(-1).contiguous()
+        if op == "edge":
+            args = {k: t for k, t in v.items() if k != "g"}
+            return mp.apply_edge(node.attrs["fn"], v["g"], **args)
+        if op == "vert":
+            return mp.apply_vert(node.attrs["fn"], v["g"], e=v["e"])
+        raise NotImplementedError("operator %r" % op)
+
+    def run(self, dataflow: ir.Dataflow, kwargs: dict):
+        """Evaluates the root (or every root of a dict) of ``dataflow``; ``kwargs``
+        are the model's arguments, plus ``stitch`` when the stitcher has run."""
+        values = {}
+        for node in ir.walk(dataflow):
+            ins = {k: values[id(c)] for k, c in node.inputs.items()}
+            values[id(node)] = self._eval(node, ins, kwargs)
+        if isinstance(dataflow, ir.Node):
+            return values[id(dataflow)]
+        return {k: values[id(n)] for k, n in dataflow.items()}

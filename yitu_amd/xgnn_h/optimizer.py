@@ -1,0 +1,110 @@
+"""Lowering of the message-passing operators to the sparse kernels (the role of
+xgnn_h/optimizer.py):
+
+* ``edge_softmax(leaky_relu(u_add_v(k, q)))``            -> ``sddmm(g, q, k)``
+* ``aggregate_sum(copy_u(x))``                            -> ``spmm(g, x)``
+* ``aggregate_sum(u_mul_e(x, e))``                        -> ``spmm(g, e, x)``
+  (optimizer.py:10-87 matches the same three shapes)
+* ``spmm(g, sddmm(g, q, k), x)`` with no other reader of the attention
+  -> ``gat(g, q, k, x)``: the fused kernel, one pass per destination row
+* the two ``linear`` nodes that produce q and k from one input
+  -> one ``bundle`` GEMM launch (what ``_bundle_gemm``, optimizer.py:89-104,
+  sets out to do and leaves empty)
+"""
+from torch.nn import functional as F
+
+from . import ir
+
+_SLOPE = 0.2  # the LeakyReLU slope the attention kernels implement (ops.cuh:1-3)
+
+
+def _leaky_input(node: ir.Node):
+    """The input of a ``leaky_relu`` call with the kernels' slope, else None."""
+    if node.op != "call" or node.attrs["fn"] is not F.leaky_relu:
+        return None
+    args, kwargs = node.attrs["args"], node.attrs["kwargs"]
+    slope = kwargs.get("negative_slope", args[1] if len(args) > 1 else 0.01)
+    if abs(slope - _SLOPE) > 1e-12 or not isinstance(args[0], ir.Slot):
+        return None
+    return node.inputs[args[0].key]
+
+
+class Optimizer:
+    def __init__(self, fuse_gat: bool = True, bundle_gemm: bool = True):
+        self.fuse_gat = fuse_gat
+        self.bundle_gemm = bundle_gemm
+
+    # -- message passing -> sddmm / spmm ------------------------------------
+    @staticmethod
+    def _lower_node(node: ir.Node) -> ir.Node:
+        if node.op == "edge" and node.attrs["fn"] == "edge_softmax":
+            logits = _leaky_input(node.inputs["e"])
+            if logits is not None and logits.op == "edge" and logits.attrs["fn"] == "u_add_v" \
+                    and logits.inputs["g"] is node.inputs["g"]:
+                return ir.Node("sddmm", {"g": node.inputs["g"], "q": logits.inputs["v"],
+                                         "k": logits.inputs["u"]}, size=node.size)
+        if node.op == "vert" and node.attrs["fn"] == "aggregate_sum":
+            msg = node.inputs["e"]
+            if msg.op == "edge" and msg.inputs["g"] is node.inputs["g"]:
+                if msg.attrs["fn"] == "copy_u":
+                    return ir.Node("spmm", {"g": node.inputs["g"], "x": msg.inputs["u"]},
+                                   size=node.size)
+                if msg.attrs["fn"] == "u_mul_e":
+                    return ir.Node("spmm", {"g": node.inputs["g"], "e": msg.inputs["e"],
+                                            "x": msg.inputs["u"]}, size=node.size)
+        return node
+
+    # -- spmm(sddmm) -> gat --------------------------------------------------
+    @staticmethod
+    def _fuse_gat(dataflow: ir.Dataflow) -> ir.Dataflow:
+        uses = ir.use_counts(dataflow)
+
+        def rule(node: ir.Node) -> ir.Node:
+            attn = node.inputs.get("e") if node.op == "spmm" else None
+            if attn is None or attn.op != "sddmm" or attn.inputs["g"] is not node.inputs["g"]:
+                return node
+            # the attention must have no other reader and one query block
+            if attn.attrs.get("uses", 0) != 1 or len(attn.inputs["q"].size) != 2:
+                return node
+            return ir.Node("gat", {"g": node.inputs["g"], "q": attn.inputs["q"],
+                                   "k": attn.inputs["k"], "x": node.inputs["x"]}, size=node.size)
+
+        # use counts refer to the nodes before rewriting: note them on the sddmm nodes
+        for node in ir.walk(dataflow):
+            if node.op == "sddmm":
+                node.attrs["uses"] = uses.get(id(node), 0)
+        return ir.rewrite(dataflow, rule)
+
+    # -- linear_q(h), linear_k(h) -> one launch ------------------------------
+    @staticmethod
+    def _bundle(dataflow: ir.Dataflow) -> ir.Dataflow:
+        bundles = {}
+
+        def rule(node: ir.Node) -> ir.Node:
+            if node.op not in ("sddmm", "gat"):
+                return node
+            q, k = node.inputs["q"], node.inputs["k"]
+            if q.op != "linear" or k.op != "linear" or q is k or q.inputs["x"] is not k.inputs["x"]:
+                return node
+            wq, wk = q.attrs["weight"], k.attrs["weight"]
+            if wq.shape != wk.shape or wq.stride() != wk.stride() or len(q.inputs["x"].size) != 2:
+                return node
+            key = (id(q), id(k))
+            if key not in bundles:
+                both = ir.Node("bundle", {"x": q.inputs["x"]},
+                               {"weights": (wq, wk), "biases": (q.attrs["bias"], k.attrs["bias"])})
+                bundles[key] = (ir.Node("select", {"x": both}, {"index": 0}, q.size),
+                                ir.Node("select", {"x": both}, {"index": 1}, k.size))
+            inputs = dict(node.inputs)
+            inputs["q"], inputs["k"] = bundles[key]
+            return node.with_inputs(inputs)
+
+        return ir.rewrite(dataflow, rule)
+
+    def lower(self, dataflow: ir.Dataflow, kwargs: dict = None) -> ir.Dataflow:
+        dataflow = ir.rewrite(dataflow, self._lower_node)
+        if self.fuse_gat:
+            dataflow = self._fuse_gat(dataflow)
+        if self.bundle_gemm:
+            dataflow = self._bundle(dataflow)
+        return dataflow
