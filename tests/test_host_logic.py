@@ -91,3 +91,15 @@ def test_input_info_auto_decider():
     assert info.set_input().dimWorker == 32 and info.set_hidden().dimWorker == 16
     with pytest.raises(ValueError):
         InputInfo(sharedMem=100)
+
+
+def test_auto_knobs_hand_computed():
+    """input_info.py:79-127 worked by hand. Average degree 50, 1000 input and 300 hidden
+    features, 8 KB budget: input estimate 8 * (200 + 4000 + 400) B = 36.8 KB -> capped at
+    8 KB -> int(8000 / 4200) = 1 row per workgroup; hidden estimate 8 * (200 + 300 + 400) B
+    = 7.2 KB (the hidden width enters unscaled) -> int(7200 / 1400) = 5."""
+    from yitu_amd.utils.input_info import auto_knobs, worth_reordering
+    k = auto_knobs(50.9, 1000, 300, 8.0)
+    assert tuple(k) == (50, 1, 5, 32, 32)
+    assert tuple(auto_knobs(11.3, 64, 16, 40.0)) == (11, 8, 8, 32, 16)
+    assert worth_reordering(3000.0, 10000) and not worth_reordering(0.5, 10000)

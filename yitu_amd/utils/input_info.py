@@ -1,10 +1,44 @@
-"""Parameter carrier consumed by the conv modules (YiTu_GNN/utils/input_info.py).
+"""The argument carrier that the conv modules read (the role of
+YiTu_GNN/utils/input_info.py): the CSR, the per-node scale, the neighbour
+partition and the three launch knobs of the reference's op signature, plus the
+rule that picks those knobs and decides on reordering in automatic mode.
 
-Holds the CSR, the per-node scale, the neighbour-group partition and the three
-tuning knobs of the reference signature. The knobs are kept because callers set
-and read them; the gfx950 kernels pick their own row split and ignore them.
+The gfx950 kernels choose their own row split, so the knobs do not steer them;
+they are kept, and computed exactly as before, because callers set them, read
+them back and pass them on.
 """
 import math
+from collections import namedtuple
+
+MAX_WARPS_PER_BLOCK = 8
+SHARED_MEMORY_SHARE = 0.4   # fraction of the device's shared memory the rule budgets
+SMEM_GAP_WORDS = 100
+
+AutoKnobs = namedtuple("AutoKnobs", "partSize warpPerBlock_input warpPerBlock_hidden "
+                                    "dimWorker_input dimWorker_hidden")
+
+
+def auto_knobs(avg_degree, input_dim, hidden_dim, shared_memory_kb) -> AutoKnobs:
+    """The automatic choice of input_info.py:79-127. Groups are as wide as the
+    average degree; a workgroup takes as many rows as fit the shared-memory budget
+    (KB), at most eight; one lane per feature up to 32. The hidden-layer estimate
+    adds ``hidden_dim`` bytes rather than words (input_info.py:93-97) and is kept so."""
+    part = int(avg_degree)
+
+    def warps(dim, estimate_bytes):
+        budget_kb = min(MAX_WARPS_PER_BLOCK * estimate_bytes / 1e3, shared_memory_kb)
+        return min(int(budget_kb * 1e3 / (4 * part + 4 * dim)), MAX_WARPS_PER_BLOCK)
+
+    gap = 4 * SMEM_GAP_WORDS
+    return AutoKnobs(part,
+                     warps(input_dim, 4 * part + 4 * input_dim + gap),
+                     warps(hidden_dim, 4 * part + hidden_dim + gap),
+                     min(input_dim, 32), min(hidden_dim, 32))
+
+
+def worth_reordering(avg_edge_span, num_nodes) -> bool:
+    """input_info.py:131-136: reorder when neighbours are far apart in id space."""
+    return math.sqrt(avg_edge_span) > math.sqrt(num_nodes) / 100
 
 
 class InputInfo(object):
@@ -13,87 +47,70 @@ class InputInfo(object):
                  dataset_obj=None, enable_rabbit=False, manual_mode=True, verbose=False):
         if dataset_obj is None:
             raise ValueError("Dataset object MUST SET !!!")
-        self.dataset_obj = dataset_obj
-        self.row_pointers = row_pointers
-        self.column_index = column_index
-        self.degrees = degrees
-        self.num_nodes = dataset_obj.num_nodes
-        self.avgNodeDegree = dataset_obj.avg_degree
-        self.avgEdgeSpan = dataset_obj.avg_edgeSpan
+        ds = self.dataset_obj = dataset_obj
+        # graph
+        self.row_pointers, self.column_index, self.degrees = row_pointers, column_index, degrees
+        self.partPtr = self.part2Node = None
+        self.num_nodes, self.avgNodeDegree, self.avgEdgeSpan = \
+            ds.num_nodes, ds.avg_degree, ds.avg_edgeSpan
+        self.inputDim, self.hiddenDim = ds.num_features, hiddenDim
+        # knobs: the current pair, and the pairs for the input and the hidden layers
         self.partSize = partSize
-        self.dimWorker = dimWorker
-        self.warpPerBlock = warpPerBlock
-        self.dimWorker_input = dimWorker
-        self.dimWorker_hidden = dimWorker
-        self.warpPerBlock_input = warpPerBlock
-        self.warpPerBlock_hidden = warpPerBlock
-        self.inputDim = dataset_obj.num_features
-        self.hiddenDim = hiddenDim
-        self.manual_mode = manual_mode
-        self.enable_rabbit = enable_rabbit
-        self.verbose_flag = verbose
+        self.dimWorker = self.dimWorker_input = self.dimWorker_hidden = dimWorker
+        self.warpPerBlock = self.warpPerBlock_input = self.warpPerBlock_hidden = warpPerBlock
+        self.MAX_warpPerBlock = MAX_WARPS_PER_BLOCK
+        self.share_memory = sharedMem * SHARED_MEMORY_SHARE
+        self.gap_smem = SMEM_GAP_WORDS
+        # mode and state
+        self.manual_mode, self.enable_rabbit, self.verbose_flag = manual_mode, enable_rabbit, verbose
         self.state_set_input = False
         self.reorder_status = False
-        self.MAX_warpPerBlock = 8
-        self.share_memory = sharedMem * 0.4
-        self.gap_smem = 100
-        self.partPtr = None
-        self.part2Node = None
+
+    def _reorder(self, wanted: bool):
+        self.dataset_obj.reorder_flag = wanted
+        self.reorder_status = wanted
 
     def decider(self):
-        """Manual mode keeps the given knobs and reorders iff asked; auto mode
-        derives them from the average degree and feature widths and reorders iff
-        sqrt(avgEdgeSpan) > sqrt(N) / 100 (input_info.py:58-143)."""
+        """Manual mode (input_info.py:65-77): the given knobs stand; the graph is
+        reordered iff asked, and the carrier then takes the dataset's new CSR.
+        Automatic mode (:78-143): knobs from ``auto_knobs``; with reordering enabled
+        the dataset's ``rabbit_reorder`` is always called and acts iff
+        ``worth_reordering`` set its flag."""
         if self.manual_mode:
+            self._reorder(bool(self.enable_rabbit))
             if self.enable_rabbit:
-                self.dataset_obj.reorder_flag = True
                 self.dataset_obj.rabbit_reorder()
-                self.reorder_status = True
                 self.row_pointers = self.dataset_obj.row_pointers
                 self.column_index = self.dataset_obj.column_index
-            else:
-                self.dataset_obj.reorder_flag = False
-                self.reorder_status = False
             return
-        self.partSize = int(self.avgNodeDegree)
-        est = self.MAX_warpPerBlock * (self.partSize * 4 + self.inputDim * 4 + self.gap_smem * 4) / 1e3
-        share_memory_input = min(est, self.share_memory)
-        # the hidden-layer estimate really adds hiddenDim unscaled (input_info.py:93-97)
-        est = self.MAX_warpPerBlock * (self.partSize * 4 + self.hiddenDim + 4 * self.gap_smem) / 1e3
-        share_memory_hidden = min(est, self.share_memory)
-        self.warpPerBlock_input = min(
-            int(share_memory_input * 1e3 / (self.partSize * 4 + self.inputDim * 4)),
-            self.MAX_warpPerBlock)
-        self.warpPerBlock_hidden = min(
-            int(share_memory_hidden * 1e3 / (self.partSize * 4 + self.hiddenDim * 4)),
-            self.MAX_warpPerBlock)
-        self.dimWorker_input = 32 if self.inputDim > 32 else self.inputDim
-        self.dimWorker_hidden = 32 if self.hiddenDim > 32 else self.hiddenDim
+        (self.partSize, self.warpPerBlock_input, self.warpPerBlock_hidden, self.dimWorker_input,
+         self.dimWorker_hidden) = auto_knobs(self.avgNodeDegree, self.inputDim, self.hiddenDim,
+                                             self.share_memory)
         if self.enable_rabbit:
-            reorder = math.sqrt(self.avgEdgeSpan) > math.sqrt(self.num_nodes) / 100
-            self.dataset_obj.reorder_flag = reorder
-            self.reorder_status = reorder
+            self._reorder(worth_reordering(self.avgEdgeSpan, self.num_nodes))
             self.dataset_obj.rabbit_reorder()
 
-    def set_input(self):
-        self.dimWorker = self.dimWorker_input
-        self.warpPerBlock = self.warpPerBlock_input
-        self.state_set_input = True
+    def _select(self, for_input: bool):
+        suffix = "_input" if for_input else "_hidden"
+        self.dimWorker = getattr(self, "dimWorker" + suffix)
+        self.warpPerBlock = getattr(self, "warpPerBlock" + suffix)
+        self.state_set_input = for_input
         return self
 
+    def set_input(self):
+        """Knobs of the first layer (width = input features); returns self."""
+        return self._select(True)
+
     def set_hidden(self):
-        self.dimWorker = self.dimWorker_hidden
-        self.warpPerBlock = self.warpPerBlock_hidden
-        self.state_set_input = False
-        return self
+        """Knobs of the later layers (width = hidden features); returns self."""
+        return self._select(False)
 
     def print_param(self):
         if not self.verbose_flag:
             return
-        mode = "manual" if self.manual_mode else "auto"
-        layer = "INPUT" if self.state_set_input else "HIDDEN"
-        print("# {} {} partSize: {}".format(mode, layer, self.partSize))
-        print("# {} {} dimWorker: {}".format(mode, layer, self.dimWorker))
-        print("# {} {} warpPerBlock: {}".format(mode, layer, self.warpPerBlock))
+        where = "%s %s" % ("manual" if self.manual_mode else "auto",
+                           "INPUT" if self.state_set_input else "HIDDEN")
+        for knob in ("partSize", "dimWorker", "warpPerBlock"):
+            print("# %s %s: %s" % (where, knob, getattr(self, knob)))
         if not self.manual_mode:
-            print("# {} {} reorder_flag: {}".format(mode, layer, self.reorder_status))
+            print("# %s reorder_flag: %s" % (where, self.reorder_status))

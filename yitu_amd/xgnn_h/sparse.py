@@ -1,99 +1,101 @@
-"""Autograd glue over the graph_ext ops (xgnn_h/sparse.py), unchanged in
-behaviour: same Function classes, saved tensors, asserts and gradients."""
+"""Differentiable sparse ops over a ``Block`` (the role of xgnn_h/sparse.py): the
+same Function classes and wrappers, each a thin autograd shell around one pair of
+``graph_ext`` calls. The sparse structure never takes a gradient; a gradient that
+the caller does not need is not computed."""
 import torch
 from torch import autograd
+from torch.autograd.function import once_differentiable
 
 from .. import graph_ext
 from . import block
 
 
+def _structure_is_constant(ctx):
+    # the [indptr, indices] pair is passed through autograd as a plain list
+    assert ctx.needs_input_grad[0] is False
+
+
 class GSPMMFunction(autograd.Function):
-    """sparse.py:7-35"""
+    """out[r,h,:] = sum_e values[e,h] x[col_e,h,:] (sparse.py:7-35)."""
 
     @staticmethod
     def forward(ctx, adj_sparse, adj_values, x):
-        indptr, indices = adj_sparse[0], adj_sparse[1]
-        y = graph_ext.spmm_forward(adj_values, indptr, indices, x)
         ctx.adj_sparse = adj_sparse
         ctx.save_for_backward(adj_values, x)
-        return y
+        return graph_ext.spmm_forward(adj_values, adj_sparse[0], adj_sparse[1], x)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_out):
-        indptr, indices = ctx.adj_sparse[0], ctx.adj_sparse[1]
-        values, x = ctx.saved_tensors
-        grad_out = grad_out.contiguous()
+        _structure_is_constant(ctx)
         assert len(ctx.needs_input_grad) == 3
-        assert ctx.needs_input_grad[0] is False
-        # a gradient nobody asked for (constant edge weights) is not computed
-        grad_a, grad_x = graph_ext.spmm_backward(values, indptr, indices, x, grad_out,
-                                                 need_grad_a=ctx.needs_input_grad[1],
-                                                 need_grad_x=ctx.needs_input_grad[2])
-        return None, grad_a, grad_x
+        values, x = ctx.saved_tensors
+        grad_values, grad_x = graph_ext.spmm_backward(
+            values, ctx.adj_sparse[0], ctx.adj_sparse[1], x, grad_out.contiguous(),
+            need_grad_a=ctx.needs_input_grad[1], need_grad_x=ctx.needs_input_grad[2])
+        return None, grad_values, grad_x
 
 
 def gspmm(block: block.Block, edge: torch.Tensor, x: torch.Tensor):
-    """sparse.py:38-51: ``edge=None`` aggregates with unit weights."""
+    """Edge-weighted aggregation of ``x [n_src, H, F]``; ``edge=None`` means unit
+    weights (sparse.py:38-51)."""
     assert x.dim() == 3
-    indices = block.adj_sparse[1]
     if edge is None:
-        edge = torch.ones(size=[indices.size(0), x.size(1)], device=x.device)
+        n_edges = block.adj_sparse[1].size(0)
+        edge = torch.ones(size=[n_edges, x.size(1)], device=x.device)
     return GSPMMFunction.apply(block.adj_sparse, edge, x)
 
 
 class GSDDMMFunction(autograd.Function):
-    """sparse.py:54-81"""
+    """attn = softmax_row(LeakyReLU(query[bid,row] + key[col])) (sparse.py:54-81)."""
 
     @staticmethod
     def forward(ctx, adj_sparse, query, key):
-        indptr, indices = adj_sparse
-        attn_values = graph_ext.sddmm_forward(indptr, indices, query, key)
         ctx.adj_sparse = adj_sparse
-        ctx.save_for_backward(query, key, attn_values)
-        return attn_values
+        attn = graph_ext.sddmm_forward(adj_sparse[0], adj_sparse[1], query, key)
+        ctx.save_for_backward(query, key, attn)
+        return attn
 
     @staticmethod
-    def backward(ctx, grad_out):
-        grad_out = grad_out.contiguous()
-        indptr, indices = ctx.adj_sparse
-        query, key, attn_values = ctx.saved_tensors
-        assert len(ctx.needs_input_grad) == 3
-        assert ctx.needs_input_grad[0] is False
-        assert ctx.needs_input_grad[1] is True
-        assert ctx.needs_input_grad[2] is True
-        grad_query, grad_key = graph_ext.sddmm_backward(indptr, indices, query, key, attn_values,
-                                                        grad_out)
+    @once_differentiable
+    def backward(ctx, grad_attn):
+        _structure_is_constant(ctx)
+        # like the reference, both projections are expected to train
+        assert ctx.needs_input_grad[1:] == (True, True)
+        query, key, attn = ctx.saved_tensors
+        grad_query, grad_key = graph_ext.sddmm_backward(
+            ctx.adj_sparse[0], ctx.adj_sparse[1], query, key, attn, grad_attn.contiguous())
         return None, grad_query, grad_key
 
 
 def fused_gsddmm(block: block.Block, query: torch.Tensor, key: torch.Tensor):
-    """sparse.py:84-91"""
-    if query.dim() == 2:
-        query = query.unsqueeze(0)
+    """``query`` [n_dst, H] or, for a stitched block, [n_blocks, n_dst, H]
+    (sparse.py:84-91)."""
+    query = query if query.dim() == 3 else query.unsqueeze(0)
     return GSDDMMFunction.apply(block.adj_sparse, query, key)
 
 
 class HFUSEDFunction(autograd.Function):
-    """sparse.py:94-110, with the backward the reference leaves unimplemented."""
+    """An SpMM on one block and an SDDMM on another, issued together
+    (sparse.py:94-110), with the backward the reference leaves unimplemented."""
 
     @staticmethod
     def forward(ctx, spmm_sparse, spmm_values, spmm_x, sddmm_sparse, sddmm_query, sddmm_key):
-        spmm_out, attn_values = graph_ext.hfused_forward(
-            spmm_values, spmm_sparse[0], spmm_sparse[1], spmm_x,
-            sddmm_sparse[0], sddmm_sparse[1], sddmm_query, sddmm_key)
-        ctx.spmm_sparse = spmm_sparse
-        ctx.sddmm_sparse = sddmm_sparse
-        ctx.save_for_backward(spmm_values, spmm_x, sddmm_query, sddmm_key, attn_values)
-        return spmm_out, attn_values
+        ctx.structures = (spmm_sparse, sddmm_sparse)
+        out, attn = graph_ext.hfused_forward(spmm_values, *spmm_sparse, spmm_x, *sddmm_sparse,
+                                             sddmm_query, sddmm_key)
+        ctx.save_for_backward(spmm_values, spmm_x, sddmm_query, sddmm_key, attn)
+        return out, attn
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_spmm, grad_attn):
-        spmm_values, spmm_x, sddmm_query, sddmm_key, attn_values = ctx.saved_tensors
-        grad_a, grad_x, grad_q, grad_k = graph_ext.hfused_backward(
-            spmm_values, ctx.spmm_sparse[0], ctx.spmm_sparse[1], spmm_x, grad_spmm.contiguous(),
-            ctx.sddmm_sparse[0], ctx.sddmm_sparse[1], sddmm_query, sddmm_key, attn_values,
-            grad_attn.contiguous())
-        return None, grad_a, grad_x, None, grad_q, grad_k
+        (a_ptr, a_idx), (b_ptr, b_idx) = ctx.structures
+        values, x, query, key, attn = ctx.saved_tensors
+        grad_values, grad_x, grad_query, grad_key = graph_ext.hfused_backward(
+            values, a_ptr, a_idx, x, grad_spmm.contiguous(),
+            b_ptr, b_idx, query, key, attn, grad_attn.contiguous())
+        return None, grad_values, grad_x, None, grad_query, grad_key
 
 
 def hfused_spddmm(spmm_block: block.Block, spmm_values, spmm_x, sddmm_block: block.Block,
@@ -151,7 +153,8 @@ class EdgeDotFunction(autograd.Function):
         grad_dst = graph_ext.spmm_forward(grad_e, indptr, indices, src_feat)
         # grad_src[c] = sum_{i: col_i = c} grad_e[i] * dst[row_i]: spmm_backward's grad_x
         # with dst_feat in the role of grad_out
-        _, grad_src = graph_ext.spmm_backward(grad_e, indptr, indices, src_feat, dst_feat)
+        _, grad_src = graph_ext.spmm_backward(grad_e, indptr, indices, src_feat, dst_feat,
+                                              need_grad_a=False)
         return None, grad_dst, grad_src
 
 
