@@ -206,7 +206,7 @@ def run_gat(args, dev):
         es[0].record()
         out, attn = graph_ext.gat_forward(rp, ci, q, k, x)
         es[1].record()
-        graph_ext.gat_backward(rp, ci, q, k, x, attn, gy)
+        graph_ext.gat_backward(rp, ci, q, k, x, attn, gy, out=out)
         es[2].record()
         if timed:
             ev["fwd"].append((es[0], es[1]))

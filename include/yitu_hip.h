@@ -194,14 +194,19 @@ int yitu_gat_forward(float *out_device, float *attn_device, const int32_t *indpt
  * xgnn_h/sparse.py:22-35,67-81) in one call, given grad_out [n_dst,H,F]:
  * grad_query [n_dst,H], grad_key [n_src,H], grad_features [n_src,H,F], all
  * fully written, no atomics. The two scratch buffers are [nnz,H] floats.
+ * out_device: the forward's output [n_dst,H,F], or NULL. With it (and rows of
+ * 256 floats) the softmax row sums come from <grad_out[row], out[row]> and one
+ * pass over the by-source edges finishes every gradient; the workspace must
+ * then be given whatever the degrees (yitu_gat_workspace_bytes).
  */
 int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       float *grad_features_device, float *grad_attn_scratch_device,
                       float *grad_edge_scratch_device, const int32_t *indptr_device,
                       const int32_t *indices_device, const float *query_device,
                       const float *key_device, const float *features_device,
-                      const float *attn_device, const float *grad_out_device,
-                      const int32_t *t_indptr_device, const int32_t *t_rows_device,
+                      const float *attn_device, const float *out_device,
+                      const float *grad_out_device, const int32_t *t_indptr_device,
+                      const int32_t *t_rows_device,
                       const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
                       int64_t n_heads, int64_t n_features, int64_t max_degree,
                       int64_t max_degree_t, const void *plan_device, const void *plan_t_device,

@@ -113,3 +113,11 @@ def test_c2_backward_is_the_adjoint_of_forward(dev, c2):
     assert abs(num - ana) < 5e-5 * scale, (num, ana, scale)
     again = graph_ext.gat_backward(rp, ci, q, k, x, attn, gy)
     assert all(torch.equal(a, b) for a, b in zip((gq, gk, gx), again))
+    # with the forward output: the one-pass backward; same gradients, reproducible
+    full = graph_ext.gat_backward(rp, ci, q, k, x, attn, gy, out=out)
+    assert torch.equal(full[2], gx)
+    for got, want in zip(full[:2], (gq, gk)):
+        scale_g = float(want.abs().max())
+        assert float((got - want).abs().max()) < 1e-4 * max(scale_g, 1.0)
+    again = graph_ext.gat_backward(rp, ci, q, k, x, attn, gy, out=out)
+    assert all(torch.equal(a, b) for a, b in zip(full, again))

@@ -676,18 +676,75 @@ struct GatSrcParams {
     SpmmParams sp;   // indptr / indices / eperm = by-source structure, values = attn,
                      // feat = grad_out, out = grad_x, plan = its row plan, partial
     const float *x;  // [n_src, L]
-    float *grad_a;   // [nnz, H], CSR order
+    float *grad_a;   // [nnz, H], CSR order: d_attn (FULL = false) or the logit gradient (FULL)
+    // FULL: the forward output is at hand, so the softmax row sum S[r,h] = sum_e a d_attn
+    // = <grad_out[r,h,:], out[r,h,:]> is known before the pass and the whole
+    // softmax + LeakyReLU backward happens per edge, here
+    const float2 *row_sq;  // [n_dst, H]: (S, query) side by side, one line per destination
+    const float *key;      // [n_src, H]
+    float *grad_k;         // [n_src, H]
+    float *partial_k;      // [plan item id, H] partial grad_k of multi-item sources
 };
 
+// (S[r,h], query[r,h]) with S[r,h] = <grad_out[r,h,:], out[r,h,:]>, 256-float rows,
+// kRowsPerWave rows per wave. The pair is what an edge needs from its destination.
 template <int LPH>
+__global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict__ row_sq,
+                                                             const float *__restrict__ grad_out,
+                                                             const float *__restrict__ out,
+                                                             const float *__restrict__ query,
+                                                             int n_rows) {
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    constexpr int H = kWave / LPH;
+    for (int i0 = 0; i0 < kRowsPerWave && r0 + i0 < n_rows; i0 += 4) {
+        float d[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int r = min(r0 + i0 + u, n_rows - 1);
+            float a[4], b[4];
+            RowLoad<4, float>::ld(grad_out + (size_t)r * 256 + lane * 4, a);
+            RowLoad<4, float>::ld(out + (size_t)r * 256 + lane * 4, b);
+            d[u] = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int o = LPH >> 1; o >= 1; o >>= 1) d[u] += __shfl_xor(d[u], o, kWave);
+            const int r = r0 + i0 + u;
+            if (lane % LPH == 0 && r < n_rows)
+                row_sq[(size_t)r * H + lane / LPH] =
+                    make_float2(d[u], query[(size_t)r * H + lane / LPH]);
+        }
+    }
+}
+
+// FULL: kc = key[c, h] of the source; gk accumulates this lane's share of grad_key[c, h].
+template <int LPH, bool FULL>
 __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const EdgeWindow &win,
                                                int first, int n, const float (&xt)[4],
-                                               float (&acc)[4]) {
+                                               float (&acc)[4], float kc, float &gk) {
     constexpr int NS = kWave / LPH;
     const int lane = lane_id();
     const int h = lane / LPH, sub = lane % LPH;
     const int L = p.sp.L, H = p.sp.H;
     const float *__restrict__ g = static_cast<const float *>(p.sp.feat);
+    // What is needed per (edge, head) is fetched once, before the row gathers, in the
+    // layout of the epilogue: lane (h, sub) owns edge j * LPH + sub. The attention
+    // weight reaches the accumulate loop by a lane shuffle.
+    float ea[NS], eS[NS], eq[NS];
+#pragma unroll
+    for (int j = 0; j < NS; j++) {
+        const int k = min(j * LPH + sub, n - 1);
+        const int vr = __shfl(win.vrow, first + k, kWave);
+        ea[j] = p.sp.values[(size_t)vr * H + h];
+        if constexpr (FULL) {
+            const int r = __shfl(win.col, first + k, kWave);
+            const float2 sq = p.row_sq[(size_t)r * H + h];
+            eS[j] = sq.x;
+            eq[j] = sq.y;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NS; j++) {
         if (j * LPH >= n) break;  // wave-uniform
@@ -699,9 +756,8 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
                 const int k = j * LPH + kk + u;
                 if (k < n) {  // wave-uniform
                     const int r = __builtin_amdgcn_readlane(win.col, first + k);
-                    const int vr = __builtin_amdgcn_readlane(win.vrow, first + k);
                     RowLoad<4, float>::ld(g + (size_t)r * L + lane * 4, v[u]);
-                    a[u] = p.sp.values[(size_t)vr * H + h];
+                    a[u] = __shfl(ea[j], (lane - sub) + kk + u, kWave);
                 }
             }
 #pragma unroll
@@ -719,13 +775,30 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
         }
         const int k = j * LPH + sub;
         const int vr = __shfl(win.vrow, first + min(k, n - 1), kWave);
-        if (k < n) p.grad_a[(size_t)vr * H + h] = keep;
+        if constexpr (FULL) {
+            if (k < n) {
+                const float gl = ea[j] * (keep - eS[j]) * (eq[j] + kc < 0.0f ? kSlope : 1.0f);
+                p.grad_a[(size_t)vr * H + h] = gl;
+                gk += gl;
+            }
+        } else {
+            if (k < n) p.grad_a[(size_t)vr * H + h] = keep;
+        }
     }
 }
 
+// sum of gk over the lanes of a head (all lanes of the head get it)
 template <int LPH>
+__device__ __forceinline__ float head_sum(float gk) {
+#pragma unroll
+    for (int o = LPH >> 1; o >= 1; o >>= 1) gk += __shfl_xor(gk, o, kWave);
+    return gk;
+}
+
+template <int LPH, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
     const int lane = lane_id();
+    const int h = lane / LPH;
     const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
@@ -742,20 +815,29 @@ __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
         const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
         if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
         float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (end > beg) RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
+        float kc = 0.0f, gk = 0.0f;
+        if (end > beg) {
+            RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
+            if constexpr (FULL) kc = p.key[(size_t)row * p.sp.H + h];
+        }
         for (int b = beg; b < end; b += kWave) {
             const int n = min(kWave, end - b);
             if (win.base < 0 || b < win.base || b + n > win.base + kWave)
                 load_window<W_EDGEHEAD>(win, p.sp, b, limit);
-            gat_src_window<LPH>(p, win, b - win.base, n, xt, acc);
+            gat_src_window<LPH, FULL>(p, win, b - win.base, n, xt, acc, kc, gk);
         }
         store_row<4>(p.sp.out + (size_t)row * L + lane * 4, acc);
+        if constexpr (FULL) {
+            gk = head_sum<LPH>(gk);
+            if (lane % LPH == 0) p.grad_k[(size_t)row * p.sp.H + h] = gk;
+        }
     }
 }
 
-template <int LPH>
+template <int LPH, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
     const int lane = lane_id();
+    const int h = lane / LPH;
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
@@ -780,37 +862,67 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
             if (n_edges[j] <= 0) continue;
             const int row = tag[j] & 0x7fffffff;
             float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float kc = 0.0f, gk = 0.0f;
             RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
-            gat_src_window<LPH>(p, win[j], 0, n_edges[j], xt, acc);
-            float *dst = tag[j] < 0 ? p.sp.out + (size_t)row * L : p.sp.partial + (size_t)item[j] * L;
+            if constexpr (FULL) kc = p.key[(size_t)row * p.sp.H + h];
+            gat_src_window<LPH, FULL>(p, win[j], 0, n_edges[j], xt, acc, kc, gk);
+            const bool single = tag[j] < 0;
+            float *dst = single ? p.sp.out + (size_t)row * L : p.sp.partial + (size_t)item[j] * L;
             store_row<4>(dst + lane * 4, acc);
+            if constexpr (FULL) {
+                gk = head_sum<LPH>(gk);
+                float *dk = single ? p.grad_k + (size_t)row * p.sp.H
+                                   : p.partial_k + (size_t)item[j] * p.sp.H;
+                if (lane % LPH == 0) dk[h] = gk;
+            }
         }
     }
 }
 
-template <int LPH>
-static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, hipStream_t stream) {
-    gat_src_rows_kernel<LPH>
+template <int LPH, bool FULL>
+static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, const float *grad_out,
+                              const float *out, const float *query, int n_dst,
+                              hipStream_t stream) {
+    if constexpr (FULL) {
+        gat_row_dot_kernel<LPH>
+            <<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(
+                const_cast<float2 *>(p.row_sq), grad_out, out, query, n_dst);
+        YITU_LAUNCH_CHECK();
+    }
+    gat_src_rows_kernel<LPH, FULL>
         <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
-    gat_src_items_kernel<LPH><<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
-                                                                kWavesPerBlock * kItemsPerWave),
-                                                       1 << 16),
-                                kBlock, 0, stream>>>(p);
+    gat_src_items_kernel<LPH, FULL>
+        <<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave),
+                                  1 << 16),
+           kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    spmm_reduce_kernel<W_NONE, 4>
-        <<<(int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16), kBlock, 0, stream>>>(p.sp);
+    const int red_grid = (int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16);
+    spmm_reduce_kernel<W_NONE, 4><<<red_grid, kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
+    if constexpr (FULL) {
+        // the item partials of grad_key, rows of H = 64 / LPH floats
+        constexpr int H = kWave / LPH;
+        SpmmParams k = p.sp;
+        k.L = k.F = H;
+        k.H = 1;
+        k.out = p.grad_k;
+        k.partial = p.partial_k;
+        spmm_reduce_kernel<W_NONE, (H >= 4 ? 4 : H)><<<red_grid, kBlock, 0, stream>>>(k);
+        YITU_LAUNCH_CHECK();
+    }
     return 0;
 }
 
-static int gat_src_launch(const GatSrcParams &p, bool has_items, hipStream_t stream) {
+template <bool FULL>
+static int gat_src_launch(const GatSrcParams &p, bool has_items, const float *grad_out,
+                          const float *out, const float *query, int n_dst, hipStream_t stream) {
     switch (p.sp.F / 4) {
-        case 8: return gat_src_launch_lph<8>(p, has_items, stream);
-        case 16: return gat_src_launch_lph<16>(p, has_items, stream);
-        case 32: return gat_src_launch_lph<32>(p, has_items, stream);
-        case 64: return gat_src_launch_lph<64>(p, has_items, stream);
+        case 8: return gat_src_launch_lph<8, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
+        case 16: return gat_src_launch_lph<16, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
+        case 32: return gat_src_launch_lph<32, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
+        case 64: return gat_src_launch_lph<64, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
     }
     set_error("gat backward: unsupported head width %d", p.sp.F);
     return -1;
@@ -1042,7 +1154,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                                float *grad_attn_scratch, float *grad_edge_scratch,
                                const int32_t *indptr, const int32_t *indices, const float *query,
                                const float *key, const float *features, const float *attn,
-                               const float *grad_out, const int32_t *t_indptr,
+                               const float *out, const float *grad_out, const int32_t *t_indptr,
                                const int32_t *t_rows, const int32_t *t_perm, int64_t n_dst,
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
                                int64_t max_degree, int64_t max_degree_t, const void *plan,
@@ -1086,19 +1198,49 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                               0x7fffffff, max_degree_t, workspace, workspace_bytes, &rest,
                               &rest_bytes, stream);
         if (rc) return rc;
-        if (has_items) {
-            const size_t need = sizeof(float) * (size_t)p.sp.plan.max_items * (size_t)L;
-            YITU_REQUIRE(rest && rest_bytes >= need, "workspace too small: need %zu more bytes",
-                         need);
-            p.sp.partial = static_cast<float *>(rest);
+        const bool full = out != nullptr && aligned16(out);
+        const size_t part = has_items ? align_up(sizeof(float) * (size_t)p.sp.plan.max_items *
+                                                     (size_t)L, 256) : 0;
+        const size_t part_k = has_items && full
+                                  ? align_up(sizeof(float) * (size_t)p.sp.plan.max_items *
+                                                 (size_t)n_heads, 256) : 0;
+        const size_t dots = full ? sizeof(float2) * (size_t)(n_dst * n_heads) : 0;
+        YITU_REQUIRE((part + part_k + dots == 0) || (rest && rest_bytes >= part + part_k + dots),
+                     "workspace too small: need %zu more bytes", part + part_k + dots);
+        char *w = static_cast<char *>(rest);
+        if (has_items) p.sp.partial = reinterpret_cast<float *>(w);
+        if (!full) {
+            rc = gat_src_launch<false>(p, has_items, grad_out, nullptr, nullptr, (int)n_dst, stream);
+            if (rc) return rc;
+            // softmax + LeakyReLU backward from d_attn; grad_key over the transposed structure
+            return sddmm_backward_run(grad_query, grad_key, grad_edge_scratch, indptr, indices,
+                                      query, key, attn, grad_attn_scratch, t_indptr, t_perm, n_dst,
+                                      n_src, nnz, n_heads, 1, max_degree, max_degree_t, plan,
+                                      plan_t, workspace, workspace_bytes, 0, stream);
         }
-        rc = gat_src_launch(p, has_items, stream);
+        // With the forward output the softmax row sums are known up front and the pass
+        // also finishes the per-edge logit gradient (left in grad_attn_scratch, CSR
+        // order) and grad_key; grad_query is its sum over each destination row.
+        p.partial_k = reinterpret_cast<float *>(w + part);
+        p.row_sq = reinterpret_cast<float2 *>(w + part + part_k);
+        p.key = key;
+        p.grad_k = grad_key;
+        rc = gat_src_launch<true>(p, has_items, grad_out, out, query, (int)n_dst, stream);
         if (rc) return rc;
-        // softmax + LeakyReLU backward from d_attn; grad_key over the transposed structure
-        return sddmm_backward_run(grad_query, grad_key, grad_edge_scratch, indptr, indices, query,
-                                  key, attn, grad_attn_scratch, t_indptr, t_perm, n_dst, n_src, nnz,
-                                  n_heads, 1, max_degree, max_degree_t, plan, plan_t, workspace,
-                                  workspace_bytes, 0, stream);
+        SpmmParams q{};
+        q.indptr = indptr;
+        q.indices = indices;
+        q.cols_are_edges = 1;
+        q.feat = grad_attn_scratch;
+        q.out = grad_query;
+        q.n_rows = (int)n_dst;
+        q.n_src = (int)n_src;
+        q.L = q.F = (int)n_heads;
+        q.H = 1;
+        q.col_mask = kColMask;
+        q.alpha = 1.0f;
+        return launch_spmm(q, W_NONE, false, nnz, max_degree, plan, workspace, workspace_bytes,
+                           stream);
     }
     // d attn = <grad_out[row], x[col]> per edge and head; grad_x = attn-weighted
     // gather of grad_out over the transposed structure

@@ -78,6 +78,14 @@ static int launch_tiny(const SpmmParams &p, bool has_items, hipStream_t stream) 
     tiny_rows_kernel<VEC>
         <<<(int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
+    if (has_items && p.cols_are_edges) {
+        // a row's edges are contiguous: sum them in place, no items
+        edge_sum_long_kernel<VEC>
+            <<<(int)std::min<int64_t>(std::max<int64_t>(p.plan.max_rows, 2), 1 << 14), kBlock, 0,
+               stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        return 0;
+    }
     if (has_items) {
         const int item_grid = (int)std::min<int64_t>(
             ceil_div(p.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);

@@ -43,6 +43,7 @@ struct SpmmParams {
     int F;         // floats per head
     int H;
     int col_mask;
+    int cols_are_edges;  // nonzero: edge e reads feat row e (a segmented sum of per-edge rows)
     float alpha;   // output scale
     PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
     float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
@@ -67,7 +68,7 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
                                             int limit) {
     const int e = min(base + lane_id(), limit - 1);
     win.base = base;
-    win.col = p.indices[e] & p.col_mask;
+    win.col = p.cols_are_edges ? e : (p.indices[e] & p.col_mask);
     win.w = 1.0f;
     win.vrow = 0;
     if constexpr (WMODE == W_DEGPROD) win.w = p.scale_col[win.col];
@@ -439,7 +440,7 @@ template <int VEC>
 __device__ __forceinline__ void load_tiny_window(TinyWindow<VEC> &w, const SpmmParams &p, int base,
                                                  int limit) {
     const int e = min(base + lane_id(), limit - 1);
-    const int c = p.indices[e] & p.col_mask;
+    const int c = p.cols_are_edges ? e : (p.indices[e] & p.col_mask);
     w.base = base;
     RowLoad<VEC, float>::ld(static_cast<const float *>(p.feat) + (size_t)c * VEC, w.v);
 }
@@ -529,6 +530,76 @@ __global__ __launch_bounds__(kBlock) void tiny_items_kernel(SpmmParams p) {
                 store_row<VEC>(single ? p.out + (size_t)(tag[j] & 0x7fffffff) * VEC
                                       : p.partial + (size_t)item[j] * VEC,
                                acc);
+            }
+        }
+    }
+}
+
+// Planned rows of a segmented sum of per-edge rows (cols_are_edges): the edges of a
+// row are contiguous, so no items are needed. Rows of up to kEdgeSumWave edges: one
+// wave per row, lanes stride the edges, four loads in flight, one butterfly at the
+// end. Longer rows: one workgroup per row, thread sums added in thread order.
+// Blocks [0, gridDim.x / 2) take the first kind. Bitwise reproducible.
+constexpr int kEdgeSumWave = 4096;
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void edge_sum_long_kernel(SpmmParams p) {
+    __shared__ float red[kBlock * VEC];
+    if (p.plan.counters->overflow) return;
+    const int n_long = min(p.plan.counters->n_rows, p.plan.max_rows);
+    const float *__restrict__ feat = static_cast<const float *>(p.feat);
+    const int half = gridDim.x / 2;
+    if ((int)blockIdx.x < half) {
+        const int lane = lane_id();
+        const int stride = half * kWavesPerBlock;
+        for (int i = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; i < n_long; i += stride) {
+            const int row = p.plan.rows[i].x;
+            const int beg = p.indptr[row], n = p.indptr[row + 1] - beg;
+            if (n > kEdgeSumWave) continue;
+            float s[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) s[k] = 0.0f;
+            sum_partials<VEC>(s, feat + (size_t)beg * VEC, VEC, lane, n, kWave);
+#pragma unroll
+            for (int o = kWave / 2; o >= 1; o >>= 1)
+#pragma unroll
+                for (int k = 0; k < VEC; k++) s[k] += __shfl_xor(s[k], o, kWave);
+            if (lane == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) s[k] *= p.alpha;
+                store_row<VEC>(p.out + (size_t)row * VEC, s);
+            }
+        }
+        return;
+    }
+    for (int i = blockIdx.x - half; i < n_long; i += gridDim.x - half) {
+        const int row = p.plan.rows[i].x;
+        const int beg = p.indptr[row], n = p.indptr[row + 1] - beg;
+        if (n <= kEdgeSumWave) continue;
+        float s[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) s[k] = 0.0f;
+        sum_partials<VEC>(s, feat + (size_t)beg * VEC, VEC, threadIdx.x, n, kBlock);
+        __syncthreads();  // red[] may still be read for the previous row
+#pragma unroll
+        for (int k = 0; k < VEC; k++) red[threadIdx.x * VEC + k] = s[k];
+        __syncthreads();
+        if (threadIdx.x < kWave) {
+            // 64 lanes add four thread sums each in thread order, then a fixed butterfly
+            float t[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) t[k] = 0.0f;
+            for (int q = 0; q < kBlock / kWave; q++)
+#pragma unroll
+                for (int k = 0; k < VEC; k++) t[k] += red[(threadIdx.x * (kBlock / kWave) + q) * VEC + k];
+#pragma unroll
+            for (int o = kWave / 2; o >= 1; o >>= 1)
+#pragma unroll
+                for (int k = 0; k < VEC; k++) t[k] += __shfl_xor(t[k], o, kWave);
+            if (threadIdx.x == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) t[k] *= p.alpha;
+                store_row<VEC>(p.out + (size_t)row * VEC, t);
             }
         }
     }

@@ -403,11 +403,19 @@ def gat_forward(indptr, indices, query, key, features):
     return [out, attn]
 
 
-def gat_backward(indptr, indices, query, key, features, attn, grad_out):
-    """Returns [grad_query, grad_key, grad_features] of gat_forward's ``out``."""
+def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None):
+    """Returns [grad_query, grad_key, grad_features] of gat_forward's ``out``.
+    Passing the forward output ``out`` [n_dst, H, F] lets the softmax backward use
+    sum_e a d_attn = <grad_out[row], out[row]> and finish in the same pass over
+    the edges that computes grad_features (256-float rows); without it the
+    attention gradient takes passes of its own."""
     _check(grad_out, torch.float32, "grad_out", 3)
     _check(attn, torch.float32, "attn", 2)
     dev = _lib.require_device(indptr, indices, query, key, features, attn, grad_out)
+    if out is not None:
+        _check(out, torch.float32, "out", 3)
+        if out.shape != grad_out.shape:
+            raise RuntimeError("out and grad_out must have the same shape")
     n_dst = indptr.numel() - 1
     n_src, h, f = features.shape
     nnz = indices.numel()
@@ -420,14 +428,15 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out):
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = 0
-    if max(maxdeg, tr.max_degree_t) >= 64:
+    if max(maxdeg, tr.max_degree_t) >= 64 or out is not None:
         need = _size_fn("yitu_gat_workspace_bytes")(c_i64(max(n_dst, n_src)), c_i64(nnz), c_i64(h),
                                                     c_i64(f), c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_gat_backward(
             ptr(grad_q), ptr(grad_k), ptr(grad_x), ptr(s1), ptr(s2), ptr(indptr), ptr(indices),
-            ptr(query), ptr(key), ptr(features), ptr(attn), ptr(grad_out), ptr(tr.t_indptr),
+            ptr(query), ptr(key), ptr(features), ptr(attn), ptr(out), ptr(grad_out),
+            ptr(tr.t_indptr),
             ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
             c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan), ptr(tr.plan_t), ptr(ws),
             c_size(ws.numel()), stream_ptr(dev))

@@ -116,15 +116,15 @@ class FusedGATFunction(autograd.Function):
         indptr, indices = adj_sparse
         out, attn = graph_ext.gat_forward(indptr, indices, query, key, x)
         ctx.adj_sparse = adj_sparse
-        ctx.save_for_backward(query, key, x, attn)
+        ctx.save_for_backward(query, key, x, attn, out)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         indptr, indices = ctx.adj_sparse
-        query, key, x, attn = ctx.saved_tensors
+        query, key, x, attn, out = ctx.saved_tensors
         grad_q, grad_k, grad_x = graph_ext.gat_backward(indptr, indices, query, key, x, attn,
-                                                        grad_out.contiguous())
+                                                        grad_out.contiguous(), out=out)
         return None, grad_q, grad_k, grad_x
 
 
