@@ -103,6 +103,19 @@ int yitu_spmm_forward(float *out_device, const float *values_device, const int32
                       size_t workspace_bytes, void *stream);
 
 /*
+ * The same product with bf16 feature rows (fp32 edge values, fp32 accumulate,
+ * fp32 out): the reference's op is fp32 only (spmm_cuda.cu:44-62); this is the
+ * aggregation step of a bf16 pipeline whose dense transforms write bf16 rows
+ * (yitu_gemm_bf16).
+ */
+int yitu_spmm_forward_bf16(float *out_device, const float *values_device,
+                           const int32_t *indptr_device, const int32_t *indices_device,
+                           const void *features_bf16_device, int64_t n_dst, int64_t n_src,
+                           int64_t nnz, int64_t n_heads, int64_t n_features, int64_t max_degree,
+                           const void *plan_device, void *workspace_device, size_t workspace_bytes,
+                           void *stream);
+
+/*
  * spmm_backward (entry.cpp:92-104; spmm_cuda.cu:24-42,64-86):
  *   grad_a[i,h]   = sum_k grad_out[row_i,h,k] * features[col_i,h,k]
  *   grad_x[c,h,k] = sum_{i: col_i = c} grad_out[row_i,h,k] * values[i,h]

@@ -83,6 +83,25 @@ def test_spmm_power_law_with_hub_rows_and_columns(dev, h, f):
     assert torch.equal(ga, ga2) and torch.equal(gx, gx2)  # no atomics: reproducible
 
 
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24), (3, 5), (1, 8)])
+def test_spmm_bf16_features(dev, h, f):
+    """bf16 feature rows, fp32 edge values and accumulation: equal to the fp32 op on the
+    rounded features (tolerance of the bf16 bar; in fact only the order of the fp32 sums
+    differs), on a power-law graph so that planned rows are covered."""
+    indptr, indices = powerlaw_graph(12, 50000, 9 * h + f)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(h + f)
+    values = torch.rand(indices.numel(), h, generator=g)
+    x16 = torch.randn(n, h, f, generator=g).to(torch.bfloat16)
+    want = oracle.mh_spmm_forward(values, indptr, indices, x16.float())
+    got = graph_ext.spmm_forward(values.to(dev), indptr.to(dev), indices.to(dev), x16.to(dev))
+    assert got.dtype == torch.float32
+    assert_close(got, want, rtol=1e-2, atol=1e-4, what="H=%d F=%d" % (h, f))
+    same = graph_ext.spmm_forward(values.to(dev), indptr.to(dev), indices.to(dev),
+                                  x16.float().to(dev))
+    assert_close(got, same, rtol=1e-5, atol=1e-4)
+
+
 def test_spmm_more_than_65535_rows(dev):
     """The reference's dim3(n_heads, n_nodes) launch is invalid above 65,535 rows."""
     n_dst, n_src, h, f = 70000, 1000, 2, 8

@@ -42,11 +42,11 @@ YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_
                        workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
-YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *indptr,
-                               const int32_t *indices, const float *features, int64_t n_dst,
-                               int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                               int64_t max_degree, const void *plan, void *workspace,
-                               size_t workspace_bytes, void *stream) {
+static int spmm_forward_any(float *out, const float *values, const int32_t *indptr,
+                            const int32_t *indices, const void *features, bool bf16_in,
+                            int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                            int64_t n_features, int64_t max_degree, const void *plan,
+                            void *workspace, size_t workspace_bytes, void *stream) {
     YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
                  "negative size");
     if (n_dst == 0 || n_heads * n_features == 0) return 0;
@@ -67,8 +67,28 @@ YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *i
     p.H = (int)n_heads;
     p.col_mask = 0xffffff;
     p.alpha = 1.0f;
-    return launch_spmm(p, W_EDGEHEAD, false, nnz, max_degree, plan, workspace, workspace_bytes,
+    return launch_spmm(p, W_EDGEHEAD, bf16_in, nnz, max_degree, plan, workspace, workspace_bytes,
                        static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *indptr,
+                               const int32_t *indices, const float *features, int64_t n_dst,
+                               int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
+                               int64_t max_degree, const void *plan, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    return spmm_forward_any(out, values, indptr, indices, features, false, n_dst, n_src, nnz,
+                            n_heads, n_features, max_degree, plan, workspace, workspace_bytes,
+                            stream);
+}
+
+YITU_API int yitu_spmm_forward_bf16(float *out, const float *values, const int32_t *indptr,
+                                    const int32_t *indices, const void *features_bf16,
+                                    int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                                    int64_t n_features, int64_t max_degree, const void *plan,
+                                    void *workspace, size_t workspace_bytes, void *stream) {
+    return spmm_forward_any(out, values, indptr, indices, features_bf16, true, n_dst, n_src, nnz,
+                            n_heads, n_features, max_degree, plan, workspace, workspace_bytes,
+                            stream);
 }
 
 

@@ -109,12 +109,10 @@ static int dispatch_type(const SpmmParams &p, bool bf16_in, bool with_hub, hipSt
     }
     // a lane's VEC elements must stay inside one head and one aligned vector
     const int unit = WMODE == W_EDGEHEAD ? p.F : p.L;
-    if constexpr (WMODE != W_EDGEHEAD) {
-      if (bf16_in) {
+    if (bf16_in) {
         if (unit % 8 == 0 && aligned16(p.feat) && aligned16(p.out))
             return dispatch_shape<WMODE, bf16_t, 8>(p, with_hub, stream);
         return dispatch_shape<WMODE, bf16_t, 1>(p, with_hub, stream);
-      }
     }
     if (unit % 4 == 0 && aligned16(p.feat) && aligned16(p.out))
         return dispatch_shape<WMODE, float, 4>(p, with_hub, stream);
@@ -146,9 +144,7 @@ int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max
     switch (wmode) {
         case W_NONE: return dispatch_type<W_NONE>(p, bf16_in, with_hub, stream);
         case W_DEGPROD: return dispatch_type<W_DEGPROD>(p, bf16_in, with_hub, stream);
-        case W_EDGEHEAD:
-            YITU_REQUIRE(!bf16_in, "edge-weighted SpMM takes fp32 features");
-            return dispatch_type<W_EDGEHEAD>(p, false, with_hub, stream);
+        case W_EDGEHEAD: return dispatch_type<W_EDGEHEAD>(p, bf16_in, with_hub, stream);
     }
     set_error("unknown weight mode %d", wmode);
     return -1;

@@ -86,11 +86,13 @@ def transposed(indptr, indices, n_src):
 # SpMM
 # --------------------------------------------------------------------------- #
 def spmm_forward(values, indptr, indices, features):
-    """out[r,h,k] = sum_i values[i,h] * features[col_i,h,k] (entry.cpp:80-90)."""
+    """out[r,h,k] = sum_i values[i,h] * features[col_i,h,k] (entry.cpp:80-90).
+    ``features`` fp32 like the reference, or bf16 (fp32 accumulate, fp32 out)."""
     _check(values, torch.float32, "values", 2)
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
-    _check(features, torch.float32, "features", 3)
+    bf16 = features.dtype == torch.bfloat16
+    _check(features, torch.bfloat16 if bf16 else torch.float32, "features", 3)
     dev = _lib.require_device(values, indptr, indices, features)
     n_dst = indptr.numel() - 1
     n_src, h, f = features.shape
@@ -103,11 +105,11 @@ def spmm_forward(values, indptr, indices, features):
     need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f), c_int(1)) \
         if plan is not None else 0
     ws = _lib.workspace(need, dev)
+    entry = _lib.lib().yitu_spmm_forward_bf16 if bf16 else _lib.lib().yitu_spmm_forward
     with torch.cuda.device(dev):
-        rc = _lib.lib().yitu_spmm_forward(ptr(out), ptr(values), ptr(indptr), ptr(indices),
-                                          ptr(features), c_i64(n_dst), c_i64(n_src), c_i64(nnz),
-                                          c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan), ptr(ws),
-                                          c_size(ws.numel()), stream_ptr(dev))
+        rc = entry(ptr(out), ptr(values), ptr(indptr), ptr(indices), ptr(features), c_i64(n_dst),
+                   c_i64(n_src), c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan), ptr(ws),
+                   c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_spmm_forward")
     return out
 
@@ -344,9 +346,10 @@ def sgemm(a, b, trans_a=False, trans_b=False, out=None):
     return c
 
 
-def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32):
+def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32, out=None):
     """a . op(b) with bf16 operands and fp32 accumulation on the matrix cores.
-    ``a`` [m, k]; ``b`` [k, n], or [n, k] with ``trans_b`` (a Linear weight)."""
+    ``a`` [m, k]; ``b`` [k, n], or [n, k] with ``trans_b`` (a Linear weight).
+    ``out``: a contiguous [m, n] fp32 or bf16 tensor to write (sets ``out_dtype``)."""
     _check(a, torch.bfloat16, "a", 2)
     _check(b, torch.bfloat16, "b", 2)
     if out_dtype not in (torch.float32, torch.bfloat16):
@@ -356,7 +359,14 @@ def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32):
     n, kb = (b.size(0), b.size(1)) if trans_b else (b.size(1), b.size(0))
     if k != kb:
         raise RuntimeError("inner dimensions differ: %d vs %d" % (k, kb))
-    c = torch.empty((m, n), dtype=out_dtype, device=dev)
+    if out is None:
+        c = torch.empty((m, n), dtype=out_dtype, device=dev)
+    else:
+        out_dtype = out.dtype
+        if out_dtype not in (torch.float32, torch.bfloat16) or tuple(out.shape) != (m, n) \
+                or out.device != dev or not out.is_contiguous():
+            raise RuntimeError("out must be a contiguous [%d, %d] fp32 or bf16 tensor" % (m, n))
+        c = out
     ws = _lib.workspace(_size_fn("yitu_gemm_bf16_workspace_bytes")(c_i64(n), c_i64(k),
                                                                   c_int(int(trans_b))), dev)
     with torch.cuda.device(dev):
