@@ -229,6 +229,32 @@ def run_gat(args, dev):
     sd_fwd_ms = _event_ms(lambda: graph_ext.sddmm_forward(rp, ci, q1, k), args.steps, args.warmup)
     sd_bwd_ms = _event_ms(lambda: graph_ext.sddmm_backward(rp, ci, q1, k, attn_sa, ga), args.steps,
                           args.warmup)
+    # layer level, through autograd. (a) the configuration's layer: per-head projections
+    # q = <a_dst, x'>, k = <a_src, x'>, fused attention, mean over heads; (b) the
+    # reference's GATLayer (test/common/model.py:61-106): linear_v 256 -> 4x64, dense
+    # 256 -> 4 projections with bias, attention, mean over heads
+    from yitu_amd.xgnn_h import block as xblock, layers as xlayers, sparse as xsparse
+    blk = xblock.Block([n, n], [rp, ci])
+    xr = x.clone().requires_grad_()
+    a_s, a_d = a_src.clone().requires_grad_(), a_dst.clone().requires_grad_()
+    g_mean = torch.randn(n, f, generator=g, device=dev)
+
+    def layer_step():
+        qq = torch.einsum("nhf,hf->nh", xr, a_d).contiguous()
+        kk = torch.einsum("nhf,hf->nh", xr, a_s).contiguous()
+        xsparse.fused_gat(blk, qq, kk, xr).mean(dim=1).backward(g_mean)
+        xr.grad = a_s.grad = a_d.grad = None
+
+    ref_layer = xlayers.GATLayer(h * f, f, h).to(dev)
+    x_in = x.reshape(n, h * f).clone().requires_grad_()
+
+    def ref_layer_step():
+        ref_layer(blk, x_in).backward(g_mean)
+        x_in.grad = None
+        ref_layer.zero_grad(set_to_none=True)
+
+    layer_ms = _event_ms(layer_step, args.steps, args.warmup)
+    ref_layer_ms = _event_ms(ref_layer_step, args.steps, args.warmup)
     alg_sd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h
     alg_fwd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h + 8 * n * h * f
     alg_bwd = (2 * 4 * n * h * f + 4 * nnz * h + 8 * nnz + 8 * (n + 1) + 4 * nnz
@@ -241,6 +267,8 @@ def run_gat(args, dev):
         "config": {"workload": "c2_gat_f32", "graph": "R-MAT scale 18, 13M draws dedup, CSR by "
                    "destination", "n_nodes": n, "n_edges": nnz, "heads": h, "head_dim": f},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "layer_fwd_bwd_ms": layer_ms,
+        "reference_gatlayer_fwd_bwd_ms": ref_layer_ms,
         "sddmm": {"fwd_ms": sd_fwd_ms, "bwd_ms": sd_bwd_ms,
                   "edges_per_s_fwd_bwd": nnz / ((sd_fwd_ms + sd_bwd_ms) * 1e-3),
                   "fwd_algorithmic_bytes": alg_sd,

@@ -48,6 +48,7 @@ def _run(dev, indptr, indices, n_dst, n_src, h, f, seed, atol=2e-4):
 
 @pytest.mark.parametrize("h,f", [(4, 64), (1, 4), (1, 128), (2, 8), (3, 12), (8, 32), (5, 20),
                                  (16, 16), (33, 4), (64, 8), (4, 256), (2, 1000),
+                                 (2, 128), (8, 64), (4, 128), (16, 64), (32, 32), (16, 32),
                                  (4, 6), (3, 5), (70, 4)])
 def test_gat_shapes(dev, h, f):
     """The last three shapes take the unfused composition inside the same entry point."""
@@ -58,7 +59,7 @@ def test_gat_shapes(dev, h, f):
     assert torch.all(out[0] == 0) and torch.all(out[202] == 0)
 
 
-@pytest.mark.parametrize("h,f", [(4, 64), (8, 8), (1, 32)])
+@pytest.mark.parametrize("h,f", [(4, 64), (8, 8), (1, 32), (8, 64), (8, 128)])
 def test_gat_power_law_hub_rows(dev, h, f):
     indptr, indices = powerlaw_graph(13, 150000, 11 * h + f)
     n = indptr.numel() - 1

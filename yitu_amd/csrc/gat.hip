@@ -664,14 +664,16 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams
     }
 }
 
-// ---- backward over the transposed structure: one gather for two results ----------
+// ---- backward over the transposed structure: one gather for every gradient -------
 // Walking the edges by source c, the source's own row x[c] is local and the
 // gathered row is grad_out[row_e]. That single gather gives both
-//   d_attn[e,h]   = <grad_out[row_e,h,:], x[c,h,:]>          (written in CSR order)
+//   d_attn[e,h]   = <grad_out[row_e,h,:], x[c,h,:]>
 //   grad_x[c,h,:] = sum_e attn[e,h] grad_out[row_e,h,:]
-// so the backward needs one pass over the 1 KB rows instead of two. Lane layout
-// as above: 4 floats per lane, a head owns LPH lanes, the dot of edge k is kept
-// by lane (k % LPH) of each head and stored through the edge permutation.
+// so the backward needs one pass over the feature rows instead of two. Rows of
+// L = 256 KT floats (KT = 1, 2, 4): lane l holds floats [256 t + 4 l, +4) of every
+// tile t, a head owns LPH = F / 4 consecutive lanes of one tile (HPT = 64 / LPH heads
+// per tile), the dot of edge k is kept by lane (k % LPH) of each head and stored
+// through the edge permutation.
 struct GatSrcParams {
     SpmmParams sp;   // indptr / indices / eperm = by-source structure, values = attn,
                      // feat = grad_out, out = grad_x, plan = its row plan, partial
@@ -686,45 +688,55 @@ struct GatSrcParams {
     float *partial_k;      // [plan item id, H] partial grad_k of multi-item sources
 };
 
-// (S[r,h], query[r,h]) with S[r,h] = <grad_out[r,h,:], out[r,h,:]>, 256-float rows,
-// kRowsPerWave rows per wave. The pair is what an edge needs from its destination.
-template <int LPH>
+// (S[r,h], query[r,h]) with S[r,h] = <grad_out[r,h,:], out[r,h,:]>, kRowsPerWave rows
+// per wave. The pair is what an edge needs from its destination.
+template <int LPH, int KT>
 __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict__ row_sq,
                                                              const float *__restrict__ grad_out,
                                                              const float *__restrict__ out,
                                                              const float *__restrict__ query,
                                                              int n_rows) {
+    constexpr int HPT = kWave / LPH, H = HPT * KT, L = 256 * KT, U = KT == 1 ? 4 : 2;
     const int lane = lane_id();
     const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
-    constexpr int H = kWave / LPH;
-    for (int i0 = 0; i0 < kRowsPerWave && r0 + i0 < n_rows; i0 += 4) {
-        float d[4];
+    for (int i0 = 0; i0 < kRowsPerWave && r0 + i0 < n_rows; i0 += U) {
+        float d[U][KT];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < U; u++) {
             const int r = min(r0 + i0 + u, n_rows - 1);
-            float a[4], b[4];
-            RowLoad<4, float>::ld(grad_out + (size_t)r * 256 + lane * 4, a);
-            RowLoad<4, float>::ld(out + (size_t)r * 256 + lane * 4, b);
-            d[u] = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                float a[4], b[4];
+                RowLoad<4, float>::ld(grad_out + (size_t)r * L + t * 256 + lane * 4, a);
+                RowLoad<4, float>::ld(out + (size_t)r * L + t * 256 + lane * 4, b);
+                d[u][t] = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-#pragma unroll
-            for (int o = LPH >> 1; o >= 1; o >>= 1) d[u] += __shfl_xor(d[u], o, kWave);
+        for (int u = 0; u < U; u++) {
             const int r = r0 + i0 + u;
-            if (lane % LPH == 0 && r < n_rows)
-                row_sq[(size_t)r * H + lane / LPH] =
-                    make_float2(d[u], query[(size_t)r * H + lane / LPH]);
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                float s = d[u][t];
+#pragma unroll
+                for (int o = LPH >> 1; o >= 1; o >>= 1) s += __shfl_xor(s, o, kWave);
+                const int head = t * HPT + lane / LPH;
+                if (lane % LPH == 0 && r < n_rows)
+                    row_sq[(size_t)r * H + head] = make_float2(s, query[(size_t)r * H + head]);
+            }
         }
     }
 }
 
-// FULL: kc = key[c, h] of the source; gk accumulates this lane's share of grad_key[c, h].
-template <int LPH, bool FULL>
+// FULL: kc[t] = key[c, head] of the source; gk[t] accumulates this lane's share of
+// grad_key[c, head], head = t HPT + lane / LPH.
+template <int LPH, int KT, bool FULL>
 __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const EdgeWindow &win,
-                                               int first, int n, const float (&xt)[4],
-                                               float (&acc)[4], float kc, float &gk) {
-    constexpr int NS = kWave / LPH;
+                                               int first, int n, const float (&xt)[KT][4],
+                                               float (&acc)[KT][4], const float (&kc)[KT],
+                                               float (&gk)[KT]) {
+    constexpr int NS = kWave / LPH;  // edge groups of LPH edges in a window; also heads per tile
+    constexpr int U = KT == 1 ? kDotUnroll : 2;  // row gathers in flight
     const int lane = lane_id();
     const int h = lane / LPH, sub = lane % LPH;
     const int L = p.sp.L, H = p.sp.H;
@@ -732,79 +744,122 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
     // What is needed per (edge, head) is fetched once, before the row gathers, in the
     // layout of the epilogue: lane (h, sub) owns edge j * LPH + sub. The attention
     // weight reaches the accumulate loop by a lane shuffle.
-    float ea[NS], eS[NS], eq[NS];
+    float ea[NS][KT], eS[NS][KT], eq[NS][KT];
 #pragma unroll
     for (int j = 0; j < NS; j++) {
         const int k = min(j * LPH + sub, n - 1);
         const int vr = __shfl(win.vrow, first + k, kWave);
-        ea[j] = p.sp.values[(size_t)vr * H + h];
-        if constexpr (FULL) {
-            const int r = __shfl(win.col, first + k, kWave);
-            const float2 sq = p.row_sq[(size_t)r * H + h];
-            eS[j] = sq.x;
-            eq[j] = sq.y;
+        const int r = __shfl(win.col, first + k, kWave);
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+            const int head = t * NS + h;
+            ea[j][t] = p.sp.values[(size_t)vr * H + head];
+            if constexpr (FULL) {
+                const float2 sq = p.row_sq[(size_t)r * H + head];
+                eS[j][t] = sq.x;
+                eq[j][t] = sq.y;
+            }
         }
     }
 #pragma unroll
     for (int j = 0; j < NS; j++) {
         if (j * LPH >= n) break;  // wave-uniform
-        float keep = 0.0f;
-        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += kDotUnroll) {
-            float v[kDotUnroll][4], a[kDotUnroll];
+        float keep[KT];
 #pragma unroll
-            for (int u = 0; u < kDotUnroll; u++) {
+        for (int t = 0; t < KT; t++) keep[t] = 0.0f;
+        for (int kk = 0; kk < LPH && j * LPH + kk < n; kk += U) {
+            float v[U][KT][4], a[U][KT];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
                 const int k = j * LPH + kk + u;
                 if (k < n) {  // wave-uniform
                     const int r = __builtin_amdgcn_readlane(win.col, first + k);
-                    RowLoad<4, float>::ld(g + (size_t)r * L + lane * 4, v[u]);
-                    a[u] = __shfl(ea[j], (lane - sub) + kk + u, kWave);
+#pragma unroll
+                    for (int t = 0; t < KT; t++) {
+                        RowLoad<4, float>::ld(g + (size_t)r * L + t * 256 + lane * 4, v[u][t]);
+                        a[u][t] = __shfl(ea[j][t], (lane - sub) + kk + u, kWave);
+                    }
                 }
             }
 #pragma unroll
-            for (int u = 0; u < kDotUnroll; u++) {
+            for (int u = 0; u < U; u++) {
                 const int k = j * LPH + kk + u;
                 if (k < n) {
-                    float d = xt[0] * v[u][0] + xt[1] * v[u][1] + xt[2] * v[u][2] + xt[3] * v[u][3];
 #pragma unroll
-                    for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
-                    if (sub == kk + u) keep = d;
+                    for (int t = 0; t < KT; t++) {
+                        float d = xt[t][0] * v[u][t][0] + xt[t][1] * v[u][t][1] +
+                                  xt[t][2] * v[u][t][2] + xt[t][3] * v[u][t][3];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) acc[i] += a[u] * v[u][i];
+                        for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                        if (sub == kk + u) keep[t] = d;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[t][i] += a[u][t] * v[u][t][i];
+                    }
                 }
             }
         }
         const int k = j * LPH + sub;
         const int vr = __shfl(win.vrow, first + min(k, n - 1), kWave);
-        if constexpr (FULL) {
-            if (k < n) {
-                const float gl = ea[j] * (keep - eS[j]) * (eq[j] + kc < 0.0f ? kSlope : 1.0f);
-                p.grad_a[(size_t)vr * H + h] = gl;
-                gk += gl;
+        if (k < n) {
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                float *dst = p.grad_a + (size_t)vr * H + t * NS + h;
+                if constexpr (FULL) {
+                    const float gl = ea[j][t] * (keep[t] - eS[j][t]) *
+                                     (eq[j][t] + kc[t] < 0.0f ? kSlope : 1.0f);
+                    *dst = gl;
+                    gk[t] += gl;
+                } else {
+                    *dst = keep[t];
+                }
             }
-        } else {
-            if (k < n) p.grad_a[(size_t)vr * H + h] = keep;
         }
     }
 }
 
-// sum of gk over the lanes of a head (all lanes of the head get it)
-template <int LPH>
-__device__ __forceinline__ float head_sum(float gk) {
+// The source's own row, its key, and zeroed accumulators.
+template <int LPH, int KT, bool FULL>
+__device__ __forceinline__ void gat_src_begin(const GatSrcParams &p, int row, bool load,
+                                              float (&xt)[KT][4], float (&acc)[KT][4],
+                                              float (&kc)[KT], float (&gk)[KT]) {
+    const int lane = lane_id();
 #pragma unroll
-    for (int o = LPH >> 1; o >= 1; o >>= 1) gk += __shfl_xor(gk, o, kWave);
-    return gk;
+    for (int t = 0; t < KT; t++) {
+        kc[t] = gk[t] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[t][i] = xt[t][i] = 0.0f;
+        if (load) {
+            RowLoad<4, float>::ld(p.x + (size_t)row * p.sp.L + t * 256 + lane * 4, xt[t]);
+            if constexpr (FULL) kc[t] = p.key[(size_t)row * p.sp.H + t * (kWave / LPH) + lane / LPH];
+        }
+    }
 }
 
-template <int LPH, bool FULL>
+// Writes the accumulated row to x_dst and (FULL) the head sums of gk to k_dst.
+template <int LPH, int KT, bool FULL>
+__device__ __forceinline__ void gat_src_end(float *x_dst, float *k_dst, const float (&acc)[KT][4],
+                                            const float (&gk)[KT]) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        store_row<4>(x_dst + t * 256 + lane * 4, acc[t]);
+        if constexpr (FULL) {
+            float s = gk[t];
+#pragma unroll
+            for (int o = LPH >> 1; o >= 1; o >>= 1) s += __shfl_xor(s, o, kWave);
+            if (lane % LPH == 0) k_dst[t * (kWave / LPH) + lane / LPH] = s;
+        }
+    }
+}
+
+template <int LPH, int KT, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
     const int lane = lane_id();
-    const int h = lane / LPH;
     const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
-    const int L = p.sp.L;
     EdgeWindow win;
     win.base = -1;
     win.col = 0;
@@ -814,34 +869,26 @@ __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
         const int row = r0 + i;
         const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
         if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
-        float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        float kc = 0.0f, gk = 0.0f;
-        if (end > beg) {
-            RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
-            if constexpr (FULL) kc = p.key[(size_t)row * p.sp.H + h];
-        }
+        float xt[KT][4], acc[KT][4], kc[KT], gk[KT];
+        gat_src_begin<LPH, KT, FULL>(p, row, end > beg, xt, acc, kc, gk);
         for (int b = beg; b < end; b += kWave) {
             const int n = min(kWave, end - b);
             if (win.base < 0 || b < win.base || b + n > win.base + kWave)
                 load_window<W_EDGEHEAD>(win, p.sp, b, limit);
-            gat_src_window<LPH, FULL>(p, win, b - win.base, n, xt, acc, kc, gk);
+            gat_src_window<LPH, KT, FULL>(p, win, b - win.base, n, xt, acc, kc, gk);
         }
-        store_row<4>(p.sp.out + (size_t)row * L + lane * 4, acc);
-        if constexpr (FULL) {
-            gk = head_sum<LPH>(gk);
-            if (lane % LPH == 0) p.grad_k[(size_t)row * p.sp.H + h] = gk;
-        }
+        gat_src_end<LPH, KT, FULL>(p.sp.out + (size_t)row * p.sp.L,
+                                   FULL ? p.grad_k + (size_t)row * p.sp.H : nullptr, acc, gk);
     }
 }
 
-template <int LPH, bool FULL>
+template <int LPH, int KT, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
     const int lane = lane_id();
-    const int h = lane / LPH;
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
-    const int L = p.sp.L;
+    const int L = p.sp.L, H = p.sp.H;
     for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
@@ -861,39 +908,34 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
         for (int j = 0; j < kItemsPerWave; j++) {
             if (n_edges[j] <= 0) continue;
             const int row = tag[j] & 0x7fffffff;
-            float xt[4], acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            float kc = 0.0f, gk = 0.0f;
-            RowLoad<4, float>::ld(p.x + (size_t)row * L + lane * 4, xt);
-            if constexpr (FULL) kc = p.key[(size_t)row * p.sp.H + h];
-            gat_src_window<LPH, FULL>(p, win[j], 0, n_edges[j], xt, acc, kc, gk);
+            float xt[KT][4], acc[KT][4], kc[KT], gk[KT];
+            gat_src_begin<LPH, KT, FULL>(p, row, true, xt, acc, kc, gk);
+            gat_src_window<LPH, KT, FULL>(p, win[j], 0, n_edges[j], xt, acc, kc, gk);
             const bool single = tag[j] < 0;
-            float *dst = single ? p.sp.out + (size_t)row * L : p.sp.partial + (size_t)item[j] * L;
-            store_row<4>(dst + lane * 4, acc);
-            if constexpr (FULL) {
-                gk = head_sum<LPH>(gk);
-                float *dk = single ? p.grad_k + (size_t)row * p.sp.H
-                                   : p.partial_k + (size_t)item[j] * p.sp.H;
-                if (lane % LPH == 0) dk[h] = gk;
-            }
+            float *x_dst = single ? p.sp.out + (size_t)row * L : p.sp.partial + (size_t)item[j] * L;
+            float *k_dst = nullptr;
+            if constexpr (FULL)
+                k_dst = single ? p.grad_k + (size_t)row * H : p.partial_k + (size_t)item[j] * H;
+            gat_src_end<LPH, KT, FULL>(x_dst, k_dst, acc, gk);
         }
     }
 }
 
-template <int LPH, bool FULL>
-static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, const float *grad_out,
-                              const float *out, const float *query, int n_dst,
-                              hipStream_t stream) {
+template <int LPH, int KT, bool FULL>
+static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const float *grad_out,
+                                const float *out, const float *query, int n_dst,
+                                hipStream_t stream) {
     if constexpr (FULL) {
-        gat_row_dot_kernel<LPH>
+        gat_row_dot_kernel<LPH, KT>
             <<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(
                 const_cast<float2 *>(p.row_sq), grad_out, out, query, n_dst);
         YITU_LAUNCH_CHECK();
     }
-    gat_src_rows_kernel<LPH, FULL>
+    gat_src_rows_kernel<LPH, KT, FULL>
         <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
-    gat_src_items_kernel<LPH, FULL>
+    gat_src_items_kernel<LPH, KT, FULL>
         <<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave),
                                   1 << 16),
            kBlock, 0, stream>>>(p);
@@ -902,17 +944,36 @@ static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, const float
     spmm_reduce_kernel<W_NONE, 4><<<red_grid, kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
     if constexpr (FULL) {
-        // the item partials of grad_key, rows of H = 64 / LPH floats
-        constexpr int H = kWave / LPH;
+        // the item partials of grad_key, rows of H floats
+        constexpr int H = kWave / LPH * KT;
         SpmmParams k = p.sp;
         k.L = k.F = H;
         k.H = 1;
         k.out = p.grad_k;
         k.partial = p.partial_k;
-        spmm_reduce_kernel<W_NONE, (H >= 4 ? 4 : H)><<<red_grid, kBlock, 0, stream>>>(k);
+        spmm_reduce_kernel<W_NONE, (H % 4 == 0 ? 4 : H)><<<red_grid, kBlock, 0, stream>>>(k);
         YITU_LAUNCH_CHECK();
     }
     return 0;
+}
+
+template <int LPH, bool FULL>
+static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, const float *grad_out,
+                              const float *out, const float *query, int n_dst,
+                              hipStream_t stream) {
+    const int kt = p.sp.L / 256;
+    if (kt == 1)
+        return gat_src_launch_shape<LPH, 1, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
+    if constexpr (FULL) {  // wider rows exist only with the forward output at hand
+        if (kt == 2)
+            return gat_src_launch_shape<LPH, 2, true>(p, has_items, grad_out, out, query, n_dst,
+                                                      stream);
+        if (kt == 4)
+            return gat_src_launch_shape<LPH, 4, true>(p, has_items, grad_out, out, query, n_dst,
+                                                      stream);
+    }
+    set_error("gat backward: unsupported row width %d", p.sp.L);
+    return -1;
 }
 
 template <bool FULL>
@@ -1166,13 +1227,15 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
     YITU_REQUIRE(t_indptr && (nnz == 0 || (t_rows && t_perm)),
                  "gat_backward needs the transposed structure (yitu_csr_transpose)");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // Rows of 256 floats with a power-of-two head width: one pass over the
-    // transposed structure gives d_attn and grad_features from a single gather.
+    // Rows of 256 floats (512 and 1024 too when the forward output is given) with a
+    // power-of-two head width of 32 to 256: one pass over the transposed structure
+    // serves every gradient from a single gather.
     const int64_t L = n_heads * n_features;
     const int lph = (int)(n_features / 4);
-    const bool one_gather = L == 256 && n_features % 4 == 0 && lph >= 8 && (lph & (lph - 1)) == 0 &&
-                            n_dst > 0 && nnz > 0 && n_dst < INT32_MAX && n_src <= (1 << 24) &&
-                            aligned16(features) && aligned16(grad_out) &&
+    const bool wide_ok = out != nullptr && aligned16(out) && (L == 512 || L == 1024);
+    const bool one_gather = (L == 256 || wide_ok) && n_features % 4 == 0 && lph >= 8 && lph <= 64 &&
+                            (lph & (lph - 1)) == 0 && n_dst > 0 && nnz > 0 && n_dst < INT32_MAX &&
+                            n_src <= (1 << 24) && aligned16(features) && aligned16(grad_out) &&
                             aligned16(grad_features);
     if (one_gather) {
         GatSrcParams p{};
