@@ -240,9 +240,7 @@ def run_gat(args, dev):
     g_mean = torch.randn(n, f, generator=g, device=dev)
 
     def layer_step():
-        qq = torch.einsum("nhf,hf->nh", xr, a_d).contiguous()
-        kk = torch.einsum("nhf,hf->nh", xr, a_s).contiguous()
-        xsparse.fused_gat(blk, qq, kk, xr).mean(dim=1).backward(g_mean)
+        xsparse.gat_heads(blk, xr, a_s, a_d, head_mean=True).backward(g_mean)
         xr.grad = a_s.grad = a_d.grad = None
 
     ref_layer = xlayers.GATLayer(h * f, f, h).to(dev)
@@ -660,7 +658,8 @@ def main():
             # the other single-GPU configurations ride along as extra fields
             args.no_cpu = True
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
-                                                "roofline", "fwd_ms", "bwd_ms", "sddmm")
+                                                "roofline", "fwd_ms", "bwd_ms", "layer_fwd_bwd_ms",
+                                                "reference_gatlayer_fwd_bwd_ms", "sddmm")
                               if k in r}
             res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
                             "c2_gat_f32": slim(run_gat(args, dev)),

@@ -211,6 +211,11 @@ int yitu_gat_forward(float *out_device, float *attn_device, const int32_t *indpt
  * 256 floats) the softmax row sums come from <grad_out[row], out[row]> and one
  * pass over the by-source edges finishes every gradient; the workspace must
  * then be given whatever the degrees (yitu_gat_workspace_bytes).
+ * grad_out_is_head_mean: nonzero when the caller's result was the mean of out over
+ * the heads (test/common/model.py:106) and grad_out_device is its gradient
+ * g [n_dst,F], standing for grad_out[r,h,:] = g[r,:] / H. The pass then gathers
+ * F floats per edge instead of H*F. One-pass shapes only (rows of 256 floats, or
+ * 512 / 1024 with out_device, head width a power of two in 32..256).
  */
 int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       float *grad_features_device, float *grad_attn_scratch_device,
@@ -223,7 +228,31 @@ int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
                       int64_t n_heads, int64_t n_features, int64_t max_degree,
                       int64_t max_degree_t, const void *plan_device, const void *plan_t_device,
-                      void *workspace_device, size_t workspace_bytes, void *stream);
+                      int grad_out_is_head_mean, void *workspace_device, size_t workspace_bytes,
+                      void *stream);
+
+/*
+ * Per-head projections of a GAT layer stated with attention vectors:
+ *   out_a[n,h] = <vec_a[h,:], x[n,h,:]>   (and out_b with vec_b; vec_b / out_b may be NULL)
+ * x [n,H,F], vec_* [H,F], out_* [n,H], fp32. The reference's example layer makes
+ * query and key with dense H*F -> H Linears (test/common/model.py:70-71); the
+ * per-head vectors are their block-diagonal, bias-free case. n_features must be
+ * 4 * a power of two (4..256) and H*F at most 1024.
+ * Backward: grad_x[n,h,:] (+)= grad_a[n,h] vec_a[h,:] + grad_b[n,h] vec_b[h,:]
+ * (accumulate != 0 adds to what grad_x holds: the gradient that reached x through
+ * the attention itself), grad_vec_a[h,:] = sum_n grad_a[n,h] x[n,h,:]. The sums over
+ * n are taken per wave and then in wave order (reproducible).
+ */
+int yitu_head_dot(float *out_a_device, float *out_b_device, const float *x_device,
+                  const float *vec_a_device, const float *vec_b_device, int64_t n, int64_t n_heads,
+                  int64_t n_features, void *stream);
+size_t yitu_head_dot_workspace_bytes(int64_t n, int64_t n_heads, int64_t n_features);
+int yitu_head_dot_backward(float *grad_x_device, int accumulate, float *grad_vec_a_device,
+                           float *grad_vec_b_device, const float *x_device,
+                           const float *vec_a_device, const float *vec_b_device,
+                           const float *grad_a_device, const float *grad_b_device, int64_t n,
+                           int64_t n_heads, int64_t n_features, void *workspace_device,
+                           size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Dense products on the matrix cores (fp32 MFMA)                              */

@@ -108,3 +108,103 @@ def test_gat_without_attn_buffer(dev):
                                      _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(dev))
     _lib.check(rc, "yitu_gat_forward")
     assert_close(out, want)
+
+
+@pytest.mark.parametrize("h,f", [(4, 64), (8, 32), (1, 256), (8, 64), (4, 256), (3, 12), (16, 16)])
+def test_gat_head_mean_gradient(dev, h, f):
+    """The layer's mean over heads taken inside the op: its gradient [n_dst, F] is handed
+    to the backward as it is (gathered F floats per edge) and gives the same gradients as
+    the explicit mean; the last two shapes fall outside the one-pass kernels and are
+    expanded by the wrapper."""
+    indptr, indices = powerlaw_graph(12, 60000, 3 * h + f)
+    n = indptr.numel() - 1
+    blk = xblock.Block([n, n], [indptr, indices]).to(dev)
+    g = torch.Generator().manual_seed(h * f)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dev).requires_grad_()
+    q, k, x = mk(n, h), mk(n, h), mk(n, h, f)
+    w = torch.randn(n, f, generator=g).to(dev)
+    y1 = sparse.fused_gat(blk, q, k, x).mean(dim=1)
+    (y1 * w).sum().backward()
+    want = [t.grad.clone() for t in (q, k, x)]
+    for t in (q, k, x):
+        t.grad = None
+    y2 = sparse.fused_gat(blk, q, k, x, head_mean=True)
+    (y2 * w).sum().backward()
+    assert_close(y2, y1, atol=2e-4)
+    for got, ref, name in zip((q.grad, k.grad, x.grad), want, "qkx"):
+        assert_close(got, ref, atol=5e-4, what="grad_%s H=%d F=%d" % (name, h, f))
+
+
+@pytest.mark.parametrize("n,h,f", [(1000, 4, 64), (37, 1, 4), (513, 8, 32), (300, 2, 256),
+                                   (129, 16, 16), (64, 4, 256), (5, 3, 8)])
+@pytest.mark.parametrize("two", [True, False])
+def test_head_dot_forward_backward(dev, n, h, f, two):
+    """Per-head projections against float64 torch algebra: outputs, grad_x written and
+    accumulated, and the attention-vector gradients (sums over all rows)."""
+    g = torch.Generator().manual_seed(n + h + f)
+    x = torch.randn(n, h, f, generator=g)
+    a, b = torch.randn(h, f, generator=g), torch.randn(h, f, generator=g)
+    ga, gb = torch.randn(n, h, generator=g), torch.randn(n, h, generator=g)
+    base = torch.randn(n, h, f, generator=g)
+    d = lambda t: t.to(dev)
+    oa, ob = graph_ext.head_dot(d(x), d(a), d(b) if two else None)
+    xd = x.double()
+    assert_close(oa, (xd * a.double()).sum(-1).float(), atol=1e-4 * f ** 0.5)
+    if two:
+        assert_close(ob, (xd * b.double()).sum(-1).float(), atol=1e-4 * f ** 0.5)
+    else:
+        assert ob is None
+    want_gx = ga.double()[:, :, None] * a.double()
+    want_gb = None
+    if two:
+        want_gx = want_gx + gb.double()[:, :, None] * b.double()
+        want_gb = (gb.double()[:, :, None] * xd).sum(0).float()
+    want_ga = (ga.double()[:, :, None] * xd).sum(0).float()
+    gx, gva, gvb = graph_ext.head_dot_backward(d(x), d(a), d(b) if two else None, d(ga),
+                                               d(gb) if two else None)
+    assert_close(gx, want_gx.float())
+    assert_close(gva, want_ga, atol=1e-4 * n ** 0.5)
+    if two:
+        assert_close(gvb, want_gb, atol=1e-4 * n ** 0.5)
+    acc = d(base.clone())
+    gx2, gva2, _ = graph_ext.head_dot_backward(d(x), d(a), d(b) if two else None, d(ga),
+                                               d(gb) if two else None, grad_x=acc)
+    assert gx2 is acc
+    assert_close(gx2, (want_gx + base.double()).float())
+    assert torch.equal(gva2, gva)  # fixed summation order
+
+
+@pytest.mark.parametrize("h,f,bipartite", [(4, 64, False), (8, 32, True), (2, 24, False),
+                                           (1, 256, True)])
+def test_gat_head_layer_equals_torch_composition(dev, h, f, bipartite):
+    """layers.GATHeadLayer (projections + attention + head mean as one op) against the same
+    layer composed of torch ops and the two-op attention, outputs and every gradient.
+    (2, 24) is a head width the projection kernels do not take: the wrapper composes."""
+    from yitu_amd.xgnn_h import layers
+    n_dst, n_src = (150, 220) if bipartite else (200, 200)
+    indptr, indices = random_csr(n_dst, n_src, 0.1, 4 * h + f, hub_rows=(3,), hub_degree=n_src - 5,
+                                 empty_rows=(0,))
+    blk = xblock.Block([n_dst, n_src], [indptr, indices]).to(dev)
+    torch.manual_seed(h * f)
+    layer = layers.GATHeadLayer(20, f, h).to(dev)
+    xs = torch.randn(n_src, 20, device=dev, requires_grad=True)
+    xd = torch.randn(n_dst, 20, device=dev, requires_grad=True)
+    w = torch.randn(n_dst, f, device=dev)
+    inputs = (xs, xd) if bipartite else (xs,)
+
+    y = layer(blk, [xs, xd] if bipartite else xs)
+    (y * w).sum().backward()
+    got = [y.detach()] + [t.grad.clone() for t in inputs] + [p.grad.clone() for p in layer.parameters()]
+    for t in inputs:
+        t.grad = None
+    layer.zero_grad()
+
+    h_src = layer.linear_v(xs).view(-1, h, f)
+    h_dst = layer.linear_v(xd).view(-1, h, f) if bipartite else h_src
+    q = (h_dst * layer.a_dst).sum(-1)
+    k = (h_src * layer.a_src).sum(-1)
+    y2 = sparse.gspmm(blk, sparse.fused_gsddmm(blk, q, k), h_src.contiguous()).mean(dim=1)
+    (y2 * w).sum().backward()
+    want = [y2.detach()] + [t.grad for t in inputs] + [p.grad for p in layer.parameters()]
+    for a_, b_ in zip(got, want):
+        assert_close(a_, b_, rtol=1e-4, atol=5e-4)

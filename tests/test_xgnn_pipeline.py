@@ -94,6 +94,11 @@ def test_lowering_gat_patterns_and_options():
     assert full["gat"] == 2 and full["bundle"] == 2 and full["select"] == 4
     assert full["linear"] == 2 and full["spmm"] == 0 and full["sddmm"] == 0
     assert not any(k.startswith(("edge", "vert")) for k in full)
+    # the mean over heads that follows each attention is taken inside the fused op
+    lowered = xgnn_h.Optimizer().lower(dataflow, kwargs)
+    assert all(n.attrs.get("head_mean") for n in ir.walk(lowered) if n.op == "gat")
+    assert not any(n.op == "call" and n.fn_name() == "mean" for n in ir.walk(lowered))
+    assert lowered.op == "gat" and lowered.size == [g.num_dst_nodes(), 3]
 
     plain = cases.ops_of(xgnn_h.Optimizer(fuse_gat=False, bundle_gemm=False).lower(dataflow, kwargs))
     assert plain["sddmm"] == 2 and plain["spmm"] == 2 and plain["gat"] == 0

@@ -686,6 +686,12 @@ struct GatSrcParams {
     const float *key;      // [n_src, H]
     float *grad_k;         // [n_src, H]
     float *partial_k;      // [plan item id, H] partial grad_k of multi-item sources
+    // The gathered rows. Normally grad_out [n_dst, L]. When the caller's output was the
+    // mean over heads, its gradient g [n_dst, F] stands for grad_out[r,h,:] = g[r,:] / H:
+    // the gather shrinks to F floats per edge, every head's lanes reading the same ones.
+    int g_ld;        // floats between gathered rows: L, or F
+    int head_mean;   // nonzero: the second form
+    float g_scale;   // 1, or 1 / H
 };
 
 // (S[r,h], query[r,h]) with S[r,h] = <grad_out[r,h,:], out[r,h,:]>, kRowsPerWave rows
@@ -695,9 +701,11 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict_
                                                              const float *__restrict__ grad_out,
                                                              const float *__restrict__ out,
                                                              const float *__restrict__ query,
-                                                             int n_rows) {
+                                                             int n_rows, int g_ld, int head_mean,
+                                                             float g_scale) {
     constexpr int HPT = kWave / LPH, H = HPT * KT, L = 256 * KT, U = KT == 1 ? 4 : 2;
     const int lane = lane_id();
+    const int g_lane = (head_mean ? lane % LPH : lane) * 4, g_tile = head_mean ? 0 : 256;
     const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
     for (int i0 = 0; i0 < kRowsPerWave && r0 + i0 < n_rows; i0 += U) {
         float d[U][KT];
@@ -707,9 +715,9 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict_
 #pragma unroll
             for (int t = 0; t < KT; t++) {
                 float a[4], b[4];
-                RowLoad<4, float>::ld(grad_out + (size_t)r * L + t * 256 + lane * 4, a);
+                RowLoad<4, float>::ld(grad_out + (size_t)r * g_ld + t * g_tile + g_lane, a);
                 RowLoad<4, float>::ld(out + (size_t)r * L + t * 256 + lane * 4, b);
-                d[u][t] = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+                d[u][t] = (a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3]) * g_scale;
             }
         }
 #pragma unroll
@@ -739,8 +747,10 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
     constexpr int U = KT == 1 ? kDotUnroll : 2;  // row gathers in flight
     const int lane = lane_id();
     const int h = lane / LPH, sub = lane % LPH;
-    const int L = p.sp.L, H = p.sp.H;
+    const int H = p.sp.H;
     const float *__restrict__ g = static_cast<const float *>(p.sp.feat);
+    const int g_lane = (p.head_mean ? sub : lane) * 4, g_tile = p.head_mean ? 0 : 256;
+    const float g_scale = p.g_scale;
     // What is needed per (edge, head) is fetched once, before the row gathers, in the
     // layout of the epilogue: lane (h, sub) owns edge j * LPH + sub. The attention
     // weight reaches the accumulate loop by a lane shuffle.
@@ -776,8 +786,8 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
                     const int r = __builtin_amdgcn_readlane(win.col, first + k);
 #pragma unroll
                     for (int t = 0; t < KT; t++) {
-                        RowLoad<4, float>::ld(g + (size_t)r * L + t * 256 + lane * 4, v[u][t]);
-                        a[u][t] = __shfl(ea[j][t], (lane - sub) + kk + u, kWave);
+                        RowLoad<4, float>::ld(g + (size_t)r * p.g_ld + t * g_tile + g_lane, v[u][t]);
+                        a[u][t] = __shfl(ea[j][t], (lane - sub) + kk + u, kWave) * g_scale;
                     }
                 }
             }
@@ -791,7 +801,7 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
                                   xt[t][2] * v[u][t][2] + xt[t][3] * v[u][t][3];
 #pragma unroll
                         for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
-                        if (sub == kk + u) keep[t] = d;
+                        if (sub == kk + u) keep[t] = d * g_scale;
 #pragma unroll
                         for (int i = 0; i < 4; i++) acc[t][i] += a[u][t] * v[u][t][i];
                     }
@@ -928,7 +938,8 @@ static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const flo
     if constexpr (FULL) {
         gat_row_dot_kernel<LPH, KT>
             <<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(
-                const_cast<float2 *>(p.row_sq), grad_out, out, query, n_dst);
+                const_cast<float2 *>(p.row_sq), grad_out, out, query, n_dst, p.g_ld, p.head_mean,
+                p.g_scale);
         YITU_LAUNCH_CHECK();
     }
     gat_src_rows_kernel<LPH, KT, FULL>
@@ -1219,8 +1230,8 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                                const int32_t *t_rows, const int32_t *t_perm, int64_t n_dst,
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
                                int64_t max_degree, int64_t max_degree_t, const void *plan,
-                               const void *plan_t, void *workspace, size_t workspace_bytes,
-                               void *stream_) {
+                               const void *plan_t, int grad_out_is_head_mean, void *workspace,
+                               size_t workspace_bytes, void *stream_) {
     YITU_REQUIRE(grad_query && grad_key && grad_features, "null output");
     YITU_REQUIRE(nnz == 0 || (grad_attn_scratch && grad_edge_scratch),
                  "gat_backward needs two [nnz, H] scratch buffers");
@@ -1237,6 +1248,10 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                             (lph & (lph - 1)) == 0 && n_dst > 0 && nnz > 0 && n_dst < INT32_MAX &&
                             n_src <= (1 << 24) && aligned16(features) && aligned16(grad_out) &&
                             aligned16(grad_features);
+    YITU_REQUIRE(!grad_out_is_head_mean || one_gather,
+                 "a head-mean gradient is taken by the one-pass shapes only (rows of 256, 512 or "
+                 "1024 floats, head width 32..256 a power of two, forward output given for the "
+                 "wider rows); expand it to [n_dst, H, F] / H for other shapes");
     if (one_gather) {
         GatSrcParams p{};
         p.sp.indptr = t_indptr;
@@ -1254,6 +1269,9 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         p.sp.alpha = 1.0f;
         p.x = features;
         p.grad_a = grad_attn_scratch;
+        p.g_ld = grad_out_is_head_mean ? (int)n_features : (int)L;
+        p.head_mean = grad_out_is_head_mean ? 1 : 0;
+        p.g_scale = grad_out_is_head_mean ? 1.0f / (float)n_heads : 1.0f;
         bool has_items = false;
         void *rest = nullptr;
         size_t rest_bytes = 0;

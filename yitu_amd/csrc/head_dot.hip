@@ -1,0 +1,315 @@
+// Per-head projections of a GAT layer with attention vectors:
+//   q[n,h] = <a_dst[h,:], x[n,h,:]>,   k[n,h] = <a_src[h,:], x[n,h,:]>
+// and their backward. The reference's example layer uses dense H*F -> H Linears
+// for the two (test/common/model.py:70-71); the per-head vectors a_src / a_dst
+// [H, F] are their block-diagonal, bias-free special case and the form GAT is
+// usually stated in. As torch ops ((x * a).sum(-1) twice, and the broadcast
+// products and sums of its backward) they take ten passes over x; here the
+// forward reads x once and the backward reads x once and updates grad_x once.
+//
+// Layout: a row of L = H * F floats is spread over the wave in tiles of 256
+// floats, 4 per lane; F = 4 * LPH with LPH a power of two <= 64, so a head is LPH
+// consecutive lanes of one tile and its dot is a butterfly inside the group.
+#include "../../include/yitu_hip.h"
+#include "spmm_rows.hpp"
+
+namespace yitu {
+
+namespace {
+
+constexpr int kMaxTiles = 4;      // rows of up to 1024 floats
+constexpr int kRowsInFlight = 4;  // rows a wave loads before it reduces
+
+struct HeadDotParams {
+    const float *x;        // [n, L]
+    const float *a1, *a2;  // [L] each (a2 may be null)
+    float *o1, *o2;        // [n, H]
+    const float *g1, *g2;  // backward: gradients of o1, o2 [n, H]
+    float *grad_x;         // backward: [n, L], written or accumulated into
+    float *partial;        // backward: [workgroups][2][L] partial sums for the vector gradients
+    int accumulate;
+    int n, L, H, lph;
+};
+
+__device__ __forceinline__ float group_sum_rt(float v, int lph) {
+    for (int o = lph >> 1; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+template <int KT, bool TWO>
+__global__ __launch_bounds__(kBlock) void head_dot_kernel(HeadDotParams p) {
+    const int lane = lane_id();
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int wave = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    float a1[KT][4], a2[KT][4];
+    bool live[KT];
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        const int col = t * 256 + lane * 4;
+        live[t] = col < p.L;
+#pragma unroll
+        for (int i = 0; i < 4; i++) a1[t][i] = a2[t][i] = 0.0f;
+        if (live[t]) {
+            RowLoad<4, float>::ld(p.a1 + col, a1[t]);
+            if constexpr (TWO) RowLoad<4, float>::ld(p.a2 + col, a2[t]);
+        }
+    }
+    for (int r0 = wave * kRowsInFlight; r0 < p.n; r0 += n_waves * kRowsInFlight) {
+        float x[kRowsInFlight][KT][4];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; u++) {
+            const int r = min(r0 + u, p.n - 1);
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+                if (live[t]) RowLoad<4, float>::ld(p.x + (size_t)r * p.L + t * 256 + lane * 4, x[u][t]);
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; u++) {
+            const int r = r0 + u;
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                float d1 = 0.0f, d2 = 0.0f;
+                if (live[t]) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        d1 += x[u][t][i] * a1[t][i];
+                        if constexpr (TWO) d2 += x[u][t][i] * a2[t][i];
+                    }
+                }
+                d1 = group_sum_rt(d1, p.lph);
+                if constexpr (TWO) d2 = group_sum_rt(d2, p.lph);
+                const int head = (t * 256 + lane * 4) / (4 * p.lph);
+                if (live[t] && r < p.n && lane % p.lph == 0) {
+                    p.o1[(size_t)r * p.H + head] = d1;
+                    if constexpr (TWO) p.o2[(size_t)r * p.H + head] = d2;
+                }
+            }
+        }
+    }
+}
+
+// grad_x[n,h,:] (+)= g1[n,h] a1[h,:] + g2[n,h] a2[h,:]; the workgroup's sums of
+// g1[n,h] x[n,h,:] and g2[n,h] x[n,h,:] go to partial[workgroup][0 / 1][:], added up by
+// the kernel below.
+template <int KT, bool TWO>
+__global__ __launch_bounds__(kBlock) void head_dot_bwd_kernel(HeadDotParams p) {
+    const int lane = lane_id();
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int wave = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    float a1[KT][4], a2[KT][4], s1[KT][4], s2[KT][4];
+    bool live[KT];
+    int head[KT];
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        const int col = t * 256 + lane * 4;
+        live[t] = col < p.L;
+        head[t] = live[t] ? col / (4 * p.lph) : 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) a1[t][i] = a2[t][i] = s1[t][i] = s2[t][i] = 0.0f;
+        if (live[t]) {
+            RowLoad<4, float>::ld(p.a1 + col, a1[t]);
+            if constexpr (TWO) RowLoad<4, float>::ld(p.a2 + col, a2[t]);
+        }
+    }
+    for (int r0 = wave * kRowsInFlight; r0 < p.n; r0 += n_waves * kRowsInFlight) {
+        float x[kRowsInFlight][KT][4], gx[kRowsInFlight][KT][4];
+        float g1[kRowsInFlight][KT], g2[kRowsInFlight][KT];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; u++) {
+            const int r = min(r0 + u, p.n - 1);
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                g1[u][t] = g2[u][t] = 0.0f;
+                if (live[t]) {
+                    const size_t off = (size_t)r * p.L + t * 256 + lane * 4;
+                    RowLoad<4, float>::ld(p.x + off, x[u][t]);
+                    if (p.accumulate) RowLoad<4, float>::ld(p.grad_x + off, gx[u][t]);
+                    g1[u][t] = p.g1[(size_t)r * p.H + head[t]];
+                    if constexpr (TWO) g2[u][t] = p.g2[(size_t)r * p.H + head[t]];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; u++) {
+            if (r0 + u >= p.n) break;  // wave-uniform
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                if (!live[t]) continue;
+                float out[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    float v = g1[u][t] * a1[t][i];
+                    s1[t][i] += g1[u][t] * x[u][t][i];
+                    if constexpr (TWO) {
+                        v += g2[u][t] * a2[t][i];
+                        s2[t][i] += g2[u][t] * x[u][t][i];
+                    }
+                    out[i] = p.accumulate ? gx[u][t][i] + v : v;
+                }
+                store_row<4>(p.grad_x + (size_t)(r0 + u) * p.L + t * 256 + lane * 4, out);
+            }
+        }
+    }
+    // the four waves of the workgroup are added in wave order; one partial row per workgroup
+    __shared__ float red[kWavesPerBlock][2][256 * KT];
+    const int w = threadIdx.x / kWave;
+#pragma unroll
+    for (int t = 0; t < KT; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            red[w][0][t * 256 + lane * 4 + i] = s1[t][i];
+            red[w][1][t * 256 + lane * 4 + i] = s2[t][i];
+        }
+    __syncthreads();
+    for (int j = threadIdx.x; j < 2 * p.L; j += kBlock) {
+        const int which = j / p.L, col = j % p.L;
+        float s = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kWavesPerBlock; q++) s += red[q][which][col];
+        p.partial[(size_t)blockIdx.x * 2 * p.L + j] = s;
+    }
+}
+
+// grad_a[j] = sum over the workgroups' partial rows. A workgroup takes 16 columns;
+// its 16 thread groups add rows g, g + 16, ... and the group sums are added in order.
+constexpr int kSumCols = 16, kSumGroups = kBlock / kSumCols;
+
+__global__ __launch_bounds__(kBlock) void head_dot_sum_kernel(float *__restrict__ grad_a1,
+                                                              float *__restrict__ grad_a2,
+                                                              const float *__restrict__ partial,
+                                                              int n_rows, int L) {
+    __shared__ float red[kSumGroups][kSumCols];
+    const int c = threadIdx.x % kSumCols, g = threadIdx.x / kSumCols;
+    const int j = blockIdx.x * kSumCols + c;
+    float s = 0.0f;
+    if (j < 2 * L)
+        for (int r = g; r < n_rows; r += kSumGroups) s += partial[(size_t)r * 2 * L + j];
+    red[g][c] = s;
+    __syncthreads();
+    if (g == 0 && j < 2 * L) {
+        float t = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kSumGroups; q++) t += red[q][c];
+        if (j < L)
+            grad_a1[j] = t;
+        else if (grad_a2)
+            grad_a2[j - L] = t;
+    }
+}
+
+// workgroups of the forward (enough to fill the chip) and of the backward (each leaves
+// one partial row for the attention-vector gradients)
+int head_dot_grid(int64_t n) {
+    return (int)std::min<int64_t>(ceil_div(n, kWavesPerBlock * kRowsInFlight), 4096);
+}
+int head_dot_bwd_grid(int64_t n) {
+    return (int)std::min<int64_t>(ceil_div(n, kWavesPerBlock * kRowsInFlight), 1024);
+}
+
+int check_shape(int64_t n, int64_t n_heads, int64_t n_features) {
+    YITU_REQUIRE(n >= 0 && n_heads > 0 && n_features > 0 && n < INT32_MAX, "size out of range");
+    const int64_t lph = n_features / 4;
+    YITU_REQUIRE(n_features % 4 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 &&
+                     n_heads * n_features <= 256 * kMaxTiles,
+                 "head_dot: head width must be 4 * a power of two up to 256 and rows at most %d "
+                 "floats (got H=%lld F=%lld)",
+                 256 * kMaxTiles, (long long)n_heads, (long long)n_features);
+    return 0;
+}
+
+template <bool BWD, bool TWO>
+int launch_tiles(const HeadDotParams &p, int grid, hipStream_t stream) {
+    switch ((p.L + 255) / 256) {
+        case 1:
+            if constexpr (BWD) head_dot_bwd_kernel<1, TWO><<<grid, kBlock, 0, stream>>>(p);
+            else head_dot_kernel<1, TWO><<<grid, kBlock, 0, stream>>>(p);
+            break;
+        case 2:
+            if constexpr (BWD) head_dot_bwd_kernel<2, TWO><<<grid, kBlock, 0, stream>>>(p);
+            else head_dot_kernel<2, TWO><<<grid, kBlock, 0, stream>>>(p);
+            break;
+        default:
+            if constexpr (BWD) head_dot_bwd_kernel<4, TWO><<<grid, kBlock, 0, stream>>>(p);
+            else head_dot_kernel<4, TWO><<<grid, kBlock, 0, stream>>>(p);
+    }
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+
+}  // namespace yitu
+
+using namespace yitu;
+#define YITU_API extern "C" __attribute__((visibility("default")))
+
+YITU_API int yitu_head_dot(float *out_a, float *out_b, const float *x, const float *vec_a,
+                           const float *vec_b, int64_t n, int64_t n_heads, int64_t n_features,
+                           void *stream) {
+    if (int rc = check_shape(n, n_heads, n_features)) return rc;
+    if (n == 0) return 0;
+    YITU_REQUIRE(out_a && x && vec_a && (!vec_b == !out_b), "null pointer");
+    YITU_REQUIRE(aligned16(x) && aligned16(vec_a) && aligned16(vec_b), "pointers must be 16-byte aligned");
+    HeadDotParams p{};
+    p.x = x;
+    p.a1 = vec_a;
+    p.a2 = vec_b;
+    p.o1 = out_a;
+    p.o2 = out_b;
+    p.n = (int)n;
+    p.L = (int)(n_heads * n_features);
+    p.H = (int)n_heads;
+    p.lph = (int)(n_features / 4);
+    const int grid = head_dot_grid(n);
+    return vec_b ? launch_tiles<false, true>(p, grid, static_cast<hipStream_t>(stream))
+                 : launch_tiles<false, false>(p, grid, static_cast<hipStream_t>(stream));
+}
+
+YITU_API size_t yitu_head_dot_workspace_bytes(int64_t n, int64_t n_heads, int64_t n_features) {
+    return sizeof(float) * 2 * (size_t)(n_heads * n_features) *
+           (size_t)head_dot_bwd_grid(std::max<int64_t>(n, 1));
+}
+
+YITU_API int yitu_head_dot_backward(float *grad_x, int accumulate, float *grad_vec_a,
+                                    float *grad_vec_b, const float *x, const float *vec_a,
+                                    const float *vec_b, const float *grad_a, const float *grad_b,
+                                    int64_t n, int64_t n_heads, int64_t n_features, void *workspace,
+                                    size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = check_shape(n, n_heads, n_features)) return rc;
+    const int64_t L = n_heads * n_features;
+    YITU_REQUIRE(grad_x && grad_vec_a && x && vec_a && grad_a, "null pointer");
+    YITU_REQUIRE(!vec_b == !grad_b && !vec_b == !grad_vec_b,
+                 "the second vector, its output gradient and its gradient go together");
+    YITU_REQUIRE(aligned16(x) && aligned16(grad_x) && aligned16(vec_a) && aligned16(vec_b),
+                 "pointers must be 16-byte aligned");
+    if (n == 0) {
+        int rc = fill_zero(grad_vec_a, L, stream);
+        if (!rc && grad_vec_b) rc = fill_zero(grad_vec_b, L, stream);
+        return rc;
+    }
+    YITU_REQUIRE(workspace && workspace_bytes >= yitu_head_dot_workspace_bytes(n, n_heads, n_features) &&
+                     aligned16(workspace),
+                 "workspace too small: need %zu bytes",
+                 yitu_head_dot_workspace_bytes(n, n_heads, n_features));
+    HeadDotParams p{};
+    p.x = x;
+    p.a1 = vec_a;
+    p.a2 = vec_b;
+    p.g1 = grad_a;
+    p.g2 = grad_b;
+    p.grad_x = grad_x;
+    p.partial = static_cast<float *>(workspace);
+    p.accumulate = accumulate;
+    p.n = (int)n;
+    p.L = (int)L;
+    p.H = (int)n_heads;
+    p.lph = (int)(n_features / 4);
+    const int grid = head_dot_bwd_grid(n);
+    int rc = vec_b ? launch_tiles<true, true>(p, grid, stream) : launch_tiles<true, false>(p, grid, stream);
+    if (rc) return rc;
+    head_dot_sum_kernel<<<(int)ceil_div(2 * L, kSumCols), kBlock, 0, stream>>>(
+        grad_vec_a, grad_vec_b, p.partial, grid, (int)L);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}

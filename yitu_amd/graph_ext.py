@@ -413,22 +413,43 @@ def gat_forward(indptr, indices, query, key, features):
     return [out, attn]
 
 
-def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None):
+def gat_one_pass_shape(n_heads, n_features, with_out=True):
+    """Whether ``yitu_gat_backward`` takes its one-pass path for [*, H, F] rows (the
+    shapes for which a head-mean gradient can be passed as it is)."""
+    row = n_heads * n_features
+    lph = n_features // 4
+    return (n_features % 4 == 0 and 8 <= lph <= 64 and lph & (lph - 1) == 0 and
+            (row == 256 or (with_out and row in (512, 1024))))
+
+
+def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None,
+                 head_mean=False):
     """Returns [grad_query, grad_key, grad_features] of gat_forward's ``out``.
     Passing the forward output ``out`` [n_dst, H, F] lets the softmax backward use
     sum_e a d_attn = <grad_out[row], out[row]> and finish in the same pass over
-    the edges that computes grad_features (256-float rows); without it the
-    attention gradient takes passes of its own."""
-    _check(grad_out, torch.float32, "grad_out", 3)
+    the edges that computes grad_features (rows of 256, 512, 1024 floats); without
+    it the attention gradient takes passes of its own.
+    ``head_mean``: ``grad_out`` is [n_dst, F], the gradient of ``out.mean(dim=1)``
+    (the layer's result, model.py:106); the pass then gathers F floats per edge."""
     _check(attn, torch.float32, "attn", 2)
     dev = _lib.require_device(indptr, indices, query, key, features, attn, grad_out)
-    if out is not None:
-        _check(out, torch.float32, "out", 3)
-        if out.shape != grad_out.shape:
-            raise RuntimeError("out and grad_out must have the same shape")
     n_dst = indptr.numel() - 1
     n_src, h, f = features.shape
     nnz = indices.numel()
+    if head_mean:
+        _check(grad_out, torch.float32, "grad_out", 2)
+        if tuple(grad_out.shape) != (n_dst, f):
+            raise RuntimeError("a head-mean grad_out must be [n_dst, n_features]")
+        if not (gat_one_pass_shape(h, f, out is not None) and n_dst > 0 and nnz > 0):
+            # shapes outside the one-pass kernels: spell the gradient out per head
+            grad_out = (grad_out / h).unsqueeze(1).expand(n_dst, h, f).contiguous()
+            head_mean = False
+    if not head_mean:
+        _check(grad_out, torch.float32, "grad_out", 3)
+    if out is not None:
+        _check(out, torch.float32, "out", 3)
+        if tuple(out.shape) != (n_dst, h, f):
+            raise RuntimeError("out must be [n_dst, n_heads, n_features]")
     tr = transposed(indptr, indices, n_src)
     grad_q = torch.empty_like(query)
     grad_k = torch.empty_like(key)
@@ -446,9 +467,66 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None
         rc = _lib.lib().yitu_gat_backward(
             ptr(grad_q), ptr(grad_k), ptr(grad_x), ptr(s1), ptr(s2), ptr(indptr), ptr(indices),
             ptr(query), ptr(key), ptr(features), ptr(attn), ptr(out), ptr(grad_out),
-            ptr(tr.t_indptr),
-            ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src), c_i64(nnz), c_i64(h),
-            c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan), ptr(tr.plan_t), ptr(ws),
-            c_size(ws.numel()), stream_ptr(dev))
+            ptr(tr.t_indptr), ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src),
+            c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan),
+            ptr(tr.plan_t), c_int(int(head_mean)), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_gat_backward")
     return [grad_q, grad_k, grad_x]
+
+
+# --------------------------------------------------------------------------- #
+# per-head projections (attention vectors)
+# --------------------------------------------------------------------------- #
+def head_dot_shape(n_heads, n_features):
+    """Shapes the projection kernels take: head width 4 * a power of two up to 256,
+    rows of at most 1024 floats."""
+    lph = n_features // 4
+    return (n_features % 4 == 0 and 1 <= lph <= 64 and lph & (lph - 1) == 0 and
+            n_heads * n_features <= 1024)
+
+
+def head_dot(x, vec_a, vec_b=None):
+    """out_a[n,h] = <vec_a[h,:], x[n,h,:]> (and out_b with ``vec_b``): x [n,H,F],
+    vec_* [H,F]. Returns (out_a, out_b or None)."""
+    _check(x, torch.float32, "x", 3)
+    _check(vec_a, torch.float32, "vec_a", 2)
+    if vec_b is not None:
+        _check(vec_b, torch.float32, "vec_b", 2)
+    dev = _lib.require_device(x, vec_a)
+    n, h, f = x.shape
+    if tuple(vec_a.shape) != (h, f) or (vec_b is not None and tuple(vec_b.shape) != (h, f)):
+        raise RuntimeError("attention vectors must be [n_heads, n_features]")
+    out_a = torch.empty((n, h), dtype=torch.float32, device=dev)
+    out_b = torch.empty((n, h), dtype=torch.float32, device=dev) if vec_b is not None else None
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_head_dot(ptr(out_a), ptr(out_b), ptr(x), ptr(vec_a), ptr(vec_b),
+                                      c_i64(n), c_i64(h), c_i64(f), stream_ptr(dev))
+    check(rc, "yitu_head_dot")
+    return out_a, out_b
+
+
+def head_dot_backward(x, vec_a, vec_b, grad_a, grad_b, grad_x=None):
+    """Returns (grad_x, grad_vec_a, grad_vec_b). ``grad_x`` given: the projections'
+    share is added to it in place (it holds the gradient that reached x by other
+    paths); otherwise a new tensor is written."""
+    _check(x, torch.float32, "x", 3)
+    _check(grad_a, torch.float32, "grad_a", 2)
+    dev = _lib.require_device(x, vec_a, grad_a)
+    n, h, f = x.shape
+    accumulate = grad_x is not None
+    if accumulate:
+        _check(grad_x, torch.float32, "grad_x", 3)
+        if grad_x.shape != x.shape:
+            raise RuntimeError("grad_x must have the shape of x")
+    else:
+        grad_x = torch.empty_like(x)
+    gva = torch.empty_like(vec_a)
+    gvb = torch.empty_like(vec_b) if vec_b is not None else None
+    ws = _lib.workspace(_size_fn("yitu_head_dot_workspace_bytes")(c_i64(n), c_i64(h), c_i64(f)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_head_dot_backward(
+            ptr(grad_x), c_int(int(accumulate)), ptr(gva), ptr(gvb), ptr(x), ptr(vec_a), ptr(vec_b),
+            ptr(grad_a), ptr(grad_b), c_i64(n), c_i64(h), c_i64(f), ptr(ws), c_size(ws.numel()),
+            stream_ptr(dev))
+    check(rc, "yitu_head_dot_backward")
+    return grad_x, gva, gvb

@@ -62,7 +62,8 @@ class Executor:
         if op == "sddmm":
             return sparse.fused_gsddmm(v["g"], v["q"], v["k"])
         if op == "gat":
-            return sparse.fused_gat(v["g"], v["q"], v["k"], v["x"])
+            return sparse.fused_gat(v["g"], v["q"], v["k"], v["x"],
+                                    head_mean=bool(node.attrs.get("head_mean")))
         if op == "bundle":
             w_a, w_b = node.attrs["weights"]
             b_a, b_b = node.attrs["biases"]

@@ -65,11 +65,42 @@ class GATLayer(nn.Module):
         k = self.linear_k(h_src)
         h_src = h_src.view(size=[-1, self.n_heads, self.n_features])
         if self.fused:
-            v = sparse.fused_gat(blk, q.contiguous(), k.contiguous(), h_src.contiguous())
+            return sparse.fused_gat(blk, q.contiguous(), k.contiguous(), h_src.contiguous(),
+                                    head_mean=True)
         else:
             attn = sparse.fused_gsddmm(blk, q.contiguous(), k.contiguous())
             v = sparse.gspmm(blk, attn, h_src.contiguous())
         return torch.mean(v, dim=1)
+
+
+class GATHeadLayer(nn.Module):
+    """GAT layer stated with per-head attention vectors: ``h = linear_v(x)`` viewed as
+    [n, H, F] (``in_features=None``: x already is that), logits
+    ``LeakyReLU_0.2(<a_dst[h], h_dst> + <a_src[h], h_src>)``, softmax over each
+    destination's in-edges, aggregate, mean over heads. The reference's example layer
+    (model.py:61-106) makes the two scalars with dense H*F -> H Linears; this is their
+    block-diagonal, bias-free case, and runs as one op (``sparse.gat_heads``)."""
+
+    def __init__(self, in_features, out_features: int, n_heads: int, head_mean: bool = True):
+        super().__init__()
+        self.n_heads, self.n_features, self.head_mean = n_heads, out_features, head_mean
+        self.linear_v = None if in_features is None else \
+            nn.Linear(in_features, n_heads * out_features)
+        self.a_src = nn.Parameter(torch.randn(n_heads, out_features) * 0.1)
+        self.a_dst = nn.Parameter(torch.randn(n_heads, out_features) * 0.1)
+
+    def _heads(self, x):
+        h = x if self.linear_v is None else self.linear_v(x)
+        return h.view(size=[-1, self.n_heads, self.n_features])
+
+    def forward(self, blk: block.Block, x):
+        if isinstance(x, (list, tuple)):
+            assert len(x) == 2
+            h_src, h_dst = self._heads(x[0]), self._heads(x[1])
+        else:
+            h_src, h_dst = self._heads(x), None
+        return sparse.gat_heads(blk, h_src, self.a_src, self.a_dst, x_dst=h_dst,
+                                head_mean=self.head_mean)
 
 
 class HeteroGraphConv(nn.Module):

@@ -73,6 +73,28 @@ class Optimizer:
         for node in ir.walk(dataflow):
             if node.op == "sddmm":
                 node.attrs["uses"] = uses.get(id(node), 0)
+        return Optimizer._fuse_head_mean(ir.rewrite(dataflow, rule))
+
+    # -- mean(gat, dim=1) -> gat with the mean inside ------------------------
+    @staticmethod
+    def _fuse_head_mean(dataflow: ir.Dataflow) -> ir.Dataflow:
+        uses = ir.use_counts(dataflow)
+        only_reader = {id(n) for n in ir.walk(dataflow) if n.op == "gat" and uses.get(id(n)) == 1}
+
+        def rule(node: ir.Node) -> ir.Node:
+            if node.op != "call" or node.fn_name() != "mean" or len(node.inputs) != 1:
+                return node
+            (inner,) = node.inputs.values()
+            kwargs = node.attrs["kwargs"]
+            if inner.op != "gat" or inner.attrs.get("origin") not in only_reader or \
+                    kwargs.get("dim") != 1 or set(kwargs) != {"dim"} or len(node.attrs["args"]) != 1:
+                return node
+            return ir.Node("gat", inner.inputs, {"head_mean": True}, node.size)
+
+        # rewriting copies nodes whose inputs change: carry the identity along
+        for n in ir.walk(dataflow):
+            if n.op == "gat":
+                n.attrs["origin"] = id(n)
         return ir.rewrite(dataflow, rule)
 
     # -- linear_q(h), linear_k(h) -> one launch ------------------------------

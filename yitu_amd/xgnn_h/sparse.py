@@ -109,29 +109,92 @@ def hfused_spddmm(spmm_block: block.Block, spmm_values, spmm_x, sddmm_block: blo
 
 class FusedGATFunction(autograd.Function):
     """The vertical fusion the reference's optimizer stops short of:
-    ``gspmm(blk, fused_gsddmm(blk, q, k), x)`` as one op, forward and backward."""
+    ``gspmm(blk, fused_gsddmm(blk, q, k), x)`` as one op, forward and backward, and
+    optionally the mean over heads that the layer applies next (model.py:106): its
+    gradient is then one F-float row per destination, which the backward gathers
+    as it is instead of H * F floats per edge."""
 
     @staticmethod
-    def forward(ctx, adj_sparse, query, key, x):
+    def forward(ctx, adj_sparse, query, key, x, head_mean):
         indptr, indices = adj_sparse
         out, attn = graph_ext.gat_forward(indptr, indices, query, key, x)
         ctx.adj_sparse = adj_sparse
+        ctx.head_mean = head_mean
         ctx.save_for_backward(query, key, x, attn, out)
-        return out
+        return out.mean(dim=1) if head_mean else out
 
     @staticmethod
     def backward(ctx, grad_out):
         indptr, indices = ctx.adj_sparse
         query, key, x, attn, out = ctx.saved_tensors
         grad_q, grad_k, grad_x = graph_ext.gat_backward(indptr, indices, query, key, x, attn,
-                                                        grad_out.contiguous(), out=out)
-        return None, grad_q, grad_k, grad_x
+                                                        grad_out.contiguous(), out=out,
+                                                        head_mean=ctx.head_mean)
+        return None, grad_q, grad_k, grad_x, None
 
 
-def fused_gat(block: block.Block, query: torch.Tensor, key: torch.Tensor, x: torch.Tensor):
-    """query [n_dst, H], key [n_src, H], x [n_src, H, F] -> [n_dst, H, F]."""
+def fused_gat(block: block.Block, query: torch.Tensor, key: torch.Tensor, x: torch.Tensor,
+              head_mean: bool = False):
+    """query [n_dst, H], key [n_src, H], x [n_src, H, F] -> [n_dst, H, F], or
+    [n_dst, F] (the mean over heads) with ``head_mean``."""
     assert x.dim() == 3 and query.dim() == 2 and key.dim() == 2
-    return FusedGATFunction.apply(block.adj_sparse, query, key, x)
+    return FusedGATFunction.apply(block.adj_sparse, query, key, x, head_mean)
+
+
+class GATHeadsFunction(autograd.Function):
+    """A GAT layer's attention stated with per-head attention vectors: query
+    ``<a_dst[h], x_dst[n,h,:]>``, key ``<a_src[h], x_src[n,h,:]>``, then the fused
+    attention, as one differentiable op. The projections read x once forward; their
+    backward is added in place into the gradient the attention already produced for x,
+    so x's three uses cost no extra adds."""
+
+    @staticmethod
+    def forward(ctx, adj_sparse, x_src, x_dst, a_src, a_dst, head_mean):
+        indptr, indices = adj_sparse
+        if x_dst is None:
+            query, key = graph_ext.head_dot(x_src, a_dst, a_src)
+        else:
+            query, _ = graph_ext.head_dot(x_dst, a_dst)
+            key, _ = graph_ext.head_dot(x_src, a_src)
+        out, attn = graph_ext.gat_forward(indptr, indices, query, key, x_src)
+        ctx.adj_sparse, ctx.head_mean, ctx.shared = adj_sparse, head_mean, x_dst is None
+        saved = (x_src, a_src, a_dst, query, key, attn, out)
+        ctx.save_for_backward(*(saved if x_dst is None else saved + (x_dst,)))
+        return out.mean(dim=1) if head_mean else out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        indptr, indices = ctx.adj_sparse
+        x_src, a_src, a_dst, query, key, attn, out = ctx.saved_tensors[:7]
+        grad_q, grad_k, grad_x = graph_ext.gat_backward(
+            indptr, indices, query, key, x_src, attn, grad_out.contiguous(), out=out,
+            head_mean=ctx.head_mean)
+        if ctx.shared:
+            grad_x, g_dst, g_src = graph_ext.head_dot_backward(x_src, a_dst, a_src, grad_q, grad_k,
+                                                               grad_x=grad_x)
+            return None, grad_x, None, g_src, g_dst, None
+        x_dst = ctx.saved_tensors[7]
+        grad_x, g_src, _ = graph_ext.head_dot_backward(x_src, a_src, None, grad_k, None,
+                                                       grad_x=grad_x)
+        grad_xd, g_dst, _ = graph_ext.head_dot_backward(x_dst, a_dst, None, grad_q, None)
+        return None, grad_x, grad_xd, g_src, g_dst, None
+
+
+def gat_heads(block: block.Block, x_src: torch.Tensor, a_src: torch.Tensor, a_dst: torch.Tensor,
+              x_dst: torch.Tensor = None, head_mean: bool = False):
+    """x_src [n_src, H, F] (x_dst [n_dst, H, F] for a bipartite block, default the
+    same tensor), a_src / a_dst [H, F] -> [n_dst, H, F], or [n_dst, F] with
+    ``head_mean``. Head widths the projection kernels do not take go through
+    ``(x * a).sum(-1)`` and ``fused_gat``."""
+    assert x_src.dim() == 3 and a_src.shape == a_dst.shape == x_src.shape[1:]
+    if graph_ext.head_dot_shape(x_src.size(1), x_src.size(2)):
+        return GATHeadsFunction.apply(block.adj_sparse, x_src.contiguous(),
+                                      None if x_dst is None else x_dst.contiguous(),
+                                      a_src.contiguous(), a_dst.contiguous(), head_mean)
+    query = ((x_src if x_dst is None else x_dst) * a_dst).sum(-1)
+    key = (x_src * a_src).sum(-1)
+    return fused_gat(block, query, key, x_src.contiguous(), head_mean=head_mean)
 
 
 class EdgeDotFunction(autograd.Function):

@@ -17,6 +17,8 @@ limits of a packed CSR allow, and the scale is kept.
 """
 from typing import Dict, List, Optional
 
+import torch
+
 from . import block, ir, mp
 
 _ADD = ("add", "__add__", "__radd__")
@@ -57,6 +59,7 @@ class _Term:
         self.root, self.scale, self.post, self.core = root, scale, post, core
         self.rel_index, self.hgraph_key = rel_index, hgraph_key
         self.attention = core.op == "gat" or "e" in core.inputs
+        self.mean_inside = core.op == "gat" and bool(core.attrs.get("head_mean"))
 
     def qkx(self):
         c = self.core
@@ -68,8 +71,8 @@ class _Term:
 
     def signature(self):
         x = self.core.inputs["x"]
-        return (self.attention, self.scale is not None, self.post.fn_name() if self.post else None,
-                tuple(x.size[1:]), self.hgraph_key)
+        post = "mean" if self.mean_inside else (self.post.fn_name() if self.post else None)
+        return (self.attention, self.scale is not None, post, tuple(x.size[1:]), self.hgraph_key)
 
 
 def _match_term(node: ir.Node, kwargs: dict) -> Optional[_Term]:
@@ -152,7 +155,11 @@ class Stitcher:
             inputs["e"] = ir.Node("edge_values", dict(g=g, **scales), size=[n_edges, 1])
         out = ir.Node("spmm", inputs, size=[new_blk.size[0]] + xs[0].size[1:])
         post = terms[0].post
-        if post is not None:
+        if terms[0].mean_inside:  # the terms carried their mean over heads inside the fused op
+            out = ir.Node("call", {"0": out}, {"fn": torch.mean, "args": (ir.Slot("0"),),
+                                               "kwargs": {"dim": 1}},
+                          size=[out.size[0]] + out.size[2:])
+        elif post is not None:
             (slot,) = post.inputs
             out = post.with_inputs({slot: out})
         return out
