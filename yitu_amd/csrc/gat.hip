@@ -931,6 +931,190 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
     }
 }
 
+// ---- head-mean gradient, rows of 256 floats: several edges per load -----------------
+// When the gathered row is the F-float gradient of the head mean, a wave-wide load of
+// the layout above fetches the same F floats once per head, and with F * 4 bytes per
+// edge the pass is bound by the number of loads in flight, not by bandwidth. Here a
+// load instruction fetches SLOTS = 64 / LPH = H different edges: lane (s, sub) holds
+// floats [4 sub, +4) of the gradient row of the s-th edge of a group, and the source's
+// own row as H slices x[c, h, 4 sub .. +4). Per group: H dots (one per head, reduced
+// over the slot's LPH lanes), H x 4 FMAs into acc[h], and the epilogue on lanes
+// sub < H (one head each). Slot sums are folded by a fixed butterfly at the end.
+template <int LPH>
+struct SlotRow {
+    static constexpr int H = kWave / LPH;  // heads = slots (rows of 256 floats)
+    float xh[H][4], acc[H][4];
+    float kc, gk;  // lanes sub < H: key[c, sub] and this slot's share of grad_key[c, sub]
+};
+
+template <int LPH>
+__device__ __forceinline__ void slot_begin(SlotRow<LPH> &row, const GatSrcParams &p, int c,
+                                           bool load) {
+    constexpr int H = SlotRow<LPH>::H;
+    const int sub = lane_id() % LPH;
+    row.kc = row.gk = 0.0f;
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) row.acc[h][i] = row.xh[h][i] = 0.0f;
+        if (load) RowLoad<4, float>::ld(p.x + (size_t)c * 256 + h * (4 * LPH) + sub * 4, row.xh[h]);
+    }
+    if (load && sub < H) row.kc = p.key[(size_t)c * H + sub];
+}
+
+template <int LPH>
+__device__ __forceinline__ void slot_window(SlotRow<LPH> &row, const GatSrcParams &p,
+                                            const EdgeWindow &win, int first, int n) {
+    constexpr int H = SlotRow<LPH>::H, SLOTS = H, U = 4;
+    const int lane = lane_id();
+    const int s = lane / LPH, sub = lane % LPH;
+    const float *__restrict__ g = static_cast<const float *>(p.sp.feat);
+    const int F = 4 * LPH;
+    for (int k0 = 0; k0 < n; k0 += SLOTS * U) {
+        float v[U][4], a[U][H];
+        float2 sq[U];
+        int vr[U];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (k0 + u * SLOTS < n) {  // wave-uniform
+                const int k = k0 + u * SLOTS + s;
+                valid[u] = k < n;
+                const int src = first + min(k, n - 1);
+                const int r = __shfl(win.col, src, kWave);
+                vr[u] = __shfl(win.vrow, src, kWave);
+                RowLoad<4, float>::ld(g + (size_t)r * F + sub * 4, v[u]);
+                if constexpr (H == 8) {  // two 16-byte halves
+                    float lo[4], hi[4];
+                    RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8, lo);
+                    RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8 + 4, hi);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        a[u][i] = lo[i];
+                        a[u][4 + i] = hi[i];
+                    }
+                } else {
+                    RowLoad<H, float>::ld(p.sp.values + (size_t)vr[u] * H, a[u]);
+                }
+                sq[u] = sub < H ? p.row_sq[(size_t)r * H + sub] : make_float2(0.0f, 0.0f);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (k0 + u * SLOTS >= n) break;  // wave-uniform
+            float mine = 0.0f;  // d_attn of (this slot's edge, head sub) on lanes sub < H
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                float d = row.xh[h][0] * v[u][0] + row.xh[h][1] * v[u][1] + row.xh[h][2] * v[u][2] +
+                          row.xh[h][3] * v[u][3];
+#pragma unroll
+                for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                if (sub == h) mine = d;
+                const float w = valid[u] ? a[u][h] * p.g_scale : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) row.acc[h][i] += w * v[u][i];
+            }
+            if (valid[u] && sub < H) {
+                float ah = 0.0f;
+#pragma unroll
+                for (int h = 0; h < H; h++)
+                    if (sub == h) ah = a[u][h];
+                const float gl = ah * (mine * p.g_scale - sq[u].x) *
+                                 (sq[u].y + row.kc < 0.0f ? kSlope : 1.0f);
+                p.grad_a[(size_t)vr[u] * H + sub] = gl;
+                row.gk += gl;
+            }
+        }
+    }
+}
+
+template <int LPH>
+__device__ __forceinline__ void slot_end(SlotRow<LPH> &row, float *x_dst, float *k_dst) {
+    constexpr int H = SlotRow<LPH>::H;
+    const int lane = lane_id();
+    const int s = lane / LPH, sub = lane % LPH;
+#pragma unroll
+    for (int o = kWave / 2; o >= LPH; o >>= 1) {
+        row.gk += __shfl_xor(row.gk, o, kWave);
+#pragma unroll
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) row.acc[h][i] += __shfl_xor(row.acc[h][i], o, kWave);
+    }
+    if (s == 0) {
+#pragma unroll
+        for (int h = 0; h < H; h++) store_row<4>(x_dst + h * (4 * LPH) + sub * 4, row.acc[h]);
+        if (sub < H) k_dst[sub] = row.gk;
+    }
+}
+
+template <int LPH>
+__global__ __launch_bounds__(kBlock) void gat_slot_rows_kernel(GatSrcParams p) {
+    constexpr int H = kWave / LPH;
+    const int lane = lane_id();
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    if (r0 >= p.sp.n_rows) return;
+    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
+    const int limit = __shfl(my_ptr, n_here, kWave);
+    EdgeWindow win;
+    win.base = -1;
+    win.col = 0;
+    win.w = 0.0f;
+    win.vrow = 0;
+    for (int i = 0; i < n_here; i++) {
+        const int row = r0 + i;
+        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
+        SlotRow<LPH> acc;
+        slot_begin<LPH>(acc, p, row, end > beg);
+        for (int b = beg; b < end; b += kWave) {
+            const int n = min(kWave, end - b);
+            if (win.base < 0 || b < win.base || b + n > win.base + kWave)
+                load_window<W_EDGEHEAD>(win, p.sp, b, limit);
+            slot_window<LPH>(acc, p, win, b - win.base, n);
+        }
+        slot_end<LPH>(acc, p.sp.out + (size_t)row * 256, p.grad_k + (size_t)row * H);
+    }
+}
+
+template <int LPH>
+__global__ __launch_bounds__(kBlock) void gat_slot_items_kernel(GatSrcParams p) {
+    constexpr int H = kWave / LPH;
+    const int lane = lane_id();
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int n_edges[kItemsPerWave], tag[kItemsPerWave], item[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            const int beg = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            item[j] = __shfl(my_rec.z, j, kWave);
+            tag[j] = __shfl(my_rec.w, j, kWave);
+            n_edges[j] = j < n_here ? end - beg : 0;
+            if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;
+            const int row = tag[j] & 0x7fffffff;
+            SlotRow<LPH> acc;
+            slot_begin<LPH>(acc, p, row, true);
+            slot_window<LPH>(acc, p, win[j], 0, n_edges[j]);
+            const bool single = tag[j] < 0;
+            slot_end<LPH>(acc,
+                          single ? p.sp.out + (size_t)row * 256 : p.sp.partial + (size_t)item[j] * 256,
+                          single ? p.grad_k + (size_t)row * H : p.partial_k + (size_t)item[j] * H);
+        }
+    }
+}
+
 template <int LPH, int KT, bool FULL>
 static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const float *grad_out,
                                 const float *out, const float *query, int n_dst,
@@ -942,15 +1126,32 @@ static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const flo
                 p.g_scale);
         YITU_LAUNCH_CHECK();
     }
-    gat_src_rows_kernel<LPH, KT, FULL>
-        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
+    const int row_grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave);
+    const int item_grid = (int)std::min<int64_t>(
+        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+    // a head-mean gradient of F < 256 floats per row: the several-edges-per-load kernels
+    constexpr bool kSlots = FULL && KT == 1 && LPH < kWave;
+    bool slots = false;
+    if constexpr (kSlots) slots = p.head_mean != 0;
+    if constexpr (kSlots) {
+        if (slots) {
+            gat_slot_rows_kernel<LPH><<<row_grid, kBlock, 0, stream>>>(p);
+            YITU_LAUNCH_CHECK();
+            if (has_items) {
+                gat_slot_items_kernel<LPH><<<item_grid, kBlock, 0, stream>>>(p);
+                YITU_LAUNCH_CHECK();
+            }
+        }
+    }
+    if (!slots) {
+        gat_src_rows_kernel<LPH, KT, FULL><<<row_grid, kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        if (has_items) {
+            gat_src_items_kernel<LPH, KT, FULL><<<item_grid, kBlock, 0, stream>>>(p);
+            YITU_LAUNCH_CHECK();
+        }
+    }
     if (!has_items) return 0;
-    gat_src_items_kernel<LPH, KT, FULL>
-        <<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave),
-                                  1 << 16),
-           kBlock, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
     const int red_grid = (int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16);
     spmm_reduce_kernel<W_NONE, 4><<<red_grid, kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
@@ -1248,6 +1449,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                             (lph & (lph - 1)) == 0 && n_dst > 0 && nnz > 0 && n_dst < INT32_MAX &&
                             n_src <= (1 << 24) && aligned16(features) && aligned16(grad_out) &&
                             aligned16(grad_features);
+    YITU_REQUIRE(!grad_out_is_head_mean || aligned16(attn), "attn must be 16-byte aligned");
     YITU_REQUIRE(!grad_out_is_head_mean || one_gather,
                  "a head-mean gradient is taken by the one-pass shapes only (rows of 256, 512 or "
                  "1024 floats, head width 32..256 a power of two, forward output given for the "
