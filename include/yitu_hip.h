@@ -254,6 +254,25 @@ int yitu_head_dot_backward(float *grad_x_device, int accumulate, float *grad_vec
                            int64_t n_heads, int64_t n_features, void *workspace_device,
                            size_t workspace_bytes, void *stream);
 
+/*
+ * Linear layers with a handful of outputs per row: y[n,J] = x[n,K] . w[J,K]^T + bias[J]
+ * (bias may be NULL). The dense query / key projections of the reference's GATLayer
+ * (nn.Linear(H*F, H), test/common/model.py:70-71) are this shape; stack the weights
+ * of the two to make both with one read of x. K a multiple of 4 up to 1024, J up to 16
+ * with J * tiles <= 16 (tiles = 1, 2, 4 for K up to 256, 512, 1024).
+ * Backward: grad_x (+)= grad_y . w (accumulate != 0 adds to what grad_x holds),
+ * grad_w [J,K], grad_bias [J] (may be NULL), summed in a fixed order.
+ */
+int yitu_skinny_linear(float *y_device, const float *x_device, const float *w_device,
+                       const float *bias_device, int64_t n, int64_t in_features,
+                       int64_t out_features, void *stream);
+size_t yitu_skinny_linear_workspace_bytes(int64_t n, int64_t in_features, int64_t out_features);
+int yitu_skinny_linear_backward(float *grad_x_device, int accumulate, float *grad_w_device,
+                                float *grad_bias_device, const float *x_device,
+                                const float *w_device, const float *grad_y_device, int64_t n,
+                                int64_t in_features, int64_t out_features, void *workspace_device,
+                                size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Dense products on the matrix cores (fp32 MFMA)                              */
 /* ------------------------------------------------------------------------- */

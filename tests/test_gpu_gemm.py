@@ -120,3 +120,38 @@ def test_gemm_bf16_rejects_unaligned_k(dev):
     b = torch.zeros(12, 4, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="multiples of 8"):
         graph_ext.gemm_bf16(a, b)
+
+
+@pytest.mark.parametrize("n,k,j,bias", [(1000, 256, 8, True), (33, 64, 1, False), (517, 512, 8, True),
+                                        (260, 1024, 4, True), (129, 100, 16, True), (5, 768, 4, False),
+                                        (2048, 256, 16, True)])
+def test_skinny_linear_forward_backward(dev, n, k, j, bias):
+    """Linear layers with a handful of outputs against float64 torch: y, grad_x written and
+    accumulated in place, grad_w, grad_b."""
+    g = torch.Generator().manual_seed(n + k + j)
+    x, w = torch.randn(n, k, generator=g), torch.randn(j, k, generator=g)
+    b = torch.randn(j, generator=g) if bias else None
+    gy, base = torch.randn(n, j, generator=g), torch.randn(n, k, generator=g)
+    d = lambda t: None if t is None else t.to(dev)
+    y = graph_ext.skinny_linear(d(x), d(w), d(b))
+    want = x.double() @ w.double().t() + (b.double() if bias else 0)
+    assert_close(y, want.float(), atol=1e-4 * k ** 0.5)
+    gx, gw, gb = graph_ext.skinny_linear_backward(d(x), d(w), d(gy), need_bias=bias)
+    assert_close(gx, (gy.double() @ w.double()).float(), atol=1e-4 * j ** 0.5)
+    assert_close(gw, (gy.double().t() @ x.double()).float(), atol=1e-4 * n ** 0.5)
+    if bias:
+        assert_close(gb, gy.double().sum(0).float(), atol=1e-4 * n ** 0.5)
+    else:
+        assert gb is None
+    acc = d(base.clone())
+    gx2, gw2, _ = graph_ext.skinny_linear_backward(d(x), d(w), d(gy), grad_x=acc, need_bias=bias)
+    assert gx2 is acc
+    assert_close(gx2, (gy.double() @ w.double() + base.double()).float(), atol=1e-4 * j ** 0.5)
+    assert torch.equal(gw2, gw)
+
+
+def test_skinny_linear_rejects_wide_outputs(dev):
+    x, w = torch.zeros(4, 1024, device=dev), torch.zeros(8, 1024, device=dev)
+    with pytest.raises(RuntimeError):
+        graph_ext.skinny_linear(x, w)
+    assert not graph_ext.skinny_linear_shape(1024, 8) and graph_ext.skinny_linear_shape(1024, 4)

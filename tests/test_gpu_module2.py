@@ -275,3 +275,54 @@ def test_dtype_and_device_checks(dev):
     with pytest.raises(RuntimeError):
         graph_ext.sddmm_forward(indptr.to(dev), indices.to(dev), torch.randn(1, 9, 2, device=dev),
                                 torch.randn(10, 2, device=dev))  # query rows != n_dst
+
+
+def test_too_small_max_degree_hint_costs_speed_not_correctness(dev, monkeypatch):
+    """The widest-row argument of the entry points is a hint: told (wrongly) that no row is
+    long, the library builds no row plan and its row kernels walk the long rows themselves.
+    Every op must still give the right answer."""
+    from yitu_amd import _lib
+    indptr, indices = powerlaw_graph(11, 40000, 77)
+    n = indptr.numel() - 1
+    assert int((indptr[1:] - indptr[:-1]).max()) > 500
+    h, f = 4, 16
+    g = torch.Generator().manual_seed(9)
+    q, k = torch.randn(1, n, h, generator=g), torch.randn(n, h, generator=g)
+    x, gy = torch.randn(n, h, f, generator=g), torch.randn(n, h, f, generator=g)
+    ga = torch.randn(indices.numel(), h, generator=g)
+    d = lambda t: t.to(dev)
+    ip, ix = d(indptr), d(indices)
+
+    def run():
+        attn = graph_ext.sddmm_forward(ip, ix, d(q), d(k))
+        gq, gk = graph_ext.sddmm_backward(ip, ix, d(q), d(k), attn, d(ga))
+        out = graph_ext.spmm_forward(attn, ip, ix, d(x))
+        gav, gx = graph_ext.spmm_backward(attn, ip, ix, d(x), d(gy))
+        fo, fattn = graph_ext.gat_forward(ip, ix, d(q[0]), d(k), d(x))
+        fb = graph_ext.gat_backward(ip, ix, d(q[0]), d(k), d(x), fattn, d(gy), out=fo)
+        return [attn, gq, gk, out, gav, gx, fo] + list(fb)
+
+    want = run()
+    graph_ext.transposed(ip, ix, n)  # built with the true degrees; only the hints lie below
+    monkeypatch.setattr(_lib, "max_degree", lambda t: 1)
+    monkeypatch.setattr(_lib, "row_plan", lambda *a: None)
+    tr = graph_ext.transposed(ip, ix, n)
+    monkeypatch.setattr(tr, "max_degree_t", 1)
+    monkeypatch.setattr(tr, "plan_t", None)
+    got = run()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert_close(a, b, rtol=1e-4, atol=5e-4, what="result %d" % i)
+
+
+def test_max_degree_cache_does_not_outlive_its_tensor(dev):
+    """Two graphs of the same size allocated one after the other land on the same device
+    address; the widest-row cache must not hand the first one's answer to the second."""
+    from yitu_amd import _lib
+    a = torch.tensor([0, 1, 2, 3], dtype=torch.int32, device=dev)
+    assert _lib.max_degree(a) == 1
+    addr = a.data_ptr()
+    del a
+    b = torch.tensor([0, 0, 0, 300], dtype=torch.int32, device=dev)
+    if b.data_ptr() == addr:  # the allocator reused the block (the case that matters)
+        assert _lib.max_degree(b) == 300
+    assert _lib.max_degree(b) == 300

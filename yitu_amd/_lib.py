@@ -96,16 +96,18 @@ _max_degree = {}
 
 
 def max_degree(indptr):
-    key = (indptr.data_ptr(), indptr.numel(), indptr._version, str(indptr.device))
+    """Longest row of a CSR, computed once per ``indptr`` tensor. The entry lives as long
+    as the tensor object: an address alone is no identity, the allocator hands a freed
+    block to the next graph of the same size."""
+    key = (id(indptr), indptr.data_ptr(), indptr.numel(), indptr._version)
     v = _max_degree.get(key)
     if v is None:
         if indptr.numel() <= 1:
             v = 0
         else:
             v = int((indptr[1:] - indptr[:-1]).max().item())
-        if len(_max_degree) > 64:
-            _max_degree.clear()
         _max_degree[key] = v
+        weakref.finalize(indptr, _max_degree.pop, key, None)
     return v
 
 
@@ -119,8 +121,8 @@ def row_plan(indptr, indices, n_src, col_mask):
     row reaches the planning threshold."""
     if max_degree(indptr) < 64:
         return None
-    key = (id(indices), indices.data_ptr(), indices._version, indptr.data_ptr(), int(n_src),
-           int(col_mask))
+    key = (id(indices), indices.data_ptr(), indices._version, id(indptr), indptr.data_ptr(),
+           indptr._version, int(n_src), int(col_mask))
     hit = _plans.get(key)
     if hit is not None:
         return hit

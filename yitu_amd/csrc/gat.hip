@@ -479,9 +479,24 @@ __global__ __launch_bounds__(kBlock) void attn_rows_kernel(GatParams p) {
         const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
         const int n = end - beg;
         if (n == 0 || n >= p.sp.plan.threshold) continue;
+        const float qv = hl < H ? p.query[(size_t)(r0 + i) * H + hl] : 0.0f;
+        if (n > kWave) {
+            // no plan although the row is long (a caller's max-degree hint was too small):
+            // two walks over the row's windows, slow but right
+            MaxSum a = ms_init();
+            for (int b = beg; b < end; b += kWave) {
+                load_window<W_NONE>(win, p.sp, b, limit);
+                a = ms_merge(a, gat_stats_window(p, win, 0, min(kWave, end - b), qv));
+            }
+            a = ms_wave_rt(a, p.HP);
+            for (int b = beg; b < end; b += kWave) {
+                load_window<W_NONE>(win, p.sp, b, limit);
+                attn_write_window(p, win, 0, min(kWave, end - b), b, qv, a.m, 1.0f / a.s);
+            }
+            continue;
+        }
         if (win.base < 0 || beg < win.base || end > win.base + kWave)
             load_window<W_NONE>(win, p.sp, beg, limit);
-        const float qv = hl < H ? p.query[(size_t)(r0 + i) * H + hl] : 0.0f;
         const MaxSum a = ms_wave_rt(gat_stats_window(p, win, beg - win.base, n, qv), p.HP);
         attn_write_window(p, win, beg - win.base, n, beg, qv, a.m, 1.0f / a.s);
     }
@@ -557,6 +572,37 @@ __device__ __forceinline__ void attn_bwd_sums_window(const GatBwdParams &p, cons
     }
 }
 
+// Per-edge logit gradient a (g - S) slope of the n edges in window lanes [first, first + n)
+// (CSR edges e0 ...), (edge, head) per lane.
+__device__ __forceinline__ void attn_bwd_write_window(const GatBwdParams &p, const EdgeWindow &win,
+                                                      int first, int n, int e0, float qv, float S) {
+    const int lane = lane_id();
+    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int H = p.sp.H;
+    for (int k0 = 0; k0 < n; k0 += 4 * eps) {
+        float a[4], g[4], kv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            const int col = __shfl(win.col, first + min(k, n - 1), kWave);
+            a[u] = g[u] = kv[u] = 0.0f;
+            if (k < n && hl < H) {
+                const size_t e = (size_t)(e0 + k) * H + hl;
+                a[u] = p.attn[e];
+                g[u] = p.grad_a[e];
+                kv[u] = p.key[(size_t)col * H + hl];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int k = k0 + u * eps + esub;
+            if (k < n && hl < H)
+                p.grad_e[(size_t)(e0 + k) * H + hl] =
+                    a[u] * (g[u] - S) * (qv + kv[u] < 0.0f ? kSlope : 1.0f);
+        }
+    }
+}
+
 __device__ __forceinline__ void attn_bwd_reduce(float &S, float &A1, float &A2, int hp) {
     for (int o = kWave / 2; o >= hp; o >>= 1) {
         S += __shfl_xor(S, o, kWave);
@@ -588,36 +634,30 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
             if (lane < p.HP && hl < H) p.grad_q[(size_t)row * H + hl] = 0.0f;
             continue;
         }
+        const float qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
+        float S = 0.0f, A1 = 0.0f, A2 = 0.0f;
+        if (n > kWave) {
+            // no plan although the row is long (a max-degree hint that was too small):
+            // sums over all windows first, then the per-edge gradients
+            for (int b = beg; b < end; b += kWave) {
+                load_window<W_NONE>(win, p.sp, b, limit);
+                attn_bwd_sums_window(p, win, 0, min(kWave, end - b), b, qv, S, A1, A2);
+            }
+            attn_bwd_reduce(S, A1, A2, p.HP);
+            if (lane < p.HP && hl < H) p.grad_q[(size_t)row * H + hl] = A1 - S * A2;
+            for (int b = beg; b < end; b += kWave) {
+                load_window<W_NONE>(win, p.sp, b, limit);
+                attn_bwd_write_window(p, win, 0, min(kWave, end - b), b, qv, S);
+            }
+            continue;
+        }
         if (win.base < 0 || beg < win.base || end > win.base + kWave)
             load_window<W_NONE>(win, p.sp, beg, limit);
         const int first = beg - win.base;
-        const float qv = hl < H ? p.query[(size_t)row * H + hl] : 0.0f;
-        float S = 0.0f, A1 = 0.0f, A2 = 0.0f;
         attn_bwd_sums_window(p, win, first, n, beg, qv, S, A1, A2);
         attn_bwd_reduce(S, A1, A2, p.HP);
         if (lane < p.HP && hl < H) p.grad_q[(size_t)row * H + hl] = A1 - S * A2;
-        for (int k0 = 0; k0 < n; k0 += 4 * eps) {
-            float a[4], g[4], kv[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int k = k0 + u * eps + esub;
-                const int col = __shfl(win.col, first + min(k, n - 1), kWave);
-                a[u] = g[u] = kv[u] = 0.0f;
-                if (k < n && hl < H) {
-                    const size_t e = (size_t)(beg + k) * H + hl;
-                    a[u] = p.attn[e];
-                    g[u] = p.grad_a[e];
-                    kv[u] = p.key[(size_t)col * H + hl];
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int k = k0 + u * eps + esub;
-                if (k < n && hl < H)
-                    p.grad_e[(size_t)(beg + k) * H + hl] =
-                        a[u] * (g[u] - S) * (qv + kv[u] < 0.0f ? kSlope : 1.0f);
-            }
-        }
+        attn_bwd_write_window(p, win, first, n, beg, qv, S);
     }
 }
 

@@ -313,3 +313,295 @@ YITU_API int yitu_head_dot_backward(float *grad_x, int accumulate, float *grad_v
     YITU_LAUNCH_CHECK();
     return 0;
 }
+
+// ---- skinny Linear: y[n, J] = x[n, K] . w[J, K]^T (+ b), J small ---------------------
+// The dense query / key projections of the reference's GATLayer (H*F -> H Linears with
+// bias, test/common/model.py:70-71) have a handful of outputs per row: as GEMMs they
+// are one read of x each with a tile that is almost empty. Here a wave takes rows of
+// K floats (4 per lane and tile), the J weight rows sit in LDS, and each output is a
+// full-wave butterfly; two Linears that read the same x are one call with their
+// weights stacked. Backward: grad_x (+)= grad_y . w in place, grad_w and grad_b as
+// per-workgroup partial sums added in a fixed order.
+namespace yitu {
+namespace {
+
+constexpr int kSkinnyMaxJ = 16;
+
+struct SkinnyParams {
+    const float *x, *w, *b;  // [n, K], [J, K], [J] or null
+    float *y;                // [n, J]
+    const float *gy;         // backward: [n, J]
+    float *grad_x;           // backward: [n, K]
+    float *partial;          // backward: [workgroups][J * K + J]
+    int accumulate;
+    int n, K, J;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+template <int KT>
+__global__ __launch_bounds__(kBlock) void skinny_linear_kernel(SkinnyParams p) {
+    extern __shared__ __align__(16) float w_lds[];  // [J][256 * KT]
+    constexpr int KP = 256 * KT;
+    for (int i = threadIdx.x; i < p.J * KP; i += kBlock) {
+        const int j = i / KP, c = i % KP;
+        w_lds[i] = c < p.K ? p.w[(size_t)j * p.K + c] : 0.0f;
+    }
+    __syncthreads();
+    const int lane = lane_id();
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int wave = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    for (int r0 = wave * kRowsInFlight; r0 < p.n; r0 += n_waves * kRowsInFlight) {
+        float x[kRowsInFlight][KT][4];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; u++) {
+            const int r = min(r0 + u, p.n - 1);
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                const int c = t * 256 + lane * 4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) x[u][t][i] = 0.0f;
+                if (c < p.K) RowLoad<4, float>::ld(p.x + (size_t)r * p.K + c, x[u][t]);
+            }
+        }
+        for (int j = 0; j < p.J; j++) {
+            float d[kRowsInFlight];
+#pragma unroll
+            for (int u = 0; u < kRowsInFlight; u++) d[u] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                const float4 w4 = *reinterpret_cast<const float4 *>(&w_lds[j * KP + t * 256 + lane * 4]);
+#pragma unroll
+                for (int u = 0; u < kRowsInFlight; u++)
+                    d[u] += x[u][t][0] * w4.x + x[u][t][1] * w4.y + x[u][t][2] * w4.z + x[u][t][3] * w4.w;
+            }
+            const float bj = p.b ? p.b[j] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < kRowsInFlight; u++) {
+                const float s = wave_sum(d[u]);
+                if (lane == 0 && r0 + u < p.n) p.y[(size_t)(r0 + u) * p.J + j] = s + bj;
+            }
+        }
+    }
+}
+
+// JT = outputs whose weight-gradient accumulators a lane keeps (J <= JT).
+template <int KT, int JT>
+__global__ __launch_bounds__(kBlock) void skinny_linear_bwd_kernel(SkinnyParams p) {
+    extern __shared__ __align__(16) float lds[];  // [J][256 * KT] weights, then the workgroup reduction
+    constexpr int KP = 256 * KT;
+    for (int i = threadIdx.x; i < p.J * KP; i += kBlock) {
+        const int j = i / KP, c = i % KP;
+        lds[i] = c < p.K ? p.w[(size_t)j * p.K + c] : 0.0f;
+    }
+    __syncthreads();
+    const int lane = lane_id();
+    const int w_id = threadIdx.x / kWave;
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int wave = blockIdx.x * kWavesPerBlock + w_id;
+    float gw[JT][KT][4], gb[JT];
+#pragma unroll
+    for (int j = 0; j < JT; j++) {
+        gb[j] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < KT; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) gw[j][t][i] = 0.0f;
+    }
+    for (int r = wave; r < p.n; r += n_waves) {
+        float x[KT][4], out[KT][4];
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+            const int c = t * 256 + lane * 4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) x[t][i] = out[t][i] = 0.0f;
+            if (c < p.K) {
+                RowLoad<4, float>::ld(p.x + (size_t)r * p.K + c, x[t]);
+                if (p.accumulate) RowLoad<4, float>::ld(p.grad_x + (size_t)r * p.K + c, out[t]);
+            }
+        }
+        const float g_lane = lane < p.J ? p.gy[(size_t)r * p.J + lane] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < JT; j++) {
+            if (j >= p.J) break;
+            const float g = __shfl(g_lane, j, kWave);
+            gb[j] += g;
+#pragma unroll
+            for (int t = 0; t < KT; t++) {
+                const float4 w4 = *reinterpret_cast<const float4 *>(&lds[j * KP + t * 256 + lane * 4]);
+                out[t][0] += g * w4.x;
+                out[t][1] += g * w4.y;
+                out[t][2] += g * w4.z;
+                out[t][3] += g * w4.w;
+#pragma unroll
+                for (int i = 0; i < 4; i++) gw[j][t][i] += g * x[t][i];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+            const int c = t * 256 + lane * 4;
+            if (c < p.K) store_row<4>(p.grad_x + (size_t)r * p.K + c, out[t]);
+        }
+    }
+    // workgroup partial: the four waves added in wave order, one output row at a time
+    float *dst = p.partial + (size_t)blockIdx.x * (p.J * p.K + p.J);
+    for (int j = 0; j < p.J; j++) {
+        __syncthreads();  // the weights (first pass) or the previous row are no longer needed
+#pragma unroll
+        for (int jj = 0; jj < JT; jj++) {
+            if (jj != j) continue;
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) lds[w_id * KP + t * 256 + lane * 4 + i] = gw[jj][t][i];
+            if (lane == 0) lds[kWavesPerBlock * KP + w_id] = gb[jj];
+        }
+        __syncthreads();
+        for (int c = threadIdx.x; c < p.K; c += kBlock) {
+            float s = 0.0f;
+#pragma unroll
+            for (int q = 0; q < kWavesPerBlock; q++) s += lds[q * KP + c];
+            dst[(size_t)j * p.K + c] = s;
+        }
+        if (threadIdx.x == 0) {
+            float s = 0.0f;
+#pragma unroll
+            for (int q = 0; q < kWavesPerBlock; q++) s += lds[kWavesPerBlock * KP + q];
+            dst[(size_t)p.J * p.K + j] = s;
+        }
+    }
+}
+
+// out[j] = sum over partial rows of partial[row][j], rows added by kSumGroups thread
+// groups and the group sums in order (the same scheme as head_dot_sum_kernel).
+__global__ __launch_bounds__(kBlock) void partial_sum_kernel(float *__restrict__ out_a, int n_a,
+                                                             float *__restrict__ out_b, int n_b,
+                                                             const float *__restrict__ partial,
+                                                             int n_rows) {
+    __shared__ float red[kSumGroups][kSumCols];
+    const int width = n_a + n_b;
+    const int c = threadIdx.x % kSumCols, g = threadIdx.x / kSumCols;
+    const int j = blockIdx.x * kSumCols + c;
+    float s = 0.0f;
+    if (j < width)
+        for (int r = g; r < n_rows; r += kSumGroups) s += partial[(size_t)r * width + j];
+    red[g][c] = s;
+    __syncthreads();
+    if (g == 0 && j < width) {
+        float t = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kSumGroups; q++) t += red[q][c];
+        if (j < n_a)
+            out_a[j] = t;
+        else if (out_b)
+            out_b[j - n_a] = t;
+    }
+}
+
+int skinny_check(int64_t n, int64_t k, int64_t j) {
+    YITU_REQUIRE(n >= 0 && n < INT32_MAX && k > 0 && j > 0, "size out of range");
+    const int64_t tiles = k <= 256 ? 1 : (k <= 512 ? 2 : 4);  // the kernels' tile counts
+    YITU_REQUIRE(k % 4 == 0 && k <= 256 * kMaxTiles && j <= kSkinnyMaxJ && j * tiles <= 16,
+                 "skinny linear: in_features a multiple of 4 up to %d, out_features up to %d with "
+                 "out_features * tiles(in_features) <= 16, tiles = 1, 2, 4 for up to 256, 512, 1024 "
+                 "(got %lld -> %lld)",
+                 256 * kMaxTiles, kSkinnyMaxJ, (long long)k, (long long)j);
+    return 0;
+}
+
+int skinny_bwd_grid(int64_t n) {
+    return (int)std::min<int64_t>(ceil_div(std::max<int64_t>(n, 1), kWavesPerBlock * 8), 1024);
+}
+
+template <int KT>
+int skinny_bwd_launch(const SkinnyParams &p, int grid, size_t lds_bytes, hipStream_t stream) {
+    if (p.J <= 4) skinny_linear_bwd_kernel<KT, 4><<<grid, kBlock, lds_bytes, stream>>>(p);
+    else if (p.J <= 8) {
+        if constexpr (KT <= 2) skinny_linear_bwd_kernel<KT, 8><<<grid, kBlock, lds_bytes, stream>>>(p);
+    } else {
+        if constexpr (KT == 1) skinny_linear_bwd_kernel<KT, 16><<<grid, kBlock, lds_bytes, stream>>>(p);
+    }
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+}  // namespace yitu
+
+YITU_API int yitu_skinny_linear(float *y, const float *x, const float *w, const float *bias,
+                                int64_t n, int64_t in_features, int64_t out_features,
+                                void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = skinny_check(n, in_features, out_features)) return rc;
+    if (n == 0) return 0;
+    YITU_REQUIRE(y && x && w && aligned16(x), "null or misaligned pointer");
+    SkinnyParams p{};
+    p.x = x;
+    p.w = w;
+    p.b = bias;
+    p.y = y;
+    p.n = (int)n;
+    p.K = (int)in_features;
+    p.J = (int)out_features;
+    const int kt = (int)((in_features + 255) / 256);
+    const int grid = head_dot_grid(n);
+    switch (kt) {
+        case 1: skinny_linear_kernel<1><<<grid, kBlock, sizeof(float) * p.J * 256, stream>>>(p); break;
+        case 2: skinny_linear_kernel<2><<<grid, kBlock, sizeof(float) * p.J * 512, stream>>>(p); break;
+        default: skinny_linear_kernel<4><<<grid, kBlock, sizeof(float) * p.J * 1024, stream>>>(p);
+    }
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+YITU_API size_t yitu_skinny_linear_workspace_bytes(int64_t n, int64_t in_features,
+                                                   int64_t out_features) {
+    return sizeof(float) * (size_t)(out_features * in_features + out_features) *
+           (size_t)skinny_bwd_grid(n);
+}
+
+YITU_API int yitu_skinny_linear_backward(float *grad_x, int accumulate, float *grad_w,
+                                         float *grad_bias, const float *x, const float *w,
+                                         const float *grad_y, int64_t n, int64_t in_features,
+                                         int64_t out_features, void *workspace,
+                                         size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (int rc = skinny_check(n, in_features, out_features)) return rc;
+    YITU_REQUIRE(grad_x && grad_w && x && w && grad_y && aligned16(x) && aligned16(grad_x),
+                 "null or misaligned pointer");
+    YITU_REQUIRE(workspace && aligned16(workspace) &&
+                     workspace_bytes >= yitu_skinny_linear_workspace_bytes(n, in_features, out_features),
+                 "workspace too small: need %zu bytes",
+                 yitu_skinny_linear_workspace_bytes(n, in_features, out_features));
+    SkinnyParams p{};
+    p.x = x;
+    p.w = w;
+    p.gy = grad_y;
+    p.grad_x = grad_x;
+    p.partial = static_cast<float *>(workspace);
+    p.accumulate = accumulate;
+    p.n = (int)n;
+    p.K = (int)in_features;
+    p.J = (int)out_features;
+    const int kt = (int)((in_features + 255) / 256);
+    const int grid = skinny_bwd_grid(n);
+    // LDS: the weights, later per-wave rows of one output plus the four bias sums
+    const size_t kp = 256 * (kt == 3 ? 4 : kt);
+    const size_t lds_bytes = sizeof(float) * std::max<size_t>(p.J * kp, kWavesPerBlock * kp + kWavesPerBlock);
+    int rc;
+    switch (kt) {
+        case 1: rc = skinny_bwd_launch<1>(p, grid, lds_bytes, stream); break;
+        case 2: rc = skinny_bwd_launch<2>(p, grid, lds_bytes, stream); break;
+        default: rc = skinny_bwd_launch<4>(p, grid, lds_bytes, stream);
+    }
+    if (rc) return rc;
+    const int width = p.J * p.K + p.J;
+    partial_sum_kernel<<<(int)ceil_div(width, kSumCols), kBlock, 0, stream>>>(
+        grad_w, p.J * p.K, grad_bias, p.J, p.partial, grid);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}

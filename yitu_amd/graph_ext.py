@@ -56,7 +56,8 @@ _transposed = {}
 def transposed(indptr, indices, n_src):
     """By-source view (t_indptr, t_rows, t_perm) of a packed CSR, built on the
     device on first use and kept for as long as ``indices`` is alive."""
-    key = (id(indices), indices.data_ptr(), indices._version, indptr.data_ptr(), int(n_src))
+    key = (id(indices), indices.data_ptr(), indices._version, id(indptr), indptr.data_ptr(),
+           indptr._version, int(n_src))
     hit = _transposed.get(key)
     if hit is not None:
         return hit
@@ -530,3 +531,54 @@ def head_dot_backward(x, vec_a, vec_b, grad_a, grad_b, grad_x=None):
             stream_ptr(dev))
     check(rc, "yitu_head_dot_backward")
     return grad_x, gva, gvb
+
+
+# --------------------------------------------------------------------------- #
+# Linear layers with few outputs
+# --------------------------------------------------------------------------- #
+def skinny_linear_shape(in_features, out_features):
+    tiles = 1 if in_features <= 256 else (2 if in_features <= 512 else 4)
+    return (in_features % 4 == 0 and 0 < in_features <= 1024 and 0 < out_features <= 16 and
+            out_features * tiles <= 16)
+
+
+def skinny_linear(x, weight, bias=None):
+    """x [n, K] . weight [J, K]^T + bias [J] for a handful of outputs J."""
+    _check(x, torch.float32, "x", 2)
+    _check(weight, torch.float32, "weight", 2)
+    if bias is not None:
+        _check(bias, torch.float32, "bias", 1)
+    dev = _lib.require_device(x, weight)
+    n, k = x.shape
+    j = weight.size(0)
+    if weight.size(1) != k or (bias is not None and bias.numel() != j):
+        raise RuntimeError("weight must be [out, in] and bias [out]")
+    y = torch.empty((n, j), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_skinny_linear(ptr(y), ptr(x), ptr(weight), ptr(bias), c_i64(n), c_i64(k),
+                                           c_i64(j), stream_ptr(dev))
+    check(rc, "yitu_skinny_linear")
+    return y
+
+
+def skinny_linear_backward(x, weight, grad_y, grad_x=None, need_bias=True):
+    """Returns (grad_x, grad_weight, grad_bias or None); a given ``grad_x`` is added to in place."""
+    _check(grad_y, torch.float32, "grad_y", 2)
+    dev = _lib.require_device(x, weight, grad_y)
+    n, k = x.shape
+    j = weight.size(0)
+    accumulate = grad_x is not None
+    if not accumulate:
+        grad_x = torch.empty_like(x)
+    else:
+        _check(grad_x, torch.float32, "grad_x", 2)
+    gw = torch.empty_like(weight)
+    gb = torch.empty(j, dtype=torch.float32, device=dev) if need_bias else None
+    ws = _lib.workspace(_size_fn("yitu_skinny_linear_workspace_bytes")(c_i64(n), c_i64(k), c_i64(j)),
+                        dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_skinny_linear_backward(
+            ptr(grad_x), c_int(int(accumulate)), ptr(gw), ptr(gb), ptr(x), ptr(weight), ptr(grad_y),
+            c_i64(n), c_i64(k), c_i64(j), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_skinny_linear_backward")
+    return grad_x, gw, gb

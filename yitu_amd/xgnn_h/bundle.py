@@ -26,3 +26,46 @@ class GEMMBundleFunction(autograd.Function):
         grads = graph_ext.b2gemm_backward(*ctx.saved_tensors, grad_1.contiguous(),
                                           grad_2.contiguous())
         return (*grads, None, None)
+
+
+class SkinnyLinearFunction(autograd.Function):
+    """``F.linear(x, weight, bias)`` for a handful of output features (the query / key
+    projections of a GAT layer): one read of x forward; backward reads x once and writes
+    grad_x once."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return graph_ext.skinny_linear(x, weight, bias)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_y):
+        x, weight = ctx.saved_tensors
+        grad_x, grad_w, grad_b = graph_ext.skinny_linear_backward(
+            x, weight, grad_y.contiguous(), need_bias=ctx.has_bias)
+        return grad_x, grad_w, grad_b
+
+
+def bundled_linear(x, w_a, w_b, b_a=None, b_b=None):
+    """``(x w_a^T + b_a, x w_b^T + b_b)`` for two weight matrices of equal shape applied
+    to one 2-D input: with a handful of outputs one skinny product over the stacked
+    weights (one read of x), otherwise the grouped GEMM launch plus the biases."""
+    import torch
+    n_out = w_a.size(0)
+    if (b_a is None) == (b_b is None) and x.dtype == torch.float32 and \
+            graph_ext.skinny_linear_shape(w_a.size(1), 2 * n_out):
+        bias = None if b_a is None else torch.cat([b_a, b_b])
+        y = SkinnyLinearFunction.apply(x.contiguous(), torch.cat([w_a, w_b], dim=0), bias)
+        return y[:, :n_out].contiguous(), y[:, n_out:].contiguous()
+    y_a, y_b = GEMMBundleFunction.apply(x, w_a, w_b, b_a, b_b)
+    return (y_a if b_a is None else y_a + b_a, y_b if b_b is None else y_b + b_b)
+
+
+def linear_pair(x, linear_a, linear_b):
+    """``(linear_a(x), linear_b(x))`` for two ``nn.Linear`` that read the same input."""
+    if x.dim() == 2 and x.is_cuda and linear_a.weight.shape == linear_b.weight.shape and \
+            linear_a.weight.stride() == linear_b.weight.stride():
+        return bundled_linear(x, linear_a.weight, linear_b.weight, linear_a.bias, linear_b.bias)
+    return linear_a(x), linear_b(x)

@@ -67,9 +67,9 @@ class Executor:
         if op == "bundle":
             w_a, w_b = node.attrs["weights"]
             b_a, b_b = node.attrs["biases"]
-            y_a, y_b = bundle.GEMMBundleFunction.apply(v["x"], w_a, w_b, b_a, b_b)
-            # the bundled GEMM leaves the biases out (bundle.py:8-14): add them here
-            return (y_a if b_a is None else y_a + b_a, y_b if b_b is None else y_b + b_b)
+            # the bundled GEMM of the reference leaves the biases out (bundle.py:8-14);
+            # bundled_linear adds them
+            return bundle.bundled_linear(v["x"], w_a, w_b, b_a, b_b)
         if op == "select":
             return v["x"][node.attrs["index"]]
         if op in ("concat", "stack"):

@@ -8,7 +8,7 @@ from typing import Union
 import torch
 from torch import nn
 
-from . import block, sparse
+from . import block, bundle, sparse
 
 
 def right_norm(blk: block.Block):
@@ -61,8 +61,11 @@ class GATLayer(nn.Module):
             h_src = h_dst = self.linear_v(x)
         else:
             raise TypeError
-        q = self.linear_q(h_dst)
-        k = self.linear_k(h_src)
+        if h_dst is h_src:  # one read of h for both projections
+            q, k = bundle.linear_pair(h_src, self.linear_q, self.linear_k)
+        else:
+            q = self.linear_q(h_dst)
+            k = self.linear_k(h_src)
         h_src = h_src.view(size=[-1, self.n_heads, self.n_features])
         if self.fused:
             return sparse.fused_gat(blk, q.contiguous(), k.contiguous(), h_src.contiguous(),
