@@ -1005,7 +1005,8 @@ __device__ __forceinline__ void slot_begin(SlotRow<LPH> &row, const GatSrcParams
 template <int LPH>
 __device__ __forceinline__ void slot_window(SlotRow<LPH> &row, const GatSrcParams &p,
                                             const EdgeWindow &win, int first, int n) {
-    constexpr int H = SlotRow<LPH>::H, SLOTS = H, U = 4;
+    // U load groups in flight: 2 measured a little better than 4 (fewer registers)
+    constexpr int H = SlotRow<LPH>::H, SLOTS = H, U = 2;
     const int lane = lane_id();
     const int s = lane / LPH, sub = lane % LPH;
     const float *__restrict__ g = static_cast<const float *>(p.sp.feat);
