@@ -530,7 +530,9 @@ def run_c5(args, dev):
                        "n_events": n_events, "batch": batch, "neighbours": k,
                        "sampled_edges": blk.num_edges()},
             "sampler_ms": sample_ms, "sampler_threads": 16, "gpu_sampler_ms": gpu_sample_ms,
-            "note": "45 MB working set, launch-bound: time only"}
+            "note": "45 MB working set, launch-bound: time only; hip_graph_ms is the same step "
+                    "captured once and replayed, reported only when every replay reproduces the "
+                    "eager gradients"}
 
 
 def _c5_graph_ms(layer, blk, gout, steps):

@@ -273,6 +273,15 @@ int yitu_skinny_linear_backward(float *grad_x_device, int accumulate, float *gra
                                 int64_t in_features, int64_t out_features, void *workspace_device,
                                 size_t workspace_bytes, void *stream);
 
+/*
+ * out[j] = sum_r x[r,j] for a row-major [n_rows, n_cols] fp32 matrix: the bias
+ * gradient of a Linear layer, in two stages with a fixed order of additions and no
+ * cleared accumulator, so the call can be recorded into a HIP graph and replayed.
+ */
+size_t yitu_column_sum_workspace_bytes(int64_t n_rows, int64_t n_cols);
+int yitu_column_sum(float *out_device, const float *x_device, int64_t n_rows, int64_t n_cols,
+                    void *workspace_device, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Dense products on the matrix cores (fp32 MFMA)                              */
 /* ------------------------------------------------------------------------- */

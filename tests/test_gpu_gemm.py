@@ -155,3 +155,12 @@ def test_skinny_linear_rejects_wide_outputs(dev):
     with pytest.raises(RuntimeError):
         graph_ext.skinny_linear(x, w)
     assert not graph_ext.skinny_linear_shape(1024, 8) and graph_ext.skinny_linear_shape(1024, 4)
+
+
+@pytest.mark.parametrize("m,n", [(1, 1), (11132, 100), (64, 272), (65, 3), (5000, 1000)])
+def test_column_sum(dev, m, n):
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, n, generator=g)
+    got = graph_ext.column_sum(x.to(dev))
+    assert_close(got, x.double().sum(0).float(), atol=1e-4 * m ** 0.5)
+    assert torch.equal(got, graph_ext.column_sum(x.to(dev)))

@@ -605,3 +605,52 @@ YITU_API int yitu_skinny_linear_backward(float *grad_x, int accumulate, float *g
     YITU_LAUNCH_CHECK();
     return 0;
 }
+
+// ---- column sums: out[j] = sum_r x[r, j] -----------------------------------------------
+// The bias gradient of a Linear layer. Two stages with a fixed order of additions and no
+// cleared accumulator (library reductions clear one with a memset node, which makes them
+// unsafe to replay from a captured graph): workgroups sum row chunks into partial rows,
+// partial_sum_kernel adds those.
+namespace yitu {
+namespace {
+
+constexpr int kColSumChunk = 64;  // rows per workgroup
+
+__global__ __launch_bounds__(kBlock) void column_chunk_sum_kernel(float *__restrict__ partial,
+                                                                  const float *__restrict__ x,
+                                                                  int n_rows, int n_cols) {
+    const int r0 = blockIdx.x * kColSumChunk, r1 = min(r0 + kColSumChunk, n_rows);
+    for (int c = threadIdx.x; c < n_cols; c += kBlock) {
+        float s = 0.0f;
+        for (int r = r0; r < r1; r++) s += x[(size_t)r * n_cols + c];
+        partial[(size_t)blockIdx.x * n_cols + c] = s;
+    }
+}
+
+}  // namespace
+}  // namespace yitu
+
+YITU_API size_t yitu_column_sum_workspace_bytes(int64_t n_rows, int64_t n_cols) {
+    return sizeof(float) * (size_t)std::max<int64_t>(ceil_div(n_rows, kColSumChunk), 1) * (size_t)n_cols;
+}
+
+YITU_API int yitu_column_sum(float *out, const float *x, int64_t n_rows, int64_t n_cols,
+                             void *workspace, size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_rows >= 0 && n_cols >= 0 && n_rows < INT32_MAX && n_cols < (1 << 24),
+                 "size out of range");
+    if (n_cols == 0) return 0;
+    YITU_REQUIRE(out && (n_rows == 0 || x), "null pointer");
+    if (n_rows == 0) return fill_zero(out, n_cols, stream);
+    YITU_REQUIRE(workspace && workspace_bytes >= yitu_column_sum_workspace_bytes(n_rows, n_cols),
+                 "workspace too small: need %zu bytes",
+                 yitu_column_sum_workspace_bytes(n_rows, n_cols));
+    const int chunks = (int)ceil_div(n_rows, kColSumChunk);
+    float *partial = static_cast<float *>(workspace);
+    column_chunk_sum_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows, (int)n_cols);
+    YITU_LAUNCH_CHECK();
+    partial_sum_kernel<<<(int)ceil_div(n_cols, kSumCols), kBlock, 0, stream>>>(
+        out, (int)n_cols, nullptr, 0, partial, chunks);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}

@@ -582,3 +582,18 @@ def skinny_linear_backward(x, weight, grad_y, grad_x=None, need_bias=True):
             c_i64(n), c_i64(k), c_i64(j), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_skinny_linear_backward")
     return grad_x, gw, gb
+
+
+def column_sum(x):
+    """Sum over the rows of a 2-D fp32 tensor (a Linear's bias gradient), in a fixed order and
+    without a cleared accumulator: safe to record into a HIP graph."""
+    _check(x, torch.float32, "x", 2)
+    dev = _lib.require_device(x)
+    m, n = x.shape
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_column_sum_workspace_bytes")(c_i64(m), c_i64(n)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_column_sum(ptr(out), ptr(x), c_i64(m), c_i64(n), ptr(ws),
+                                        c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_column_sum")
+    return out

@@ -17,6 +17,33 @@ from ..xgnn_h import block as xblock
 from ..xgnn_h import sparse
 
 
+class _ReplayableLinear(torch.autograd.Function):
+    """``F.linear`` whose bias gradient is a fixed-order column sum. torch's own reduction
+    clears an accumulator with a memset node, and such nodes do not replay reliably from a
+    captured HIP graph; with this the whole training step of the layer can be captured."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, weight = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_x = grad_y @ weight if ctx.needs_input_grad[0] else None
+        grad_w = grad_y.t() @ x if ctx.needs_input_grad[1] else None
+        grad_b = graph_ext.column_sum(grad_y) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return grad_x, grad_w, grad_b
+
+
+def _linear(layer: torch.nn.Linear, x):
+    if x.is_cuda and x.dtype == torch.float32 and x.dim() == 2:
+        return _ReplayableLinear.apply(x, layer.weight, layer.bias)
+    return layer(x)
+
+
 class TimeEncode(torch.nn.Module):
     """cos(t * w + b), w_i = 10^(-9 i / (dim - 1)), b = 0, both trainable (layers.py:6-17)."""
 
@@ -29,7 +56,7 @@ class TimeEncode(torch.nn.Module):
         self.w.bias = torch.nn.Parameter(torch.zeros(dim))
 
     def forward(self, t):
-        return torch.cos(self.w(t.reshape((-1, 1))))
+        return torch.cos(_linear(self.w, t.reshape((-1, 1))))
 
 
 class TemporalBlock:
@@ -139,11 +166,11 @@ class TransfomerAttentionLayer(torch.nn.Module):
         kv_in = torch.cat(parts_kv, dim=1)
         head_dim = self.dim_out // self.num_head
         if parts_q:
-            Q = self.w_q(torch.cat(parts_q, dim=1))
+            Q = _linear(self.w_q, torch.cat(parts_q, dim=1))
         else:  # edge features only (layers.py:104-107)
             Q = torch.ones((n_dst, self.dim_out), device=dev)
-        K = self.w_k(kv_in).reshape(-1, self.num_head, head_dim).contiguous()
-        V = self.w_v(kv_in).reshape(-1, self.num_head, head_dim).contiguous()
+        K = _linear(self.w_k, kv_in).reshape(-1, self.num_head, head_dim).contiguous()
+        V = _linear(self.w_v, kv_in).reshape(-1, self.num_head, head_dim).contiguous()
         Q = Q.reshape(n_dst, self.num_head, head_dim).contiguous()
         # att = edge_softmax(LeakyReLU(sum_d Q*K)); fused_gsddmm applies LeakyReLU(0.2) +
         # softmax to (query + key): query = 0, key = the dot-product logits, one key per edge
@@ -157,6 +184,6 @@ class TransfomerAttentionLayer(torch.nn.Module):
         att = self.att_dropout(att)
         agg = sparse.gspmm(b.blk, att, V).reshape(n_dst, self.dim_out)
         rst = torch.cat([agg, b.h[:n_dst]], dim=1) if self.dim_node_feat != 0 else agg
-        rst = self.w_out(rst)
+        rst = _linear(self.w_out, rst)
         rst = torch.nn.functional.relu(self.dropout(rst))
         return self.layer_norm(rst)
