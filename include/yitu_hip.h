@@ -192,21 +192,28 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
  * reading each destination row once. attn_device [nnz,H] receives the
  * probabilities for the backward pass; it may be NULL when the shape takes the
  * fused kernel (n_features % 4 == 0, n_heads <= 64, 16-byte aligned pointers).
+ * row_stats_device [n_dst,H,2] (optional, fused kernel only) receives each row's
+ * softmax (max, 1 / sum): with it the backward recomputes a probability from
+ * query, key and these two numbers instead of reading attn, so attn need not be
+ * stored at all.
  */
 size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads, int64_t n_features,
                                 int with_plans);
-int yitu_gat_forward(float *out_device, float *attn_device, const int32_t *indptr_device,
-                     const int32_t *indices_device, const float *query_device,
-                     const float *key_device, const float *features_device, int64_t n_dst,
-                     int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
-                     int64_t max_degree, const void *plan_device, void *workspace_device,
-                     size_t workspace_bytes, void *stream);
+int yitu_gat_forward(float *out_device, float *attn_device, float *row_stats_device,
+                     const int32_t *indptr_device, const int32_t *indices_device,
+                     const float *query_device, const float *key_device,
+                     const float *features_device, int64_t n_dst, int64_t n_src, int64_t nnz,
+                     int64_t n_heads, int64_t n_features, int64_t max_degree,
+                     const void *plan_device, void *workspace_device, size_t workspace_bytes,
+                     void *stream);
 
 /*
  * Backward of the composition (spmm_backward then sddmm_backward,
  * xgnn_h/sparse.py:22-35,67-81) in one call, given grad_out [n_dst,H,F]:
  * grad_query [n_dst,H], grad_key [n_src,H], grad_features [n_src,H,F], all
  * fully written, no atomics. The two scratch buffers are [nnz,H] floats.
+ * attn_device may be NULL when row_stats_device (the forward's statistics) and
+ * out_device are given and the shape is a one-pass shape.
  * out_device: the forward's output [n_dst,H,F], or NULL. With it (and rows of
  * 256 floats) the softmax row sums come from <grad_out[row], out[row]> and one
  * pass over the by-source edges finishes every gradient; the workspace must
@@ -222,8 +229,9 @@ int yitu_gat_backward(float *grad_query_device, float *grad_key_device,
                       float *grad_edge_scratch_device, const int32_t *indptr_device,
                       const int32_t *indices_device, const float *query_device,
                       const float *key_device, const float *features_device,
-                      const float *attn_device, const float *out_device,
-                      const float *grad_out_device, const int32_t *t_indptr_device,
+                      const float *attn_device, const float *row_stats_device,
+                      const float *out_device, const float *grad_out_device,
+                      const int32_t *t_indptr_device,
                       const int32_t *t_rows_device,
                       const int32_t *t_perm_device, int64_t n_dst, int64_t n_src, int64_t nnz,
                       int64_t n_heads, int64_t n_features, int64_t max_degree,

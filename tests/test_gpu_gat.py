@@ -43,6 +43,17 @@ def _run(dev, indptr, indices, n_dst, n_src, h, f, seed, atol=2e-4):
         assert_close(gq, want_gq, atol=atol, what="grad_q " + tag)
         assert_close(gk, want_gk, atol=atol, what="grad_k " + tag)
         assert_close(gx, want_gx, atol=atol, what="grad_x " + tag)
+    if graph_ext.gat_one_pass_shape(h, f):
+        # the probabilities never stored: row statistics out of the forward, recomputed
+        # per edge in the backward
+        out2, none, stats = graph_ext.gat_forward(d(indptr), d(indices), d(q), d(k), d(x),
+                                                  stats_only=True)
+        assert none is None and torch.equal(out2, out)
+        gq, gk, gx = graph_ext.gat_backward(d(indptr), d(indices), d(q), d(k), d(x), None, d(gy),
+                                            out=out2, stats=stats)
+        assert_close(gq, want_gq, atol=atol, what="grad_q (stats) " + what)
+        assert_close(gk, want_gk, atol=atol, what="grad_k (stats) " + what)
+        assert_close(gx, want_gx, atol=atol, what="grad_x (stats) " + what)
     return out
 
 
@@ -101,7 +112,8 @@ def test_gat_without_attn_buffer(dev):
     ip, ix, qd, kd, xd = d(indptr), d(indices), d(q), d(k), d(x)
     out = torch.empty(100, 4, 16, device=dev)
     ws = _lib.workspace(256, dev)
-    rc = _lib.lib().yitu_gat_forward(_lib.ptr(out), _lib.ptr(None), _lib.ptr(ip), _lib.ptr(ix),
+    rc = _lib.lib().yitu_gat_forward(_lib.ptr(out), _lib.ptr(None), _lib.ptr(None), _lib.ptr(ip),
+                                     _lib.ptr(ix),
                                      _lib.ptr(qd), _lib.ptr(kd), _lib.ptr(xd), _lib.c_i64(100),
                                      _lib.c_i64(100), _lib.c_i64(ix.numel()), _lib.c_i64(4),
                                      _lib.c_i64(16), _lib.c_i64(_lib.max_degree(ip)), _lib.ptr(None),

@@ -32,6 +32,7 @@ struct GatParams {
     int HP;              // heads rounded up to a power of two (<= 64)
     float *item_stats;   // [plan item id][H][2]: (max, sum) of the item's logits
     float *row_stats;    // [n_dst][H][2]: (max, 1/sum) of the planned rows
+    float *stats_out;    // optional output, same layout, for every row (then row_stats == stats_out)
 };
 
 // (max, sum) over the lanes that share lane % hp, hp a runtime power of two
@@ -166,6 +167,10 @@ __global__ __launch_bounds__(kBlock) void gat_rows_kernel(GatParams p) {
             a = ms_wave_rt(a, p.HP);
             m = a.m;
             inv = 1.0f / a.s;
+        }
+        if (p.stats_out && lane < p.HP && hl < H) {
+            p.stats_out[((size_t)row * H + hl) * 2] = m;
+            p.stats_out[((size_t)row * H + hl) * 2 + 1] = inv;
         }
         for (int c0 = 0; c0 < L; c0 += G * VEC * KT) {
             const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
@@ -722,7 +727,11 @@ struct GatSrcParams {
     // FULL: the forward output is at hand, so the softmax row sum S[r,h] = sum_e a d_attn
     // = <grad_out[r,h,:], out[r,h,:]> is known before the pass and the whole
     // softmax + LeakyReLU backward happens per edge, here
-    const float2 *row_sq;  // [n_dst, H]: (S, query) side by side, one line per destination
+    // [n_dst, H]: (S, query, softmax max, 1 / softmax sum) side by side: everything an edge
+    // needs from its destination, in one line (max and 1 / sum only with `recompute`)
+    const float4 *row_sq;
+    const float *stats;  // forward's row statistics [n_dst, H, 2] = (max, 1 / sum), or null
+    int recompute;       // attn is not read: a = exp(LeakyReLU(query + key) - max) / sum
     const float *key;      // [n_src, H]
     float *grad_k;         // [n_src, H]
     float *partial_k;      // [plan item id, H] partial grad_k of multi-item sources
@@ -737,10 +746,11 @@ struct GatSrcParams {
 // (S[r,h], query[r,h]) with S[r,h] = <grad_out[r,h,:], out[r,h,:]>, kRowsPerWave rows
 // per wave. The pair is what an edge needs from its destination.
 template <int LPH, int KT>
-__global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict__ row_sq,
+__global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float4 *__restrict__ row_sq,
                                                              const float *__restrict__ grad_out,
                                                              const float *__restrict__ out,
                                                              const float *__restrict__ query,
+                                                             const float *__restrict__ stats,
                                                              int n_rows, int g_ld, int head_mean,
                                                              float g_scale) {
     constexpr int HPT = kWave / LPH, H = HPT * KT, L = 256 * KT, U = KT == 1 ? 4 : 2;
@@ -769,8 +779,11 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float2 *__restrict_
 #pragma unroll
                 for (int o = LPH >> 1; o >= 1; o >>= 1) s += __shfl_xor(s, o, kWave);
                 const int head = t * HPT + lane / LPH;
-                if (lane % LPH == 0 && r < n_rows)
-                    row_sq[(size_t)r * H + head] = make_float2(s, query[(size_t)r * H + head]);
+                if (lane % LPH == 0 && r < n_rows) {
+                    const size_t at = (size_t)r * H + head;
+                    row_sq[at] = make_float4(s, query[at], stats ? stats[at * 2] : 0.0f,
+                                             stats ? stats[at * 2 + 1] : 0.0f);
+                }
             }
         }
     }
@@ -803,11 +816,14 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
 #pragma unroll
         for (int t = 0; t < KT; t++) {
             const int head = t * NS + h;
-            ea[j][t] = p.sp.values[(size_t)vr * H + head];
             if constexpr (FULL) {
-                const float2 sq = p.row_sq[(size_t)r * H + head];
+                const float4 sq = p.row_sq[(size_t)r * H + head];
                 eS[j][t] = sq.x;
                 eq[j][t] = sq.y;
+                ea[j][t] = p.recompute ? expf(leaky(sq.y + kc[t]) - sq.z) * sq.w
+                                       : p.sp.values[(size_t)vr * H + head];
+            } else {
+                ea[j][t] = p.sp.values[(size_t)vr * H + head];
             }
         }
     }
@@ -1025,19 +1041,36 @@ __device__ __forceinline__ void slot_window(SlotRow<LPH> &row, const GatSrcParam
                 const int r = __shfl(win.col, src, kWave);
                 vr[u] = __shfl(win.vrow, src, kWave);
                 RowLoad<4, float>::ld(g + (size_t)r * F + sub * 4, v[u]);
-                if constexpr (H == 8) {  // two 16-byte halves
-                    float lo[4], hi[4];
-                    RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8, lo);
-                    RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8 + 4, hi);
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        a[u][i] = lo[i];
-                        a[u][4 + i] = hi[i];
+                sq[u] = make_float2(0.0f, 0.0f);
+                if (p.recompute) {
+                    // no read of attn: lane sub < H makes the probability of (edge, head sub)
+                    // from the destination's line, the slot's lanes then share the H values
+                    float mine_a = 0.0f;
+                    if (sub < H) {
+                        const float4 t4 = p.row_sq[(size_t)r * H + sub];
+                        sq[u] = make_float2(t4.x, t4.y);
+                        mine_a = expf(leaky(t4.y + row.kc) - t4.z) * t4.w;
                     }
+#pragma unroll
+                    for (int h = 0; h < H; h++) a[u][h] = __shfl(mine_a, (lane - sub) + h, kWave);
                 } else {
-                    RowLoad<H, float>::ld(p.sp.values + (size_t)vr[u] * H, a[u]);
+                    if constexpr (H == 8) {  // two 16-byte halves
+                        float lo[4], hi[4];
+                        RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8, lo);
+                        RowLoad<4, float>::ld(p.sp.values + (size_t)vr[u] * 8 + 4, hi);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            a[u][i] = lo[i];
+                            a[u][4 + i] = hi[i];
+                        }
+                    } else {
+                        RowLoad<H, float>::ld(p.sp.values + (size_t)vr[u] * H, a[u]);
+                    }
+                    if (sub < H) {
+                        const float4 t4 = p.row_sq[(size_t)r * H + sub];
+                        sq[u] = make_float2(t4.x, t4.y);
+                    }
                 }
-                sq[u] = sub < H ? p.row_sq[(size_t)r * H + sub] : make_float2(0.0f, 0.0f);
             }
         }
 #pragma unroll
@@ -1163,8 +1196,8 @@ static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const flo
     if constexpr (FULL) {
         gat_row_dot_kernel<LPH, KT>
             <<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(
-                const_cast<float2 *>(p.row_sq), grad_out, out, query, n_dst, p.g_ld, p.head_mean,
-                p.g_scale);
+                const_cast<float4 *>(p.row_sq), grad_out, out, query, p.stats, n_dst, p.g_ld,
+                p.head_mean, p.g_scale);
         YITU_LAUNCH_CHECK();
     }
     const int row_grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave);
@@ -1246,7 +1279,7 @@ static int gat_src_launch(const GatSrcParams &p, bool has_items, const float *gr
 // workspace beyond the plan: item statistics, row statistics, partial rows
 static size_t gat_own_bytes(int64_t n_dst, int64_t nnz, int64_t H, int64_t L) {
     return align_up(sizeof(float) * 2 * (size_t)(plan_max_items(nnz) * H), 256) +
-           align_up(sizeof(float) * 2 * (size_t)(n_dst * H), 256) +
+           align_up(sizeof(float) * 4 * (size_t)(n_dst * H), 256) +
            align_up(sizeof(float) * (size_t)(plan_max_items(nnz) * L), 256);
 }
 
@@ -1396,7 +1429,7 @@ YITU_API size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_h
     return b + 256;
 }
 
-YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
+YITU_API int yitu_gat_forward(float *out, float *attn, float *row_stats, const int32_t *indptr,
                               const int32_t *indices, const float *query, const float *key,
                               const float *features, int64_t n_dst, int64_t n_src, int64_t nnz,
                               int64_t n_heads, int64_t n_features, int64_t max_degree,
@@ -1416,6 +1449,7 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
     if (!fused_ok) {
         // shapes outside the fused kernel's vector layout: the two-op composition
         YITU_REQUIRE(attn, "this shape needs the attn buffer (unfused path)");
+        YITU_REQUIRE(!row_stats, "row statistics are produced by the fused kernels only");
         int rc = yitu_sddmm_forward(attn, indptr, indices, query, key, n_dst, n_src, nnz, n_heads,
                                     1, max_degree, plan, workspace, workspace_bytes, stream_);
         if (rc) return rc;
@@ -1438,6 +1472,7 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
     p.query = query;
     p.key = key;
     p.attn = attn;
+    p.stats_out = row_stats;
     p.HP = 1;
     while (p.HP < p.sp.H) p.HP <<= 1;
     bool has_items = false;
@@ -1452,8 +1487,9 @@ YITU_API int yitu_gat_forward(float *out, float *attn, const int32_t *indptr,
         char *w = static_cast<char *>(rest);
         p.item_stats = reinterpret_cast<float *>(w);
         w += align_up(sizeof(float) * 2 * (size_t)(plan_max_items(nnz) * n_heads), 256);
-        p.row_stats = reinterpret_cast<float *>(w);
-        w += align_up(sizeof(float) * 2 * (size_t)(n_dst * n_heads), 256);
+        // the planned rows' statistics go straight to the caller's buffer when there is one
+        p.row_stats = row_stats ? row_stats : reinterpret_cast<float *>(w);
+        w += align_up(sizeof(float) * 4 * (size_t)(n_dst * n_heads), 256);
         p.sp.partial = reinterpret_cast<float *>(w);
     }
     const int lanes = (int)(L / 4);
@@ -1468,13 +1504,15 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                                float *grad_attn_scratch, float *grad_edge_scratch,
                                const int32_t *indptr, const int32_t *indices, const float *query,
                                const float *key, const float *features, const float *attn,
-                               const float *out, const float *grad_out, const int32_t *t_indptr,
+                               const float *row_stats, const float *out, const float *grad_out,
+                               const int32_t *t_indptr,
                                const int32_t *t_rows, const int32_t *t_perm, int64_t n_dst,
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
                                int64_t max_degree, int64_t max_degree_t, const void *plan,
                                const void *plan_t, int grad_out_is_head_mean, void *workspace,
                                size_t workspace_bytes, void *stream_) {
     YITU_REQUIRE(grad_query && grad_key && grad_features, "null output");
+    YITU_REQUIRE(nnz == 0 || attn || row_stats, "the backward needs attn or the row statistics");
     YITU_REQUIRE(nnz == 0 || (grad_attn_scratch && grad_edge_scratch),
                  "gat_backward needs two [nnz, H] scratch buffers");
     YITU_REQUIRE(t_indptr && (nnz == 0 || (t_rows && t_perm)),
@@ -1491,6 +1529,8 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                             n_src <= (1 << 24) && aligned16(features) && aligned16(grad_out) &&
                             aligned16(grad_features);
     YITU_REQUIRE(!grad_out_is_head_mean || aligned16(attn), "attn must be 16-byte aligned");
+    YITU_REQUIRE(nnz == 0 || attn || (one_gather && out && aligned16(out)),
+                 "without attn the backward needs a one-pass shape and the forward output");
     YITU_REQUIRE(!grad_out_is_head_mean || one_gather,
                  "a head-mean gradient is taken by the one-pass shapes only (rows of 256, 512 or "
                  "1024 floats, head width 32..256 a power of two, forward output given for the "
@@ -1528,7 +1568,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         const size_t part_k = has_items && full
                                   ? align_up(sizeof(float) * (size_t)p.sp.plan.max_items *
                                                  (size_t)n_heads, 256) : 0;
-        const size_t dots = full ? sizeof(float2) * (size_t)(n_dst * n_heads) : 0;
+        const size_t dots = full ? sizeof(float4) * (size_t)(n_dst * n_heads) : 0;
         YITU_REQUIRE((part + part_k + dots == 0) || (rest && rest_bytes >= part + part_k + dots),
                      "workspace too small: need %zu more bytes", part + part_k + dots);
         char *w = static_cast<char *>(rest);
@@ -1546,7 +1586,9 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         // also finishes the per-edge logit gradient (left in grad_attn_scratch, CSR
         // order) and grad_key; grad_query is its sum over each destination row.
         p.partial_k = reinterpret_cast<float *>(w + part);
-        p.row_sq = reinterpret_cast<float2 *>(w + part + part_k);
+        p.row_sq = reinterpret_cast<float4 *>(w + part + part_k);
+        p.stats = row_stats;
+        p.recompute = row_stats != nullptr;
         p.key = key;
         p.grad_k = grad_key;
         rc = gat_src_launch<true>(p, has_items, grad_out, out, query, (int)n_dst, stream);

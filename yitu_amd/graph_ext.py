@@ -382,9 +382,12 @@ def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32, out=None):
 # --------------------------------------------------------------------------- #
 # fused GAT attention (extension: the composition sddmm_forward -> spmm_forward)
 # --------------------------------------------------------------------------- #
-def gat_forward(indptr, indices, query, key, features):
+def gat_forward(indptr, indices, query, key, features, stats_only=False):
     """Returns [out [Nd,H,F], attn [E,H]] = the reference's two-op GAT lowering
-    (sddmm_forward then spmm_forward, n_bid = 1) in one pass per destination row."""
+    (sddmm_forward then spmm_forward, n_bid = 1) in one pass per destination row.
+    ``stats_only``: returns [out, None, stats] instead, stats [Nd,H,2] = each row's
+    softmax (max, 1 / sum): all that ``gat_backward`` needs of the attention for the
+    one-pass shapes (``gat_one_pass_shape``); the probabilities are then never stored."""
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
     _check(query, torch.float32, "query", 2)
@@ -396,8 +399,11 @@ def gat_forward(indptr, indices, query, key, features):
     nnz = indices.numel()
     if query.shape != (n_dst, h) or key.shape != (n_src, h):
         raise RuntimeError("query must be [n_dst, H] and key [n_src, H]")
+    if stats_only and not gat_one_pass_shape(h, f):
+        raise RuntimeError("stats_only needs a one-pass shape (see gat_one_pass_shape)")
     out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
-    attn = torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    attn = None if stats_only else torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    stats = torch.empty((n_dst, h, 2), dtype=torch.float32, device=dev) if stats_only else None
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = 0
@@ -406,12 +412,12 @@ def gat_forward(indptr, indices, query, key, features):
                                                     c_int(1))
     ws = _lib.workspace(need, dev)
     with torch.cuda.device(dev):
-        rc = _lib.lib().yitu_gat_forward(ptr(out), ptr(attn), ptr(indptr), ptr(indices), ptr(query),
-                                         ptr(key), ptr(features), c_i64(n_dst), c_i64(n_src),
-                                         c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan),
-                                         ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+        rc = _lib.lib().yitu_gat_forward(ptr(out), ptr(attn), ptr(stats), ptr(indptr), ptr(indices),
+                                         ptr(query), ptr(key), ptr(features), c_i64(n_dst),
+                                         c_i64(n_src), c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg),
+                                         ptr(plan), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_gat_forward")
-    return [out, attn]
+    return [out, None, stats] if stats_only else [out, attn]
 
 
 def gat_one_pass_shape(n_heads, n_features, with_out=True):
@@ -424,16 +430,23 @@ def gat_one_pass_shape(n_heads, n_features, with_out=True):
 
 
 def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None,
-                 head_mean=False):
+                 head_mean=False, stats=None):
     """Returns [grad_query, grad_key, grad_features] of gat_forward's ``out``.
     Passing the forward output ``out`` [n_dst, H, F] lets the softmax backward use
     sum_e a d_attn = <grad_out[row], out[row]> and finish in the same pass over
     the edges that computes grad_features (rows of 256, 512, 1024 floats); without
     it the attention gradient takes passes of its own.
     ``head_mean``: ``grad_out`` is [n_dst, F], the gradient of ``out.mean(dim=1)``
-    (the layer's result, model.py:106); the pass then gathers F floats per edge."""
-    _check(attn, torch.float32, "attn", 2)
-    dev = _lib.require_device(indptr, indices, query, key, features, attn, grad_out)
+    (the layer's result, model.py:106); the pass then gathers F floats per edge.
+    ``stats``: the row statistics of ``gat_forward(stats_only=True)``; ``attn`` may then
+    be None (needs ``out`` and a one-pass shape)."""
+    if attn is not None:
+        _check(attn, torch.float32, "attn", 2)
+    elif stats is None or out is None:
+        raise RuntimeError("without attn the backward needs stats and out")
+    if stats is not None:
+        _check(stats, torch.float32, "stats", 3)
+    dev = _lib.require_device(indptr, indices, query, key, features, grad_out)
     n_dst = indptr.numel() - 1
     n_src, h, f = features.shape
     nnz = indices.numel()
@@ -455,8 +468,8 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None
     grad_q = torch.empty_like(query)
     grad_k = torch.empty_like(key)
     grad_x = torch.empty_like(features)
-    s1 = torch.empty_like(attn)
-    s2 = torch.empty_like(attn)
+    s1 = torch.empty((nnz, h), dtype=torch.float32, device=dev)
+    s2 = s1 if attn is None else torch.empty_like(s1)  # unused by the one-pass path
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = 0
@@ -467,7 +480,7 @@ def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None
     with torch.cuda.device(dev):
         rc = _lib.lib().yitu_gat_backward(
             ptr(grad_q), ptr(grad_k), ptr(grad_x), ptr(s1), ptr(s2), ptr(indptr), ptr(indices),
-            ptr(query), ptr(key), ptr(features), ptr(attn), ptr(out), ptr(grad_out),
+            ptr(query), ptr(key), ptr(features), ptr(attn), ptr(stats), ptr(out), ptr(grad_out),
             ptr(tr.t_indptr), ptr(tr.t_rows), ptr(tr.t_perm), c_i64(n_dst), c_i64(n_src),
             c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), c_i64(tr.max_degree_t), ptr(plan),
             ptr(tr.plan_t), c_int(int(head_mean)), ptr(ws), c_size(ws.numel()), stream_ptr(dev))

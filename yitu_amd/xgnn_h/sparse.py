@@ -117,19 +117,24 @@ class FusedGATFunction(autograd.Function):
     @staticmethod
     def forward(ctx, adj_sparse, query, key, x, head_mean):
         indptr, indices = adj_sparse
-        out, attn = graph_ext.gat_forward(indptr, indices, query, key, x)
+        # one-pass shapes: keep each row's softmax statistics instead of the probabilities
+        ctx.stats_only = graph_ext.gat_one_pass_shape(x.size(1), x.size(2)) and \
+            indices.numel() > 0
+        out, attn, *stats = graph_ext.gat_forward(indptr, indices, query, key, x,
+                                                  stats_only=ctx.stats_only)
         ctx.adj_sparse = adj_sparse
         ctx.head_mean = head_mean
-        ctx.save_for_backward(query, key, x, attn, out)
+        ctx.save_for_backward(query, key, x, stats[0] if ctx.stats_only else attn, out)
         return out.mean(dim=1) if head_mean else out
 
     @staticmethod
     def backward(ctx, grad_out):
         indptr, indices = ctx.adj_sparse
-        query, key, x, attn, out = ctx.saved_tensors
+        query, key, x, kept, out = ctx.saved_tensors
+        attn, stats = (None, kept) if ctx.stats_only else (kept, None)
         grad_q, grad_k, grad_x = graph_ext.gat_backward(indptr, indices, query, key, x, attn,
                                                         grad_out.contiguous(), out=out,
-                                                        head_mean=ctx.head_mean)
+                                                        head_mean=ctx.head_mean, stats=stats)
         return None, grad_q, grad_k, grad_x, None
 
 
@@ -156,9 +161,12 @@ class GATHeadsFunction(autograd.Function):
         else:
             query, _ = graph_ext.head_dot(x_dst, a_dst)
             key, _ = graph_ext.head_dot(x_src, a_src)
-        out, attn = graph_ext.gat_forward(indptr, indices, query, key, x_src)
+        ctx.stats_only = graph_ext.gat_one_pass_shape(x_src.size(1), x_src.size(2)) and \
+            indices.numel() > 0
+        out, attn, *stats = graph_ext.gat_forward(indptr, indices, query, key, x_src,
+                                                  stats_only=ctx.stats_only)
         ctx.adj_sparse, ctx.head_mean, ctx.shared = adj_sparse, head_mean, x_dst is None
-        saved = (x_src, a_src, a_dst, query, key, attn, out)
+        saved = (x_src, a_src, a_dst, query, key, stats[0] if ctx.stats_only else attn, out)
         ctx.save_for_backward(*(saved if x_dst is None else saved + (x_dst,)))
         return out.mean(dim=1) if head_mean else out
 
@@ -166,10 +174,11 @@ class GATHeadsFunction(autograd.Function):
     @once_differentiable
     def backward(ctx, grad_out):
         indptr, indices = ctx.adj_sparse
-        x_src, a_src, a_dst, query, key, attn, out = ctx.saved_tensors[:7]
+        x_src, a_src, a_dst, query, key, kept, out = ctx.saved_tensors[:7]
+        attn, stats = (None, kept) if ctx.stats_only else (kept, None)
         grad_q, grad_k, grad_x = graph_ext.gat_backward(
             indptr, indices, query, key, x_src, attn, grad_out.contiguous(), out=out,
-            head_mean=ctx.head_mean)
+            head_mean=ctx.head_mean, stats=stats)
         if ctx.shared:
             grad_x, g_dst, g_src = graph_ext.head_dot_backward(x_src, a_dst, a_src, grad_q, grad_k,
                                                                grad_x=grad_x)
