@@ -253,6 +253,27 @@ def run_gat(args, dev):
 
     layer_ms = _event_ms(layer_step, args.steps, args.warmup)
     ref_layer_ms = _event_ms(ref_layer_step, args.steps, args.warmup)
+    # model level: the reference's 2-layer GATModel written against mp.Graph, captured and
+    # lowered (fused attention, bundled projections), against the reference's own lowering
+    # (sddmm + spmm, separate Linears) executed on the same kernels
+    from yitu_amd import xgnn_h
+    from yitu_amd.xgnn_h import models as xmodels, mp as xmp
+    model = xmodels.GATModel(h * f, f, f, n_heads=h).to(dev)
+    m_kwargs = {"graph": xmp.Graph(blk), "x": x.reshape(n, h * f)}
+    captured = xgnn_h.Module2IR().transform(model, m_kwargs)
+    executor = xgnn_h.Executor()
+    executor.train()
+    g_model = torch.randn(n, f, generator=g, device=dev)
+
+    def model_step(dataflow):
+        def run():
+            executor.run(dataflow, m_kwargs).backward(g_model)
+            model.zero_grad(set_to_none=True)
+        return _event_ms(run, args.steps, args.warmup)
+
+    model_ms = model_step(xgnn_h.Optimizer().lower(captured, m_kwargs))
+    model_plain_ms = model_step(
+        xgnn_h.Optimizer(fuse_gat=False, bundle_gemm=False).lower(captured, m_kwargs))
     alg_sd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h
     alg_fwd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h + 8 * n * h * f
     alg_bwd = (2 * 4 * n * h * f + 4 * nnz * h + 8 * nnz + 8 * (n + 1) + 4 * nnz
@@ -267,6 +288,8 @@ def run_gat(args, dev):
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
         "layer_fwd_bwd_ms": layer_ms,
         "reference_gatlayer_fwd_bwd_ms": ref_layer_ms,
+        "gat_model_2_layers": {"captured_and_lowered_fwd_bwd_ms": model_ms,
+                               "reference_lowering_only_fwd_bwd_ms": model_plain_ms},
         "sddmm": {"fwd_ms": sd_fwd_ms, "bwd_ms": sd_bwd_ms,
                   "edges_per_s_fwd_bwd": nnz / ((sd_fwd_ms + sd_bwd_ms) * 1e-3),
                   "fwd_algorithmic_bytes": alg_sd,
@@ -661,7 +684,8 @@ def main():
             args.no_cpu = True
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
                                                 "roofline", "fwd_ms", "bwd_ms", "layer_fwd_bwd_ms",
-                                                "reference_gatlayer_fwd_bwd_ms", "sddmm")
+                                                "reference_gatlayer_fwd_bwd_ms", "gat_model_2_layers",
+                                                "sddmm")
                               if k in r}
             res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
                             "c2_gat_f32": slim(run_gat(args, dev)),
