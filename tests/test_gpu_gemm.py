@@ -164,3 +164,24 @@ def test_column_sum(dev, m, n):
     got = graph_ext.column_sum(x.to(dev))
     assert_close(got, x.double().sum(0).float(), atol=1e-4 * m ** 0.5)
     assert torch.equal(got, graph_ext.column_sum(x.to(dev)))
+
+
+@pytest.mark.parametrize("n,k,m,bias", [(1000, 256, 256, True), (77, 24, 64, True), (513, 100, 172, False),
+                                        (300, 64, 4, True)])
+def test_bundle_linear_matches_torch(dev, n, k, m, bias):
+    """bundle.linear (MFMA GEMM or skinny product, fixed-order bias gradient) == F.linear,
+    outputs and all three gradients."""
+    torch.manual_seed(n + k + m)
+    lin = nn.Linear(k, m, bias=bias).to(dev)
+    x = torch.randn(n, k, device=dev, requires_grad=True)
+    w = torch.randn(n, m, device=dev)
+    y = bundle.linear(x, lin.weight, lin.bias)
+    (y * w).sum().backward()
+    got = [y.detach(), x.grad.clone(), lin.weight.grad.clone()] + ([lin.bias.grad.clone()] if bias else [])
+    x.grad = None
+    lin.zero_grad()
+    y2 = lin(x)
+    (y2 * w).sum().backward()
+    want = [y2.detach(), x.grad, lin.weight.grad] + ([lin.bias.grad] if bias else [])
+    for a, b in zip(got, want):
+        assert_close(a, b, rtol=1e-4, atol=2e-4 * (n ** 0.5 if a.dim() < 2 or a.shape == lin.weight.shape else 1))

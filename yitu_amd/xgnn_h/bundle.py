@@ -69,3 +69,39 @@ def linear_pair(x, linear_a, linear_b):
             linear_a.weight.stride() == linear_b.weight.stride():
         return bundled_linear(x, linear_a.weight, linear_b.weight, linear_a.bias, linear_b.bias)
     return linear_a(x), linear_b(x)
+
+
+class MfmaLinearFunction(autograd.Function):
+    """``F.linear(x, weight, bias)`` on the library's fp32 MFMA GEMM: ``x . weight^T`` and both
+    gradient products at the same rate whatever the operand layout, the bias gradient as
+    a fixed-order column sum."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        y = graph_ext.sgemm(x, weight, trans_b=True)
+        return y if bias is None else y.add_(bias)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_y):
+        x, weight = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_x = graph_ext.sgemm(grad_y, weight) if ctx.needs_input_grad[0] else None
+        grad_w = graph_ext.sgemm(grad_y, x, trans_a=True) if ctx.needs_input_grad[1] else None
+        grad_b = graph_ext.column_sum(grad_y) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return grad_x, grad_w, grad_b
+
+
+def linear(x, weight, bias=None):
+    """``F.linear`` for 2-D fp32 device tensors on the library's kernels: the skinny product
+    for a handful of outputs, the MFMA GEMM otherwise; anything else goes to torch."""
+    import torch
+    from torch.nn import functional as F
+    if x.dim() == 2 and x.is_cuda and x.dtype == torch.float32 and weight.dtype == torch.float32 \
+            and x.size(0) > 0:
+        if graph_ext.skinny_linear_shape(weight.size(1), weight.size(0)):
+            return SkinnyLinearFunction.apply(x.contiguous(), weight.contiguous(), bias)
+        return MfmaLinearFunction.apply(x.contiguous(), weight.contiguous(), bias)
+    return F.linear(x, weight, bias)

@@ -52,7 +52,7 @@ class Executor:
         if op == "call":
             return node.attrs["fn"](*_fill(node.attrs["args"], v), **_fill(node.attrs["kwargs"], v))
         if op == "linear":
-            return F.linear(v["x"], node.attrs["weight"], node.attrs["bias"])
+            return bundle.linear(v["x"], node.attrs["weight"], node.attrs["bias"])
         if op == "dropout":
             if self._is_training is None:
                 raise RuntimeError("call train() or eval() on the executor first")

@@ -30,7 +30,7 @@ class GCNLayer(nn.Module):
         if isinstance(x, (list, tuple)):
             assert len(x) == 2
             x = x[0]
-        h = self.fc(x)
+        h = bundle.linear(x, self.fc.weight, self.fc.bias)
         h = h.view(size=[-1, 1, h.size(-1)])
         h = torch.squeeze(sparse.gspmm(blk, None, h), dim=1)
         return torch.multiply(norm, h)
@@ -55,10 +55,10 @@ class GATLayer(nn.Module):
     def forward(self, blk: block.Block, x):
         if isinstance(x, (list, tuple)):
             assert len(x) == 2
-            h_src = self.linear_v(x[0])
-            h_dst = self.linear_v(x[1])
+            h_src = bundle.linear(x[0], self.linear_v.weight, self.linear_v.bias)
+            h_dst = bundle.linear(x[1], self.linear_v.weight, self.linear_v.bias)
         elif isinstance(x, torch.Tensor):
-            h_src = h_dst = self.linear_v(x)
+            h_src = h_dst = bundle.linear(x, self.linear_v.weight, self.linear_v.bias)
         else:
             raise TypeError
         if h_dst is h_src:  # one read of h for both projections
@@ -93,7 +93,8 @@ class GATHeadLayer(nn.Module):
         self.a_dst = nn.Parameter(torch.randn(n_heads, out_features) * 0.1)
 
     def _heads(self, x):
-        h = x if self.linear_v is None else self.linear_v(x)
+        h = x if self.linear_v is None else \
+            bundle.linear(x, self.linear_v.weight, self.linear_v.bias)
         return h.view(size=[-1, self.n_heads, self.n_features])
 
     def forward(self, blk: block.Block, x):
