@@ -103,8 +103,10 @@ def test_lowering_gat_patterns_and_options():
     plain = cases.ops_of(xgnn_h.Optimizer(fuse_gat=False, bundle_gemm=False).lower(dataflow, kwargs))
     assert plain["sddmm"] == 2 and plain["spmm"] == 2 and plain["gat"] == 0
     assert plain["bundle"] == 0 and plain["linear"] == 6
-    # lowering rebuilds the graph: the captured dataflow is unchanged
+    # lowering rebuilds the graph: the captured dataflow is unchanged, attributes included
     assert cases.ops_of(dataflow) == before
+    assert all(set(n.attrs) <= {"fn", "args", "kwargs", "weight", "bias", "p", "width", "dtype"}
+               for n in ir.walk(dataflow))
 
 
 def test_lowering_leaves_other_slopes_and_shared_attention_alone():

@@ -1,4 +1,11 @@
-// Per-head projections of a GAT layer with attention vectors:
+// Row-wise dense helpers around the sparse ops, three families in this file:
+//   1. per-head projections of a GAT layer (yitu_head_dot*),
+//   2. Linear layers with a handful of outputs (yitu_skinny_linear*),
+//   3. column sums = bias gradients, replayable from a HIP graph (yitu_column_sum).
+// They share the row layout (tiles of 256 floats over the wave, 4 per lane) and the
+// fixed-order two-stage sums.
+//
+// 1. Per-head projections of a GAT layer with attention vectors:
 //   q[n,h] = <a_dst[h,:], x[n,h,:]>,   k[n,h] = <a_src[h,:], x[n,h,:]>
 // and their backward. The reference's example layer uses dense H*F -> H Linears
 // for the two (test/common/model.py:70-71); the per-head vectors a_src / a_dst

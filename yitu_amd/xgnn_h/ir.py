@@ -107,10 +107,12 @@ def use_counts(dataflow: Dataflow) -> Dict[int, int]:
     return uses
 
 
-def rewrite(dataflow: Dataflow, rule: Callable[[Node], Node]) -> Dataflow:
-    """Rebuilds the graph bottom-up. ``rule`` receives each node with its inputs
-    already rewritten and returns the node to use in its place (possibly the same
-    one). Shared sub-graphs stay shared."""
+def rewrite(dataflow: Dataflow, rule: Callable[[Node, Node], Node]) -> Dataflow:
+    """Rebuilds the graph bottom-up. ``rule(node, original)`` receives each node with
+    its inputs already rewritten, and the node of the input graph it stands for (for
+    facts gathered beforehand, such as use counts); it returns the node to use in its
+    place (possibly the same one). Shared sub-graphs stay shared; the input graph is
+    not modified."""
     done: Dict[int, Node] = {}
     for node in walk(dataflow):
         new_inputs = {k: done[id(v)] for k, v in node.inputs.items()}
@@ -118,7 +120,7 @@ def rewrite(dataflow: Dataflow, rule: Callable[[Node], Node]) -> Dataflow:
             node_in = node.with_inputs(new_inputs)
         else:
             node_in = node
-        done[id(node)] = rule(node_in)
+        done[id(node)] = rule(node_in, node)
     if isinstance(dataflow, Node):
         return done[id(dataflow)]
     return {k: done[id(v)] for k, v in dataflow.items()}

@@ -36,7 +36,7 @@ class Optimizer:
 
     # -- message passing -> sddmm / spmm ------------------------------------
     @staticmethod
-    def _lower_node(node: ir.Node) -> ir.Node:
+    def _lower_node(node: ir.Node, _original: ir.Node = None) -> ir.Node:
         if node.op == "edge" and node.attrs["fn"] == "edge_softmax":
             logits = _leaky_input(node.inputs["e"])
             if logits is not None and logits.op == "edge" and logits.attrs["fn"] == "u_add_v" \
@@ -58,43 +58,40 @@ class Optimizer:
     @staticmethod
     def _fuse_gat(dataflow: ir.Dataflow) -> ir.Dataflow:
         uses = ir.use_counts(dataflow)
+        attention_of = {}  # id(rewritten sddmm) -> readers of the sddmm it stands for
 
-        def rule(node: ir.Node) -> ir.Node:
+        def rule(node: ir.Node, original: ir.Node) -> ir.Node:
+            if node.op == "sddmm":
+                attention_of[id(node)] = uses.get(id(original), 0)
             attn = node.inputs.get("e") if node.op == "spmm" else None
             if attn is None or attn.op != "sddmm" or attn.inputs["g"] is not node.inputs["g"]:
                 return node
             # the attention must have no other reader and one query block
-            if attn.attrs.get("uses", 0) != 1 or len(attn.inputs["q"].size) != 2:
+            if attention_of.get(id(attn)) != 1 or len(attn.inputs["q"].size) != 2:
                 return node
             return ir.Node("gat", {"g": node.inputs["g"], "q": attn.inputs["q"],
                                    "k": attn.inputs["k"], "x": node.inputs["x"]}, size=node.size)
 
-        # use counts refer to the nodes before rewriting: note them on the sddmm nodes
-        for node in ir.walk(dataflow):
-            if node.op == "sddmm":
-                node.attrs["uses"] = uses.get(id(node), 0)
         return Optimizer._fuse_head_mean(ir.rewrite(dataflow, rule))
 
     # -- mean(gat, dim=1) -> gat with the mean inside ------------------------
     @staticmethod
     def _fuse_head_mean(dataflow: ir.Dataflow) -> ir.Dataflow:
         uses = ir.use_counts(dataflow)
-        only_reader = {id(n) for n in ir.walk(dataflow) if n.op == "gat" and uses.get(id(n)) == 1}
+        sole_reader = set()  # ids of rewritten gat nodes whose original has one reader
 
-        def rule(node: ir.Node) -> ir.Node:
+        def rule(node: ir.Node, original: ir.Node) -> ir.Node:
+            if node.op == "gat" and uses.get(id(original)) == 1:
+                sole_reader.add(id(node))
             if node.op != "call" or node.fn_name() != "mean" or len(node.inputs) != 1:
                 return node
             (inner,) = node.inputs.values()
             kwargs = node.attrs["kwargs"]
-            if inner.op != "gat" or inner.attrs.get("origin") not in only_reader or \
-                    kwargs.get("dim") != 1 or set(kwargs) != {"dim"} or len(node.attrs["args"]) != 1:
+            if inner.op != "gat" or id(inner) not in sole_reader or kwargs.get("dim") != 1 or \
+                    set(kwargs) != {"dim"} or len(node.attrs["args"]) != 1:
                 return node
             return ir.Node("gat", inner.inputs, {"head_mean": True}, node.size)
 
-        # rewriting copies nodes whose inputs change: carry the identity along
-        for n in ir.walk(dataflow):
-            if n.op == "gat":
-                n.attrs["origin"] = id(n)
         return ir.rewrite(dataflow, rule)
 
     # -- linear_q(h), linear_k(h) -> one launch ------------------------------
@@ -102,7 +99,7 @@ class Optimizer:
     def _bundle(dataflow: ir.Dataflow) -> ir.Dataflow:
         bundles = {}
 
-        def rule(node: ir.Node) -> ir.Node:
+        def rule(node: ir.Node, _original: ir.Node) -> ir.Node:
             if node.op not in ("sddmm", "gat"):
                 return node
             q, k = node.inputs["q"], node.inputs["k"]
