@@ -123,7 +123,9 @@ def test_c2_backward_is_the_adjoint_of_forward(dev, c2):
     assert all(torch.equal(a, b) for a, b in zip(full, again))
     # probabilities never stored: row statistics from the forward, recomputed per edge
     out2, _, stats = graph_ext.gat_forward(rp, ci, q, k, x, stats_only=True)
-    assert torch.equal(out2, out)
+    assert float((out2 - out).abs().max()) < 1e-5 * max(float(out.abs().max()), 1.0)
+    again, _, _ = graph_ext.gat_forward(rp, ci, q, k, x, stats_only=True)
+    assert torch.equal(again, out2)  # fixed summation order
     lean = graph_ext.gat_backward(rp, ci, q, k, x, None, gy, out=out2, stats=stats)
     for got, want in zip(lean, full):
         assert float((got - want).abs().max()) < 1e-5 * max(float(want.abs().max()), 1.0)

@@ -48,7 +48,9 @@ def _run(dev, indptr, indices, n_dst, n_src, h, f, seed, atol=2e-4):
         # per edge in the backward
         out2, none, stats = graph_ext.gat_forward(d(indptr), d(indices), d(q), d(k), d(x),
                                                   stats_only=True)
-        assert none is None and torch.equal(out2, out)
+        assert none is None
+        # long rows are summed from unnormalised item sums here: another rounding, same bar
+        assert_close(out2, want_out, atol=atol, what="out (stats) " + what)
         gq, gk, gx = graph_ext.gat_backward(d(indptr), d(indices), d(q), d(k), d(x), None, d(gy),
                                             out=out2, stats=stats)
         assert_close(gq, want_gq, atol=atol, what="grad_q (stats) " + what)

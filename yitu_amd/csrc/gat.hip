@@ -327,6 +327,190 @@ __global__ __launch_bounds__(kBlock) void gat_item_apply_kernel(GatParams p) {
     }
 }
 
+// ---- planned rows without the probabilities as an output ------------------------
+// When no [nnz, H] probabilities are asked for, an item does not wait for its
+// row's statistics: it weighs its edges by exp(logit - the item's own max) and
+// leaves the sum unnormalised, next to its (max, sum). The reduction then scales
+// item c of a row by exp(max_c - max_row) / sum_row. That drops the separate pass
+// over the items' keys. Rows of one item are normalised and written at once.
+template <int VEC, int G, int KT>
+__global__ __launch_bounds__(kBlock) void gat_item_local_kernel(GatParams p) {
+    const int lane = lane_id();
+    const int sub = lane % G, slot = lane / G;
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int hl = lane & (p.HP - 1);
+    const int H = p.sp.H, L = p.sp.L;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        EdgeWindow win[kItemsPerWave];
+        int e_beg[kItemsPerWave], n_edges[kItemsPerWave], item_id[kItemsPerWave],
+            row_tag[kItemsPerWave];
+        float qv[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            e_beg[j] = __shfl(my_rec.x, j, kWave);
+            const int end = __shfl(my_rec.y, j, kWave);
+            item_id[j] = __shfl(my_rec.z, j, kWave);
+            row_tag[j] = __shfl(my_rec.w, j, kWave);
+            n_edges[j] = j < n_here ? end - e_beg[j] : 0;
+            qv[j] = 0.0f;
+            if (n_edges[j] > 0) {
+                load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
+                if (hl < H) qv[j] = p.query[(size_t)(row_tag[j] & 0x7fffffff) * H + hl];
+            }
+        }
+        MaxSum st[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            st[j] = ms_init();
+            if (n_edges[j] > 0)
+                st[j] = ms_wave_rt(gat_stats_window(p, win[j], 0, n_edges[j], qv[j]), p.HP);
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;
+            const bool single = row_tag[j] < 0;
+            const int row = row_tag[j] & 0x7fffffff;
+            if (lane < p.HP && lane < H) {
+                p.item_stats[((size_t)item_id[j] * H + lane) * 2] = st[j].m;
+                p.item_stats[((size_t)item_id[j] * H + lane) * 2 + 1] = st[j].s;
+            }
+            const float inv = single ? 1.0f / st[j].s : 1.0f;
+            float *dst = single ? p.sp.out + (size_t)row * L
+                                : p.sp.partial + (size_t)item_id[j] * L;
+            for (int c0 = 0; c0 < L; c0 += G * VEC * KT) {
+                const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+                float acc[KT][VEC];
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) acc[t][k] = 0.0f;
+                gat_apply_window<VEC, G, KT>(acc, p, tl, win[j], 0, n_edges[j], e_beg[j], qv[j],
+                                             st[j].m, inv, false);
+                fold_slots<VEC, G, KT>(acc);
+                if (slot == 0) {
+#pragma unroll
+                    for (int t = 0; t < KT; t++) {
+                        const int o = c0 + (t * G + sub) * VEC;
+                        if (o < L) store_row<VEC>(dst + o, acc[t]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// s += exp(max_c - m_row) * src[c * L] for c = first, first + step, ... < n, in
+// that order; st points at the first item's (max, sum) of this lane's head.
+__device__ __forceinline__ void sum_scaled_partials(float (&s)[4], const float *src,
+                                                    const float *st, int H, float m_row, int L,
+                                                    int first, int n, int step) {
+    int c = first;
+    for (; c + 3 * step < n; c += 4 * step) {
+        float v[4][4], w[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            RowLoad<4, float>::ld(src + (size_t)(c + u * step) * L, v[u]);
+            w[u] = st[(size_t)(c + u * step) * H * 2];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const float f = expf(w[u] - m_row);
+#pragma unroll
+            for (int i = 0; i < 4; i++) s[i] += f * v[u][i];
+        }
+    }
+    for (; c < n; c += step) {
+        float v[4];
+        RowLoad<4, float>::ld(src + (size_t)c * L, v);
+        const float f = expf(st[(size_t)c * H * 2] - m_row);
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[i] += f * v[i];
+    }
+}
+
+// Adds the unnormalised item sums of every planned row with more than one item
+// (after gat_row_combine_kernel), four columns per lane; the head width is a
+// multiple of four, so a lane's columns share a head. Work split and summation
+// order as in spmm_reduce_kernel.
+__global__ __launch_bounds__(kBlock) void gat_scaled_reduce_kernel(GatParams p) {
+    __shared__ float red[kBlock * 4];
+    if (p.sp.plan.counters->overflow) return;
+    const int n_hub = min(p.sp.plan.counters->n_rows, p.sp.plan.max_rows);
+    const int L = p.sp.L, H = p.sp.H, F = p.sp.F;
+    const int lanes_total = L / 4;
+    const int half = gridDim.x / 2;
+    if ((int)blockIdx.x < half) {
+        const int lane = lane_id();
+        int lanes = 1;
+        while (lanes < lanes_total && lanes < kWave) lanes <<= 1;
+        const int slots = kWave / lanes;
+        const int slot = lane / lanes, sub = lane % lanes;
+        const int stride = half * kWavesPerBlock;
+        for (int h = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; h < n_hub; h += stride) {
+            const int4 r = p.sp.plan.rows[h];
+            if (r.z <= 1 || r.z > kReduceWaveItems) continue;
+            for (int l0 = 0; l0 < lanes_total; l0 += lanes) {
+                const bool live = l0 + sub < lanes_total;
+                float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                float inv = 0.0f;
+                if (live) {
+                    const int head = (l0 + sub) * 4 / F;
+                    const float *rs = p.row_stats + ((size_t)r.x * H + head) * 2;
+                    inv = rs[1];
+                    sum_scaled_partials(s, p.sp.partial + (size_t)r.y * L + (size_t)(l0 + sub) * 4,
+                                        p.item_stats + ((size_t)r.y * H + head) * 2, H, rs[0], L,
+                                        slot, r.z, slots);
+                }
+                for (int o = kWave / 2; o >= lanes; o >>= 1)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) s[i] += __shfl_xor(s[i], o, kWave);
+                if (live && slot == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) s[i] *= inv;
+                    store_row<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + sub) * 4, s);
+                }
+            }
+        }
+        return;
+    }
+    for (int h = blockIdx.x - half; h < n_hub; h += gridDim.x - half) {
+        const int4 r = p.sp.plan.rows[h];
+        if (r.z <= kReduceWaveItems) continue;
+        for (int l0 = 0; l0 < lanes_total; l0 += kBlock) {
+            const int lanes = min(kBlock, lanes_total - l0);
+            const int groups = kBlock / lanes;
+            const int g = threadIdx.x / lanes, l = threadIdx.x % lanes;
+            float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float inv = 0.0f;
+            if (g < groups) {
+                const int head = (l0 + l) * 4 / F;
+                const float *rs = p.row_stats + ((size_t)r.x * H + head) * 2;
+                inv = rs[1];
+                sum_scaled_partials(s, p.sp.partial + (size_t)r.y * L + (size_t)(l0 + l) * 4,
+                                    p.item_stats + ((size_t)r.y * H + head) * 2, H, rs[0], L, g,
+                                    r.z, groups);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 4; i++) red[threadIdx.x * 4 + i] = s[i];
+            __syncthreads();
+            if (g == 0) {
+                for (int gg = 1; gg < groups; gg++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) s[i] += red[(gg * lanes + l) * 4 + i];
+#pragma unroll
+                for (int i = 0; i < 4; i++) s[i] *= inv;
+                store_row<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + l) * 4, s);
+            }
+        }
+    }
+}
+
 // ---- backward of the softmax + LeakyReLU ----------------------------------------
 // Given d_attn per edge and head, the three row sums
 //   S = sum a d_attn,  A1 = sum a d_attn s,  A2 = sum a s   (s = LeakyReLU slope)
@@ -623,7 +807,7 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
     const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
-    const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
+    const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
     EdgeWindow win;
     win.base = -1;
@@ -1291,17 +1475,26 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
     if (!has_items) return 0;
     const int item_grid = (int)std::min<int64_t>(
         ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+    const int combine_grid =
+        (int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15);
+    const int reduce_grid = (int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16);
+    if (!p.attn && p.sp.F % 4 == 0) {
+        gat_item_local_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        gat_row_combine_kernel<<<combine_grid, kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        gat_scaled_reduce_kernel<<<reduce_grid, kBlock, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        return 0;
+    }
     gat_item_stats_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    gat_row_combine_kernel<<<(int)std::min<int64_t>(
-                                 ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15),
-                             kBlock, 0, stream>>>(p);
+    gat_row_combine_kernel<<<combine_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     gat_item_apply_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     p.sp.alpha = 1.0f;
-    spmm_reduce_kernel<W_NONE, 4>
-        <<<(int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16), kBlock, 0, stream>>>(p.sp);
+    spmm_reduce_kernel<W_NONE, 4><<<reduce_grid, kBlock, 0, stream>>>(p.sp);
     YITU_LAUNCH_CHECK();
     return 0;
 }
