@@ -105,6 +105,35 @@ def cpu_baseline_spmm(rp, ci, deg, x, dy):
             "seconds": t}
 
 
+def cpu_library_cross_check(rp, ci, deg, x, with_scipy=False):
+    """One forward aggregation through general-purpose CPU libraries on the same
+    cores, beside the restatement's figure: torch's CSR product (all threads) and,
+    for small graphs, scipy's (one thread)."""
+    import warnings
+    rp_t, ci_t, deg_t, x_t = rp.cpu(), ci.cpu(), deg.cpu().float(), x.float().cpu()
+    n = rp_t.numel() - 1
+    rows = torch.repeat_interleave(torch.arange(n), (rp_t[1:] - rp_t[:-1]).long())
+    vals = deg_t[rows] * deg_t[ci_t.long()]
+    del rows
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        a = torch.sparse_csr_tensor(rp_t, ci_t, vals, size=(n, x_t.shape[0]))
+        torch.sparse.mm(a, x_t[:, :4].contiguous())  # warm-up on a narrow operand
+        t0 = time.perf_counter()
+        torch.sparse.mm(a, x_t)
+        res = {"torch_sparse_csr_mm_fwd_edges_per_s": ci_t.numel() / (time.perf_counter() - t0),
+               "torch_threads": torch.get_num_threads()}
+    if with_scipy:
+        import scipy.sparse as sp
+        m = sp.csr_matrix((vals.numpy(), ci_t.numpy(), rp_t.numpy()), shape=(n, x_t.shape[0]))
+        x_h = x_t.numpy()
+        m @ x_h
+        t0 = time.perf_counter()
+        m @ x_h
+        res["scipy_csr_matmul_fwd_edges_per_s"] = ci_t.numel() / (time.perf_counter() - t0)
+    return res
+
+
 def run_spmm(args, dev, bf16):
     from yitu_amd import _lib
     n, rp, ci, deg, info = build_c3(dev)
@@ -172,6 +201,7 @@ def run_spmm(args, dev, bf16):
     }
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_spmm(rp, ci, deg, x, dy)
+        res["cpu_baseline"]["library_cross_check"] = cpu_library_cross_check(rp, ci, deg, x)
     return res
 
 
@@ -354,7 +384,11 @@ def run_c1(args, dev):
 
     layer_ms = _event_ms(layer, max(args.steps, 50), args.warmup)
     agg_ms = _event_ms(agg_only, max(args.steps, 50), args.warmup)
+    cross = None
+    if getattr(args, "cpu_cross_check", not args.no_cpu):
+        cross = cpu_library_cross_check(rp, ci, deg, x, with_scipy=True)
     return {"value": nnz / (agg_ms * 1e-3), "unit": "edges/s", "ms_per_step": agg_ms, "dtype": "f32",
+            "cpu_library_cross_check": cross,
             "config": {"workload": "c1_gcn_f32", "graph": "Erdos-Renyi 10^4 nodes, 10^5 draws + self "
                        "loops", "n_edges": nnz, "feature_dim": dim,
                        "step": "aggregate(X) + aggregate(dY) (two launches)"},
@@ -681,6 +715,7 @@ def main():
         res["copy_calibration"] = calibration_copy(dev)
         if not args.no_extra:
             # the other single-GPU configurations ride along as extra fields
+            args.cpu_cross_check = not args.no_cpu  # the small first configuration keeps its own
             args.no_cpu = True
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
                                                 "roofline", "fwd_ms", "bwd_ms", "layer_fwd_bwd_ms",
