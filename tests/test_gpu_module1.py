@@ -205,3 +205,28 @@ def test_rejects_cpu_tensors_and_bad_dtypes(dev):
         K.SAG(x.to(dev), rp.long(), ci, deg, pp, p2n, PS, DW, WPB)
     with pytest.raises(RuntimeError):
         K.SAG(x.to(dev).t(), rp, ci, deg, pp, p2n, PS, DW, WPB)  # not contiguous
+
+
+@pytest.mark.parametrize("n", [30, 0])
+def test_graph_without_edges(dev, n):
+    """Rows without any edge, and no rows at all: zeros of the right shape."""
+    rp = torch.zeros(n + 1, dtype=torch.int32)
+    ci = torch.zeros(0, dtype=torch.int32, device=dev)
+    pp, p2n = K.build_part(PS, rp)
+    assert pp.numel() == 1 and p2n.numel() == 0
+    rp, pp, p2n = rp.to(dev), pp.to(dev), p2n.to(dev)
+    x = torch.randn(n, 32, device=dev)
+    w = torch.randn(32, 16, device=dev)
+    dy = torch.randn(n, 16, device=dev)
+    deg = torch.ones(n, device=dev)
+
+    def zeros(t, *shape):
+        return tuple(t.shape) == shape and not bool(t.any())
+
+    (out,) = K.forward(x, w, rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert zeros(out, n, 16)
+    dx, dw = K.backward(dy, x, w, rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert zeros(dx, n, 32) and zeros(dw, 32, 16)
+    out, agg = K.forward_gin(x, w, rp, ci, 0.5, pp, p2n, PS, DW, WPB)
+    assert zeros(out, n, 16) and zeros(agg, n, 32)
+    assert zeros(K.SAG(x, rp, ci, deg, pp, p2n, PS, DW, WPB), n, 32)

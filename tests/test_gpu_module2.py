@@ -326,3 +326,39 @@ def test_max_degree_cache_does_not_outlive_its_tensor(dev):
     if b.data_ptr() == addr:  # the allocator reused the block (the case that matters)
         assert _lib.max_degree(b) == 300
     assert _lib.max_degree(b) == 300
+
+
+# ---- degenerate graphs --------------------------------------------------------------
+
+@pytest.mark.parametrize("n_dst,n_src", [(50, 40), (0, 40), (50, 0), (0, 0)])
+def test_graph_without_edges(dev, n_dst, n_src):
+    """No edges, and no rows on either side: every op returns zeros of the right
+    shape (empty tensors have no address, so the library must not insist on one)."""
+    h, f = 4, 16
+    indptr = torch.zeros(n_dst + 1, dtype=torch.int32, device=dev)
+    indices = torch.zeros(0, dtype=torch.int32, device=dev)
+    g = torch.Generator().manual_seed(n_dst + n_src)
+    x = torch.randn(n_src, h, f, generator=g).to(dev)
+    q = torch.randn(n_dst, h, generator=g).to(dev)
+    k = torch.randn(n_src, h, generator=g).to(dev)
+    gy = torch.randn(n_dst, h, f, generator=g).to(dev)
+    none = torch.zeros(0, h, device=dev)
+
+    def zeros(t, *shape):
+        return tuple(t.shape) == shape and not bool(t.any())
+
+    assert zeros(graph_ext.spmm_forward(none, indptr, indices, x), n_dst, h, f)
+    ga, gx = graph_ext.spmm_backward(none, indptr, indices, x, gy)
+    assert zeros(ga, 0, h) and zeros(gx, n_src, h, f)
+    assert zeros(graph_ext.sddmm_forward(indptr, indices, q[None], k), 0, h)
+    gq, gk = graph_ext.sddmm_backward(indptr, indices, q[None], k, none, none)
+    assert zeros(gq, 1, n_dst, h) and zeros(gk, n_src, h)
+    out, attn = graph_ext.gat_forward(indptr, indices, q, k, x)
+    assert zeros(out, n_dst, h, f) and zeros(attn, 0, h)
+    gq, gk, gx = graph_ext.gat_backward(indptr, indices, q, k, x, attn, gy)
+    assert zeros(gq, n_dst, h) and zeros(gk, n_src, h) and zeros(gx, n_src, h, f)
+    # and through autograd
+    blk = xblock.Block([n_dst, n_src], [indptr, indices])
+    leaves = [t.clone().requires_grad_() for t in (q, k, x)]
+    sparse.fused_gat(blk, *leaves).sum().backward()
+    assert all(zeros(t.grad, *t.shape) for t in leaves)

@@ -1704,7 +1704,11 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                                int64_t max_degree, int64_t max_degree_t, const void *plan,
                                const void *plan_t, int grad_out_is_head_mean, void *workspace,
                                size_t workspace_bytes, void *stream_) {
-    YITU_REQUIRE(grad_query && grad_key && grad_features, "null output");
+    YITU_REQUIRE(n_dst >= 0 && n_src >= 0 && nnz >= 0 && n_heads >= 0 && n_features >= 0,
+                 "negative size");
+    YITU_REQUIRE((grad_query || n_dst * n_heads == 0) && (grad_key || n_src * n_heads == 0) &&
+                     (grad_features || n_src * n_heads * n_features == 0),
+                 "null output");
     YITU_REQUIRE(nnz == 0 || attn || row_stats, "the backward needs attn or the row statistics");
     YITU_REQUIRE(nnz == 0 || (grad_attn_scratch && grad_edge_scratch),
                  "gat_backward needs two [nnz, H] scratch buffers");

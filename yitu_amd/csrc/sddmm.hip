@@ -177,7 +177,7 @@ int sddmm_backward_run(float *grad_query, float *grad_key, float *grad_edge, con
     int rc = sddmm_check(indptr, indices, query, key, n_dst, n_src, nnz, n_heads, n_bid);
     if (rc) return rc;
     if (n_heads == 0) return 0;
-    YITU_REQUIRE(grad_query && grad_key, "null output");
+    YITU_REQUIRE((grad_query || n_dst == 0) && (grad_key || n_src == 0), "null output");
     const bool gather = t_indptr != nullptr;
     YITU_REQUIRE(!gather || (t_perm && grad_edge) || nnz == 0,
                  "the gather form needs t_perm and a grad_edge buffer");

@@ -219,6 +219,7 @@ int spmm_backward_run(float *grad_a, float *grad_x, const float *values, const i
     YITU_REQUIRE(n_dst < INT32_MAX && n_src <= (1 << 24) && L < (1 << 20) && nnz < INT32_MAX,
                  "size out of range (columns are 24-bit)");
     YITU_REQUIRE(indptr && (nnz == 0 || (indices && features && grad_out)), "null input");
+    if (nnz == 0 && n_src == 0) return 0;  // both gradients are empty
     YITU_REQUIRE(grad_a || grad_x, "no output requested");
     YITU_REQUIRE(!grad_x || nnz == 0 || values, "grad_x needs the edge values");
     YITU_REQUIRE(!grad_x || (t_indptr && (nnz == 0 || (t_rows && t_perm))),
