@@ -7,7 +7,14 @@ test-suite, the smoke check and the benchmark's ``cpu_baseline`` leg may import
 this package; the shipped ``yitu_amd`` package never does.
 
 Every function cites the reference lines it restates; paths are relative to the
-reference checkout.
+reference checkout. Each is pinned in tests/test_oracle_module1.py and
+tests/test_oracle_module2.py against an independent formulation (scipy's CSR
+product, dense torch algebra with autograd, closed forms, brute-force loops).
+
+Parity unpinned: the exact permutation of the Rabbit-Order reorder. Its reference
+(rabbit_order.hpp) needs boost, which is absent, and holds no golden permutation,
+so there is no function for it here; tests/test_rabbit.py pins the algorithm's
+definition on small graphs and its invariants instead.
 """
 import ctypes
 import os

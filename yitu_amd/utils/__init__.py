@@ -1,0 +1,1 @@
+"""Per-graph bookkeeping of the GCN / GIN layers (``input_info.InputInfo``)."""
