@@ -1,8 +1,11 @@
-"""Size-independent properties at the full sizes of the second and third
+"""Size-independent properties at the full sizes of the second to fifth
 configurations (R-MAT 2^18 nodes / 13 M draws, 4 heads x 64; R-MAT 2^21 nodes /
-63 M draws, 128 features), where the CPU oracle would take minutes: exact row
-counts, column-sum checksums in float64, the adjoint identity between forward
-and backward, softmax rows that sum to one, reproducibility."""
+63 M draws, 128 features; 4 node types with 8 relations at 256 features; 2^20
+temporal events with 2,048 roots x 20 neighbours), where the CPU oracle would
+take minutes: exact row counts, column-sum checksums in float64, the adjoint
+identity between forward and backward, softmax rows that sum to one, closed
+forms, sampled rows against float64, host and device sampler bit for bit,
+reproducibility."""
 import pytest
 import torch
 
@@ -129,3 +132,146 @@ def test_c2_backward_is_the_adjoint_of_forward(dev, c2):
     lean = graph_ext.gat_backward(rp, ci, q, k, x, None, gy, out=out2, stats=stats)
     for got, want in zip(lean, full):
         assert float((got - want).abs().max()) < 1e-5 * max(float(want.abs().max()), 1.0)
+
+
+# ---- fourth configuration: 4 node types, 8 relations, 256 features --------------------
+
+@pytest.fixture(scope="module")
+def c4(dev):
+    from yitu_amd.xgnn_h import block as xblock
+    sizes = [1 << 18, 1 << 17, 1 << 16, 1 << 15]
+    off = [0]
+    for n in sizes:
+        off.append(off[-1] + n)
+    rels = []
+    for r in range(8):
+        s_t, d_t = r % 4, (r + 1 + r // 4) % 4
+        rp, ci = graphgen.bipartite_uniform(sizes[d_t], sizes[s_t], 8, 20243 + r, device=dev)
+        indeg = (rp[1:] - rp[:-1]).float()
+        norm = torch.where(indeg > 0, 1.0 / indeg.clamp(min=1), torch.zeros_like(indeg))[:, None]
+        rels.append((s_t, d_t, rp, ci, norm))
+    per_dst = [sum(1 for r in rels if r[1] == t) for t in range(4)]
+    stacked, values = xblock.stack_blocks(
+        [xblock.Block([sizes[d], sizes[s]], [rp, ci]) for s, d, rp, ci, _ in rels],
+        [off[d] for _, d, _, _, _ in rels], [off[s] for s, _, _, _, _ in rels], off[-1], off[-1],
+        [norm / per_dst[d] for _, d, _, _, norm in rels])
+    return sizes, off, rels, per_dst, stacked.adj_sparse, values
+
+
+def test_c4_stacked_relations_closed_form_and_adjoint(dev, c4):
+    """Mean over each relation's neighbours, then mean over the relations of the
+    destination type, as one edge-weighted product over the stacked structure:
+    constant features give (relations with at least one edge into the row) /
+    (relations of the type) exactly up to rounding; the result equals the
+    relation-by-relation composition; <A x, y> = <x, A^T y> in float64."""
+    sizes, off, rels, per_dst, (indptr, indices), values = c4
+    n_all, dim = off[-1], 256
+    assert indices.numel() == sum(int(r[3].numel()) for r in rels) > 7_000_000
+    ones = torch.ones(n_all, 1, dim, device=dev)
+    got = graph_ext.spmm_forward(values, indptr, indices, ones).view(n_all, dim)
+    want = torch.zeros(n_all, device=dev)
+    for _, d, rp, _, _ in rels:
+        want[off[d]:off[d + 1]] += (rp[1:] > rp[:-1]).float() / per_dst[d]
+    assert float((got - want[:, None]).abs().max()) < 1e-6
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn(n_all, dim, generator=g, device=dev)
+    y = torch.randn(n_all, dim, generator=g, device=dev)
+    ax = graph_ext.spmm_forward(values, indptr, indices, x.view(n_all, 1, dim)).view(n_all, dim)
+    by_rel = torch.zeros(n_all, dim, device=dev)
+    for s, d, rp, ci, norm in rels:
+        by_rel[off[d]:off[d + 1]] += K._aggregate(x[off[s]:off[s + 1]], rp, ci, None, 1.0) * \
+            (norm / per_dst[d])
+    assert torch.allclose(ax, by_rel, rtol=1e-5, atol=1e-4)
+    aty = graph_ext.spmm_backward(values, indptr, indices, x.view(n_all, 1, dim),
+                                  y.view(n_all, 1, dim), need_grad_a=False)[1].view(n_all, dim)
+    lhs = float((ax.double() * y.double()).sum())
+    rhs = float((x.double() * aty.double()).sum())
+    scale = float((ax.double().abs() * y.double().abs()).sum())
+    assert abs(lhs - rhs) < 1e-6 * scale, (lhs, rhs, scale)
+    # bf16 rows: exactly representable inputs give the fp32 result up to summation order
+    xb = x.to(torch.bfloat16)
+    ab = graph_ext.spmm_forward(values, indptr, indices, xb.view(n_all, 1, dim))
+    af = graph_ext.spmm_forward(values, indptr, indices, xb.float().view(n_all, 1, dim))
+    assert torch.allclose(ab, af, rtol=1e-5, atol=1e-4)
+
+
+def test_c4_typed_gemms_against_float64(dev, c4):
+    """[n_t, 256] x [256, 256] per node type, forward and both gradients, on a
+    sample of rows against float64 (dW over all rows)."""
+    sizes = c4[0]
+    dim = 256
+    g = torch.Generator(device=dev).manual_seed(11)
+    for n in sizes:
+        x = torch.randn(n, dim, generator=g, device=dev)
+        w = torch.randn(dim, dim, generator=g, device=dev) * 0.02
+        dy = torch.randn(n, dim, generator=g, device=dev)
+        rows = torch.randint(0, n, (4096,), generator=g, device=dev)
+        y = graph_ext.sgemm(x, w)
+        assert torch.allclose(y[rows].double(), x[rows].double() @ w.double(), rtol=1e-5, atol=1e-5)
+        dx = graph_ext.sgemm(dy, w, trans_b=True)
+        assert torch.allclose(dx[rows].double(), dy[rows].double() @ w.double().t(), rtol=1e-5,
+                              atol=1e-5)
+        dw = graph_ext.sgemm(x, dy, trans_a=True)
+        want = x.double().t() @ dy.double()
+        # n products per element: the bar scales with sqrt(n)
+        assert float((dw.double() - want).abs().max()) < 2e-6 * (n ** 0.5) * 4
+        y16 = graph_ext.gemm_bf16(x.bfloat16(), w.bfloat16())
+        want16 = x.bfloat16()[rows].double() @ w.bfloat16().double()
+        assert torch.allclose(y16[rows].double(), want16, rtol=1e-2, atol=1e-2)
+
+
+# ---- fifth configuration: 2^20 events, 2^17 nodes, 2,048 roots x 20 neighbours --------
+
+def test_c5_device_sampler_equals_host_and_layer_equals_dense_attention(dev):
+    import numpy as np
+    from helpers import assert_close, dense_temporal_attention
+    from yitu_amd import sampler_core
+    from yitu_amd.temporal import TemporalBlock, TransfomerAttentionLayer
+    rng = np.random.default_rng(20244)
+    n_nodes, n_events, k, batch = 1 << 17, 1 << 20, 20, 2048
+    src = ((rng.zipf(1.2, n_events) - 1) % n_nodes).astype(np.int64)
+    dst = ((rng.zipf(1.2, n_events) - 1) % n_nodes).astype(np.int64)
+    ts = np.sort(rng.uniform(0, 1e6, n_events)).astype(np.float32)
+    node = np.concatenate([src, dst])
+    other = np.concatenate([dst, src])
+    eid = np.concatenate([np.arange(n_events), np.arange(n_events)])
+    tt = np.concatenate([ts, ts])
+    order = np.lexsort((eid, tt, node))
+    indptr = np.zeros(n_nodes + 1, np.int64)
+    indptr[1:] = np.cumsum(np.bincount(node, minlength=n_nodes))
+    args = (indptr, other[order], eid[order], tt[order], 16, 1, 1, [k], True, False, 1, 0.0)
+    host = sampler_core.ParallelSampler(*args)
+    device = sampler_core.GpuParallelSampler(*args, device=dev)
+    # three consecutive batches in time order: the cursors carry over between them
+    for lo in (0.90, 0.93, 0.96):
+        ev = np.sort(rng.integers(int(n_events * lo), int(n_events * (lo + 0.03)), batch // 2))
+        roots = np.concatenate([src[ev], dst[ev]])
+        root_ts = np.concatenate([ts[ev], ts[ev]])
+        host.sample(roots, root_ts)
+        device.sample(torch.as_tensor(roots, dtype=torch.int32, device=dev),
+                      torch.as_tensor(root_ts, dtype=torch.float32, device=dev))
+        tgb, dblk = host.get_ret()[0], device.get_ret()[0].cpu_block()
+        for f in ("row", "col", "eid", "ts", "dts", "nodes"):
+            assert np.array_equal(getattr(dblk, f)(), getattr(tgb, f)()), f
+    # every root's neighbours are its k most recent events before its time
+    row, dts = tgb.row(), tgb.dts()
+    assert np.bincount(row, minlength=batch).max() <= k and (dts[batch:] >= 0).all()
+    torch.manual_seed(20244)
+    memory = torch.randn(n_nodes, 172, device=dev)
+    layer = TransfomerAttentionLayer(172, 0, 100, 1, 0.0, 0.0, 100).to(dev)
+    blk = TemporalBlock.from_sampler(tgb, memory, device=dev)
+    assert blk.n_dst == batch and blk.num_edges() > batch
+    blk.h.requires_grad_()
+    out = layer(blk)
+    w = torch.randn_like(out)
+    (out * w).sum().backward()
+    grads = [blk.h.grad.clone()] + [p.grad.clone() for p in layer.parameters()]
+    blk.h.grad = None
+    layer.zero_grad()
+    want = dense_temporal_attention(layer, blk.h, blk.row, blk.dt, blk.n_dst, k)
+    (want * w).sum().backward()
+    assert_close(out, want, atol=2e-4)
+    names = ["h"] + [n for n, _ in layer.named_parameters()]
+    for got, ref, name in zip(grads, [blk.h.grad] + [p.grad for p in layer.parameters()], names):
+        # parameter gradients sum over 2,048 roots (and up to 40,960 edges)
+        assert_close(got, ref, rtol=1e-4, atol=5e-3 if name != "h" else 5e-4, what=name)
