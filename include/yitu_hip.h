@@ -309,6 +309,23 @@ int yitu_sgemm(float *c_device, const float *a_device, const float *b_device, in
                int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
+ * Typed products in one launch per 8 problems: C_i[m_i,n] (+)= op(A_i)[m_i,k_i] .
+ * op(B_i)[k_i,n] for i < n_problems, with shared n, transposes and leading
+ * dimensions. c, a, b, m, k are HOST arrays (of device pointers and sizes).
+ * Replaces the loop of per-relation / per-type Linear layers of the
+ * heterogeneous models (test/common/model.py:137-171 over :7-30, one cuBLAS SGEMM each and
+ * its two gradient products): the row tiles of all node types fill the chip
+ * together instead of one short launch after another. Workspace for the split
+ * products (X_t^T . G_t): yitu_sgemm_workspace_bytes(max m_i, n, max k_i,
+ * min(n_problems, 8)); the same workspace serves every group of 8.
+ */
+int yitu_sgemm_typed(float *const *c_device_ptrs, const float *const *a_device_ptrs,
+                     const float *const *b_device_ptrs, const int64_t *m, const int64_t *k,
+                     int64_t n_problems, int64_t n, int trans_a, int trans_b, int64_t lda,
+                     int64_t ldb, int64_t ldc, int accumulate, void *workspace_device,
+                     size_t workspace_bytes, void *stream);
+
+/*
  * b2gemm (entry.cpp:56-64; fc_cuda.cu:4-75): y_a = x . w_a^T, y_b = x . w_b^T
  * as one grouped launch. x [n,k], w_* [m,k], y_* [n,m], contiguous.
  */

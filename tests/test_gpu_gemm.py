@@ -50,6 +50,50 @@ def test_sgemm_typed_gemm_shape(dev):
     assert_close(graph_ext.sgemm(x.to(dev), w.to(dev)), _ref(x, w, False, False))
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("sizes", [[(300, 64), (1, 64), (0, 64), (129, 64)],
+                                   [(1024, 256), (512, 256), (256, 256)],
+                                   [(50, 8)] * 11,                  # more than one group of 8
+                                   [(40, 70001), (33, 5000), (64, 0)]])  # long, uneven, empty K
+def test_sgemm_typed_equals_one_product_at_a_time(dev, ta, tb, sizes):
+    """Problems of different height (and inner length) in one launch: each result is
+    bit for bit what the single-problem entry point gives when no K split is
+    involved, and within the bar of a float64 product always."""
+    n = 96
+    g = torch.Generator().manual_seed(len(sizes) * 5 + ta * 2 + tb)
+    if ta:  # the gradient form: a_i [k_i, m], b_i [k_i, n] with m shared
+        sizes = [(64, k) for _, k in sizes]
+    a_list = [torch.randn((k, m) if ta else (m, k), generator=g).to(dev) for m, k in sizes]
+    b_list = [torch.randn((n, k) if tb else (k, n), generator=g).to(dev) for _, k in sizes]
+    if len({a.size(1) for a in a_list}) > 1 or len({b.size(1) for b in b_list}) > 1:
+        pytest.skip("row strides differ: the wrapper takes the products one at a time")
+    got = graph_ext.sgemm_typed(a_list, b_list, ta, tb)
+    for (m, k), a, b, c in zip(sizes, a_list, b_list, got):
+        assert tuple(c.shape) == (m, n)
+        assert_close(c, _ref(a.cpu(), b.cpu(), ta, tb), atol=1e-4 * max(1.0, np.sqrt(k) / 4),
+                     what="m=%d k=%d" % (m, k))
+        if k < 4096:
+            assert torch.equal(c, graph_ext.sgemm(a, b, ta, tb))
+    again = graph_ext.sgemm_typed(a_list, b_list, ta, tb)
+    assert all(torch.equal(x, y) for x, y in zip(got, again))
+
+
+def test_sgemm_typed_writes_row_slices_of_one_buffer(dev):
+    g = torch.Generator().manual_seed(4)
+    heights = [384, 128, 257, 5]
+    xs = [torch.randn(m, 256, generator=g).to(dev) for m in heights]
+    ws = [(torch.randn(256, 256, generator=g) * 0.02).to(dev) for _ in heights]
+    buf = torch.full((sum(heights) + 3, 256), 7.0, device=dev)
+    parts, off = [], 0
+    for m in heights:
+        parts.append(buf[off:off + m])
+        off += m
+    graph_ext.sgemm_typed(xs, ws, out_list=parts)
+    for x, w, part in zip(xs, ws, parts):
+        assert_close(part, _ref(x.cpu(), w.cpu(), False, False))
+    assert torch.all(buf[off:] == 7.0)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_check_bundle(dev, seed):
     """test_kernel.py:187-233 with seeded shapes: b2gemm vs two bias-free Linear layers,

@@ -6,7 +6,8 @@
 //   C[M,N] (+)= A[M,K] . B[K,N],  element (i,k) of A at A + i*a_si + k*a_sk,
 //                                  element (k,j) of B at B + k*b_sk + j*b_sj,
 // one of each stride pair being 1, C row-major. Up to 8 problems that share
-// N, K and the strides are grouped into one launch (blockIdx.z).
+// N and the strides, each with its own M and K, are grouped into one launch
+// (blockIdx.z walks the problems and their K splits).
 //
 // Tiling: 128x128 output tile per 256-thread workgroup, each of the 4 waves
 // owns 64x64 = 2x2 MFMA tiles (64 accumulator registers); K advances in steps
@@ -28,22 +29,29 @@ struct GemmProblem {
     const float *A;
     const float *B;
     float *C;
-    int M;
+    int M, K;
+    // split-K: this problem owns blockIdx.z in [z0, z0 + n_split); split s covers
+    // the K range [s * k_chunk, min(K, (s+1) * k_chunk)) and, when n_split > 1,
+    // writes its own [M, N] slab of `partial` (slab index = blockIdx.z)
+    int z0, n_split, k_chunk;
 };
 
 struct GemmParams {
     GemmProblem prob[kMaxGroup];
     int n_prob;
-    int N, K;
+    int N;
     int64_t a_si, a_sk, b_sk, b_sj;
     int ldc;
     int accumulate;  // C += A.B instead of C = A.B
-    // split-K: blockIdx.z = problem * n_split + split; split s covers K range
-    // [s * k_chunk, min(K, (s+1) * k_chunk)) and writes its own [M, N] slab of
-    // `partial` (slab index = blockIdx.z, all problems sized by max_m)
-    int n_split, k_chunk, max_m;
+    int max_m;       // slabs of `partial` are [max_m, N]
     float *partial;
 };
+
+__device__ __forceinline__ int problem_of(const GemmParams &p, int z) {
+    int i = 0;
+    while (i + 1 < p.n_prob && z >= p.prob[i + 1].z0) i++;
+    return i;
+}
 
 // Loads this thread's 8 elements of a [128 x 16] operand tile into regs.
 // KCONT: the operand is contiguous along K (thread owns 8 consecutive k of one row),
@@ -98,9 +106,9 @@ template <bool A_KCONT, bool B_KCONT, bool FAST>
 __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
     __shared__ float As[2][BK][LDP];
     __shared__ float Bs[2][BK][LDP];
-    const GemmProblem pr = p.prob[blockIdx.z / p.n_split];
-    const int split = blockIdx.z % p.n_split;
-    const int kb = split * p.k_chunk, ke = min(p.K, kb + p.k_chunk);
+    const GemmProblem pr = p.prob[problem_of(p, blockIdx.z)];
+    const int split = blockIdx.z - pr.z0;
+    const int kb = split * pr.k_chunk, ke = min(pr.K, kb + pr.k_chunk);
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     if (m0 >= pr.M) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -152,7 +160,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
     float *cbase = pr.C;
     int ldc = p.ldc;
     bool accumulate = p.accumulate != 0;
-    if (p.n_split > 1) {
+    if (pr.n_split > 1) {
         cbase = p.partial + (size_t)blockIdx.z * p.max_m * p.N;
         ldc = p.N;
         accumulate = false;
@@ -179,13 +187,14 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
 // C (+)= sum over splits of the partial slabs, in split order (reproducible)
 __global__ __launch_bounds__(256) void sgemm_splitk_reduce_kernel(GemmParams p) {
     const GemmProblem pr = p.prob[blockIdx.y];
+    if (pr.n_split <= 1) return;  // written in place by the product kernel
     const int64_t total = (int64_t)pr.M * p.N;
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total;
          e += (int64_t)gridDim.x * 256) {
         const int row = (int)(e / p.N), col = (int)(e % p.N);
         float s = 0.0f;
-        for (int z = 0; z < p.n_split; z++)
-            s += p.partial[((size_t)(blockIdx.y * p.n_split + z) * p.max_m + row) * p.N + col];
+        for (int z = 0; z < pr.n_split; z++)
+            s += p.partial[((size_t)(pr.z0 + z) * p.max_m + row) * p.N + col];
         float *c = pr.C + (int64_t)row * p.ldc + col;
         *c = p.accumulate ? *c + s : s;
     }
@@ -193,37 +202,51 @@ __global__ __launch_bounds__(256) void sgemm_splitk_reduce_kernel(GemmParams p) 
 
 // Few output tiles and a long inner dimension (dW = X^T.G with K = number of
 // nodes): split K so the whole chip works, partials summed by a second kernel.
-static void choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
-    p.n_split = 1;
-    p.k_chunk = ((p.K + BK - 1) / BK) * BK;
+// Returns the number of blockIdx.z values.
+static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
     p.max_m = max_m;
-    const int64_t tiles = ceil_div(p.N, BN) * ceil_div(max_m, BM) * p.n_prob;
-    if (tiles >= 256 || p.K < 4096) return;
-    int64_t want = std::min<int64_t>(ceil_div(p.K, 1024), ceil_div(1024, tiles));
-    const int64_t slab = (int64_t)max_m * p.N * sizeof(float) * p.n_prob;
-    want = std::min<int64_t>(want, slab > 0 ? (int64_t)(workspace_bytes / slab) : 1);
-    if (want <= 1) return;
-    p.k_chunk = (int)(ceil_div(ceil_div(p.K, want), BK) * BK);
-    p.n_split = (int)ceil_div(p.K, p.k_chunk);
+    int64_t tiles = 0;
+    for (int i = 0; i < p.n_prob; i++) tiles += ceil_div(p.N, BN) * ceil_div(p.prob[i].M, BM);
+    const int64_t slab = (int64_t)max_m * p.N * sizeof(float);
+    const int64_t slab_cap = slab > 0 ? (int64_t)(workspace_bytes / slab) / p.n_prob : 0;
+    int z = 0;
+    for (int i = 0; i < p.n_prob; i++) {
+        GemmProblem &pr = p.prob[i];
+        pr.z0 = z;
+        pr.n_split = 1;
+        pr.k_chunk = (int)(ceil_div(pr.K, BK) * BK);
+        if (tiles < 256 && pr.K >= 4096 && pr.M > 0) {
+            int64_t want = std::min<int64_t>(ceil_div(pr.K, 1024), ceil_div(1024, tiles));
+            want = std::min<int64_t>(want, slab_cap);
+            if (want > 1) {
+                pr.k_chunk = (int)(ceil_div(ceil_div(pr.K, want), BK) * BK);
+                pr.n_split = (int)ceil_div(pr.K, pr.k_chunk);
+            }
+        }
+        z += pr.n_split;
+    }
+    return z;
 }
 
 template <bool A_KCONT, bool B_KCONT>
-static int sgemm_launch(const GemmParams &p, int max_m, hipStream_t stream) {
-    bool fast = p.N % BN == 0 && p.K % BK == 0;
+static int sgemm_launch(const GemmParams &p, int max_m, int n_z, hipStream_t stream) {
+    bool fast = p.N % BN == 0, any_split = false;
     for (int i = 0; i < p.n_prob; i++) {
-        fast = fast && p.prob[i].M % BM == 0 && aligned16(p.prob[i].A) && aligned16(p.prob[i].B);
+        const GemmProblem &pr = p.prob[i];
+        fast = fast && pr.M % BM == 0 && pr.K % BK == 0 && pr.K > 0 && aligned16(pr.A) &&
+               aligned16(pr.B);
+        any_split = any_split || pr.n_split > 1;
     }
     // vector loads also need every row / k-line to start 16-byte aligned
     fast = fast && (A_KCONT ? p.a_si % 4 == 0 : p.a_sk % 4 == 0) &&
            (B_KCONT ? p.b_sj % 4 == 0 : p.b_sk % 4 == 0);
-    dim3 grid((unsigned)ceil_div(p.N, BN), (unsigned)ceil_div(max_m, BM),
-              (unsigned)(p.n_prob * p.n_split));
+    dim3 grid((unsigned)ceil_div(p.N, BN), (unsigned)ceil_div(max_m, BM), (unsigned)n_z);
     if (fast)
         sgemm_mfma_kernel<A_KCONT, B_KCONT, true><<<grid, 256, 0, stream>>>(p);
     else
         sgemm_mfma_kernel<A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    if (p.n_split > 1) {
+    if (any_split) {
         dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)max_m * p.N, 256), 2048),
                 (unsigned)p.n_prob);
         sgemm_splitk_reduce_kernel<<<rg, 256, 0, stream>>>(p);
@@ -236,27 +259,32 @@ static int sgemm_launch(const GemmParams &p, int max_m, hipStream_t stream) {
 // [N, K] row-major (else [K, N]).
 int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, void *workspace,
                   size_t workspace_bytes, hipStream_t stream) {
+    // problems with an empty inner dimension: C = 0 (or unchanged); they leave the group
+    int kept = 0;
+    for (int i = 0; i < p.n_prob; i++) {
+        const GemmProblem pr = p.prob[i];
+        if (pr.M == 0) continue;
+        if (pr.K > 0) {
+            p.prob[kept++] = pr;
+            continue;
+        }
+        if (p.accumulate) continue;
+        if (p.ldc == p.N) {
+            int rc = fill_zero(pr.C, (int64_t)pr.M * p.N, stream);
+            if (rc) return rc;
+        } else {
+            for (int r = 0; r < pr.M; r++) {
+                int rc = fill_zero(pr.C + (int64_t)r * p.ldc, p.N, stream);
+                if (rc) return rc;
+            }
+        }
+    }
+    p.n_prob = kept;
     int max_m = 0;
     for (int i = 0; i < p.n_prob; i++) max_m = std::max(max_m, p.prob[i].M);
     if (max_m == 0 || p.N == 0) return 0;
-    choose_split(p, max_m, workspace ? workspace_bytes : 0);
+    const int n_z = choose_split(p, max_m, workspace ? workspace_bytes : 0);
     p.partial = static_cast<float *>(workspace);
-    if (p.K == 0) {
-        if (p.accumulate) return 0;
-        // empty inner dimension: C = 0
-        for (int i = 0; i < p.n_prob; i++) {
-            if (p.ldc == p.N) {
-                int rc = fill_zero(p.prob[i].C, (int64_t)p.prob[i].M * p.N, stream);
-                if (rc) return rc;
-            } else {
-                for (int r = 0; r < p.prob[i].M; r++) {
-                    int rc = fill_zero(p.prob[i].C + (int64_t)r * p.ldc, p.N, stream);
-                    if (rc) return rc;
-                }
-            }
-        }
-        return 0;
-    }
     if (trans_a) {  // element (i,k) at A[k*lda + i]: contiguous along rows
         p.a_si = 1;
         p.a_sk = lda;
@@ -271,10 +299,10 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
         p.b_sk = ldb;
         p.b_sj = 1;
     }
-    if (!trans_a && trans_b) return sgemm_launch<true, true>(p, max_m, stream);
-    if (!trans_a && !trans_b) return sgemm_launch<true, false>(p, max_m, stream);
-    if (trans_a && !trans_b) return sgemm_launch<false, false>(p, max_m, stream);
-    return sgemm_launch<false, true>(p, max_m, stream);
+    if (!trans_a && trans_b) return sgemm_launch<true, true>(p, max_m, n_z, stream);
+    if (!trans_a && !trans_b) return sgemm_launch<true, false>(p, max_m, n_z, stream);
+    if (trans_a && !trans_b) return sgemm_launch<false, false>(p, max_m, n_z, stream);
+    return sgemm_launch<false, true>(p, max_m, n_z, stream);
 }
 
 }  // namespace yitu
@@ -299,14 +327,45 @@ YITU_API int yitu_sgemm(float *c, const float *a, const float *b, int64_t m, int
     YITU_REQUIRE(m < INT32_MAX && n < INT32_MAX && k < INT32_MAX && ldc >= n, "size out of range");
     YITU_REQUIRE(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n), "leading dimension too small");
     GemmParams p{};
-    p.prob[0] = GemmProblem{a, b, c, (int)m};
+    p.prob[0] = GemmProblem{a, b, c, (int)m, (int)k};
     p.n_prob = 1;
     p.N = (int)n;
-    p.K = (int)k;
     p.ldc = (int)ldc;
     p.accumulate = accumulate;
     return sgemm_grouped(p, trans_a != 0, trans_b != 0, (int)lda, (int)ldb, workspace,
                          workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_sgemm_typed(float *const *c, const float *const *a, const float *const *b,
+                              const int64_t *m, const int64_t *k, int64_t n_problems, int64_t n,
+                              int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldc,
+                              int accumulate, void *workspace, size_t workspace_bytes,
+                              void *stream) {
+    YITU_REQUIRE(n_problems >= 0 && n >= 0, "negative size");
+    if (n_problems == 0 || n == 0) return 0;
+    YITU_REQUIRE(c && a && b && m && k, "null problem table");
+    YITU_REQUIRE(n < INT32_MAX && ldc >= n, "size out of range");
+    for (int64_t first = 0; first < n_problems; first += kMaxGroup) {
+        GemmParams p{};
+        p.n_prob = (int)std::min<int64_t>(kMaxGroup, n_problems - first);
+        p.N = (int)n;
+        p.ldc = (int)ldc;
+        p.accumulate = accumulate;
+        for (int i = 0; i < p.n_prob; i++) {
+            const int64_t mi = m[first + i], ki = k[first + i];
+            YITU_REQUIRE(mi >= 0 && ki >= 0 && mi < INT32_MAX && ki < INT32_MAX,
+                         "problem %d: size out of range", (int)(first + i));
+            YITU_REQUIRE(mi == 0 || (c[first + i] && (ki == 0 || (a[first + i] && b[first + i]))),
+                         "problem %d: null operand", (int)(first + i));
+            YITU_REQUIRE(lda >= (trans_a ? mi : ki) && ldb >= (trans_b ? ki : n),
+                         "problem %d: leading dimension too small", (int)(first + i));
+            p.prob[i] = GemmProblem{a[first + i], b[first + i], c[first + i], (int)mi, (int)ki};
+        }
+        int rc = sgemm_grouped(p, trans_a != 0, trans_b != 0, (int)lda, (int)ldb, workspace,
+                               workspace_bytes, static_cast<hipStream_t>(stream));
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 YITU_API int yitu_b2gemm(float *y_a, float *y_b, const float *x, const float *w_a,
@@ -316,11 +375,10 @@ YITU_API int yitu_b2gemm(float *y_a, float *y_b, const float *x, const float *w_
     YITU_REQUIRE(y_a && y_b && (k == 0 || (x && w_a && w_b)), "null operand");
     YITU_REQUIRE(n < INT32_MAX && k < INT32_MAX && m < INT32_MAX, "size out of range");
     GemmParams p{};
-    p.prob[0] = GemmProblem{x, w_a, y_a, (int)n};
-    p.prob[1] = GemmProblem{x, w_b, y_b, (int)n};
+    p.prob[0] = GemmProblem{x, w_a, y_a, (int)n, (int)k};
+    p.prob[1] = GemmProblem{x, w_b, y_b, (int)n, (int)k};
     p.n_prob = 2;
     p.N = (int)m;
-    p.K = (int)k;
     p.ldc = (int)m;
     return sgemm_grouped(p, false, true, (int)k, (int)k, nullptr, 0,
                          static_cast<hipStream_t>(stream));
@@ -337,11 +395,10 @@ YITU_API int yitu_b2gemm_backward(float *dx, float *dw_a, float *dw_b, const flo
     // dw_* [m,k] = grad_*^T [m,n] . x [n,k]: one grouped launch of two problems
     if (m > 0 && k > 0) {
         GemmParams p{};
-        p.prob[0] = GemmProblem{grad_a, x, dw_a, (int)m};
-        p.prob[1] = GemmProblem{grad_b, x, dw_b, (int)m};
+        p.prob[0] = GemmProblem{grad_a, x, dw_a, (int)m, (int)n};
+        p.prob[1] = GemmProblem{grad_b, x, dw_b, (int)m, (int)n};
         p.n_prob = 2;
         p.N = (int)k;
-        p.K = (int)n;
         p.ldc = (int)k;
         int rc = sgemm_grouped(p, true, false, (int)m, (int)k, workspace, workspace_bytes, stream);
         if (rc) return rc;
@@ -350,10 +407,9 @@ YITU_API int yitu_b2gemm_backward(float *dx, float *dw_a, float *dw_b, const flo
     if (n > 0 && k > 0) {
         for (int pass = 0; pass < 2; pass++) {
             GemmParams p{};
-            p.prob[0] = GemmProblem{pass ? grad_b : grad_a, pass ? w_b : w_a, dx, (int)n};
+            p.prob[0] = GemmProblem{pass ? grad_b : grad_a, pass ? w_b : w_a, dx, (int)n, (int)m};
             p.n_prob = 1;
             p.N = (int)k;
-            p.K = (int)m;
             p.ldc = (int)k;
             p.accumulate = pass;
             int rc = sgemm_grouped(p, false, false, (int)m, (int)k, nullptr, 0, stream);

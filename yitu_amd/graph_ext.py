@@ -347,6 +347,54 @@ def sgemm(a, b, trans_a=False, trans_b=False, out=None):
     return c
 
 
+def sgemm_typed(a_list, b_list, trans_a=False, trans_b=False, out_list=None):
+    """[op(a_i) . op(b_i)] for operand pairs that share the output width, the
+    transposes and the row strides (the per-type Linear layers of a heterogeneous
+    model and their gradient products), eight products per launch so that the
+    row tiles of all types fill the chip together. ``out_list``: contiguous
+    [m_i, n] tensors to write (e.g. row slices of one buffer)."""
+    import ctypes
+    if len(a_list) != len(b_list) or not a_list:
+        raise RuntimeError("sgemm_typed needs as many a as b operands, at least one")
+    for a, b in zip(a_list, b_list):
+        _check(a, torch.float32, "a", 2)
+        _check(b, torch.float32, "b", 2)
+    dev = _lib.require_device(*a_list, *b_list)
+    ms = [a.size(1) if trans_a else a.size(0) for a in a_list]
+    ks = [a.size(0) if trans_a else a.size(1) for a in a_list]
+    n = b_list[0].size(0) if trans_b else b_list[0].size(1)
+    lda, ldb = a_list[0].size(1), b_list[0].size(1)
+    shared = True
+    for a, b, k in zip(a_list, b_list, ks):
+        kb, nb = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
+        if kb != k:
+            raise RuntimeError("inner dimensions differ: %d vs %d" % (k, kb))
+        shared = shared and nb == n and a.size(1) == lda and b.size(1) == ldb
+    if not shared:  # widths differ between the types: one product at a time
+        outs = out_list if out_list is not None else [None] * len(a_list)
+        return [sgemm(a, b, trans_a, trans_b, out=c) for a, b, c in zip(a_list, b_list, outs)]
+    if out_list is None:
+        out_list = [torch.empty((m, n), dtype=torch.float32, device=dev) for m in ms]
+    else:
+        for c, m in zip(out_list, ms):
+            _check(c, torch.float32, "out", 2)
+            if tuple(c.shape) != (m, n) or c.device != dev:
+                raise RuntimeError("out must be [%d, %d] on the operands' device" % (m, n))
+    count = len(a_list)
+    ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(
+        c_i64(max(ms)), c_i64(n), c_i64(max(ks)), c_i64(min(count, 8))), dev)
+    pointers = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() or None for t in ts])
+    sizes = lambda v: (ctypes.c_int64 * count)(*v)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_sgemm_typed(pointers(out_list), pointers(a_list), pointers(b_list),
+                                         sizes(ms), sizes(ks), c_i64(count), c_i64(n),
+                                         c_int(int(trans_a)), c_int(int(trans_b)), c_i64(lda),
+                                         c_i64(ldb), c_i64(n), c_int(0), ptr(ws),
+                                         c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_sgemm_typed")
+    return list(out_list)
+
+
 def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32, out=None):
     """a . op(b) with bf16 operands and fp32 accumulation on the matrix cores.
     ``a`` [m, k]; ``b`` [k, n], or [n, k] with ``trans_b`` (a Linear weight).

@@ -141,13 +141,15 @@ class _TypedLinear(torch.autograd.Function):
         xs, ws, bs = args[:n_parts], args[n_parts:2 * n_parts], args[2 * n_parts:]
         total = sum(x.size(0) for x in xs)
         y = torch.empty((total, ws[0].size(0)), dtype=torch.float32, device=xs[0].device)
-        off = 0
-        for x, w, b in zip(xs, ws, bs):
-            part = y[off:off + x.size(0)]
-            graph_ext.sgemm(x.contiguous(), w.contiguous(), trans_b=True, out=part)
+        parts, off = [], 0
+        for x in xs:
+            parts.append(y[off:off + x.size(0)])
+            off += x.size(0)
+        graph_ext.sgemm_typed([x.contiguous() for x in xs], [w.contiguous() for w in ws],
+                              trans_b=True, out_list=parts)
+        for part, b in zip(parts, bs):
             if b is not None:
                 part += b
-            off += x.size(0)
         ctx.n_parts = n_parts
         ctx.has_bias = [b is not None for b in bs]
         ctx.save_for_backward(*xs, *ws)
@@ -159,15 +161,24 @@ class _TypedLinear(torch.autograd.Function):
         n = ctx.n_parts
         xs, ws = ctx.saved_tensors[:n], ctx.saved_tensors[n:]
         grad_y = grad_y.contiguous()
-        gx, gw, gb = [], [], []
-        off = 0
-        for i, (x, w) in enumerate(zip(xs, ws)):
-            g = grad_y[off:off + x.size(0)]
-            gx.append(graph_ext.sgemm(g, w.contiguous()) if ctx.needs_input_grad[1 + i] else None)
-            gw.append(graph_ext.sgemm(g, x.contiguous(), trans_a=True)
-                      if ctx.needs_input_grad[1 + n + i] else None)
-            gb.append(g.sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None)
+        gs, off = [], 0
+        for x in xs:
+            gs.append(grad_y[off:off + x.size(0)])
             off += x.size(0)
+        gx, gw = [None] * n, [None] * n
+        want = [i for i in range(n) if ctx.needs_input_grad[1 + i]]
+        if want:
+            for i, g in zip(want, graph_ext.sgemm_typed([gs[i] for i in want],
+                                                        [ws[i].contiguous() for i in want])):
+                gx[i] = g
+        want = [i for i in range(n) if ctx.needs_input_grad[1 + n + i]]
+        if want:
+            for i, g in zip(want, graph_ext.sgemm_typed([gs[i] for i in want],
+                                                        [xs[i].contiguous() for i in want],
+                                                        trans_a=True)):
+                gw[i] = g
+        gb = [gs[i].sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None
+              for i in range(n)]
         return (None, *gx, *gw, *gb)
 
 
