@@ -37,11 +37,10 @@ struct HGemmParams {
     int64_t lda, ldbt, ldc;
 };
 
+// round to nearest even; gfx950 converts in hardware (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x7fffffu)) return (uint16_t)((u >> 16) | 0x40u);  // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    const __bf16 h = static_cast<__bf16>(f);
+    return __builtin_bit_cast(uint16_t, h);
 }
 
 template <bool OUT_BF16>
