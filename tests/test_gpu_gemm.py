@@ -65,8 +65,7 @@ def test_sgemm_typed_equals_one_product_at_a_time(dev, ta, tb, sizes):
         sizes = [(64, k) for _, k in sizes]
     a_list = [torch.randn((k, m) if ta else (m, k), generator=g).to(dev) for m, k in sizes]
     b_list = [torch.randn((n, k) if tb else (k, n), generator=g).to(dev) for _, k in sizes]
-    if len({a.size(1) for a in a_list}) > 1 or len({b.size(1) for b in b_list}) > 1:
-        pytest.skip("row strides differ: the wrapper takes the products one at a time")
+    # (where the row strides differ between the problems the wrapper takes them one at a time)
     got = graph_ext.sgemm_typed(a_list, b_list, ta, tb)
     for (m, k), a, b, c in zip(sizes, a_list, b_list, got):
         assert tuple(c.shape) == (m, n)
