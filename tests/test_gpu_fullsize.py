@@ -274,4 +274,5 @@ def test_c5_device_sampler_equals_host_and_layer_equals_dense_attention(dev):
     names = ["h"] + [n for n, _ in layer.named_parameters()]
     for got, ref, name in zip(grads, [blk.h.grad] + [p.grad for p in layer.parameters()], names):
         # parameter gradients sum over 2,048 roots (and up to 40,960 edges)
-        assert_close(got, ref, rtol=1e-4, atol=5e-3 if name != "h" else 5e-4, what=name)
+        rtol = 1e-3 if name == "time_enc.w.weight" else 1e-4  # products with dt up to 10^6
+        assert_close(got, ref, rtol=rtol, atol=5e-3 if name != "h" else 5e-4, what=name)

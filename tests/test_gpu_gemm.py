@@ -57,8 +57,8 @@ def test_sgemm_typed_gemm_shape(dev):
                                    [(40, 70001), (33, 5000), (64, 0)]])  # long, uneven, empty K
 def test_sgemm_typed_equals_one_product_at_a_time(dev, ta, tb, sizes):
     """Problems of different height (and inner length) in one launch: each result is
-    bit for bit what the single-problem entry point gives when no K split is
-    involved, and within the bar of a float64 product always."""
+    bit for bit what the single-problem entry point gives when the inner dimension is
+    too short for a K split, and within the bar of a float64 product always."""
     n = 96
     g = torch.Generator().manual_seed(len(sizes) * 5 + ta * 2 + tb)
     if ta:  # the gradient form: a_i [k_i, m], b_i [k_i, n] with m shared
@@ -71,7 +71,7 @@ def test_sgemm_typed_equals_one_product_at_a_time(dev, ta, tb, sizes):
         assert tuple(c.shape) == (m, n)
         assert_close(c, _ref(a.cpu(), b.cpu(), ta, tb), atol=1e-4 * max(1.0, np.sqrt(k) / 4),
                      what="m=%d k=%d" % (m, k))
-        if k < 4096:
+        if k < 256:  # no K split either way: the same sums in the same order
             assert torch.equal(c, graph_ext.sgemm(a, b, ta, tb))
     again = graph_ext.sgemm_typed(a_list, b_list, ta, tb)
     assert all(torch.equal(x, y) for x, y in zip(got, again))

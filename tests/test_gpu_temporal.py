@@ -52,7 +52,10 @@ def test_layer_matches_dense_masked_attention(dev, num_head):
     assert_close(out, want, atol=2e-4)
     ref_grads = [blk.h.grad] + [p.grad for p in layer.parameters()]
     for g, r, name in zip(grads, ref_grads, ["h"] + [n for n, _ in layer.named_parameters()]):
-        assert_close(g, r, rtol=1e-4, atol=5e-4, what=name)
+        # the frequency gradients sum products with time deltas of up to 10^6 that largely
+        # cancel: both sides carry fp32 summation noise well above their other gradients'
+        rtol = 1e-3 if name == "time_enc.w.weight" else 1e-4
+        assert_close(g, r, rtol=rtol, atol=5e-4, what=name)
 
 
 def test_time_encode_closed_form(dev):

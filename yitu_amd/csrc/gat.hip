@@ -131,14 +131,15 @@ __device__ __forceinline__ void gat_apply_window(float (&acc)[KT][VEC], const Ga
     }
 }
 
-// Short rows, fully fused: a wave walks kRowsPerWave rows; per row statistics,
+// Short rows, fully fused: a wave walks rows_per_wave rows; per row statistics,
 // then probabilities + aggregate, all from the sliding edge window.
 template <int VEC, int G, int KT>
 __global__ __launch_bounds__(kBlock) void gat_rows_kernel(GatParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     const int sub = lane % G, slot = lane / G;
@@ -649,12 +650,13 @@ __device__ __forceinline__ void attn_write_window(const GatParams &p, const Edge
     }
 }
 
-// Short rows: kRowsPerWave rows per wave through the sliding edge window.
+// Short rows: rows_per_wave rows per wave through the sliding edge window.
 __global__ __launch_bounds__(kBlock) void attn_rows_kernel(GatParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     const int hl = lane & (p.HP - 1);
@@ -802,9 +804,10 @@ __device__ __forceinline__ void attn_bwd_reduce(float &S, float &A1, float &A2, 
 
 __global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     const int hl = lane & (p.HP - 1);
@@ -1105,9 +1108,10 @@ __device__ __forceinline__ void gat_src_end(float *x_dst, float *k_dst, const fl
 template <int LPH, int KT, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     EdgeWindow win;
@@ -1310,9 +1314,10 @@ template <int LPH>
 __global__ __launch_bounds__(kBlock) void gat_slot_rows_kernel(GatSrcParams p) {
     constexpr int H = kWave / LPH;
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     EdgeWindow win;
@@ -1384,7 +1389,7 @@ static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const flo
                 p.head_mean, p.g_scale);
         YITU_LAUNCH_CHECK();
     }
-    const int row_grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave);
+    const int row_grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows));
     const int item_grid = (int)std::min<int64_t>(
         ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
     // a head-mean gradient of F < 256 floats per row: the several-edges-per-load kernels
@@ -1470,7 +1475,8 @@ static size_t gat_own_bytes(int64_t n_dst, int64_t nnz, int64_t H, int64_t L) {
 template <int VEC, int G, int KT>
 static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
     gat_rows_kernel<VEC, G, KT>
-        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)), kBlock, 0,
+           stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const int item_grid = (int)std::min<int64_t>(
@@ -1529,7 +1535,8 @@ int attn_forward_run(float *attn, const int32_t *indptr, const int32_t *indices,
                           max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
     if (rc) return rc;
     if (!has_items) p.sp.plan.threshold = 0x7fffffff;
-    attn_rows_kernel<<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+    attn_rows_kernel<<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
+                       kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);
@@ -1581,8 +1588,9 @@ int attn_backward_run(float *grad_query, float *grad_edge, const int32_t *indptr
                           max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
     if (rc) return rc;
     if (!has_items) p.sp.plan.threshold = 0x7fffffff;
-    attn_bwd_rows_kernel<<<(int)ceil_div(n_dst, kWavesPerBlock * kRowsPerWave), kBlock, 0,
-                           stream>>>(p);
+    attn_bwd_rows_kernel<<<(int)ceil_div(p.sp.n_rows,
+                                         kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
+                           kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);

@@ -22,6 +22,7 @@ namespace yitu {
 
 constexpr int BM = 128, BN = 128, BK = 16, LDP = 132;  // LDP: padded LDS row (floats)
 constexpr int kMaxGroup = 8;
+constexpr int kMinSplitK = 128;  // shortest K range worth a workgroup of its own
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 
@@ -43,6 +44,7 @@ struct GemmParams {
     int64_t a_si, a_sk, b_sk, b_sj;
     int ldc;
     int accumulate;  // C += A.B instead of C = A.B
+    int a_vec4, b_vec4;  // bounds-checked tiles: 16-byte loads are all-or-nothing for this operand
     int max_m;       // slabs of `partial` are [max_m, N]
     float *partial;
 };
@@ -59,7 +61,7 @@ __device__ __forceinline__ int problem_of(const GemmParams &p, int z) {
 template <bool KCONT, bool FAST>
 __device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict__ base,
                                           int64_t s_row, int64_t s_k, int row0, int k0, int n_rows,
-                                          int K) {
+                                          int K, bool vec4) {
     const int t = threadIdx.x;
     if constexpr (KCONT) {
         const int row = row0 + (t >> 1), k = k0 + (t & 1) * 8;
@@ -69,6 +71,14 @@ __device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict
             const float4 b = *reinterpret_cast<const float4 *>(p + 4);
             r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
             r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+        } else if (vec4) {  // K and the row stride are multiples of 4: whole float4 or nothing
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float4 v = (row < n_rows && k + 4 * h + 4 <= K)
+                                     ? *reinterpret_cast<const float4 *>(p + 4 * h)
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                r[4 * h] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) r[i] = (row < n_rows && k + i < K) ? p[i] : 0.0f;
@@ -81,6 +91,14 @@ __device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict
             const float4 b = *reinterpret_cast<const float4 *>(p + 4);
             r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
             r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+        } else if (vec4) {  // the row count and the k stride are multiples of 4
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float4 v = (k < K && row + 4 * h + 4 <= n_rows)
+                                     ? *reinterpret_cast<const float4 *>(p + 4 * h)
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                r[4 * h] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) r[i] = (k < K && row + i < n_rows) ? p[i] : 0.0f;
@@ -124,8 +142,8 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     float ra[8], rb[8];
-    load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb, pr.M, ke);
-    load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb, p.N, ke);
+    load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb, pr.M, ke, p.a_vec4 != 0);
+    load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb, p.N, ke, p.b_vec4 != 0);
     store_tile<A_KCONT>(As[0], ra);
     store_tile<B_KCONT>(Bs[0], rb);
     __syncthreads();
@@ -134,8 +152,10 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
     for (int s = 0; s < n_steps; s++) {
         const int cur = s & 1;
         if (s + 1 < n_steps) {
-            load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb + (s + 1) * BK, pr.M, ke);
-            load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb + (s + 1) * BK, p.N, ke);
+            load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb + (s + 1) * BK, pr.M, ke,
+                                     p.a_vec4 != 0);
+            load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb + (s + 1) * BK, p.N, ke,
+                                     p.b_vec4 != 0);
         }
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
@@ -215,8 +235,8 @@ static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
         pr.z0 = z;
         pr.n_split = 1;
         pr.k_chunk = (int)(ceil_div(pr.K, BK) * BK);
-        if (tiles < 256 && pr.K >= 4096 && pr.M > 0) {
-            int64_t want = std::min<int64_t>(ceil_div(pr.K, 1024), ceil_div(1024, tiles));
+        if (tiles < 256 && pr.K >= 2 * kMinSplitK && pr.M > 0) {
+            int64_t want = std::min<int64_t>(ceil_div(pr.K, kMinSplitK), ceil_div(1024, tiles));
             want = std::min<int64_t>(want, slab_cap);
             if (want > 1) {
                 pr.k_chunk = (int)(ceil_div(ceil_div(pr.K, want), BK) * BK);
@@ -241,10 +261,23 @@ static int sgemm_launch(const GemmParams &p, int max_m, int n_z, hipStream_t str
     fast = fast && (A_KCONT ? p.a_si % 4 == 0 : p.a_sk % 4 == 0) &&
            (B_KCONT ? p.b_sj % 4 == 0 : p.b_sk % 4 == 0);
     dim3 grid((unsigned)ceil_div(p.N, BN), (unsigned)ceil_div(max_m, BM), (unsigned)n_z);
-    if (fast)
+    if (fast) {
         sgemm_mfma_kernel<A_KCONT, B_KCONT, true><<<grid, 256, 0, stream>>>(p);
-    else
-        sgemm_mfma_kernel<A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(p);
+    } else {
+        // ragged tiles: 16-byte loads still work where each one lies wholly inside or
+        // wholly outside the operand (contiguous extent a multiple of 4, aligned lines)
+        GemmParams q = p;
+        bool a4 = A_KCONT ? p.a_si % 4 == 0 : p.a_sk % 4 == 0;
+        bool b4 = (B_KCONT ? p.b_sj % 4 == 0 : p.b_sk % 4 == 0) && (B_KCONT || p.N % 4 == 0);
+        for (int i = 0; i < p.n_prob; i++) {
+            const GemmProblem &pr = p.prob[i];
+            a4 = a4 && aligned16(pr.A) && (A_KCONT ? pr.K % 4 == 0 : pr.M % 4 == 0);
+            b4 = b4 && aligned16(pr.B) && (!B_KCONT || pr.K % 4 == 0);
+        }
+        q.a_vec4 = a4;
+        q.b_vec4 = b4;
+        sgemm_mfma_kernel<A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(q);
+    }
     YITU_LAUNCH_CHECK();
     if (any_split) {
         dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)max_m * p.N, 256), 2048),
@@ -313,8 +346,8 @@ using namespace yitu;
 // Enough for the widest split the policy picks: 1024 / tiles slabs of [m, n].
 YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems) {
     const int64_t tiles = ceil_div(n, BN) * ceil_div(m, BM) * n_problems;
-    if (tiles <= 0 || tiles >= 256 || k < 4096) return 256;
-    const int64_t splits = std::min<int64_t>(ceil_div(k, 1024), ceil_div(1024, tiles));
+    if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return 256;
+    const int64_t splits = std::min<int64_t>(ceil_div(k, kMinSplitK), ceil_div(1024, tiles));
     return align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256);
 }
 

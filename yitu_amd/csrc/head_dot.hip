@@ -621,14 +621,21 @@ YITU_API int yitu_skinny_linear_backward(float *grad_x, int accumulate, float *g
 namespace yitu {
 namespace {
 
-constexpr int kColSumChunk = 64;  // rows per workgroup
+// rows per workgroup: 64 on large inputs, fewer on small ones so that a few thousand
+// rows still make a few hundred workgroups (and as many partial rows for the second step) (a function of n_rows alone: the workspace
+// size and the summation order follow from it)
+inline int col_sum_chunk(int64_t n_rows) {
+    const int64_t c = n_rows / 512;
+    return c < 8 ? 8 : (c > 64 ? 64 : (int)c);
+}
 
 __global__ __launch_bounds__(kBlock) void column_chunk_sum_kernel(float *__restrict__ partial,
                                                                   const float *__restrict__ x,
-                                                                  int n_rows, int n_cols) {
-    const int r0 = blockIdx.x * kColSumChunk, r1 = min(r0 + kColSumChunk, n_rows);
+                                                                  int n_rows, int n_cols, int chunk) {
+    const int r0 = blockIdx.x * chunk, r1 = min(r0 + chunk, n_rows);
     for (int c = threadIdx.x; c < n_cols; c += kBlock) {
         float s = 0.0f;
+#pragma unroll 8
         for (int r = r0; r < r1; r++) s += x[(size_t)r * n_cols + c];
         partial[(size_t)blockIdx.x * n_cols + c] = s;
     }
@@ -638,7 +645,8 @@ __global__ __launch_bounds__(kBlock) void column_chunk_sum_kernel(float *__restr
 }  // namespace yitu
 
 YITU_API size_t yitu_column_sum_workspace_bytes(int64_t n_rows, int64_t n_cols) {
-    return sizeof(float) * (size_t)std::max<int64_t>(ceil_div(n_rows, kColSumChunk), 1) * (size_t)n_cols;
+    return sizeof(float) * (size_t)std::max<int64_t>(ceil_div(n_rows, col_sum_chunk(n_rows)), 1) *
+           (size_t)n_cols;
 }
 
 YITU_API int yitu_column_sum(float *out, const float *x, int64_t n_rows, int64_t n_cols,
@@ -652,9 +660,11 @@ YITU_API int yitu_column_sum(float *out, const float *x, int64_t n_rows, int64_t
     YITU_REQUIRE(workspace && workspace_bytes >= yitu_column_sum_workspace_bytes(n_rows, n_cols),
                  "workspace too small: need %zu bytes",
                  yitu_column_sum_workspace_bytes(n_rows, n_cols));
-    const int chunks = (int)ceil_div(n_rows, kColSumChunk);
+    const int chunk = col_sum_chunk(n_rows);
+    const int chunks = (int)ceil_div(n_rows, chunk);
     float *partial = static_cast<float *>(workspace);
-    column_chunk_sum_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows, (int)n_cols);
+    column_chunk_sum_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows, (int)n_cols,
+                                                           chunk);
     YITU_LAUNCH_CHECK();
     partial_sum_kernel<<<(int)ceil_div(n_cols, kSumCols), kBlock, 0, stream>>>(
         out, (int)n_cols, nullptr, 0, partial, chunks);

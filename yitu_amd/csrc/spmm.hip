@@ -37,7 +37,7 @@ size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan) {
 
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 static int launch_variant(const SpmmParams &p, bool has_items, hipStream_t stream) {
-    const int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave);
+    const int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * rows_per_wave(p.n_rows));
     spmm_rows_kernel<VEC, G, KT, WMODE, TIN><<<grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (has_items) {
@@ -76,7 +76,7 @@ static int dispatch_shape(const SpmmParams &p, bool with_hub, hipStream_t stream
 template <int VEC>
 static int launch_tiny(const SpmmParams &p, bool has_items, hipStream_t stream) {
     tiny_rows_kernel<VEC>
-        <<<(int)ceil_div(p.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+        <<<(int)ceil_div(p.n_rows, kWavesPerBlock * rows_per_wave(p.n_rows)), kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (has_items && p.cols_are_edges) {
         // a row's edges are contiguous: sum them in place, no items

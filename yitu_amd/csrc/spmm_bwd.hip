@@ -104,13 +104,14 @@ __device__ __forceinline__ void load_grad_tile(float (&gt)[KT][VEC], const DotPa
     }
 }
 
-// Short rows: a wave walks kRowsPerWave consecutive rows through a sliding edge window.
+// Short rows: a wave walks rows_per_wave consecutive rows through a sliding edge window.
 template <int VEC, int G, int KT>
 __global__ __launch_bounds__(kBlock) void dot_rows_kernel(DotParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.sp.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.sp.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.sp.n_rows - r0);
+    const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     EdgeWindow win;
@@ -173,7 +174,7 @@ template <int VEC, int G, int KT>
 static int dot_launch(const DotParams &p, bool has_items, hipStream_t stream) {
     if (!p.long_rows_only) {
         dot_rows_kernel<VEC, G, KT>
-            <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * kRowsPerWave), kBlock, 0, stream>>>(p);
+            <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)), kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
     }
     if (has_items) {

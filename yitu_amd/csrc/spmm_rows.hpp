@@ -187,9 +187,18 @@ __device__ __forceinline__ void fold_slots(float (&acc)[KT][VEC]) {
             for (int i = 0; i < VEC; i++) acc[t][i] += __shfl_xor(acc[t][i], o, kWave);
 }
 
-constexpr int kRowsPerWave = 16;  // consecutive rows handled by one wave of the row kernel
+constexpr int kRowsPerWave = 16;  // most consecutive rows one wave of a row kernel handles
 
-// Row kernel: a wave walks kRowsPerWave consecutive rows. Their bounds come from
+// Rows per wave of the row kernels: 16 where that still leaves several thousand
+// waves, fewer on small graphs (one root per wave at 2,048 sampled roots), so a
+// small problem is spread over the chip instead of walked by a few waves. Host
+// (grid size) and device (row range of a wave) both derive it from n_rows.
+__host__ __device__ inline int rows_per_wave(int n_rows) {
+    const int r = n_rows / 4096;
+    return r < 1 ? 1 : (r > kRowsPerWave ? kRowsPerWave : r);
+}
+
+// Row kernel: a wave walks rows_per_wave consecutive rows. Their bounds come from
 // one coalesced indptr load, their edges from a sliding 64-edge window, so a
 // short row costs one round of feature gathers and nothing else that waits on
 // memory. Rows that the plan covers are skipped.
@@ -197,9 +206,10 @@ template <int VEC, int G, int KT, int WMODE, typename TIN>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
-    const int r0 = (blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave) * rpw;
     if (r0 >= p.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.n_rows - r0);
+    const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);  // end of this wave's edges
     const int sub = lane % G;
@@ -465,9 +475,10 @@ __device__ __forceinline__ void tiny_sum(float (&acc)[VEC], const TinyWindow<VEC
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
     const int lane = lane_id();
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int rpw = rows_per_wave(p.n_rows);
+    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.n_rows) return;
-    const int n_here = min(kRowsPerWave, p.n_rows - r0);
+    const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
     const int limit = __shfl(my_ptr, n_here, kWave);
     TinyWindow<VEC> win;

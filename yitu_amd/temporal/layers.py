@@ -14,33 +14,17 @@ import torch
 
 from .. import graph_ext
 from ..xgnn_h import block as xblock
-from ..xgnn_h import sparse
-
-
-class _ReplayableLinear(torch.autograd.Function):
-    """``F.linear`` whose bias gradient is a fixed-order column sum. torch's own reduction
-    clears an accumulator with a memset node, and such nodes do not replay reliably from a
-    captured HIP graph; with this the whole training step of the layer can be captured."""
-
-    @staticmethod
-    def forward(ctx, x, weight, bias):
-        ctx.save_for_backward(x, weight)
-        ctx.has_bias = bias is not None
-        return torch.nn.functional.linear(x, weight, bias)
-
-    @staticmethod
-    def backward(ctx, grad_y):
-        x, weight = ctx.saved_tensors
-        grad_y = grad_y.contiguous()
-        grad_x = grad_y @ weight if ctx.needs_input_grad[0] else None
-        grad_w = grad_y.t() @ x if ctx.needs_input_grad[1] else None
-        grad_b = graph_ext.column_sum(grad_y) if ctx.has_bias and ctx.needs_input_grad[2] else None
-        return grad_x, grad_w, grad_b
+from ..xgnn_h import bundle, sparse
 
 
 def _linear(layer: torch.nn.Linear, x):
+    """``layer(x)`` on the library's GEMM, with the bias gradient as a fixed-order column
+    sum: at these sizes (a few thousand rows, 100 to 272 columns) the products are several
+    times faster than the BLAS library's choice of kernel, and torch's own bias reduction
+    records a memset node that does not replay reliably from a captured HIP graph, so with
+    this the whole training step of the layer can be captured."""
     if x.is_cuda and x.dtype == torch.float32 and x.dim() == 2:
-        return _ReplayableLinear.apply(x, layer.weight, layer.bias)
+        return bundle.linear(x, layer.weight, layer.bias)
     return layer(x)
 
 
@@ -169,8 +153,9 @@ class TransfomerAttentionLayer(torch.nn.Module):
             Q = _linear(self.w_q, torch.cat(parts_q, dim=1))
         else:  # edge features only (layers.py:104-107)
             Q = torch.ones((n_dst, self.dim_out), device=dev)
-        K = _linear(self.w_k, kv_in).reshape(-1, self.num_head, head_dim).contiguous()
-        V = _linear(self.w_v, kv_in).reshape(-1, self.num_head, head_dim).contiguous()
+        K, V = bundle.linear_pair(kv_in, self.w_k, self.w_v)  # one grouped launch
+        K = K.reshape(-1, self.num_head, head_dim).contiguous()
+        V = V.reshape(-1, self.num_head, head_dim).contiguous()
         Q = Q.reshape(n_dst, self.num_head, head_dim).contiguous()
         # att = edge_softmax(LeakyReLU(sum_d Q*K)); fused_gsddmm applies LeakyReLU(0.2) +
         # softmax to (query + key): query = 0, key = the dot-product logits, one key per edge

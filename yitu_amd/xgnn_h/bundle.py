@@ -48,6 +48,30 @@ class SkinnyLinearFunction(autograd.Function):
         return grad_x, grad_w, grad_b
 
 
+class BiasAddFunction(autograd.Function):
+    """``y + bias`` whose bias gradient is the library's fixed-order column sum (torch's own
+    reduction clears an accumulator with a memset node, which does not replay reliably
+    from a captured HIP graph)."""
+
+    @staticmethod
+    def forward(ctx, y, bias):
+        return y + bias
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad):
+        grad_b = graph_ext.column_sum(grad.contiguous()) if ctx.needs_input_grad[1] else None
+        return grad, grad_b
+
+
+def _add_bias(y, bias):
+    if bias is None:
+        return y
+    if y.is_cuda and y.dim() == 2 and y.dtype == bias.dtype:
+        return BiasAddFunction.apply(y, bias)
+    return y + bias
+
+
 def bundled_linear(x, w_a, w_b, b_a=None, b_b=None):
     """``(x w_a^T + b_a, x w_b^T + b_b)`` for two weight matrices of equal shape applied
     to one 2-D input: with a handful of outputs one skinny product over the stacked
@@ -60,7 +84,7 @@ def bundled_linear(x, w_a, w_b, b_a=None, b_b=None):
         y = SkinnyLinearFunction.apply(x.contiguous(), torch.cat([w_a, w_b], dim=0), bias)
         return y[:, :n_out].contiguous(), y[:, n_out:].contiguous()
     y_a, y_b = GEMMBundleFunction.apply(x, w_a, w_b, b_a, b_b)
-    return (y_a if b_a is None else y_a + b_a, y_b if b_b is None else y_b + b_b)
+    return _add_bias(y_a, b_a), _add_bias(y_b, b_b)
 
 
 def linear_pair(x, linear_a, linear_b):
