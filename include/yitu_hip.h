@@ -195,7 +195,10 @@ int yitu_sddmm_backward(float *grad_query_device, float *grad_key_device, float 
  * row_stats_device [n_dst,H,2] (optional, fused kernel only) receives each row's
  * softmax (max, 1 / sum): with it the backward recomputes a probability from
  * query, key and these two numbers instead of reading attn, so attn need not be
- * stored at all.
+ * stored at all. With attn_device NULL the rows of 64 edges and more are summed
+ * from per-piece sums taken against each piece's own maximum: out then differs
+ * from the attn_device != NULL result in the last bits (same tolerance against
+ * the reference), and is reproducible from call to call like every other result.
  */
 size_t yitu_gat_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t n_heads, int64_t n_features,
                                 int with_plans);
