@@ -222,3 +222,29 @@ def test_gat_head_layer_equals_torch_composition(dev, h, f, bipartite):
     want = [y2.detach()] + [t.grad for t in inputs] + [p.grad for p in layer.parameters()]
     for a_, b_ in zip(got, want):
         assert_close(a_, b_, rtol=1e-4, atol=5e-4)
+
+
+@pytest.mark.parametrize("n_dst", [12288 + 5, 30000, 50001])
+def test_row_counts_between_the_rows_per_wave_steps(dev, n_dst):
+    """A wave of the row kernels takes n_rows / 4096 rows (1 to 16): row counts that give
+    3, 7 and 12 rows per wave, with a ragged last wave, a hub row and empty rows, through
+    the fused attention (4 x 64: every one-pass kernel), the attention-only ops and the
+    plain multi-head product."""
+    n_src, h, f = 3000, 4, 64
+    g = torch.Generator().manual_seed(n_dst)
+    deg = torch.randint(0, 9, (n_dst,), generator=g)
+    deg[n_dst // 2] = 300
+    indptr = torch.zeros(n_dst + 1, dtype=torch.int32)
+    indptr[1:] = torch.cumsum(deg, 0)
+    indices = torch.randint(0, n_src, (int(indptr[-1]),), generator=g, dtype=torch.int32)
+    _run(dev, indptr, indices, n_dst, n_src, h, f, seed=1, atol=5e-4)
+    d = lambda t: t.to(dev)
+    values = torch.randn(indices.numel(), h, generator=g)
+    x = torch.randn(n_src, h, 20, generator=g)
+    gy = torch.randn(n_dst, h, 20, generator=g)
+    got = graph_ext.spmm_forward(d(values), d(indptr), d(indices), d(x))
+    assert_close(got, oracle.mh_spmm_forward(values, indptr, indices, x))
+    ga, gx = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
+    want_ga, want_gx = oracle.mh_spmm_backward(values, indptr, indices, x, gy)
+    assert_close(ga, want_ga, atol=2e-4)
+    assert_close(gx, want_gx, atol=5e-4)
