@@ -20,7 +20,7 @@
 
 namespace yitu {
 
-constexpr int BM = 128, BN = 128, BK = 16, LDP = 132;  // LDP: padded LDS row (floats)
+constexpr int BK = 16;  // K-step
 constexpr int kMaxGroup = 8;
 constexpr int kMinSplitK = 128;  // shortest K range worth a workgroup of its own
 
@@ -55,25 +55,39 @@ __device__ __forceinline__ int problem_of(const GemmParams &p, int z) {
     return i;
 }
 
-// Loads this thread's 8 elements of a [128 x 16] operand tile into regs.
-// KCONT: the operand is contiguous along K (thread owns 8 consecutive k of one row),
-// otherwise contiguous along the row dimension (8 consecutive rows of one k).
-template <bool KCONT, bool FAST>
-__device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict__ base,
+// Tile geometry: a workgroup of 4 waves (2 x 2) owns a square tile of 64 * TM rows
+// and columns, each wave TM x TM MFMA tiles. TM = 2 (128 x 128) is the shape for
+// large products; TM = 1 (64 x 64, a quarter of the MFMAs per K-step and four
+// times the workgroups) is taken when the larger tiles would leave most CUs idle.
+template <int TM>
+struct TileGeom {
+    static constexpr int R = 64 * TM;       // rows (and columns) per workgroup tile
+    static constexpr int PER = 4 * TM;      // elements per thread and operand tile
+    static constexpr int LD = R + 4;        // padded LDS row, floats
+};
+
+// Loads this thread's PER elements of an [R x 16] operand tile into regs.
+// KCONT: the operand is contiguous along K (thread owns PER consecutive k of one row),
+// otherwise contiguous along the row dimension (PER consecutive rows of one k).
+template <int TM, bool KCONT, bool FAST>
+__device__ __forceinline__ void load_tile(float (&r)[4 * TM], const float *__restrict__ base,
                                           int64_t s_row, int64_t s_k, int row0, int k0, int n_rows,
                                           int K, bool vec4) {
+    constexpr int PER = TileGeom<TM>::PER;
     const int t = threadIdx.x;
     if constexpr (KCONT) {
-        const int row = row0 + (t >> 1), k = k0 + (t & 1) * 8;
+        constexpr int TPR = BK / PER;  // threads per row
+        const int row = row0 + t / TPR, k = k0 + (t % TPR) * PER;
         const float *p = base + (int64_t)row * s_row + k;
         if constexpr (FAST) {
-            const float4 a = *reinterpret_cast<const float4 *>(p);
-            const float4 b = *reinterpret_cast<const float4 *>(p + 4);
-            r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
-            r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+#pragma unroll
+            for (int h = 0; h < TM; h++) {
+                const float4 v = *reinterpret_cast<const float4 *>(p + 4 * h);
+                r[4 * h] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+            }
         } else if (vec4) {  // K and the row stride are multiples of 4: whole float4 or nothing
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < TM; h++) {
                 const float4 v = (row < n_rows && k + 4 * h + 4 <= K)
                                      ? *reinterpret_cast<const float4 *>(p + 4 * h)
                                      : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -81,19 +95,20 @@ __device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; i++) r[i] = (row < n_rows && k + i < K) ? p[i] : 0.0f;
+            for (int i = 0; i < PER; i++) r[i] = (row < n_rows && k + i < K) ? p[i] : 0.0f;
         }
     } else {
-        const int k = k0 + (t >> 4), row = row0 + (t & 15) * 8;
+        const int k = k0 + (t >> 4), row = row0 + (t & 15) * PER;
         const float *p = base + (int64_t)k * s_k + row;
         if constexpr (FAST) {
-            const float4 a = *reinterpret_cast<const float4 *>(p);
-            const float4 b = *reinterpret_cast<const float4 *>(p + 4);
-            r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
-            r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+#pragma unroll
+            for (int h = 0; h < TM; h++) {
+                const float4 v = *reinterpret_cast<const float4 *>(p + 4 * h);
+                r[4 * h] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+            }
         } else if (vec4) {  // the row count and the k stride are multiples of 4
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < TM; h++) {
                 const float4 v = (k < K && row + 4 * h + 4 <= n_rows)
                                      ? *reinterpret_cast<const float4 *>(p + 4 * h)
                                      : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -101,77 +116,84 @@ __device__ __forceinline__ void load_tile(float (&r)[8], const float *__restrict
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; i++) r[i] = (k < K && row + i < n_rows) ? p[i] : 0.0f;
+            for (int i = 0; i < PER; i++) r[i] = (k < K && row + i < n_rows) ? p[i] : 0.0f;
         }
     }
 }
 
-template <bool KCONT>
-__device__ __forceinline__ void store_tile(float (*tile)[LDP], const float (&r)[8]) {
+template <int TM, bool KCONT>
+__device__ __forceinline__ void store_tile(float (*tile)[TileGeom<TM>::LD], const float (&r)[4 * TM]) {
+    constexpr int PER = TileGeom<TM>::PER;
     const int t = threadIdx.x;
     if constexpr (KCONT) {
-        const int row = t >> 1, k = (t & 1) * 8;
+        constexpr int TPR = BK / PER;
+        const int row = t / TPR, k = (t % TPR) * PER;
 #pragma unroll
-        for (int i = 0; i < 8; i++) tile[k + i][row] = r[i];
+        for (int i = 0; i < PER; i++) tile[k + i][row] = r[i];
     } else {
-        const int k = t >> 4, row = (t & 15) * 8;
-        *reinterpret_cast<float4 *>(&tile[k][row]) = make_float4(r[0], r[1], r[2], r[3]);
-        *reinterpret_cast<float4 *>(&tile[k][row + 4]) = make_float4(r[4], r[5], r[6], r[7]);
+        const int k = t >> 4, row = (t & 15) * PER;
+#pragma unroll
+        for (int h = 0; h < TM; h++)
+            *reinterpret_cast<float4 *>(&tile[k][row + 4 * h]) =
+                make_float4(r[4 * h], r[4 * h + 1], r[4 * h + 2], r[4 * h + 3]);
     }
 }
 
-template <bool A_KCONT, bool B_KCONT, bool FAST>
+template <int TM, bool A_KCONT, bool B_KCONT, bool FAST>
 __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
-    __shared__ float As[2][BK][LDP];
-    __shared__ float Bs[2][BK][LDP];
+    constexpr int R = TileGeom<TM>::R, LD = TileGeom<TM>::LD, PER = TileGeom<TM>::PER;
+    __shared__ float As[2][BK][LD];
+    __shared__ float Bs[2][BK][LD];
     const GemmProblem pr = p.prob[problem_of(p, blockIdx.z)];
     const int split = blockIdx.z - pr.z0;
     const int kb = split * pr.k_chunk, ke = min(pr.K, kb + pr.k_chunk);
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int m0 = blockIdx.y * R, n0 = blockIdx.x * R;
     if (m0 >= pr.M) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int wm = (wave >> 1) * 32 * TM, wn = (wave & 1) * 32 * TM;
     const int l32 = lane & 31, lk = lane >> 5;
 
-    float16v acc[2][2];
+    float16v acc[TM][TM];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TM; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    float ra[8], rb[8];
-    load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb, pr.M, ke, p.a_vec4 != 0);
-    load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb, p.N, ke, p.b_vec4 != 0);
-    store_tile<A_KCONT>(As[0], ra);
-    store_tile<B_KCONT>(Bs[0], rb);
+    float ra[PER], rb[PER];
+    load_tile<TM, A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb, pr.M, ke, p.a_vec4 != 0);
+    load_tile<TM, B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb, p.N, ke, p.b_vec4 != 0);
+    store_tile<TM, A_KCONT>(As[0], ra);
+    store_tile<TM, B_KCONT>(Bs[0], rb);
     __syncthreads();
 
     const int n_steps = (ke - kb + BK - 1) / BK;
     for (int s = 0; s < n_steps; s++) {
         const int cur = s & 1;
         if (s + 1 < n_steps) {
-            load_tile<A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb + (s + 1) * BK, pr.M, ke,
-                                     p.a_vec4 != 0);
-            load_tile<B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb + (s + 1) * BK, p.N, ke,
-                                     p.b_vec4 != 0);
+            load_tile<TM, A_KCONT, FAST>(ra, pr.A, p.a_si, p.a_sk, m0, kb + (s + 1) * BK, pr.M, ke,
+                                         p.a_vec4 != 0);
+            load_tile<TM, B_KCONT, FAST>(rb, pr.B, p.b_sj, p.b_sk, n0, kb + (s + 1) * BK, p.N, ke,
+                                         p.b_vec4 != 0);
         }
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            const float a0 = As[cur][kk + lk][wm + l32];
-            const float a1 = As[cur][kk + lk][wm + 32 + l32];
-            const float b0 = Bs[cur][kk + lk][wn + l32];
-            const float b1 = Bs[cur][kk + lk][wn + 32 + l32];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            float a[TM], b[TM];
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[i] = As[cur][kk + lk][wm + 32 * i + l32];
+#pragma unroll
+            for (int j = 0; j < TM; j++) b[j] = Bs[cur][kk + lk][wn + 32 * j + l32];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         if (s + 1 < n_steps) {
             // the other buffer was last read in step s-1, before the barrier below
-            store_tile<A_KCONT>(As[cur ^ 1], ra);
-            store_tile<B_KCONT>(Bs[cur ^ 1], rb);
+            store_tile<TM, A_KCONT>(As[cur ^ 1], ra);
+            store_tile<TM, B_KCONT>(Bs[cur ^ 1], rb);
         }
         __syncthreads();
     }
@@ -186,9 +208,9 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
         accumulate = false;
     }
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int j = 0; j < TM; j++) {
             const int col = n0 + wn + 32 * j + l32;
 #pragma unroll
             for (int jj = 0; jj < 4; jj++)
@@ -223,10 +245,10 @@ __global__ __launch_bounds__(256) void sgemm_splitk_reduce_kernel(GemmParams p) 
 // Few output tiles and a long inner dimension (dW = X^T.G with K = number of
 // nodes): split K so the whole chip works, partials summed by a second kernel.
 // Returns the number of blockIdx.z values.
-static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
+static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes, int tile) {
     p.max_m = max_m;
     int64_t tiles = 0;
-    for (int i = 0; i < p.n_prob; i++) tiles += ceil_div(p.N, BN) * ceil_div(p.prob[i].M, BM);
+    for (int i = 0; i < p.n_prob; i++) tiles += ceil_div(p.N, tile) * ceil_div(p.prob[i].M, tile);
     const int64_t slab = (int64_t)max_m * p.N * sizeof(float);
     const int64_t slab_cap = slab > 0 ? (int64_t)(workspace_bytes / slab) / p.n_prob : 0;
     int z = 0;
@@ -248,21 +270,30 @@ static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes) {
     return z;
 }
 
-template <bool A_KCONT, bool B_KCONT>
-static int sgemm_launch(const GemmParams &p, int max_m, int n_z, hipStream_t stream) {
-    bool fast = p.N % BN == 0, any_split = false;
+// 128 x 128 tiles when they give the chip enough workgroups, 64 x 64 otherwise
+constexpr int kFillTiles = 192;
+static int pick_tile(int64_t n, const int64_t *m, int n_prob, int64_t same_m) {
+    int64_t tiles = 0;
+    for (int i = 0; i < n_prob; i++) tiles += ceil_div(n, 128) * ceil_div(m ? m[i] : same_m, 128);
+    return tiles >= kFillTiles ? 128 : 64;
+}
+
+template <int TM, bool A_KCONT, bool B_KCONT>
+static int sgemm_launch_tile(const GemmParams &p, int max_m, int n_z, hipStream_t stream) {
+    constexpr int R = TileGeom<TM>::R;
+    bool fast = p.N % R == 0, any_split = false;
     for (int i = 0; i < p.n_prob; i++) {
         const GemmProblem &pr = p.prob[i];
-        fast = fast && pr.M % BM == 0 && pr.K % BK == 0 && pr.K > 0 && aligned16(pr.A) &&
+        fast = fast && pr.M % R == 0 && pr.K % BK == 0 && pr.K > 0 && aligned16(pr.A) &&
                aligned16(pr.B);
         any_split = any_split || pr.n_split > 1;
     }
     // vector loads also need every row / k-line to start 16-byte aligned
     fast = fast && (A_KCONT ? p.a_si % 4 == 0 : p.a_sk % 4 == 0) &&
            (B_KCONT ? p.b_sj % 4 == 0 : p.b_sk % 4 == 0);
-    dim3 grid((unsigned)ceil_div(p.N, BN), (unsigned)ceil_div(max_m, BM), (unsigned)n_z);
+    dim3 grid((unsigned)ceil_div(p.N, R), (unsigned)ceil_div(max_m, R), (unsigned)n_z);
     if (fast) {
-        sgemm_mfma_kernel<A_KCONT, B_KCONT, true><<<grid, 256, 0, stream>>>(p);
+        sgemm_mfma_kernel<TM, A_KCONT, B_KCONT, true><<<grid, 256, 0, stream>>>(p);
     } else {
         // ragged tiles: 16-byte loads still work where each one lies wholly inside or
         // wholly outside the operand (contiguous extent a multiple of 4, aligned lines)
@@ -276,7 +307,7 @@ static int sgemm_launch(const GemmParams &p, int max_m, int n_z, hipStream_t str
         }
         q.a_vec4 = a4;
         q.b_vec4 = b4;
-        sgemm_mfma_kernel<A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(q);
+        sgemm_mfma_kernel<TM, A_KCONT, B_KCONT, false><<<grid, 256, 0, stream>>>(q);
     }
     YITU_LAUNCH_CHECK();
     if (any_split) {
@@ -286,6 +317,12 @@ static int sgemm_launch(const GemmParams &p, int max_m, int n_z, hipStream_t str
         YITU_LAUNCH_CHECK();
     }
     return 0;
+}
+
+template <bool A_KCONT, bool B_KCONT>
+static int sgemm_launch(const GemmParams &p, int tile, int max_m, int n_z, hipStream_t stream) {
+    if (tile == 128) return sgemm_launch_tile<2, A_KCONT, B_KCONT>(p, max_m, n_z, stream);
+    return sgemm_launch_tile<1, A_KCONT, B_KCONT>(p, max_m, n_z, stream);
 }
 
 // trans_a: A is given as [K, M] row-major (else [M, K]); trans_b: B is given as
@@ -316,7 +353,10 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
     int max_m = 0;
     for (int i = 0; i < p.n_prob; i++) max_m = std::max(max_m, p.prob[i].M);
     if (max_m == 0 || p.N == 0) return 0;
-    const int n_z = choose_split(p, max_m, workspace ? workspace_bytes : 0);
+    int64_t heights[kMaxGroup];
+    for (int i = 0; i < p.n_prob; i++) heights[i] = p.prob[i].M;
+    const int tile = pick_tile(p.N, heights, p.n_prob, 0);
+    const int n_z = choose_split(p, max_m, workspace ? workspace_bytes : 0, tile);
     p.partial = static_cast<float *>(workspace);
     if (trans_a) {  // element (i,k) at A[k*lda + i]: contiguous along rows
         p.a_si = 1;
@@ -332,10 +372,10 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
         p.b_sk = ldb;
         p.b_sj = 1;
     }
-    if (!trans_a && trans_b) return sgemm_launch<true, true>(p, max_m, n_z, stream);
-    if (!trans_a && !trans_b) return sgemm_launch<true, false>(p, max_m, n_z, stream);
-    if (trans_a && !trans_b) return sgemm_launch<false, false>(p, max_m, n_z, stream);
-    return sgemm_launch<false, true>(p, max_m, n_z, stream);
+    if (!trans_a && trans_b) return sgemm_launch<true, true>(p, tile, max_m, n_z, stream);
+    if (!trans_a && !trans_b) return sgemm_launch<true, false>(p, tile, max_m, n_z, stream);
+    if (trans_a && !trans_b) return sgemm_launch<false, false>(p, tile, max_m, n_z, stream);
+    return sgemm_launch<false, true>(p, tile, max_m, n_z, stream);
 }
 
 }  // namespace yitu
@@ -345,7 +385,8 @@ using namespace yitu;
 
 // Enough for the widest split the policy picks: 1024 / tiles slabs of [m, n].
 YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems) {
-    const int64_t tiles = ceil_div(n, BN) * ceil_div(m, BM) * n_problems;
+    const int tile = pick_tile(n, nullptr, (int)std::min<int64_t>(n_problems, kMaxGroup), m);
+    const int64_t tiles = ceil_div(n, tile) * ceil_div(m, tile) * n_problems;
     if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return 256;
     const int64_t splits = std::min<int64_t>(ceil_div(k, kMinSplitK), ceil_div(1024, tiles));
     return align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256);
