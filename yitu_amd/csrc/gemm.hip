@@ -270,8 +270,9 @@ static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes, int ti
     return z;
 }
 
-// 128 x 128 tiles when they give the chip enough workgroups, 64 x 64 otherwise
-constexpr int kFillTiles = 192;
+// 128 x 128 tiles when they fill every CU to the kernel's occupancy (3 workgroups each),
+// 64 x 64 otherwise
+constexpr int kFillTiles = 768;
 static int pick_tile(int64_t n, const int64_t *m, int n_prob, int64_t same_m) {
     int64_t tiles = 0;
     for (int i = 0; i < n_prob; i++) tiles += ceil_div(n, 128) * ceil_div(m ? m[i] : same_m, 128);

@@ -625,7 +625,7 @@ namespace {
 // rows still make a few hundred workgroups (and as many partial rows for the second step) (a function of n_rows alone: the workspace
 // size and the summation order follow from it)
 inline int col_sum_chunk(int64_t n_rows) {
-    const int64_t c = n_rows / 512;
+    const int64_t c = n_rows / 256;
     return c < 8 ? 8 : (c > 64 ? 64 : (int)c);
 }
 
