@@ -28,6 +28,34 @@ def _linear(layer: torch.nn.Linear, x):
     return layer(x)
 
 
+class _DotAttentionFunction(torch.autograd.Function):
+    """agg[r] = sum_e softmax_r(LeakyReLU_0.2(<Q[r], K[e]>)) V[e] over a block whose edge e
+    has its own source row e: ``sparse.edge_dot`` -> ``sparse.fused_gsddmm`` (zero query,
+    the logits as per-edge keys) -> ``sparse.gspmm`` on the same kernels, as one autograd
+    node (each node costs more host time than its kernels take at these sizes)."""
+
+    @staticmethod
+    def forward(ctx, adj_sparse, Q, K, V):
+        indptr, indices = adj_sparse
+        logits = graph_ext.edge_dot(indptr, indices, Q, K)
+        zeros = torch.zeros((1, Q.size(0), Q.size(1)), device=Q.device)
+        att = graph_ext.sddmm_forward(indptr, indices, zeros, logits)
+        ctx.adj_sparse = adj_sparse
+        ctx.save_for_backward(Q, K, V, logits, att, zeros)
+        return graph_ext.spmm_forward(att, indptr, indices, V)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_agg):
+        indptr, indices = ctx.adj_sparse
+        Q, K, V, logits, att, zeros = ctx.saved_tensors
+        grad_att, grad_v = graph_ext.spmm_backward(att, indptr, indices, V, grad_agg.contiguous())
+        _, grad_logits = graph_ext.sddmm_backward(indptr, indices, zeros, logits, att, grad_att)
+        grad_q = graph_ext.spmm_forward(grad_logits, indptr, indices, K)
+        _, grad_k = graph_ext.spmm_backward(grad_logits, indptr, indices, K, Q, need_grad_a=False)
+        return None, grad_q, grad_k, grad_v
+
+
 class TimeEncode(torch.nn.Module):
     """cos(t * w + b), w_i = 10^(-9 i / (dim - 1)), b = 0, both trainable (layers.py:6-17)."""
 
@@ -159,15 +187,14 @@ class TransfomerAttentionLayer(torch.nn.Module):
         Q = Q.reshape(n_dst, self.num_head, head_dim).contiguous()
         # att = edge_softmax(LeakyReLU(sum_d Q*K)); fused_gsddmm applies LeakyReLU(0.2) +
         # softmax to (query + key): query = 0, key = the dot-product logits, one key per edge
-        logits = sparse.edge_dot(b.blk, Q, K)
-        zeros = torch.zeros((n_dst, self.num_head), device=dev)
-        if logits.requires_grad:
+        if self.training and self.att_dropout.p > 0:
+            logits = sparse.edge_dot(b.blk, Q, K)
+            zeros = torch.zeros((n_dst, self.num_head), device=dev)
             att = sparse.fused_gsddmm(b.blk, zeros.requires_grad_(), logits)
+            agg = sparse.gspmm(b.blk, self.att_dropout(att), V)
         else:
-            att = graph_ext.sddmm_forward(b.blk.adj_sparse[0], b.blk.adj_sparse[1],
-                                          zeros.unsqueeze(0), logits)
-        att = self.att_dropout(att)
-        agg = sparse.gspmm(b.blk, att, V).reshape(n_dst, self.dim_out)
+            agg = _DotAttentionFunction.apply(b.blk.adj_sparse, Q, K, V)
+        agg = agg.reshape(n_dst, self.dim_out)
         rst = torch.cat([agg, b.h[:n_dst]], dim=1) if self.dim_node_feat != 0 else agg
         rst = _linear(self.w_out, rst)
         rst = torch.nn.functional.relu(self.dropout(rst))

@@ -48,28 +48,30 @@ class SkinnyLinearFunction(autograd.Function):
         return grad_x, grad_w, grad_b
 
 
-class BiasAddFunction(autograd.Function):
-    """``y + bias`` whose bias gradient is the library's fixed-order column sum (torch's own
-    reduction clears an accumulator with a memset node, which does not replay reliably
-    from a captured HIP graph)."""
+class LinearPairFunction(autograd.Function):
+    """``(x w_a^T + b_a, x w_b^T + b_b)``: the grouped product of ``GEMMBundleFunction`` with
+    the biases inside, their gradients as the library's fixed-order column sums (torch's own
+    reduction clears an accumulator with a memset node, which does not replay reliably from
+    a captured HIP graph)."""
 
     @staticmethod
-    def forward(ctx, y, bias):
-        return y + bias
+    def forward(ctx, x, w_a, w_b, b_a, b_b):
+        ctx.save_for_backward(x, w_a, w_b)
+        y_a, y_b = graph_ext.b2gemm(x, w_a, w_b)
+        if b_a is not None:
+            y_a.add_(b_a)
+        if b_b is not None:
+            y_b.add_(b_b)
+        return y_a, y_b
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, grad):
-        grad_b = graph_ext.column_sum(grad.contiguous()) if ctx.needs_input_grad[1] else None
-        return grad, grad_b
-
-
-def _add_bias(y, bias):
-    if bias is None:
-        return y
-    if y.is_cuda and y.dim() == 2 and y.dtype == bias.dtype:
-        return BiasAddFunction.apply(y, bias)
-    return y + bias
+    def backward(ctx, grad_a, grad_b):
+        grad_a, grad_b = grad_a.contiguous(), grad_b.contiguous()
+        dx, dw_a, dw_b = graph_ext.b2gemm_backward(*ctx.saved_tensors, grad_a, grad_b)
+        db_a = graph_ext.column_sum(grad_a) if ctx.needs_input_grad[3] else None
+        db_b = graph_ext.column_sum(grad_b) if ctx.needs_input_grad[4] else None
+        return dx, dw_a, dw_b, db_a, db_b
 
 
 def bundled_linear(x, w_a, w_b, b_a=None, b_b=None):
@@ -83,8 +85,9 @@ def bundled_linear(x, w_a, w_b, b_a=None, b_b=None):
         bias = None if b_a is None else torch.cat([b_a, b_b])
         y = SkinnyLinearFunction.apply(x.contiguous(), torch.cat([w_a, w_b], dim=0), bias)
         return y[:, :n_out].contiguous(), y[:, n_out:].contiguous()
-    y_a, y_b = GEMMBundleFunction.apply(x, w_a, w_b, b_a, b_b)
-    return _add_bias(y_a, b_a), _add_bias(y_b, b_b)
+    if b_a is None and b_b is None:
+        return GEMMBundleFunction.apply(x, w_a, w_b, None, None)
+    return LinearPairFunction.apply(x, w_a, w_b, b_a, b_b)
 
 
 def linear_pair(x, linear_a, linear_b):
