@@ -270,13 +270,18 @@ static int choose_split(GemmParams &p, int max_m, size_t workspace_bytes, int ti
     return z;
 }
 
-// 128 x 128 tiles when they fill every CU to the kernel's occupancy (3 workgroups each),
-// 64 x 64 otherwise
+// 128 x 128 tiles when they, times the K splits a long inner dimension allows, fill every
+// CU to the kernel's occupancy (3 workgroups each); 64 x 64 tiles otherwise
 constexpr int kFillTiles = 768;
-static int pick_tile(int64_t n, const int64_t *m, int n_prob, int64_t same_m) {
+static int pick_tile(int64_t n, const int64_t *m, int n_prob, int64_t same_m, int64_t k_max) {
     int64_t tiles = 0;
     for (int i = 0; i < n_prob; i++) tiles += ceil_div(n, 128) * ceil_div(m ? m[i] : same_m, 128);
-    return tiles >= kFillTiles ? 128 : 64;
+    if (tiles <= 0) return 64;
+    int64_t splits = 1;
+    if (k_max >= 2 * kMinSplitK)
+        splits = std::max<int64_t>(1, std::min<int64_t>(ceil_div(k_max, kMinSplitK),
+                                                        ceil_div(1024, tiles)));
+    return tiles * splits >= kFillTiles ? 128 : 64;
 }
 
 template <int TM, bool A_KCONT, bool B_KCONT>
@@ -355,8 +360,13 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
     for (int i = 0; i < p.n_prob; i++) max_m = std::max(max_m, p.prob[i].M);
     if (max_m == 0 || p.N == 0) return 0;
     int64_t heights[kMaxGroup];
-    for (int i = 0; i < p.n_prob; i++) heights[i] = p.prob[i].M;
-    const int tile = pick_tile(p.N, heights, p.n_prob, 0);
+    int64_t k_max = 0;
+    for (int i = 0; i < p.n_prob; i++) {
+        heights[i] = p.prob[i].M;
+        k_max = std::max<int64_t>(k_max, p.prob[i].K);
+    }
+    // (without a workspace there are no splits to count on)
+    const int tile = pick_tile(p.N, heights, p.n_prob, 0, workspace ? k_max : 0);
     const int n_z = choose_split(p, max_m, workspace ? workspace_bytes : 0, tile);
     p.partial = static_cast<float *>(workspace);
     if (trans_a) {  // element (i,k) at A[k*lda + i]: contiguous along rows
@@ -386,7 +396,7 @@ using namespace yitu;
 
 // Enough for the widest split the policy picks: 1024 / tiles slabs of [m, n].
 YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems) {
-    const int tile = pick_tile(n, nullptr, (int)std::min<int64_t>(n_problems, kMaxGroup), m);
+    const int tile = pick_tile(n, nullptr, (int)std::min<int64_t>(n_problems, kMaxGroup), m, k);
     const int64_t tiles = ceil_div(n, tile) * ceil_div(m, tile) * n_problems;
     if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return 256;
     const int64_t splits = std::min<int64_t>(ceil_div(k, kMinSplitK), ceil_div(1024, tiles));
