@@ -495,6 +495,7 @@ def run_c4(args, dev):
     t_torch16 = _event_ms(lambda: [torch.mm(x, w) for x, w in zip(xs16, wts16)], steps, warm)
     bytes16 = sum(2 * n * dim * 2 + 2 * dim * dim for n in sizes)
     gather = n_edges * dim * 4
+    module_ms = _c4_module_ms(sizes, rels, dim, dev, steps, warm)
     peak = 157.3  # fp32 matrix TFLOP/s, published
     return {"value": n_edges / (total * 1e-3), "unit": "edges/s", "ms_per_step": total, "dtype": "f32",
             "config": {"workload": "c4_rgcn_f32", "node_types": sizes, "relations": 8,
@@ -504,6 +505,7 @@ def run_c4(args, dev):
             "gemm_bwd_ms": t_gemm_b, "torch_mm_fwd_ms": t_torch,
             "agg_fwd_by_relation_ms": t_agg_rel,
             "agg_gather_GBps": gather / (t_agg_f * 1e-3) / 1e9,
+            "modules": module_ms,
             "bf16": {"gemm_fwd_ms": t_gemm16, "agg_fwd_ms": t_agg16,
                      "torch_mm_fwd_ms": t_torch16,
                      "gemm_TFLOPs": flops_f / (t_gemm16 * 1e-3) / 1e12,
@@ -518,6 +520,67 @@ def run_c4(args, dev):
                                    "grouped launch",
                          "kernel_ms": t_gemm_f, "flops": flops_f,
                          "bwd_achieved": 2 * flops_f / (t_gemm_b * 1e-3) / 1e12}}
+
+
+def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
+    """The same layer at module level, through autograd: the stacked layer module with one
+    Linear per node type and with one per relation (the reference model's form), and the
+    reference's own 2-layer RGCN model (embedding, HeteroGraphConv over GCNLayers, ReLU,
+    HeteroGraphConv) captured, lowered and executed relation by relation on these kernels,
+    beside the same model built from two stacked layer modules."""
+    from yitu_amd import xgnn_h
+    from yitu_amd.xgnn_h import block as xblock, layers as xl, models, mp
+    names = ["t%d" % i for i in range(4)]
+    ntypes = {names[i]: sizes[i] for i in range(4)}
+    blocks, norms = {}, {}
+    for r, (s_t, d_t, rp, ci, norm) in enumerate(rels):
+        key = (names[s_t], "r%d" % r, names[d_t])
+        blocks[key] = xblock.Block([sizes[d_t], sizes[s_t]], [rp, ci])
+        blocks[key].right_norm = norm
+        norms[str(key)] = norm
+    g = torch.Generator(device=dev).manual_seed(7)
+    xs = {n: torch.randn(c, dim, generator=g, device=dev).requires_grad_() for n, c in ntypes.items()}
+    gy = {n: torch.randn(c, dim, generator=g, device=dev) for n, c in ntypes.items()}
+    res = {}
+
+    def train_step(forward, params):
+        def run():
+            out = forward()
+            torch.autograd.backward([out[n] for n in out], [gy[n] for n in out])
+            for t in params:
+                t.grad = None
+        return run
+
+    for per_relation, tag in ((False, "stacked_layer_per_type_fwd_bwd_ms"),
+                              (True, "stacked_layer_per_relation_fwd_bwd_ms")):
+        layer = xl.StackedHeteroGCN(ntypes, list(blocks), dim, dim, per_relation=per_relation).to(dev)
+        layer.stack(blocks, norms)
+        params = list(xs.values()) + list(layer.parameters())
+        res[tag] = _event_ms(train_step(lambda: layer(xs), params), steps, warm)
+        del layer
+    # the reference's model code, unchanged, through capture -> lower -> execute
+    hg = mp.HeteroGraph.from_blocks(ntypes, blocks, device=dev)
+    torch.manual_seed(7)
+    model = models.RGCNModel(hg, dim, dim, dim).to(dev)
+    kwargs = {"hgraph": hg, "xs": {n: torch.arange(c, device=dev) for n, c in ntypes.items()},
+              "norms": {str(rel): gr.right_norm() for rel, gr in hg.hetero_graph.items()}}
+    lowered = xgnn_h.Optimizer().lower(xgnn_h.Module2IR().transform(model, kwargs), kwargs)
+    executor = xgnn_h.Executor()
+    executor.train()
+    res["reference_model_2_layers_lowered_fwd_bwd_ms"] = _event_ms(
+        train_step(lambda: executor.run(lowered, kwargs), list(model.parameters())), steps, warm)
+    # the same model from two stacked layer modules
+    l1 = xl.StackedHeteroGCN(ntypes, list(blocks), dim, dim, per_relation=True).to(dev)
+    l2 = xl.StackedHeteroGCN(ntypes, list(blocks), dim, dim, per_relation=True).to(dev)
+    stacked = l1.stack(blocks, norms)
+
+    def two_layers():
+        hidden = l1(model.em(hg, kwargs["xs"]), stacked)
+        return l2({n: torch.relu(h) for n, h in hidden.items()}, stacked)
+
+    params = list(model.em.parameters()) + list(l1.parameters()) + list(l2.parameters())
+    res["stacked_model_2_layers_fwd_bwd_ms"] = _event_ms(train_step(two_layers, params), steps, warm)
+    return res
 
 
 def run_c5(args, dev):

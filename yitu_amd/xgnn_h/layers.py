@@ -245,5 +245,7 @@ class StackedHeteroGCN(nn.Module):
                                *[fc.bias for fc in fcs])
         out = sparse.gspmm(blk, values, h.unsqueeze(1)).squeeze(1)
         reached = {dty for _, _, dty in self.relations}
-        return {nty: out[self.row_offset[nty]:self.row_offset[nty] + n]
-                for nty, n in self.ntypes.items() if nty in reached}
+        # one split (its backward is one concatenation) rather than a slice per type (each
+        # slice's backward would be a zero-filled buffer of the full height)
+        pieces = out.split(list(self.ntypes.values()))
+        return {nty: piece for nty, piece in zip(self.ntypes, pieces) if nty in reached}
