@@ -58,7 +58,13 @@ def ptr(t):
     return c_ptr(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device):
+    """The current HIP stream of ``device`` as a pointer argument."""
+    if _raw_stream is not None and device.index is not None:
+        return c_ptr(_raw_stream(device.index))  # no Stream object on the way
     return c_ptr(torch.cuda.current_stream(device).cuda_stream)
 
 
