@@ -259,6 +259,13 @@ def run_gat(args, dev):
     sd_fwd_ms = _event_ms(lambda: graph_ext.sddmm_forward(rp, ci, q1, k), args.steps, args.warmup)
     sd_bwd_ms = _event_ms(lambda: graph_ext.sddmm_backward(rp, ci, q1, k, attn_sa, ga), args.steps,
                           args.warmup)
+    # and the stand-alone edge-weighted multi-head product with those probabilities
+    gy_sp = torch.randn(n, h, f, generator=g, device=dev)
+    sp_fwd_ms = _event_ms(lambda: graph_ext.spmm_forward(attn_sa, rp, ci, x), args.steps, args.warmup)
+    sp_bwd_ms = _event_ms(lambda: graph_ext.spmm_backward(attn_sa, rp, ci, x, gy_sp), args.steps,
+                          args.warmup)
+    alg_sp = 4 * (n + 1) + 4 * nnz + 4 * nnz * h + 2 * 4 * n * h * f
+    del gy_sp
     # layer level, through autograd. (a) the configuration's layer: per-head projections
     # q = <a_dst, x'>, k = <a_src, x'>, fused attention, mean over heads; (b) the
     # reference's GATLayer (test/common/model.py:61-106): linear_v 256 -> 4x64, dense
@@ -325,12 +332,17 @@ def run_gat(args, dev):
                   "fwd_algorithmic_bytes": alg_sd,
                   "fwd_GBps": alg_sd / (sd_fwd_ms * 1e-3) / 1e9,
                   "fwd_hbm_frac": alg_sd / (sd_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "weighted_spmm": {"fwd_ms": sp_fwd_ms, "bwd_ms": sp_bwd_ms,
+                          "edges_per_s_fwd_bwd": nnz / ((sp_fwd_ms + sp_bwd_ms) * 1e-3),
+                          "fwd_algorithmic_bytes": alg_sp,
+                          "fwd_hbm_frac": alg_sp / (sp_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "achieved": alg_fwd / (fwd_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get("c2_gat_f32"),
-                     "kernel": "yitu_gat_forward = gat_rows_kernel + gat_item_stats + "
-                               "gat_row_combine + gat_item_apply + spmm_reduce",
+                     "kernel": "yitu_gat_forward (row statistics out, no stored probabilities) = "
+                               "gat_rows_kernel + gat_item_local_kernel + gat_row_combine_kernel "
+                               "+ gat_scaled_reduce_kernel",
                      "kernel_ms": fwd_ms, "algorithmic_bytes": alg_fwd,
                      "bwd_achieved": alg_bwd / (bwd_ms * 1e-3) / 1e9,
                      "bwd_algorithmic_bytes": alg_bwd},
@@ -785,7 +797,7 @@ def main():
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
                                                 "roofline", "fwd_ms", "bwd_ms", "layer_fwd_bwd_ms",
                                                 "reference_gatlayer_fwd_bwd_ms", "gat_model_2_layers",
-                                                "sddmm")
+                                                "sddmm", "weighted_spmm")
                               if k in r}
             res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
                             "c2_gat_f32": slim(run_gat(args, dev)),
