@@ -362,3 +362,29 @@ def test_graph_without_edges(dev, n_dst, n_src):
     leaves = [t.clone().requires_grad_() for t in (q, k, x)]
     sparse.fused_gat(blk, *leaves).sum().backward()
     assert all(zeros(t.grad, *t.shape) for t in leaves)
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (2, 128), (1, 256)])
+def test_spmm_backward_one_gather_shapes(dev, h, f):
+    """Rows of 256 floats: both gradients come from one pass over the by-source
+    structure; against the oracle, with hub rows on both sides, and equal to the
+    two-pass form (asked for one gradient at a time)."""
+    indptr, indices = powerlaw_graph(12, 70000, 31 * h + f)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(h + f)
+    values = torch.randn(indices.numel(), h, generator=g)
+    x = torch.randn(n, h, f, generator=g)
+    gy = torch.randn(n, h, f, generator=g)
+    d = lambda t: t.to(dev)
+    ga, gx = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
+    want_ga, want_gx = oracle.mh_spmm_backward(values, indptr, indices, x, gy)
+    assert_close(ga, want_ga, atol=5e-4)
+    assert_close(gx, want_gx, atol=1e-3)
+    ga2, _ = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy),
+                                     need_grad_x=False)
+    _, gx2 = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy),
+                                     need_grad_a=False)
+    assert_close(ga, ga2, atol=5e-4)
+    assert_close(gx, gx2, atol=1e-3)
+    again = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
+    assert torch.equal(again[0], ga) and torch.equal(again[1], gx)

@@ -1464,6 +1464,59 @@ static int gat_src_launch(const GatSrcParams &p, bool has_items, const float *gr
     return -1;
 }
 
+// ---- the by-source pass for a plain edge-weighted product -------------------------
+// grad_a[e,h] = <grad_out[row_e,h,:], x[col_e,h,:]> and grad_x[c] = sum_e values[e,h]
+// grad_out[row_e] from the same single gather of grad_out rows (rows of 256 floats, head
+// width 32 to 256 a power of two): what yitu_spmm_backward otherwise does in two passes,
+// one gathering x[col] by destination and one gathering grad_out[row] by source.
+bool spmm_backward_one_gather_shape(int64_t n_heads, int64_t n_features, const float *features,
+                                    const float *grad_out, const float *grad_x) {
+    const int64_t lph = n_features / 4;
+    return n_heads * n_features == 256 && n_features % 4 == 0 && lph >= 8 && lph <= 64 &&
+           (lph & (lph - 1)) == 0 && aligned16(features) && aligned16(grad_out) &&
+           aligned16(grad_x);
+}
+
+int spmm_backward_one_gather(float *grad_a, float *grad_x, const float *values,
+                             const float *features, const float *grad_out,
+                             const int32_t *t_indptr, const int32_t *t_rows, const int32_t *t_perm,
+                             int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                             int64_t n_features, int64_t max_degree_t, const void *plan_t,
+                             void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    const int64_t L = n_heads * n_features;
+    GatSrcParams p{};
+    p.sp.indptr = t_indptr;
+    p.sp.indices = t_rows;
+    p.sp.eperm = t_perm;
+    p.sp.values = values;
+    p.sp.feat = grad_out;
+    p.sp.out = grad_x;
+    p.sp.n_rows = (int)n_src;
+    p.sp.n_src = (int)n_dst;
+    p.sp.L = (int)L;
+    p.sp.F = (int)n_features;
+    p.sp.H = (int)n_heads;
+    p.sp.col_mask = 0x7fffffff;
+    p.sp.alpha = 1.0f;
+    p.x = features;
+    p.grad_a = grad_a;
+    p.g_ld = (int)L;
+    p.g_scale = 1.0f;
+    bool has_items = false;
+    void *rest = nullptr;
+    size_t rest_bytes = 0;
+    int rc = plan_resolve(p.sp.plan, has_items, plan_t, t_indptr, t_rows, n_src, n_dst, nnz,
+                          0x7fffffff, max_degree_t, workspace, workspace_bytes, &rest, &rest_bytes,
+                          stream);
+    if (rc) return rc;
+    const size_t part =
+        has_items ? align_up(sizeof(float) * (size_t)p.sp.plan.max_items * (size_t)L, 256) : 0;
+    YITU_REQUIRE(part == 0 || (rest && rest_bytes >= part),
+                 "workspace too small: need %zu more bytes", part);
+    if (has_items) p.sp.partial = static_cast<float *>(rest);
+    return gat_src_launch<false>(p, has_items, grad_out, nullptr, nullptr, (int)n_dst, stream);
+}
+
 // ---- host side ----------------------------------------------------------------
 // workspace beyond the plan: item statistics, row statistics, partial rows
 static size_t gat_own_bytes(int64_t n_dst, int64_t nnz, int64_t H, int64_t L) {

@@ -226,6 +226,11 @@ int spmm_backward_run(float *grad_a, float *grad_x, const float *values, const i
     YITU_REQUIRE(!grad_x || (t_indptr && (nnz == 0 || (t_rows && t_perm))),
                  "grad_x needs the transposed structure (yitu_csr_transpose)");
 
+    if (grad_a && grad_x && nnz > 0 && n_dst > 0 && n_src > 0 && !long_rows_only &&
+        spmm_backward_one_gather_shape(n_heads, n_features, features, grad_out, grad_x))
+        return spmm_backward_one_gather(grad_a, grad_x, values, features, grad_out, t_indptr,
+                                        t_rows, t_perm, n_dst, n_src, nnz, n_heads, n_features,
+                                        max_degree_t, plan_t, workspace, workspace_bytes, stream);
     if (grad_a && nnz > 0 && n_dst > 0) {
         DotParams p{};
         p.sp.indptr = indptr;

@@ -623,6 +623,16 @@ int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max
                 const void *plan, void *workspace, size_t workspace_bytes, hipStream_t stream);
 // Workspace of launch_spmm: partial rows, plus the temporary plan when none is given.
 size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan);
+// Both gradients of an edge-weighted product from one gather over the by-source
+// structure (gat.hip), for the shapes spmm_backward_one_gather_shape accepts.
+bool spmm_backward_one_gather_shape(int64_t n_heads, int64_t n_features, const float *features,
+                                    const float *grad_out, const float *grad_x);
+int spmm_backward_one_gather(float *grad_a, float *grad_x, const float *values,
+                             const float *features, const float *grad_out,
+                             const int32_t *t_indptr, const int32_t *t_rows, const int32_t *t_perm,
+                             int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                             int64_t n_features, int64_t max_degree_t, const void *plan_t,
+                             void *workspace, size_t workspace_bytes, hipStream_t stream);
 // The body of yitu_spmm_backward (spmm_bwd.hip).
 int spmm_backward_run(float *grad_a, float *grad_x, const float *values, const int32_t *indptr,
                       const int32_t *indices, const float *features, const float *grad_out,
