@@ -388,3 +388,24 @@ def test_spmm_backward_one_gather_shapes(dev, h, f):
     assert_close(gx, gx2, atol=1e-3)
     again = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
     assert torch.equal(again[0], ga) and torch.equal(again[1], gx)
+
+
+def test_spmm_backward_constant_weights_take_the_by_source_copy(dev):
+    """grad_x alone with the same weight tensor passed again: from the second call on the
+    weights are read from a copy in by-source order; same result, and an in-place change
+    of the weights is noticed."""
+    indptr, indices = powerlaw_graph(12, 50000, 17)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(3)
+    values = torch.rand(indices.numel(), 2, generator=g).to(dev)
+    x = torch.randn(n, 2, 24, generator=g)
+    gy = torch.randn(n, 2, 24, generator=g)
+    ip, ix, xd, gyd = indptr.to(dev), indices.to(dev), x.to(dev), gy.to(dev)
+    want = oracle.mh_spmm_backward(values.cpu(), indptr, indices, x, gy)[1]
+    for _ in range(3):  # first call: through the permutation; then: the kept copy
+        got = graph_ext.spmm_backward(values, ip, ix, xd, gyd, need_grad_a=False)[1]
+        assert_close(got, want, atol=5e-4)
+    values.mul_(2.0)
+    for _ in range(3):
+        got = graph_ext.spmm_backward(values, ip, ix, xd, gyd, need_grad_a=False)[1]
+        assert_close(got, 2 * torch.as_tensor(want), atol=1e-3)

@@ -115,6 +115,37 @@ def spmm_forward(values, indptr, indices, features):
     return out
 
 
+# Edge weights that take no gradient are usually constants of the graph (norms), passed
+# again every step. The backward reads them through the edge permutation, a scattered
+# 4-byte read per edge and head; the second time the same tensor (same version) comes
+# by, a copy in by-source order is made and kept for as long as the tensor lives.
+_values_seen = {}       # id(values) -> state of the tensor when it last came by
+_values_by_source = {}  # id(values) -> (that state, the copy in by-source order)
+
+
+def _by_source_values(values, indptr, indices, n_src):
+    ident = id(values)
+    state = (values.data_ptr(), values._version, id(indices), indices._version, int(n_src))
+    hit = _values_by_source.get(ident)
+    if hit is not None and hit[0] == state:
+        return hit[1]
+    if _values_seen.get(ident) != state:
+        if ident not in _values_seen:
+            weakref.finalize(values, _forget_values, ident)
+        _values_seen[ident] = state
+        _values_by_source.pop(ident, None)
+        return None
+    tr = transposed(indptr, indices, n_src)
+    copy = values.index_select(0, tr.t_perm)
+    _values_by_source[ident] = (state, copy)
+    return copy
+
+
+def _forget_values(ident):
+    _values_seen.pop(ident, None)
+    _values_by_source.pop(ident, None)
+
+
 def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
                   need_grad_x=True):
     """Returns [grad_a [E,H], grad_x [Ns,H,F]] (entry.cpp:92-104). A gradient
@@ -132,6 +163,13 @@ def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
         raise RuntimeError("grad_out must be [n_dst, n_heads, n_features]")
     if not (need_grad_a or need_grad_x):
         return [None, None]
+    if not need_grad_a and nnz > 0 and n_dst <= COL_MASK:
+        values_t = _by_source_values(values, indptr, indices, n_src)
+        if values_t is not None:
+            # constant edge weights, seen before: grad_x is a forward product over the
+            # by-source structure, its weights already in that order
+            tr = transposed(indptr, indices, n_src)
+            return [None, spmm_forward(values_t, tr.t_indptr, tr.t_rows, grad_out)]
     grad_a = torch.empty_like(values) if need_grad_a else None
     grad_x = torch.empty_like(features) if need_grad_x else None
     tr = transposed(indptr, indices, n_src)
