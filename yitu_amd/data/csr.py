@@ -2,8 +2,6 @@
 rows ascending, columns ascending inside a row, duplicates merged, int32 -- what
 ``scipy.sparse.coo_matrix(...).tocsr()`` gives the reference
 (YiTu_GNN/data/dataset.py:116-129)."""
-import ctypes
-
 import torch
 
 from .. import _lib

@@ -7,7 +7,7 @@ against."""
 import torch
 from torch.nn import functional as F
 
-from . import block, bundle, ir, mp, sparse
+from . import bundle, ir, mp, sparse
 
 
 def _fill(template, values):
