@@ -539,7 +539,8 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
     Linear per node type and with one per relation (the reference model's form), and the
     reference's own 2-layer RGCN model (embedding, HeteroGraphConv over GCNLayers, ReLU,
     HeteroGraphConv) captured, lowered and executed relation by relation on these kernels,
-    beside the same model built from two stacked layer modules."""
+    the same after the stitcher has joined the relations of each destination type, and the
+    same model built from two stacked layer modules."""
     from yitu_amd import xgnn_h
     from yitu_amd.xgnn_h import block as xblock, layers as xl, models, mp
     names = ["t%d" % i for i in range(4)]
@@ -581,6 +582,9 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
     executor.train()
     res["reference_model_2_layers_lowered_fwd_bwd_ms"] = _event_ms(
         train_step(lambda: executor.run(lowered, kwargs), list(model.parameters())), steps, warm)
+    stitched_flow = xgnn_h.Stitcher().transform(lowered, kwargs)
+    res["reference_model_2_layers_stitched_fwd_bwd_ms"] = _event_ms(
+        train_step(lambda: executor.run(stitched_flow, kwargs), list(model.parameters())), steps, warm)
     # the same model from two stacked layer modules
     l1 = xl.StackedHeteroGCN(ntypes, list(blocks), dim, dim, per_relation=True).to(dev)
     l2 = xl.StackedHeteroGCN(ntypes, list(blocks), dim, dim, per_relation=True).to(dev)

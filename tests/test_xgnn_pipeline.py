@@ -184,10 +184,14 @@ def test_stitching_replaces_sums_of_relations(which):
     # layer 2 reads all three types of layer 1: one stitched term per destination type
     # with several relations (paper: 4 -> 1, author: 2 -> 1), venue keeps its single one
     assert ops["spmm"] + ops["gat"] == 1 + 3
-    assert ops["concat"] >= 3
     if which == "rgcn":
+        # the relations' Linears feed nothing else: one typed Linear per stitched term
+        # writes the feature rows, nothing is concatenated
+        assert ops["typed_linear"] == 3 and ops["concat"] == 0
         assert ops["edge_values"] == 3 and ops["sddmm"] == 0
     else:
+        # the transformed features are also read by the projections: they stay as they are
+        assert ops["concat"] >= 3 and ops["typed_linear"] == 0
         assert ops["sddmm"] == 3 and ops["stack"] == 3 and ops["gat"] == 1
     new = kwargs["stitch"]
     assert isinstance(new, mp.HeteroGraph) and len(new.hetero_graph) == 2

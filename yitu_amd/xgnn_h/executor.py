@@ -7,7 +7,7 @@ against."""
 import torch
 from torch.nn import functional as F
 
-from . import bundle, ir, mp, sparse
+from . import bundle, ir, layers, mp, sparse
 
 
 def _fill(template, values):
@@ -23,6 +23,7 @@ def _fill(template, values):
 class Executor:
     def __init__(self):
         self._is_training = None
+        self._edge_values = {}  # edge_values node -> (state of its inputs, result, inputs)
 
     def eval(self):
         self._is_training = False
@@ -75,10 +76,25 @@ class Executor:
         if op in ("concat", "stack"):
             parts = [v[str(i)] for i in range(len(node.inputs))]
             return torch.cat(parts, dim=0) if op == "concat" else torch.stack(parts, dim=0)
+        if op == "typed_linear":
+            count = len(node.inputs)
+            return layers._TypedLinear.apply(count, *[v[str(i)] for i in range(count)],
+                                             *node.attrs["weights"], *node.attrs["biases"])
         if op == "edge_values":
-            scales = torch.stack([v[str(i)].reshape(-1) for i in range(len(node.inputs) - 1)])
-            rows, _, bids = mp.edge_endpoints(v["g"])
-            return scales[bids, rows].unsqueeze(-1).contiguous()
+            # per-edge weights of a stitched block from the relations' row scales: constants
+            # of the graph, so they are kept for as long as the same scale tensors come by
+            parts = [v[str(i)] for i in range(len(node.inputs) - 1)]
+            state = tuple((id(t), t.data_ptr(), t._version) for t in parts) + (id(v["g"]),)
+            kept = self._edge_values.get(id(node))
+            if any(t.requires_grad for t in parts):
+                kept = None  # scales that train: compute (and differentiate) every time
+            if kept is None or kept[0] != state:
+                scales = torch.stack([t.reshape(-1) for t in parts])
+                rows, _, bids = mp.edge_endpoints(v["g"])
+                kept = (state, scales[bids, rows].unsqueeze(-1).contiguous(), parts)
+                if not any(t.requires_grad for t in parts):
+                    self._edge_values[id(node)] = kept
+            return kept[1]
         if op == "edge":
             args = {k: t for k, t in v.items() if k != "g"}
             return mp.apply_edge(node.attrs["fn"], v["g"], **args)

@@ -109,6 +109,7 @@ class Stitcher:
         assert 2 <= max_blocks <= 16
         self.max_blocks = max_blocks
         self.max_columns = max_columns
+        self._readers: Dict[int, int] = {}
 
     def _pack(self, terms: List[_Term], hgraph: mp.HeteroGraph) -> List[List[_Term]]:
         """First-fit decreasing by edge count into bins of at most ``max_blocks``
@@ -126,6 +127,32 @@ class Stitcher:
                 bins.append([t])
         return bins
 
+    def _concat_features(self, xs, n_rows: int) -> ir.Node:
+        """The feature rows of the stitched block: the relations' features one below the
+        other. Where each of them is ``view(linear(x_i))`` read by nobody else, the
+        Linears become one ``typed_linear`` node that writes its products straight into
+        the row ranges of one buffer (a grouped GEMM launch, no concatenation pass)."""
+        tail = xs[0].size[1:]
+        inner = []
+        for x in xs:
+            ops = _call_operands(x, ("view", "reshape")) if len(x.size) == 3 else None
+            lin = ops[0] if ops is not None and len(ops) == 1 else None
+            if lin is None or lin.op != "linear" or len(lin.size) != 2 or \
+                    lin.size[1] != tail[0] * tail[1] or self._readers.get(id(lin), 0) != 1 or \
+                    self._readers.get(id(x), 0) != 1 or len(lin.inputs["x"].size) != 2:
+                inner = None
+                break
+            inner.append(lin)
+        if not inner:
+            return ir.Node("concat", {str(i): n for i, n in enumerate(xs)}, size=[n_rows] + tail)
+        flat = ir.Node("typed_linear", {str(i): lin.inputs["x"] for i, lin in enumerate(inner)},
+                       {"weights": [lin.attrs["weight"] for lin in inner],
+                        "biases": [lin.attrs["bias"] for lin in inner]},
+                       size=[n_rows, tail[0] * tail[1]])
+        return ir.Node("call", {"0": flat},
+                       {"fn": torch.Tensor.view, "args": (ir.Slot("0"), [-1] + tail), "kwargs": {}},
+                       size=[n_rows] + tail)
+
     def _stitch_bin(self, terms: List[_Term], hgraph: mp.HeteroGraph,
                     stitched: mp.HeteroGraph) -> ir.Node:
         rels = [tuple(hgraph.idx2rel[t.rel_index]) for t in terms]
@@ -140,8 +167,7 @@ class Stitcher:
         idx = stitched.rel2idx[new_sty, new_ety, dty]
         g = ir.Node("graph", size=new_blk.size, name="stitch.%d" % idx)
         qs, ks, xs = zip(*(t.qkx() for t in terms))
-        x = ir.Node("concat", {str(i): n for i, n in enumerate(xs)},
-                    size=[new_blk.size[1]] + xs[0].size[1:])
+        x = self._concat_features(xs, new_blk.size[1])
         inputs = {"g": g, "x": x}
         n_edges = new_blk.num_edges()
         if terms[0].attention:
@@ -172,6 +198,7 @@ class Stitcher:
         for node in ir.walk(dataflow):
             for child in node.inputs.values():
                 consumers.setdefault(id(child), []).append(node)
+        self._readers = {key: len(nodes) for key, nodes in consumers.items()}
 
         def inner_add(node):  # an add whose only reader is another add
             readers = consumers.get(id(node), [])
@@ -203,6 +230,8 @@ class Stitcher:
                 changed = any(ins[k] is not node.inputs[k] for k in ins)
                 new = node.with_inputs(ins) if changed else node
             memo[id(node)] = new
+            # a rebuilt node has the readers of the node it stands for
+            self._readers.setdefault(id(new), self._readers.get(id(node), 0))
             return new
 
         if isinstance(dataflow, ir.Node):
