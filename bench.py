@@ -35,9 +35,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # profiles/bench_c3_spmm_gat_rocprofv3.md. Per yitu_agg_csr call for the C3 workloads,
 # per yitu_gat_forward call for C2.
 MEASURED_TRAFFIC_BYTES = {
-    "c3_spmm_f32": 21_418_030_250,
-    "c3_spmm_bf16": 10_964_550_332,
-    "c2_gat_f32": 5_473_633_168,
+    "c3_spmm_f32": 21_418_734_739,
+    "c3_spmm_bf16": 10_965_161_440,
+    "c2_gat_f32": 5_478_204_769,
 }
 
 
