@@ -364,9 +364,10 @@ def test_graph_without_edges(dev, n_dst, n_src):
     assert all(zeros(t.grad, *t.shape) for t in leaves)
 
 
-@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (2, 128), (1, 256)])
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (2, 128), (1, 256), (8, 64), (2, 256),
+                                 (16, 64), (4, 256)])
 def test_spmm_backward_one_gather_shapes(dev, h, f):
-    """Rows of 256 floats: both gradients come from one pass over the by-source
+    """Rows of 256, 512 or 1024 floats: both gradients come from one pass over the by-source
     structure; against the oracle, with hub rows on both sides, and equal to the
     two-pass form (asked for one gradient at a time)."""
     indptr, indices = powerlaw_graph(12, 70000, 31 * h + f)

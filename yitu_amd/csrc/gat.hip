@@ -1439,14 +1439,10 @@ static int gat_src_launch_lph(const GatSrcParams &p, bool has_items, const float
     const int kt = p.sp.L / 256;
     if (kt == 1)
         return gat_src_launch_shape<LPH, 1, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
-    if constexpr (FULL) {  // wider rows exist only with the forward output at hand
-        if (kt == 2)
-            return gat_src_launch_shape<LPH, 2, true>(p, has_items, grad_out, out, query, n_dst,
-                                                      stream);
-        if (kt == 4)
-            return gat_src_launch_shape<LPH, 4, true>(p, has_items, grad_out, out, query, n_dst,
-                                                      stream);
-    }
+    if (kt == 2)
+        return gat_src_launch_shape<LPH, 2, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
+    if (kt == 4)
+        return gat_src_launch_shape<LPH, 4, FULL>(p, has_items, grad_out, out, query, n_dst, stream);
     set_error("gat backward: unsupported row width %d", p.sp.L);
     return -1;
 }
@@ -1471,8 +1467,8 @@ static int gat_src_launch(const GatSrcParams &p, bool has_items, const float *gr
 // one gathering x[col] by destination and one gathering grad_out[row] by source.
 bool spmm_backward_one_gather_shape(int64_t n_heads, int64_t n_features, const float *features,
                                     const float *grad_out, const float *grad_x) {
-    const int64_t lph = n_features / 4;
-    return n_heads * n_features == 256 && n_features % 4 == 0 && lph >= 8 && lph <= 64 &&
+    const int64_t lph = n_features / 4, L = n_heads * n_features;
+    return (L == 256 || L == 512 || L == 1024) && n_features % 4 == 0 && lph >= 8 && lph <= 64 &&
            (lph & (lph - 1)) == 0 && aligned16(features) && aligned16(grad_out) &&
            aligned16(grad_x);
 }
@@ -1776,13 +1772,12 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
     YITU_REQUIRE(t_indptr && (nnz == 0 || (t_rows && t_perm)),
                  "gat_backward needs the transposed structure (yitu_csr_transpose)");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // Rows of 256 floats (512 and 1024 too when the forward output is given) with a
-    // power-of-two head width of 32 to 256: one pass over the transposed structure
-    // serves every gradient from a single gather.
+    // Rows of 256, 512 or 1024 floats with a power-of-two head width of 32 to 256: one
+    // pass over the transposed structure serves every gradient from a single gather.
     const int64_t L = n_heads * n_features;
     const int lph = (int)(n_features / 4);
-    const bool wide_ok = out != nullptr && aligned16(out) && (L == 512 || L == 1024);
-    const bool one_gather = (L == 256 || wide_ok) && n_features % 4 == 0 && lph >= 8 && lph <= 64 &&
+    const bool one_gather = (L == 256 || L == 512 || L == 1024) && n_features % 4 == 0 && lph >= 8 &&
+                            lph <= 64 &&
                             (lph & (lph - 1)) == 0 && n_dst > 0 && nnz > 0 && n_dst < INT32_MAX &&
                             n_src <= (1 << 24) && aligned16(features) && aligned16(grad_out) &&
                             aligned16(grad_features);
@@ -1791,8 +1786,8 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
                  "without attn the backward needs a one-pass shape and the forward output");
     YITU_REQUIRE(!grad_out_is_head_mean || one_gather,
                  "a head-mean gradient is taken by the one-pass shapes only (rows of 256, 512 or "
-                 "1024 floats, head width 32..256 a power of two, forward output given for the "
-                 "wider rows); expand it to [n_dst, H, F] / H for other shapes");
+                 "1024 floats, head width 32..256 a power of two); expand it to [n_dst, H, F] / H "
+                 "for other shapes");
     if (one_gather) {
         GatSrcParams p{};
         p.sp.indptr = t_indptr;

@@ -512,7 +512,7 @@ def gat_one_pass_shape(n_heads, n_features, with_out=True):
     row = n_heads * n_features
     lph = n_features // 4
     return (n_features % 4 == 0 and 8 <= lph <= 64 and lph & (lph - 1) == 0 and
-            (row == 256 or (with_out and row in (512, 1024))))
+            row in (256, 512, 1024))
 
 
 def gat_backward(indptr, indices, query, key, features, attn, grad_out, out=None,
