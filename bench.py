@@ -73,14 +73,14 @@ def build_c3(dev, reorder=True, scale=21, draws=63_000_000, seed=20242):
     return _c3_cache[reorder]
 
 
-def agg_call(out, x, rp, ci, deg, plan, ws, maxdeg):
+def agg_call(out, x, rp, ci, deg, plan, ws, maxdeg, edge_scale=None):
     from yitu_amd import _lib
     n, dim = x.shape
     rc = _lib.lib().yitu_agg_csr(
         _lib.ptr(out), _lib.ptr(x), _lib.c_int(1 if x.dtype == torch.bfloat16 else 0), _lib.ptr(rp),
         _lib.ptr(ci), _lib.ptr(deg), _lib.c_i64(rp.numel() - 1), _lib.c_i64(n),
         _lib.c_i64(ci.numel()), _lib.c_i64(dim), _lib.c_f32(1.0), _lib.c_i64(maxdeg), _lib.ptr(plan),
-        _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(x.device))
+        _lib.ptr(edge_scale), _lib.ptr(ws), _lib.c_size(ws.numel()), _lib.stream_ptr(x.device))
     _lib.check(rc, "yitu_agg_csr")
 
 
@@ -149,6 +149,12 @@ def run_spmm(args, dev, bf16):
     maxdeg = int((rp[1:] - rp[:-1]).max().item())
     # per-graph preparation, outside the timed region like the reference's build_part
     plan = _lib.row_plan(rp, ci, n, 0x7FFFFFFF)
+    edge_scale = torch.empty(nnz, device=dev)  # s[col[e]]: per-graph, like the plan
+    _lib.check(_lib.lib().yitu_edge_scale(_lib.ptr(edge_scale), _lib.ptr(ci), _lib.ptr(deg),
+                                          _lib.c_i64(nnz), _lib.c_i64(n), _lib.stream_ptr(dev)),
+               "yitu_edge_scale")
+    if os.environ.get("YITU_BENCH_NO_EDGE_SCALE"):
+        edge_scale = None
     ws = torch.empty(int(_lib.size_fn("yitu_spmm_workspace_bytes")(
         _lib.c_i64(nnz), _lib.c_i64(dim), _lib.c_int(1))), dtype=torch.uint8, device=dev)
 
@@ -158,7 +164,7 @@ def run_spmm(args, dev, bf16):
                 e0 = torch.cuda.Event(enable_timing=True)
                 e1 = torch.cuda.Event(enable_timing=True)
                 e0.record()
-            agg_call(dst_t, src_t, rp, ci, deg, plan, ws, maxdeg)
+            agg_call(dst_t, src_t, rp, ci, deg, plan, ws, maxdeg, edge_scale)
             if events is not None:
                 e1.record()
                 events.append((e0, e1))

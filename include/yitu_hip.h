@@ -39,8 +39,9 @@ int yitu_stream_copy(void *dst_device, const void *src_device, int64_t n_bytes, 
  * The counterpart of the reference's neighbour-group partition build_part
  * (ccsrc/kernel/YiTu_GNN.cpp:203-245), which its callers compute once per graph
  * and pass to every op as part_pointers / part2Node: rows with >= 64 edges are
- * cut into items of 64 edges, listed in ascending order of the source id in the
- * middle of each item. The gather kernels (aggregation, SpMM, per-edge dot, GAT
+ * cut where their columns cross the boundaries of source bands (2^17 ids) and
+ * into items of at most 64 edges, listed in ascending order of the source id in
+ * the middle of each item. The gather kernels (aggregation, SpMM, per-edge dot, GAT
  * aggregate) run one wave per item in that order, which keeps the hot rows of
  * the feature table in L2. The plan depends on (indptr, indices) only.
  * Every op that takes `plan_device` also accepts NULL and then builds a
@@ -79,12 +80,25 @@ size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with_plan);
  * The neighbour-group arguments of the reference (part_pointers, part2Node,
  * partSize, dimWorker, warpPerBlock) are replaced by the row plan (or nothing).
  * max_degree: widest row if known, else -1.
+ * edge_scale_device: NULL, or the per-edge column scales s[col[e]] of this graph
+ * and this degrees array, written once by yitu_edge_scale: the kernels then read
+ * them in edge order instead of one random 4-byte read of s per edge. On a large
+ * graph those reads cost more than their bytes: the lines of s (32 sources each)
+ * are all warm and push the feature rows out of L2 (2^21 nodes, F = 128 fp32:
+ * 3.08 ms per call without, 2.69 ms with). Ignored when degrees is NULL.
  */
 int yitu_agg_csr(float *out_device, const void *x_device, int x_is_bf16,
                  const int32_t *row_pointers_device, const int32_t *column_index_device,
                  const float *degrees_device, int64_t n_rows, int64_t n_src, int64_t nnz,
                  int64_t dim, float alpha, int64_t max_degree, const void *plan_device,
-                 void *workspace_device, size_t workspace_bytes, void *stream);
+                 const float *edge_scale_device, void *workspace_device, size_t workspace_bytes,
+                 void *stream);
+
+/* edge_scale[e] = degrees[column_index[e]] for the nnz edges of a CSR: per-graph
+ * preparation for yitu_agg_csr, like the row plan (the reference's callers hold
+ * `degrees` per graph, data/dataset.py:131-136, and pass it to every call). */
+int yitu_edge_scale(float *edge_scale_device, const int32_t *column_index_device,
+                    const float *degrees_device, int64_t nnz, int64_t n_src, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Module 2: graph_ext  (YiTu_GNN/YiTu_H/src/entry.cpp:184-193)                */

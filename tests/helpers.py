@@ -9,12 +9,33 @@ RTOL_F32, ATOL_F32 = 1e-5, 1e-4
 RTOL_BF16, ATOL_BF16 = 1e-2, 1e-4
 
 
-def assert_close(got, want, rtol=RTOL_F32, atol=ATOL_F32, what=""):
-    got = got.detach().cpu().numpy() if isinstance(got, torch.Tensor) else np.asarray(got)
-    want = want.detach().cpu().numpy() if isinstance(want, torch.Tensor) else np.asarray(want)
+# Error model of a long fp32 sum. An output element y = sum_i t_i added in fp32 in an
+# order other than the oracle's differs from it by rounding noise proportional to
+# sum_i |t_i|, not to |y| (cancellation) and not to a constant (hub rows add 10^3..10^5
+# terms). With unit roundoff u = 2^-24 a sequential sum of n terms of random sign has a
+# standard error of about 0.35 u sum|t|, a tree sum less; SUM_ULPS * u * sum|t| with
+# SUM_ULPS = 4 is beyond ten standard errors of either and still 25 times below the
+# worst case of a 100-deep order. Tests pass ``abs_sum`` (the same reduction evaluated
+# on absolute values, usually by the oracle itself) and the bound becomes
+#     atol 1e-4 + rtol 1e-5 |want| + SUM_ULPS * 2^-24 * abs_sum,
+# so that rows of a few dozen terms keep the plain bar and long rows get exactly the
+# allowance their own data justifies. ``ulps`` raises the factor for quantities that
+# carry the relative error of expf of a softmax argument (|argument| * u each).
+UNIT_ROUNDOFF = 2.0 ** -24
+SUM_ULPS = 4.0
+
+
+def _np(a):
+    return a.detach().cpu().numpy() if isinstance(a, torch.Tensor) else np.asarray(a)
+
+
+def assert_close(got, want, rtol=RTOL_F32, atol=ATOL_F32, what="", abs_sum=None, ulps=SUM_ULPS):
+    got, want = _np(got), _np(want)
     assert got.shape == want.shape, "%s shape %s vs %s" % (what, got.shape, want.shape)
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     bound = atol + rtol * np.abs(want.astype(np.float64))
+    if abs_sum is not None:
+        bound = bound + ulps * UNIT_ROUNDOFF * np.abs(_np(abs_sum).astype(np.float64))
     bad = err > bound
     if bad.any():
         i = np.unravel_index(np.argmax(err - bound), err.shape)

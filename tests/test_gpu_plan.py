@@ -1,12 +1,12 @@
 """Structure of the row plan written by yitu_plan_build (integer work: exact).
 
 The plan's layout is read back from the device buffer: a 512-byte header
-(counters; slab bounds), the long-row table and the item records. The checks
+(counters; band width and count), the long-row table and the item records. The checks
 are invariants that any correct plan must satisfy, stated independently of how
 the builder derives it: the items of a long row tile the row's edge range
 without gap or overlap in item-id order, no item exceeds 64 edges, every item
 appears exactly once in the record list, the list is in ascending order of the
-items' middle source ids, the slab bounds are ordered, and the number of items
+items' middle source ids, the bands cover the source ids, and the number of items
 stays inside the bound that sizes the callers' workspaces.
 """
 import numpy as np
@@ -19,7 +19,7 @@ from yitu_amd import _lib
 pytestmark = pytest.mark.gpu
 
 CHUNK = 64
-SLABS = 4
+BAND_SHIFT, MAX_BANDS, MIN_SEGMENT = 17, 64, 16
 
 
 def read_plan(plan, nnz):
@@ -27,13 +27,13 @@ def read_plan(plan, nnz):
     max_rows = nnz // CHUNK + 1
     max_items = nnz // CHUNK + nnz // 16 + max_rows + 1
     n_items, n_rows, overflow = raw[0], raw[1], raw[2]
-    slab_bound = raw[64:64 + SLABS + 1]
+    band_shift, n_bands = int(raw[64]), int(raw[65])
     rows_off = 128
     rows = raw[rows_off:rows_off + 4 * max_rows].reshape(-1, 4)[:n_rows]
     rec_off = rows_off + ((16 * max_rows + 255) // 256 * 256) // 4
     records = raw[rec_off:rec_off + 4 * max_items].reshape(-1, 4)
     return dict(n_items=int(n_items), n_rows=int(n_rows), overflow=int(overflow),
-                slab_bound=slab_bound, rows=rows,
+                band_shift=band_shift, n_bands=n_bands, rows=rows,
                 records=records[:n_items], tail=records[n_items:], max_items=max_items)
 
 
@@ -63,14 +63,16 @@ def check_plan(indptr, indices, n_src, col_mask, dev):
     b, e, r, s = beg[by_item], end[by_item], row[by_item], single[by_item]
     for rr, first, count, _ in p["rows"]:
         assert count >= 1
-        assert count <= deg[rr] // CHUNK + min(SLABS, deg[rr] // 16)         # workspace bound
+        assert count <= deg[rr] // CHUNK + min(p["n_bands"], deg[rr] // MIN_SEGMENT)  # workspace bound
         sl = slice(first, first + count)
         assert np.all(r[sl] == rr)
         assert b[sl][0] == ip[rr] and e[sl][-1] == ip[rr + 1]                # tiles the row ...
         assert np.array_equal(b[sl][1:], e[sl][:-1])                         # ... in item order
         assert np.all(s[sl] == (count == 1))
-    sb = p["slab_bound"].astype(np.int64)
-    assert sb[0] == 0 and np.all(np.diff(sb) >= 0)
+    # bands of 2^17 ids, wider only when that would give more than 64 of them
+    assert p["band_shift"] >= BAND_SHIFT and 1 <= p["n_bands"] <= MAX_BANDS
+    assert ((max(n_src, 1) - 1) >> p["band_shift"]) + 1 == p["n_bands"]
+    assert p["band_shift"] == BAND_SHIFT or ((max(n_src, 1) - 1) >> (p["band_shift"] - 1)) + 1 > MAX_BANDS
     # the records are in ascending band (middle source id, 16 bits) order
     cols = (indices.numpy() & col_mask).astype(np.int64)
     mid = cols[(beg + end) // 2]
@@ -78,16 +80,25 @@ def check_plan(indptr, indices, n_src, col_mask, dev):
     while ((max(n_src, 1) - 1) >> shift) >= (1 << 16):
         shift += 1
     assert np.all(np.diff(mid >> shift) >= 0)
-    p["pure"] = (np.searchsorted(sb[1:SLABS], cols[beg], side="right") ==
-                 np.searchsorted(sb[1:SLABS], cols[end - 1], side="right"))
+    # an item is pure when it gathers from one group of bands of its row: a row of deg
+    # edges may be cut into the largest power of two <= deg / 16 pieces (at most the
+    # number of bands), i.e. at the boundaries of groups of ceil(bands / pieces) bands
+    d = deg[row]
+    allowed = np.minimum(2 ** np.floor(np.log2(np.maximum(d // MIN_SEGMENT, 1))).astype(np.int64),
+                         p["n_bands"])
+    allowed = np.where(2 * allowed * MIN_SEGMENT <= d, p["n_bands"], allowed)
+    per_group = -(-p["n_bands"] // allowed)
+    p["pure"] = ((cols[beg] >> p["band_shift"]) // per_group ==
+                 (cols[end - 1] >> p["band_shift"]) // per_group)
     return p
 
 
 def test_power_law_graph(dev):
-    indptr, indices = powerlaw_graph(14, 600000, 5)
-    p = check_plan(indptr, indices, 1 << 14, 0x7fffffff, dev)
-    # the slabs split the sources for real, and most items gather from one slab only
-    assert len(set(p["slab_bound"].tolist())) == SLABS + 1
+    indptr, indices = powerlaw_graph(19, 6000000, 5)
+    p = check_plan(indptr, indices, 1 << 19, 0x7fffffff, dev)
+    # 4 bands of 2^17 sources: the cuts happen for real, and most items gather from
+    # one band group only (segments shorter than 16 edges are merged into a neighbour)
+    assert p["n_bands"] == 4
     assert p["pure"].mean() > 0.6
 
 
@@ -116,8 +127,8 @@ def test_columns_not_sorted_inside_rows(dev):
 
 
 def test_more_sources_than_edges(dev):
-    """Popularity buckets are bounded by the edge count: a huge, mostly unused
-    source range must still give a valid plan."""
+    """A huge, mostly unused source range (32 bands of 2^17 ids) must still give a
+    valid plan."""
     n_dst, n_src = 64, 1 << 22
     rng = np.random.default_rng(1)
     rows = np.repeat(np.arange(n_dst), 200)

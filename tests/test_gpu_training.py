@@ -80,6 +80,9 @@ def _prepare(tmp_path, dev, manual_mode):
     info.column_index = info.column_index.to(dev)
     info.partPtr = part_ptr.int().to(dev)
     info.part2Node = part2node.int().to(dev)
+    if manual_mode:  # one of the two modes also trains with the per-edge column scales
+        info.prepare_edge_scale()
+        assert info.edge_scale.shape == info.column_index.shape
     # dense form of the CSR the model will run on
     rp, ci = info.row_pointers.cpu(), info.column_index.cpu().long()
     rows = torch.repeat_interleave(torch.arange(n), (rp[1:] - rp[:-1]).long())
@@ -131,6 +134,8 @@ def test_gcn_two_layers_from_npz_follows_dense_autograd(dev, tmp_path):
     info.degrees = dataset.degrees
     s = 1.0 / info.degrees            # the example passes sqrt(deg); the op multiplies by it, so
     info.degrees = s                  # the symmetric normalisation needs the reciprocal
+    assert info.edge_scale is None    # replacing the scale vector dropped the per-edge scales
+    info.prepare_edge_scale()
     norm_adj = s[:, None] * adj * s[None, :]
     y = (norm_adj @ (x @ torch.randn(dim, classes, device=dev))).argmax(1)
     torch.manual_seed(19)

@@ -141,6 +141,44 @@ def test_stitched_sddmm_spmm_equals_sum_over_relations():
     assert_close(got, want)
 
 
+@pytest.mark.parametrize("n_bid,h,seed", [(2, 3, 0), (5, 1, 1), (16, 4, 2)])
+def test_sddmm_multi_bid_forward_backward_equal_dense_per_block_softmax(n_bid, h, seed):
+    """A stitched block tags every edge with a query block id (sddmm_cuda.cu:11-31,
+    block.py:46-55); the softmax runs per (row, block id) (sddmm_cuda.cu:15-31) and the
+    backward per the same groups (sddmm_cuda.cu:43-66). Independent statement: one dense
+    masked softmax per block over that block's own columns, joined by autograd."""
+    rng = np.random.default_rng(100 + seed)
+    n_dst = 27
+    blocks = []
+    for b in range(n_bid):
+        n_src = int(rng.integers(3, 30))
+        ip, ix = random_csr(n_dst, n_src, 0.2, 1000 * seed + b, empty_rows=((b * 5) % n_dst,))
+        blocks.append((ip, ix, n_src))
+    sp, si, n_cols = oracle.stitch_csr(blocks)
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(n_bid, n_dst, h, generator=g, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(n_cols, h, generator=g, dtype=torch.float64, requires_grad=True)
+    # dense attention of block b lives in columns [off_b, off_b + n_src_b) of a [H, n_dst, n_cols] tensor
+    dense = torch.zeros(h, n_dst, n_cols, dtype=torch.float64)
+    off = 0
+    for b, (ip, ix, n_src) in enumerate(blocks):
+        mask = _dense_mask(ip, ix, n_dst, n_src).double()
+        dense = dense + nn.functional.pad(_dense_gat(q[b], k[off:off + n_src], mask),
+                                          (off, n_cols - off - n_src))
+        off += n_src
+    deg = np.diff(sp).astype(np.int64)
+    rows = torch.from_numpy(np.repeat(np.arange(n_dst), deg))
+    cols = torch.from_numpy((si & 0xFFFFFF).astype(np.int64))
+    attn_edges = dense[:, rows, cols].t()  # [E, H] in stitched CSR order
+    ge = torch.randn(si.shape[0], h, generator=g, dtype=torch.float64)
+    attn_edges.backward(ge)
+    got = oracle.sddmm_forward(sp, si, q.detach().numpy(), k.detach().numpy())
+    assert_close(got, attn_edges.detach().float())
+    gq, gk = oracle.sddmm_backward(sp, si, q.detach().numpy(), k.detach().numpy(), got, ge.numpy())
+    assert_close(gq, q.grad.float())
+    assert_close(gk, k.grad.float())
+
+
 def test_b2gemm_equals_two_linears():
     """check_bundle (test_kernel.py:187-233)."""
     g = torch.Generator().manual_seed(0)

@@ -32,7 +32,25 @@ def _check_inputs(*tensors):
     return _lib.require_device(*tensors)
 
 
-def _aggregate(x, row_pointers, column_index, degrees, alpha):
+def edge_scale(column_index, degrees):
+    """Per-edge column scales ``degrees[column_index[e]]`` of a graph (float32 [nnz]):
+    per-graph preparation, like ``build_part``. Passed as ``edge_scale=`` to ``forward`` /
+    ``backward`` the aggregation reads them in edge order instead of gathering ``degrees``
+    once per edge. The caller owns the tensor: it must be rebuilt when ``column_index`` or
+    ``degrees`` change."""
+    _lib.require_device(column_index, degrees)
+    _lib.require_dtype(column_index, torch.int32, "column_index")
+    _lib.require_dtype(degrees, torch.float32, "degrees")
+    out = torch.empty(column_index.numel(), dtype=torch.float32, device=column_index.device)
+    with torch.cuda.device(column_index.device):
+        rc = _lib.lib().yitu_edge_scale(ptr(out), ptr(column_index), ptr(degrees),
+                                        c_i64(column_index.numel()), c_i64(degrees.numel()),
+                                        stream_ptr(column_index.device))
+    check(rc, "yitu_edge_scale")
+    return out
+
+
+def _aggregate(x, row_pointers, column_index, degrees, alpha, edge_scale=None):
     """out[r] = alpha * s_r * sum_j s_j x[j] over the CSR row r (s = degrees or 1)."""
     _lib.require_dtype(row_pointers, torch.int32, "row_pointers")
     _lib.require_dtype(column_index, torch.int32, "column_index")
@@ -47,6 +65,11 @@ def _aggregate(x, row_pointers, column_index, degrees, alpha):
     nnz = column_index.numel()
     if degrees is not None and degrees.numel() < max(n_rows, n_src):
         raise RuntimeError("degrees is shorter than the number of nodes")
+    if edge_scale is not None:
+        _lib.require_device(edge_scale)
+        _lib.require_dtype(edge_scale, torch.float32, "edge_scale")
+        if edge_scale.numel() != nnz:
+            raise RuntimeError("edge_scale must hold one value per edge")
     out = torch.empty((n_rows, dim), dtype=torch.float32, device=x.device)
     maxdeg = _lib.max_degree(row_pointers)
     plan = _lib.row_plan(row_pointers, column_index, n_src, 0x7FFFFFFF)
@@ -57,7 +80,7 @@ def _aggregate(x, row_pointers, column_index, degrees, alpha):
         rc = _lib.lib().yitu_agg_csr(
             ptr(out), ptr(x), c_int(1 if x.dtype == torch.bfloat16 else 0), ptr(row_pointers),
             ptr(column_index), ptr(degrees), c_i64(n_rows), c_i64(n_src), c_i64(nnz), c_i64(dim),
-            c_f32(alpha), c_i64(maxdeg), ptr(plan), ptr(ws), c_size(ws.numel()),
+            c_f32(alpha), c_i64(maxdeg), ptr(plan), ptr(edge_scale), ptr(ws), c_size(ws.numel()),
             stream_ptr(x.device))
     check(rc, "yitu_agg_csr")
     return out
@@ -71,20 +94,21 @@ def SAG(input, row_pointers, column_index, degrees, part_pointers, part2Node, pa
 
 
 def forward(input, weight, row_pointers, column_index, degrees, part_pointers, part2Node, partSize,
-            dimWorker, warpPerBlock):
-    """GCN: out = aggregate_{s_i s_j}(X.W) (YiTu_GNN.cpp:94-117; cu:264-317). Returns [out]."""
+            dimWorker, warpPerBlock, edge_scale=None):
+    """GCN: out = aggregate_{s_i s_j}(X.W) (YiTu_GNN.cpp:94-117; cu:264-317). Returns [out].
+    ``edge_scale`` (optional, not in the reference): see ``edge_scale()``."""
     _check_inputs(input, weight, row_pointers, column_index, degrees, part_pointers, part2Node)
     tmp = _mm(input, weight)
-    return [_aggregate(tmp, row_pointers, column_index, degrees, 1.0)]
+    return [_aggregate(tmp, row_pointers, column_index, degrees, 1.0, edge_scale)]
 
 
 def backward(d_output, X, W, row_pointers, column_index, degrees, part_pointers, part2Node,
-             partSize, dimWorker, warpPerBlock):
+             partSize, dimWorker, warpPerBlock, edge_scale=None):
     """GCN backward with the reference's semantics: the SAME CSR aggregates dY
     (not its transpose), then dX = G.W^T, dW = X^T.G (YiTu_GNN.cpp:119-145;
     cu:422-475). Returns [d_input, d_weight]."""
     _check_inputs(d_output, X, W, row_pointers, column_index, degrees, part_pointers, part2Node)
-    g = _aggregate(d_output, row_pointers, column_index, degrees, 1.0)
+    g = _aggregate(d_output, row_pointers, column_index, degrees, 1.0, edge_scale)
     return [_mm(g, W, trans_b=True), _mm(X, g, trans_a=True)]
 
 

@@ -8,7 +8,7 @@ using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
 YITU_API const char *yitu_last_error(void) { return last_error(); }
-YITU_API int yitu_abi_version(void) { return 2; }
+YITU_API int yitu_abi_version(void) { return 3; }
 
 YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with_plan) {
     return spmm_workspace_bytes(nnz, row_len, with_plan != 0);
@@ -17,8 +17,8 @@ YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with
 YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_t *row_pointers,
                           const int32_t *column_index, const float *degrees, int64_t n_rows,
                           int64_t n_src, int64_t nnz, int64_t dim, float alpha,
-                          int64_t max_degree, const void *plan, void *workspace,
-                          size_t workspace_bytes, void *stream) {
+                          int64_t max_degree, const void *plan, const float *edge_scale,
+                          void *workspace, size_t workspace_bytes, void *stream) {
     YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0 && dim >= 0, "negative size");
     if (n_rows == 0 || dim == 0) return 0;
     YITU_REQUIRE(out && row_pointers, "null output or row_pointers");
@@ -31,6 +31,7 @@ YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_
     p.out = out;
     p.scale_row = degrees;
     p.scale_col = degrees;
+    p.edge_scale = degrees ? edge_scale : nullptr;
     p.n_rows = (int)n_rows;
     p.n_src = (int)n_src;
     p.L = (int)dim;
@@ -40,6 +41,15 @@ YITU_API int yitu_agg_csr(float *out, const void *x, int x_is_bf16, const int32_
     p.alpha = alpha;
     return launch_spmm(p, degrees ? W_DEGPROD : W_NONE, x_is_bf16 != 0, nnz, max_degree, plan,
                        workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+YITU_API int yitu_edge_scale(float *edge_scale, const int32_t *column_index, const float *degrees,
+                            int64_t nnz, int64_t n_src, void *stream) {
+    YITU_REQUIRE(nnz >= 0 && nnz < INT32_MAX && n_src >= 0, "size out of range");
+    if (nnz == 0) return 0;
+    YITU_REQUIRE(edge_scale && column_index && degrees, "null pointer");
+    return edge_scale_fill(edge_scale, column_index, degrees, nnz, 0x7fffffff,
+                           static_cast<hipStream_t>(stream));
 }
 
 static int spmm_forward_any(float *out, const float *values, const int32_t *indptr,

@@ -1,13 +1,12 @@
 // Builds the row plan on the device: queue the long rows (one atomic per
-// workgroup), count the edges per source and place the slab boundaries, cut
-// every long row at the boundaries and into items of at most 64 edges, key every
-// item by its middle source id, stable radix sort, write the records.
+// workgroup), cut every long row where its sorted columns cross the boundaries
+// of its source bands and into items of at most 64 edges, key every item by its
+// middle source id, stable radix sort, write the records.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
 
 #include "../../include/yitu_hip.h"
 #include "plan.hpp"
@@ -22,23 +21,17 @@ struct BuildBuffers {
     PlanCounters *counters;
     int4 *rows;
     int4 *records;
-    int *slab_bound;  // [kPlanSlabs + 1] first source id of every slab, in the plan
+    int *band_info;   // {log2 of the band width, number of bands}, in the plan header
     int4 *items;      // {first edge, end edge, index into rows[], row} in queue order
     uint32_t *keys_in, *keys_out;
     int32_t *vals_in, *order;
     void *sort_temp;
     size_t sort_temp_bytes;
-    uint32_t *pop;           // [n_buckets] edges per bucket of 2^bucket_shift consecutive sources
-    unsigned long long *cost;  // [n_buckets] inclusive prefix sums of popularity^0.75
-    void *scan_temp;
-    size_t scan_temp_bytes;
-    int n_buckets, bucket_shift, band_shift;
+    int key_shift;    // sort key = middle source id >> key_shift (16 bits)
+    int band_shift;   // band of a source = id >> band_shift
+    int n_bands;      // 1 = no cuts
     int max_rows, max_items;
 };
-
-// Number of popularity buckets a graph of nnz edges gets (bounds the workspace
-// by the edge count whatever the number of sources).
-inline int64_t pop_buckets(int64_t nnz) { return std::max<int64_t>(4096, nnz / 4); }
 
 __global__ __launch_bounds__(kBlock) void plan_init_kernel(BuildBuffers b) {
     const int64_t i0 = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -49,8 +42,10 @@ __global__ __launch_bounds__(kBlock) void plan_init_kernel(BuildBuffers b) {
         b.counters->overflow = 0;
         b.counters->pad = 0;
     }
-    if (i0 <= kPlanSlabs) b.slab_bound[i0] = i0 == 0 ? 0 : 0x7fffffff;
-    for (int64_t i = i0; i < b.n_buckets; i += stride) b.pop[i] = 0u;
+    if (i0 == 0) {
+        b.band_info[0] = b.band_shift;
+        b.band_info[1] = b.n_bands;
+    }
     // slots that get no item sort behind every real key
     for (int64_t i = i0; i < b.max_items; i += stride) {
         b.keys_in[i] = 0xffffu;
@@ -61,91 +56,62 @@ __global__ __launch_bounds__(kBlock) void plan_init_kernel(BuildBuffers b) {
 // Every lane owns one row; the long rows of a workgroup are numbered with a
 // block-level prefix sum and ONE atomic (hundreds of thousands of same-address
 // atomics serialise in L2).
-__global__ __launch_bounds__(kBlock) void plan_queue_kernel(BuildBuffers b,
-                                                            const int32_t *__restrict__ indptr,
-                                                            int n_rows) {
-    __shared__ int wave_rows[kWavesPerBlock];
-    __shared__ int block_first_row;
+__device__ __forceinline__ int block_rank(bool flag, int *wave_sums, int *block_base, int *counter) {
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
-    const int row = blockIdx.x * kBlock + threadIdx.x;
-    int deg = 0;
-    if (row < n_rows) deg = indptr[row + 1] - indptr[row];
-    const bool longrow = deg >= kPlanThreshold;
-    int pre = longrow ? 1 : 0;
+    int pre = flag ? 1 : 0;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
         const int x = __shfl_up(pre, o, kWave);
         if (lane >= o) pre += x;
     }
-    if (lane == kWave - 1) wave_rows[wave] = pre;
-    pre -= longrow ? 1 : 0;
+    if (lane == kWave - 1) wave_sums[wave] = pre;
+    pre -= flag ? 1 : 0;
     __syncthreads();
     if (threadIdx.x == 0) {
         int br = 0;
-        for (int w = 0; w < kWavesPerBlock; w++) br += wave_rows[w];
-        block_first_row = br > 0 ? atomicAdd(&b.counters->n_rows, br) : 0;
+        for (int w = 0; w < kWavesPerBlock; w++) br += wave_sums[w];
+        *block_base = br > 0 ? atomicAdd(counter, br) : 0;
     }
     __syncthreads();
-    if (!longrow) return;
-    int slot = block_first_row + pre;
-    for (int w = 0; w < wave; w++) slot += wave_rows[w];
-    if (slot >= b.max_rows) {
-        atomicExch(&b.counters->overflow, 1);
-        return;
+    int slot = *block_base + pre;
+    for (int w = 0; w < wave; w++) slot += wave_sums[w];
+    __syncthreads();  // the shared words are reused by the next call
+    return slot;
+}
+
+__global__ __launch_bounds__(kBlock) void plan_queue_kernel(BuildBuffers b,
+                                                            const int32_t *__restrict__ indptr,
+                                                            int n_rows) {
+    __shared__ int wave_sums[kWavesPerBlock];
+    __shared__ int block_base;
+    const int row = blockIdx.x * kBlock + threadIdx.x;
+    int deg = 0;
+    if (row < n_rows) deg = indptr[row + 1] - indptr[row];
+    const bool longrow = deg >= kPlanThreshold;
+    const int slot = block_rank(longrow, wave_sums, &block_base, &b.counters->n_rows);
+    if (longrow) {
+        if (slot >= b.max_rows)
+            atomicExch(&b.counters->overflow, 1);
+        else
+            b.rows[slot] = make_int4(row, 0, 0, 0);
     }
-    b.rows[slot] = make_int4(row, 0, 0, 0);
 }
 
-__global__ __launch_bounds__(kBlock) void plan_popularity_kernel(BuildBuffers b,
-                                                                 const int32_t *__restrict__ indices,
-                                                                 int64_t nnz, int col_mask,
-                                                                 int n_src) {
-    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (; i < nnz; i += stride) {
-        const int c = indices[i] & col_mask;
-        if (c < n_src) atomicAdd(&b.pop[c >> b.bucket_shift], 1u);
-    }
-}
-
-// Cost of a bucket of sources: popularity^0.75 in quarter units. A source that
-// many edges read is fetched into L2 once and then hit, so what it costs grows
-// more slowly than its edge count.
-__global__ __launch_bounds__(kBlock) void plan_cost_kernel(BuildBuffers b) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= b.n_buckets) return;
-    const float r = sqrtf((float)b.pop[i]);
-    b.cost[i] = (unsigned long long)(r * sqrtf(r) * 4.0f + 0.5f);
-}
-
-// Slab k starts at the first bucket where the running cost reaches k/8 of the total.
-__global__ void plan_bounds_kernel(BuildBuffers b) {
-    const int k = threadIdx.x;
-    if (k < 1 || k >= kPlanSlabs) return;
-    const unsigned long long total = b.cost[b.n_buckets - 1];
-    const unsigned long long target = total / kPlanSlabs * k;
-    int lo = 0, hi = b.n_buckets;  // first index with cost >= target
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (b.cost[mid] < target) lo = mid + 1; else hi = mid;
-    }
-    const long long bound = ((long long)lo + 1) << b.bucket_shift;
-    b.slab_bound[k] = (int)(bound < 0x7fffffffLL ? bound : 0x7fffffffLL);
-}
-
-// One wave per long row. Lanes 0..4 find where the row's columns cross the slab
-// boundaries; lane 0 turns the crossings into at most min(4, deg / 16) segments
-// (none shorter than kPlanMinSegment), the wave then writes the items of every
-// segment: ceil(len / 64) pieces of equal size. Item ids of a row are
-// consecutive; a workgroup takes its ids with one atomic.
+// One wave per long row. A row of deg edges may be cut into P = the largest
+// power of two <= deg / 16 pieces (at most the number of bands), so its cut points
+// are the boundaries of groups of ceil(n_bands / P) consecutive bands: the lanes
+// find where the row's columns cross them (binary search), lane 0 turns the
+// crossings into segments (none shorter than kPlanMinSegment), the wave then
+// writes the items of every segment: ceil(len / 64) pieces of equal size. Item
+// ids of a row are consecutive; a workgroup takes its ids with one atomic.
 __global__ __launch_bounds__(kBlock) void plan_items_kernel(BuildBuffers b,
                                                             const int32_t *__restrict__ indptr,
                                                             const int32_t *__restrict__ indices,
-                                                            int col_mask, int with_slabs) {
-    __shared__ int cut[kWavesPerBlock][kPlanSlabs + 1];
-    __shared__ int seg_beg[kWavesPerBlock][kPlanSlabs + 1];    // [n_seg] = end of the row
-    __shared__ int seg_first[kWavesPerBlock][kPlanSlabs + 1];  // first item of the segment, [n_seg] = total
+                                                            int col_mask) {
+    __shared__ int cut[kWavesPerBlock][kPlanMaxBands + 1];
+    __shared__ int seg_beg[kWavesPerBlock][kPlanMaxBands + 1];    // [n_seg] = end of the row
+    __shared__ int seg_first[kWavesPerBlock][kPlanMaxBands + 1];  // first item of the segment, [n_seg] = total
     __shared__ int n_seg[kWavesPerBlock];
     __shared__ int wave_first[kWavesPerBlock];
     const int lane = lane_id();
@@ -159,35 +125,38 @@ __global__ __launch_bounds__(kBlock) void plan_items_kernel(BuildBuffers b,
         beg = indptr[row];
         end = indptr[row + 1];
     }
-    constexpr int NS = kPlanSlabs;
-    if (active && lane <= NS) {
-        int c = lane == 0 ? beg : end;
-        if (with_slabs && lane > 0 && lane < NS) {
-            const int bound = b.slab_bound[lane];
+    const int deg = end - beg;
+    // pieces allowed, bands per group, groups
+    int allowed = 1;
+    while (allowed * 2 * kPlanMinSegment <= deg && allowed * 2 <= b.n_bands) allowed *= 2;
+    if (b.n_bands > 1 && allowed * 2 * kPlanMinSegment <= deg) allowed = b.n_bands;
+    const int per_group = (b.n_bands + allowed - 1) / allowed;
+    const int n_groups = active ? (b.n_bands + per_group - 1) / per_group : 0;
+    for (int k = lane; k <= n_groups; k += kWave) {
+        int c = k == 0 ? beg : end;
+        if (k > 0 && k < n_groups) {
+            const long long bound = ((long long)k * per_group) << b.band_shift;
             int lo = beg, hi = end;  // first edge whose column is >= bound
             while (lo < hi) {
                 const int mid = (lo + hi) >> 1;
-                if ((indices[mid] & col_mask) < bound) lo = mid + 1; else hi = mid;
+                if ((long long)(indices[mid] & col_mask) < bound) lo = mid + 1; else hi = mid;
             }
             c = lo;
         }
-        cut[wave][lane] = c;
+        cut[wave][k] = c;
     }
-    if (active && lane == 0) cut[wave][NS] = end;
     __syncthreads();
     if (active && lane == 0) {
         // columns that are not sorted inside the row give crossings out of order;
         // a running maximum keeps the pieces a partition of the row
-        const int deg = end - beg;
-        const int max_seg = max(1, min(NS, deg / kPlanMinSegment));
         int n = 0, cur = beg, total = 0, reach = beg;
-        for (int k = 1; k <= NS; k++) {
+        for (int k = 1; k <= n_groups; k++) {
             reach = min(end, max(reach, cut[wave][k]));
-            const bool last = k == NS;
+            const bool last = k == n_groups;
             const int len = reach - cur;
             if (last ? len > 0
                      : (len >= kPlanMinSegment && end - reach >= kPlanMinSegment &&
-                        n < max_seg - 1)) {
+                        n < allowed - 1)) {
                 seg_beg[wave][n] = cur;
                 seg_first[wave][n] = total;
                 total += (len + kPlanChunk - 1) / kPlanChunk;
@@ -223,8 +192,8 @@ __global__ __launch_bounds__(kBlock) void plan_items_kernel(BuildBuffers b,
         return;
     }
     if (lane == 0) b.rows[slot] = make_int4(row, first_item, total, 0);
+    int s = 0;  // items of a lane come in ascending order: the segment search resumes
     for (int i = lane; i < total; i += kWave) {
-        int s = 0;
         while (s + 1 < n && seg_first[wave][s + 1] <= i) s++;
         const int sb = seg_beg[wave][s], se = seg_beg[wave][s + 1];
         const int pieces = seg_first[wave][s + 1] - seg_first[wave][s];
@@ -234,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void plan_items_kernel(BuildBuffers b,
         const int mid_col = indices[(ib + ie) >> 1] & col_mask;
         b.items[first_item + i] = make_int4(ib, ie, slot, row);
         b.keys_in[first_item + i] =
-            min((uint32_t)mid_col >> b.band_shift, (1u << kBandBits) - 1u);
+            min((uint32_t)mid_col >> b.key_shift, (1u << kBandBits) - 1u);
     }
 }
 
@@ -261,15 +230,7 @@ size_t sort_temp_bytes(int64_t n) {
     return bytes;
 }
 
-size_t scan_temp_bytes(int64_t n) {
-    size_t bytes = 0;
-    unsigned long long *c = nullptr;
-    (void)rocprim::inclusive_scan(nullptr, bytes, c, c, (size_t)n,
-                                  rocprim::plus<unsigned long long>());
-    return bytes;
-}
-
-constexpr size_t kHeaderBytes = 512;  // counters | slab_bound[kPlanSlabs + 1]
+constexpr size_t kHeaderBytes = 512;  // counters | at byte 256: {log2 band width, bands}
 
 }  // namespace
 
@@ -280,12 +241,8 @@ size_t plan_bytes(int64_t nnz) {
 
 size_t plan_build_workspace_bytes(int64_t nnz) {
     const size_t items = (size_t)plan_max_items(nnz);
-    const size_t buckets = (size_t)pop_buckets(nnz);
     return align_up(sizeof(int4) * items, 256) + 4 * align_up(sizeof(int32_t) * items, 256) +
-           align_up(sort_temp_bytes((int64_t)items), 256) +
-           align_up(sizeof(uint32_t) * buckets, 256) +
-           align_up(sizeof(unsigned long long) * buckets, 256) +
-           align_up(scan_temp_bytes((int64_t)buckets), 256);
+           align_up(sort_temp_bytes((int64_t)items), 256);
 }
 
 size_t plan_temp_bytes(int64_t nnz) { return plan_bytes(nnz) + plan_build_workspace_bytes(nnz); }
@@ -305,7 +262,7 @@ PlanView plan_view(const void *plan, int64_t nnz) {
 }
 
 int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_t *indices,
-               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, bool with_slabs,
+               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, bool with_bands,
                void *workspace, size_t workspace_bytes, hipStream_t stream) {
     YITU_REQUIRE(plan && plan_size >= plan_bytes(nnz), "plan buffer too small: need %zu bytes",
                  plan_bytes(nnz));
@@ -318,7 +275,7 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
     const PlanView v = plan_view(plan, nnz);
     BuildBuffers b{};
     b.counters = const_cast<PlanCounters *>(v.counters);
-    b.slab_bound = reinterpret_cast<int *>(static_cast<char *>(plan) + 256);
+    b.band_info = reinterpret_cast<int *>(static_cast<char *>(plan) + 256);
     b.rows = const_cast<int4 *>(v.rows);
     b.records = const_cast<int4 *>(v.records);
     b.max_rows = v.max_rows;
@@ -335,19 +292,12 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
     b.sort_temp = w;
     b.sort_temp_bytes = sort_temp_bytes(b.max_items);
     w += align_up(b.sort_temp_bytes, 256);
-    const int64_t max_buckets = pop_buckets(nnz);
-    b.bucket_shift = 0;
-    while (((std::max<int64_t>(n_src, 1) - 1) >> b.bucket_shift) + 1 > max_buckets) b.bucket_shift++;
-    b.n_buckets = with_slabs ? (int)(((std::max<int64_t>(n_src, 1) - 1) >> b.bucket_shift) + 1) : 0;
-    b.pop = reinterpret_cast<uint32_t *>(w);
-    w += align_up(sizeof(uint32_t) * (size_t)max_buckets, 256);
-    b.cost = reinterpret_cast<unsigned long long *>(w);
-    w += align_up(sizeof(unsigned long long) * (size_t)max_buckets, 256);
-    b.scan_temp = w;
-    b.scan_temp_bytes = scan_temp_bytes(max_buckets);
-    b.band_shift = 0;
-    while (((std::max<int64_t>(n_src, 1) - 1) >> b.band_shift) >= ((int64_t)1 << kBandBits))
-        b.band_shift++;
+    const int64_t span = std::max<int64_t>(n_src, 1) - 1;  // largest source id
+    b.key_shift = 0;
+    while ((span >> b.key_shift) >= ((int64_t)1 << kBandBits)) b.key_shift++;
+    b.band_shift = kPlanBandShift;
+    while ((span >> b.band_shift) + 1 > kPlanMaxBands) b.band_shift++;
+    b.n_bands = with_bands ? (int)((span >> b.band_shift) + 1) : 1;
 
     const int item_grid = (int)ceil_div(b.max_items, kBlock);
     plan_init_kernel<<<std::min(item_grid, 4096), kBlock, 0, stream>>>(b);
@@ -357,21 +307,8 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
                                                                                 (int)n_rows);
         YITU_LAUNCH_CHECK();
     }
-    if (with_slabs && nnz > 0) {
-        plan_popularity_kernel<<<(int)std::min<int64_t>(ceil_div(nnz, kBlock), 16384), kBlock, 0,
-                                 stream>>>(b, indices, nnz, col_mask, (int)n_src);
-        YITU_LAUNCH_CHECK();
-        plan_cost_kernel<<<(int)ceil_div(b.n_buckets, kBlock), kBlock, 0, stream>>>(b);
-        YITU_LAUNCH_CHECK();
-        size_t scan_bytes = b.scan_temp_bytes;
-        YITU_HIP(rocprim::inclusive_scan(b.scan_temp, scan_bytes, b.cost, b.cost,
-                                         (size_t)b.n_buckets,
-                                         rocprim::plus<unsigned long long>(), stream));
-        plan_bounds_kernel<<<1, kWave, 0, stream>>>(b);
-        YITU_LAUNCH_CHECK();
-    }
     plan_items_kernel<<<(int)ceil_div(b.max_rows, kWavesPerBlock), kBlock, 0, stream>>>(
-        b, indptr, indices, col_mask, with_slabs && nnz > 0 ? 1 : 0);
+        b, indptr, indices, col_mask);
     YITU_LAUNCH_CHECK();
     size_t temp_bytes = b.sort_temp_bytes;
     YITU_HIP(rocprim::radix_sort_pairs(b.sort_temp, temp_bytes, b.keys_in, b.keys_out, b.vals_in,

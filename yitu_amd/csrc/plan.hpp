@@ -8,19 +8,20 @@
 // speed. Short rows are not in the plan; a wave of the row kernels walks 16 of
 // them in a row.
 //
-// Slabs: the source ids are cut into 4 contiguous ranges and a long row is cut
-// where its (sorted) columns cross a range boundary (at most deg / 16 pieces,
-// none shorter than 16 edges), so most items gather from one range only. With
-// items that straddle the whole id space, the band that the chip reads at one
-// moment is polluted by the far ends of every item; with the cuts it is not
-// (measured on a 2^21-node R-MAT graph: 3 to 7 % less time for the fp32 SpMM;
-// 8 and 16 ranges cut the rows into smaller items and cost the bf16 path more
-// than they gain).
-// Boundaries are placed so that the ranges have equal sums of popularity^0.75
-// over their sources: a hot source is fetched into L2 once and then hit, so its
-// cost grows more slowly than its edge count, and equal-cost ranges keep the
-// pieces of a row from being either tiny or huge. A plan built without slabs
-// (the temporary plan of a call that was given none) makes no such cuts.
+// Bands: the source ids are cut into bands of 2^17 consecutive ids (wider when
+// that would give more than 64 bands) and a long row is cut where its (sorted)
+// columns cross band boundaries, so that most items gather from one band and
+// the items of a band, which the sort puts side by side, share their sources.
+// A row of deg edges is cut into at most deg / 16 pieces, none shorter than 16
+// edges: rows too short for one piece per band are cut at the boundaries of
+// groups of 2, 4, ... bands. With items that straddle the whole id space, the
+// band that the chip reads at one moment is polluted by the far ends of every
+// item; with the cuts it is not. Measured on a 2^21-node R-MAT graph (fp32,
+// F = 128, 3.08 ms per call without cuts): bands of 2^12 .. 2^19 ids give 2.78,
+// 2.79, 2.78, 2.76, 2.69, 2.71 ms: a band is far wider than what an L2 holds
+// (8 k rows of 512 bytes) at any of these widths, so narrow bands only add
+// partial rows. A plan built without bands (the temporary plan of a call that
+// was given none) makes no such cuts.
 //
 // The plan depends on the graph only. It is the counterpart of the reference's
 // neighbour-group partition (build_part, ccsrc/kernel/YiTu_GNN.cpp:203-245):
@@ -33,7 +34,8 @@ namespace yitu {
 
 constexpr int kPlanChunk = 64;      // edges per item = one edge window of a wave
 constexpr int kPlanThreshold = 64;  // rows with at least this many edges are planned
-constexpr int kPlanSlabs = 4;       // source ranges at whose boundaries long rows are cut
+constexpr int kPlanBandShift = 17;  // log2 of the narrowest source band
+constexpr int kPlanMaxBands = 64;   // bands get wider beyond 2^23 sources
 constexpr int kPlanMinSegment = 16; // a row of deg edges is cut into at most deg / 16 pieces,
                                     // none shorter than this
 
@@ -55,7 +57,7 @@ struct PlanView {
 };
 
 inline int64_t plan_max_rows(int64_t nnz) { return nnz / kPlanThreshold + 1; }
-// A row of deg >= 64 edges gives at most deg / 64 + min(4, deg / 16) items.
+// A row of deg >= 64 edges gives at most deg / 64 + min(bands, deg / 16) items.
 inline int64_t plan_max_items(int64_t nnz) {
     return nnz / kPlanChunk + nnz / kPlanMinSegment + plan_max_rows(nnz) + 1;
 }
@@ -63,9 +65,9 @@ inline int64_t plan_max_items(int64_t nnz) {
 size_t plan_bytes(int64_t nnz);
 size_t plan_build_workspace_bytes(int64_t nnz);
 // Builds into `plan` (plan_bytes(nnz) of device memory, 256-byte aligned).
-// with_slabs = false skips the popularity pass and puts every item in slab 0.
+// with_bands = false cuts no row at band boundaries.
 int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_t *indices,
-               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, bool with_slabs,
+               int64_t n_rows, int64_t n_src, int64_t nnz, int32_t col_mask, bool with_bands,
                void *workspace, size_t workspace_bytes, hipStream_t stream);
 PlanView plan_view(const void *plan, int64_t nnz);
 // A view that plans nothing (every row is handled by the row kernels).

@@ -29,6 +29,26 @@ int fill_zero(float *p, int64_t n, hipStream_t stream) {
     return 0;
 }
 
+// w[e] = scale[col[e]]: the per-edge column scale of the GCN norm, computed once
+// per graph so that the aggregation kernels read it in edge order.
+__global__ __launch_bounds__(kBlock) void edge_scale_kernel(float *__restrict__ w,
+                                                            const int32_t *__restrict__ indices,
+                                                            const float *__restrict__ scale,
+                                                            int64_t nnz, int col_mask) {
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (; i < nnz; i += stride) w[i] = scale[indices[i] & col_mask];
+}
+
+int edge_scale_fill(float *w, const int32_t *indices, const float *scale, int64_t nnz, int col_mask,
+                    hipStream_t stream) {
+    if (nnz <= 0) return 0;
+    edge_scale_kernel<<<(int)std::min<int64_t>(ceil_div(nnz, kBlock), 16384), kBlock, 0, stream>>>(
+        w, indices, scale, nnz, col_mask);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
 size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan) {
     size_t b = align_up(sizeof(float) * (size_t)plan_max_items(nnz) * (size_t)L, 256);
     if (!with_plan) b += plan_temp_bytes(nnz);

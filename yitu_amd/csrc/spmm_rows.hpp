@@ -35,6 +35,8 @@ struct SpmmParams {
     float *out;              // [n_rows, L]
     const float *scale_row;  // W_DEGPROD: s[n_rows]; otherwise unused
     const float *scale_col;  // W_DEGPROD: s[n_src]
+    const float *edge_scale; // W_DEGPROD, optional: [nnz] = s[col of the edge], read in edge
+                             // order instead of one random read of scale_col per edge
     const float *values;     // W_EDGEHEAD: [nnz, H]
     const int32_t *eperm;    // optional: values row of edge i is eperm[i] (transposed pass)
     int n_rows;
@@ -71,7 +73,8 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
     win.col = p.cols_are_edges ? e : (p.indices[e] & p.col_mask);
     win.w = 1.0f;
     win.vrow = 0;
-    if constexpr (WMODE == W_DEGPROD) win.w = p.scale_col[win.col];
+    if constexpr (WMODE == W_DEGPROD)
+        win.w = p.edge_scale ? p.edge_scale[e] : p.scale_col[win.col];
     if constexpr (WMODE == W_EDGEHEAD) win.vrow = p.eperm ? p.eperm[e] : e;
 }
 
@@ -641,6 +644,9 @@ int spmm_backward_run(float *grad_a, float *grad_x, const float *values, const i
                       int64_t n_features, int64_t max_degree, int64_t max_degree_t,
                       const void *plan, const void *plan_t, void *workspace,
                       size_t workspace_bytes, bool long_rows_only, hipStream_t stream);
+// w[e] = scale[indices[e] & col_mask] for every edge.
+int edge_scale_fill(float *w, const int32_t *indices, const float *scale, int64_t nnz, int col_mask,
+                    hipStream_t stream);
 const char *last_error();
 // Zero-fill by kernel (safe to record into a captured graph, unlike a memset node).
 int fill_zero(float *p, int64_t n, hipStream_t stream);

@@ -16,12 +16,14 @@ class GNNAFunction(th.autograd.Function):
     def forward(ctx, X, weight, inputInfo):
         ctx.save_for_backward(X, weight)
         ctx.tail = graph_arguments(inputInfo, inputInfo.degrees)
-        return YiTu_GNN_kernel.forward(X, weight, *ctx.tail)[0]
+        # per-edge column scales, when the carrier has prepared them (prepare_edge_scale)
+        ctx.edge_scale = getattr(inputInfo, "edge_scale", None)
+        return YiTu_GNN_kernel.forward(X, weight, *ctx.tail, edge_scale=ctx.edge_scale)[0]
 
     @staticmethod
     def backward(ctx, d_output):
         d_input, d_weight = YiTu_GNN_kernel.backward(d_output.contiguous(), *ctx.saved_tensors,
-                                                     *ctx.tail)
+                                                     *ctx.tail, edge_scale=ctx.edge_scale)
         return d_input, d_weight, None
 
 

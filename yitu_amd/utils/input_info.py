@@ -42,6 +42,27 @@ def worth_reordering(avg_edge_span, num_nodes) -> bool:
 
 
 class InputInfo(object):
+    # Replacing the column ids or the scale vector drops the per-edge scales derived from
+    # them (prepare_edge_scale); writing INTO those tensors in place does not, and then
+    # prepare_edge_scale has to be called again by whoever wrote.
+    @property
+    def column_index(self):
+        return self._column_index
+
+    @column_index.setter
+    def column_index(self, value):
+        self._column_index = value
+        self.edge_scale = None
+
+    @property
+    def degrees(self):
+        return self._degrees
+
+    @degrees.setter
+    def degrees(self, value):
+        self._degrees = value
+        self.edge_scale = None
+
     def __init__(self, row_pointers=None, column_index=None, degrees=None, partSize=None,
                  dimWorker=None, warpPerBlock=None, sharedMem=None, hiddenDim=None,
                  dataset_obj=None, enable_rabbit=False, manual_mode=True, verbose=False):
@@ -65,6 +86,9 @@ class InputInfo(object):
         self.manual_mode, self.enable_rabbit, self.verbose_flag = manual_mode, enable_rabbit, verbose
         self.state_set_input = False
         self.reorder_status = False
+        # per-edge column scales for the GCN aggregation (see prepare_edge_scale); not in
+        # the reference's carrier
+        self.edge_scale = None
 
     def _reorder(self, wanted: bool):
         self.dataset_obj.reorder_flag = wanted
@@ -89,6 +113,16 @@ class InputInfo(object):
         if self.enable_rabbit:
             self._reorder(worth_reordering(self.avgEdgeSpan, self.num_nodes))
             self.dataset_obj.rabbit_reorder()
+
+    def prepare_edge_scale(self):
+        """Per-graph preparation for the GCN layers: ``edge_scale[e] = degrees[column_index[e]]``
+        (YiTu_GNN_kernel.edge_scale), so the aggregation reads the column scale of an edge
+        in edge order instead of gathering ``degrees``. Call after ``decider`` (a reorder
+        replaces the CSR) and again whenever ``column_index`` or ``degrees`` are replaced;
+        setting ``self.edge_scale = None`` returns to the reference's form. Returns self."""
+        from .. import YiTu_GNN_kernel
+        self.edge_scale = YiTu_GNN_kernel.edge_scale(self.column_index, self.degrees)
+        return self
 
     def _select(self, for_input: bool):
         suffix = "_input" if for_input else "_hidden"
