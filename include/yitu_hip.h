@@ -94,6 +94,24 @@ int yitu_agg_csr(float *out_device, const void *x_device, int x_is_bf16,
                  const float *edge_scale_device, void *workspace_device, size_t workspace_bytes,
                  void *stream);
 
+/*
+ * yitu_agg_csr for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same result as
+ * yitu_agg_csr given no plan and no edge scales, but its scratch (the temporary
+ * row plan and the partial rows of long rows) is a static device array of
+ * yitu_agg_csr_noalloc_max_bytes() = 32 MiB inside the library instead of a
+ * caller's workspace. No counterpart in the reference. It calls no hipMalloc /
+ * hipFree or any allocating routine; problems whose
+ * yitu_spmm_workspace_bytes(nnz, dim, 0) exceeds the array are rejected (< 0).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (different streams or threads) race and must be serialised by the caller.
+ */
+size_t yitu_agg_csr_noalloc_max_bytes(void);
+int yitu_agg_csr_noalloc(float *out_device, const void *x_device, int x_is_bf16,
+                         const int32_t *row_pointers_device, const int32_t *column_index_device,
+                         const float *degrees_device, int64_t n_rows, int64_t n_src, int64_t nnz,
+                         int64_t dim, float alpha, int64_t max_degree, void *stream);
+
 /* edge_scale[e] = degrees[column_index[e]] for the nnz edges of a CSR: per-graph
  * preparation for yitu_agg_csr, like the row plan (the reference's callers hold
  * `degrees` per graph, data/dataset.py:131-136, and pass it to every call). */

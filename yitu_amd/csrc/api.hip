@@ -3,6 +3,8 @@
 
 #include "spmm_rows.hpp"
 
+#include <mutex>
+
 using namespace yitu;
 
 #define YITU_API extern "C" __attribute__((visibility("default")))
@@ -50,6 +52,55 @@ YITU_API int yitu_edge_scale(float *edge_scale, const int32_t *column_index, con
     YITU_REQUIRE(edge_scale && column_index && degrees, "null pointer");
     return edge_scale_fill(edge_scale, column_index, degrees, nnz, 0x7fffffff,
                            static_cast<hipStream_t>(stream));
+}
+
+// ---- aggregation without any allocation ------------------------------------------
+// The scratch of yitu_agg_csr (temporary row plan + partial rows) taken from a
+// file-scope device array instead of a caller's workspace. Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process
+// ends; the name below is only a host-side handle, the address on the current
+// device comes from hipGetSymbolAddress, once per device.
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int static_scratch(void **ptr) {
+    int dev = 0;
+    YITU_HIP(hipGetDevice(&dev));
+    YITU_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        YITU_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        YITU_REQUIRE(p != nullptr, "no device address for the static scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+YITU_API size_t yitu_agg_csr_noalloc_max_bytes(void) { return kStaticScratchBytes; }
+
+YITU_API int yitu_agg_csr_noalloc(float *out, const void *x, int x_is_bf16,
+                                  const int32_t *row_pointers, const int32_t *column_index,
+                                  const float *degrees, int64_t n_rows, int64_t n_src,
+                                  int64_t nnz, int64_t dim, float alpha, int64_t max_degree,
+                                  void *stream) {
+    YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0 && dim >= 0, "negative size");
+    const size_t need = spmm_workspace_bytes(nnz, dim, false);
+    YITU_REQUIRE(need <= kStaticScratchBytes,
+                 "problem needs %zu bytes of scratch, the static array holds %zu: use "
+                 "yitu_agg_csr with a workspace",
+                 need, kStaticScratchBytes);
+    void *ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    return yitu_agg_csr(out, x, x_is_bf16, row_pointers, column_index, degrees, n_rows, n_src, nnz,
+                        dim, alpha, max_degree, nullptr, nullptr, ws, kStaticScratchBytes, stream);
 }
 
 static int spmm_forward_any(float *out, const float *values, const int32_t *indptr,
