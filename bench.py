@@ -29,16 +29,25 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM-side bytes per call (reads + writes leaving L2) measured with two rocprofv3 --pmc
-# runs of this file, FETCH_SIZE then WRITE_SIZE, each scaled by what the same counter
-# reads for the library's 1 GiB copy kernel (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000):
-# profiles/bench_c3_spmm_gat_rocprofv3.md. Per yitu_agg_csr call for the C3 workloads,
-# per yitu_gat_forward call for C2.
-MEASURED_TRAFFIC_BYTES = {
-    "c3_spmm_f32": 21_418_734_739,
-    "c3_spmm_bf16": 10_965_161_440,
-    "c2_gat_f32": 5_478_204_769,
-}
+# Bytes per call that left L2 towards the fabric (Infinity Cache or HBM), reads + writes:
+# two rocprofv3 --pmc runs of this file, FETCH_SIZE then WRITE_SIZE, each scaled by what
+# the same counter reads for the library's 1 GiB copy kernel. The figures live beside the
+# profile summary they were taken with, together with the commit they were measured on;
+# this run does not measure them itself.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "l2_miss_traffic.json")
+
+
+def measured_traffic(name):
+    """(bytes per call, provenance) from profiles/l2_miss_traffic.json, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+        entry = table["workloads"][name]
+        return int(entry["bytes_per_call"]), {
+            "file": "profiles/l2_miss_traffic.json", "measured_on_commit": table.get("commit"),
+            "what": "L2-miss traffic (FETCH_SIZE + WRITE_SIZE, copy-calibrated), not HBM bytes"}
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def _sync():
@@ -93,14 +102,14 @@ def cpu_baseline_spmm(rp, ci, deg, x, dy):
     oracle.row_agg(x_h[:1024], rp_h[:1025] - rp_h[0], ci_h[:rp_h[1024]], deg_h, oracle.MODE_GCN,
                    f64=False)  # warm-up: loads the library, spins up the team
     times = []
-    for _ in range(2):
+    for _ in range(5):
         t0 = time.perf_counter()
         oracle.row_agg(x_h, rp_h, ci_h, deg_h, oracle.MODE_GCN, f64=False)
         oracle.row_agg(dy_h, rp_h, ci_h, deg_h, oracle.MODE_GCN, f64=False)
         times.append(time.perf_counter() - t0)
-    t = min(times)
+    t = sorted(times)[len(times) // 2]
     return {"value": ci_h.shape[0] / t, "unit": "edges/s", "cores": cores, "kind": "port",
-            "sample": "full workload (2^21 nodes, %d edges, F=128), fwd+bwd, best of 2, "
+            "sample": "full workload (2^21 nodes, %d edges, F=128), fwd+bwd, median of 5, "
                       "OpenMP float restatement oracle/yitu_oracle.c" % ci_h.shape[0],
             "seconds": t}
 
@@ -185,6 +194,7 @@ def run_spmm(args, dev, bf16):
     alg = 4 * (n + 1) + 4 * nnz + 4 * n + b_in * n * dim + 4 * n * dim  # per aggregation call
     achieved = alg / (call_ms * 1e-3) / 1e9
     name = "c3_spmm_bf16" if bf16 else "c3_spmm_f32"
+    traffic, traffic_source = measured_traffic(name)
     res = {
         "metric": "SpMM edges/sec (GCN aggregation fwd+bwd, n_edges / step time)",
         "value": nnz / (ms_per_step * 1e-3),
@@ -199,9 +209,10 @@ def run_spmm(args, dev, bf16):
                    "step": "aggregate(X) + aggregate(dY), same CSR, W = I"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "one yitu_agg_csr call = spmm_rows_kernel + spmm_items_kernel + "
-                               "spmm_reduce_kernel (row plan built once per graph, untimed)",
+                               "spmm_reduce_kernel (row plan and per-edge column scales built "
+                               "once per graph, untimed)",
                      "kernel_ms": call_ms, "algorithmic_bytes": alg,
                      "gather_bytes_no_reuse": nnz * dim * b_in},
     }
@@ -345,7 +356,8 @@ def run_gat(args, dev):
         "roofline": {"bound": "hbm", "achieved": alg_fwd / (fwd_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("c2_gat_f32"),
+                     "traffic": measured_traffic("c2_gat_f32")[0],
+                     "traffic_source": measured_traffic("c2_gat_f32")[1],
                      "kernel": "yitu_gat_forward (row statistics out, no stored probabilities) = "
                                "gat_rows_kernel + gat_item_local_kernel + gat_row_combine_kernel "
                                "+ gat_scaled_reduce_kernel",
@@ -507,9 +519,33 @@ def run_c4(args, dev):
     def agg16():
         return graph_ext.spmm_forward(values, indptr, indices, h_all16.view(n_all, 1, dim))
 
+    d_out16 = d_out.to(torch.bfloat16)
+
+    def agg_bwd16():
+        # bf16 gradient rows in, fp32 sums, fp32 rows out
+        return graph_ext.spmm_backward(values, indptr, indices, h_all16.view(n_all, 1, dim),
+                                       d_out16.view(n_all, 1, dim), need_grad_a=False)[1]
+
+    def gemm_bwd16(dh):
+        dh16 = dh.view(n_all, dim).to(torch.bfloat16)  # one rounding pass over the gradient rows
+        parts = [dh16[off[t]:off[t + 1]] for t in range(4)]
+        dws = [graph_ext.gemm_bf16_tn(xs16[t], parts[t]) for t in range(4)]
+        dxs = [graph_ext.gemm_bf16(parts[t], wts16[t], trans_b=True, out_dtype=torch.bfloat16)
+               for t in range(4)]
+        return dws, dxs
+
     gemm16()
+    dh_16 = agg_bwd16()
+    dws16, _ = gemm_bwd16(dh_16)
+    dws32 = graph_ext.sgemm_typed(xs, [dh.view(n_all, dim)[off[t]:off[t + 1]] for t in range(4)],
+                                  trans_a=True)
+    for a16, a32 in zip(dws16, dws32):
+        if not torch.allclose(a16, a32, rtol=3e-2, atol=3e-2 * float(a32.abs().max())):
+            raise RuntimeError("bf16 weight gradient differs from the fp32 one beyond bf16 rounding")
     t_gemm16 = _event_ms(gemm16, steps, warm)
     t_agg16 = _event_ms(agg16, steps, warm)
+    t_agg_b16 = _event_ms(agg_bwd16, steps, warm)
+    t_gemm_b16 = _event_ms(lambda: gemm_bwd16(dh_16), steps, warm)
     t_torch16 = _event_ms(lambda: [torch.mm(x, w) for x, w in zip(xs16, wts16)], steps, warm)
     bytes16 = sum(2 * n * dim * 2 + 2 * dim * dim for n in sizes)
     gather = n_edges * dim * 4
@@ -525,6 +561,8 @@ def run_c4(args, dev):
             "agg_gather_GBps": gather / (t_agg_f * 1e-3) / 1e9,
             "modules": module_ms,
             "bf16": {"gemm_fwd_ms": t_gemm16, "agg_fwd_ms": t_agg16,
+                     "agg_bwd_ms": t_agg_b16, "gemm_bwd_ms": t_gemm_b16,
+                     "layer_fwd_bwd_ms": t_gemm16 + t_agg16 + t_agg_b16 + t_gemm_b16,
                      "torch_mm_fwd_ms": t_torch16,
                      "gemm_TFLOPs": flops_f / (t_gemm16 * 1e-3) / 1e12,
                      "gemm_GBps": bytes16 / (t_gemm16 * 1e-3) / 1e9,

@@ -395,6 +395,20 @@ int yitu_gemm_bf16(void *c_device, int c_is_bf16, const void *a_bf16_device,
                    int64_t lda, int64_t ldb, int64_t ldc, void *workspace_device,
                    size_t workspace_bytes, void *stream);
 
+/*
+ * C[ki, no] (+)= A^T . B with bf16 operands A [m, lda], B [m, ldb] (row-major,
+ * summed over their m rows) and fp32 accumulation on the matrix cores; C fp32
+ * [ki, ldc]. The weight gradient dW = X^T . dY of a bf16 layer (fc_cuda.cu:77-215,
+ * which the reference computes in fp32). ki, no and the leading dimensions must be
+ * multiples of 8. The rows are split over the chip and the partial products are
+ * added in a fixed order (bitwise reproducible); accumulate != 0 adds to C.
+ * Workspace: yitu_gemm_bf16_tn_workspace_bytes(m, ki, no).
+ */
+size_t yitu_gemm_bf16_tn_workspace_bytes(int64_t m, int64_t ki, int64_t no);
+int yitu_gemm_bf16_tn(float *c_device, const void *a_bf16_device, const void *b_bf16_device,
+                      int64_t m, int64_t ki, int64_t no, int64_t lda, int64_t ldb, int64_t ldc,
+                      int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Temporal most-recent-neighbour sampling on the device                       */
 /* ------------------------------------------------------------------------- */

@@ -158,6 +158,38 @@ def test_gemm_bf16_against_double(dev, tb, out_dtype, m, n, k):
                      atol=1e-4 * max(1.0, np.sqrt(k) / 4))
 
 
+@pytest.mark.parametrize("m,ki,no", [(1, 8, 8), (33, 8, 16), (100, 72, 40), (4096, 256, 256),
+                                     (5000, 128, 264), (70000, 256, 256), (0, 16, 8)])
+def test_gemm_bf16_tn_against_double(dev, m, ki, no):
+    """The weight gradient X^T . dY with bf16 operands: exact products, fp32 sums over
+    the m rows in a fixed order; the allowance follows sum |x| |g| (helpers.assert_close)."""
+    g = torch.Generator().manual_seed(m + 3 * ki + 5 * no)
+    a = torch.randn(m, ki, generator=g).to(torch.bfloat16)
+    b = torch.randn(m, no, generator=g).to(torch.bfloat16)
+    got = graph_ext.gemm_bf16_tn(a.to(dev), b.to(dev))
+    want = (a.double().t() @ b.double()).float()
+    abs_sum = (a.double().abs().t() @ b.double().abs()).float()
+    assert got.dtype == torch.float32 and got.shape == (ki, no)
+    assert_close(got, want, abs_sum=abs_sum, what="m=%d ki=%d no=%d" % (m, ki, no))
+    assert torch.equal(got, graph_ext.gemm_bf16_tn(a.to(dev), b.to(dev)))  # reproducible
+    # accumulate, and operands that are column slices of wider buffers
+    if m > 0 and ki >= 16:
+        wide_a = torch.randn(m, ki + 24, generator=g).to(torch.bfloat16).to(dev)
+        wide_b = torch.randn(m, no + 8, generator=g).to(torch.bfloat16).to(dev)
+        acc = torch.ones(ki, no, device=dev)
+        graph_ext.gemm_bf16_tn(wide_a[:, 8:8 + ki], wide_b[:, :no], out=acc, accumulate=True)
+        want2 = 1.0 + (wide_a[:, 8:8 + ki].double().t() @ wide_b[:, :no].double())
+        abs2 = 1.0 + (wide_a[:, 8:8 + ki].double().abs().t() @ wide_b[:, :no].double().abs())
+        assert_close(acc, want2.float(), abs_sum=abs2.float())
+
+
+def test_gemm_bf16_tn_rejects_unaligned_width(dev):
+    a = torch.zeros(16, 12, dtype=torch.bfloat16, device=dev)
+    b = torch.zeros(16, 8, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        graph_ext.gemm_bf16_tn(a, b)
+
+
 def test_gemm_bf16_rejects_unaligned_k(dev):
     a = torch.zeros(4, 12, dtype=torch.bfloat16, device=dev)
     b = torch.zeros(12, 4, dtype=torch.bfloat16, device=dev)

@@ -61,3 +61,47 @@ def test_common_dataset_builds_its_csr_on_the_device(dev):
     assert np.array_equal(ds.column_index.numpy(), want_idx)
     assert torch.allclose(ds.degrees.cpu(), torch.sqrt(torch.clamp(
         torch.from_numpy(np.diff(want_ptr)).float(), min=1.0)))
+
+
+def test_forget_after_a_raw_pointer_refill(dev):
+    """The plan / by-source caches key on torch's version counter, which a kernel that
+    writes through the raw pointer does not move: after such a refill ``forget`` must be
+    called, and then the next op sees the new graph. A second stream that uses a plan built
+    on another stream waits for the build."""
+    import oracle
+    from helpers import assert_close, powerlaw_graph
+    from yitu_amd import _lib, graph_ext
+    n = 1 << 12
+    ip_a, ix_a = powerlaw_graph(12, 60000, 1)
+    ip_b, ix_b = powerlaw_graph(12, 60000, 2)
+    m = min(ix_a.numel(), ix_b.numel())
+    # same-sized buffers: truncate both graphs to m edges
+    def clip(ip, ix):
+        ip = torch.clamp(ip, max=m)
+        return ip.contiguous(), ix[:m].contiguous()
+    ip_a, ix_a = clip(ip_a, ix_a)
+    ip_b, ix_b = clip(ip_b, ix_b)
+    indptr, indices = ip_a.to(dev), ix_a.to(dev)
+    g = torch.Generator().manual_seed(0)
+    values = torch.rand(m, 2, generator=g)
+    x = torch.randn(n, 2, 16, generator=g)
+    got_a = graph_ext.spmm_forward(values.to(dev), indptr, indices, x.to(dev))
+    assert_close(got_a, oracle.mh_spmm_forward(values, ip_a, ix_a, x))
+    # refill in place through raw pointers (what a device-side CSR builder does)
+    version = indices._version
+    torch.cuda.synchronize()
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    for dst, src in ((indptr, ip_b), (indices, ix_b)):
+        assert hip.hipMemcpy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()),
+                             ctypes.c_size_t(src.numel() * 4), 1) == 0
+    assert indices._version == version  # torch did not notice
+    graph_ext.forget(indptr, indices)
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        got_b = graph_ext.spmm_forward(values.to(dev), indptr, indices, x.to(dev))
+    side.synchronize()
+    assert_close(got_b, oracle.mh_spmm_forward(values, ip_b, ix_b, x))
+    # the plan built on the side stream, used from the default stream
+    got_b2 = graph_ext.spmm_forward(values.to(dev), indptr, indices, x.to(dev))
+    assert torch.equal(got_b2, got_b)

@@ -102,6 +102,29 @@ def test_spmm_bf16_features(dev, h, f):
     assert_close(got, same, rtol=1e-5, atol=1e-4)
 
 
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24)])
+def test_spmm_backward_bf16_rows(dev, h, f):
+    """grad_x of the product from bf16 gradient rows (fp32 weights, fp32 sums, fp32 out):
+    equal to the fp32 op on the same (exactly representable) rows, hence to the oracle,
+    on a power-law graph so that the by-source structure has planned rows."""
+    indptr, indices = powerlaw_graph(12, 50000, 7 * h + f)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(h * f)
+    values = torch.rand(indices.numel(), h, generator=g)
+    x = torch.randn(n, h, f, generator=g)
+    gy16 = torch.randn(n, h, f, generator=g).to(torch.bfloat16)
+    args = (values.to(dev), indptr.to(dev), indices.to(dev))
+    ga, gx = graph_ext.spmm_backward(*args, x.to(dev).to(torch.bfloat16), gy16.to(dev),
+                                     need_grad_a=False)
+    assert ga is None and gx.dtype == torch.float32
+    want = oracle.mh_spmm_backward(values, indptr, indices, x, gy16.float())[1]
+    abs_sum = oracle.mh_spmm_backward(values.abs(), indptr, indices, x.abs(), gy16.float().abs())[1]
+    assert_close(gx, want, rtol=1e-2, atol=1e-4, what="bf16 bar")
+    assert_close(gx, want, abs_sum=abs_sum, what="fp32 bar")
+    with pytest.raises(RuntimeError, match="grad_x only"):
+        graph_ext.spmm_backward(*args, x.to(dev), gy16.to(dev))
+
+
 def test_spmm_more_than_65535_rows(dev):
     """The reference's dim3(n_heads, n_nodes) launch is invalid above 65,535 rows."""
     n_dst, n_src, h, f = 70000, 1000, 2, 8

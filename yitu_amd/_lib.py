@@ -96,6 +96,45 @@ def workspace(n_bytes, device):
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
+# ---- state derived from a graph ----------------------------------------------------
+# The widest row, the row plan, the by-source view and by-source weight copies are
+# functions of the index tensors and are kept per tensor OBJECT (id, address, version
+# counter) for as long as the tensor lives. The version counter moves when torch writes
+# the tensor; it does NOT move when a buffer is refilled through its raw pointer, which is
+# how every kernel of this library (yitu_coo_to_csr, the device sampler, ...), DLPack
+# consumers and foreign extensions write. Whoever refills an index or weight tensor in
+# place must call ``forget`` on it (graph_ext.forget also drops the by-source state);
+# the builders in data/csr.py and the samplers return fresh tensors and need not.
+#
+# Derived buffers are built on the stream that was current at the time; a later use on
+# another stream waits for the build through an event recorded right behind it.
+
+
+class _Built:
+    __slots__ = ("value", "event", "raw_stream")
+
+    def __init__(self, value, device):
+        self.value = value
+        self.raw_stream = stream_ptr(device).value
+        self.event = torch.cuda.Event()
+        self.event.record(torch.cuda.current_stream(device))
+
+    def get(self, device):
+        if stream_ptr(device).value != self.raw_stream:  # two integers in the common case
+            torch.cuda.current_stream(device).wait_event(self.event)
+        return self.value
+
+
+def forget(*tensors):
+    """Drops every cached widest row and row plan derived from the given index tensors
+    (call after refilling one of them in place through a raw pointer)."""
+    idents = {id(t) for t in tensors if t is not None}
+    for key in [k for k in _max_degree if k[0] in idents]:
+        _max_degree.pop(key, None)
+    for key in [k for k in _plans if k[0] in idents or k[3] in idents]:
+        _plans.pop(key, None)
+
+
 # Widest-row cache: the kernels skip their hub-row machinery when they are told
 # that no row reaches the hub threshold. Computed once per indptr tensor.
 _max_degree = {}
@@ -131,7 +170,7 @@ def row_plan(indptr, indices, n_src, col_mask):
            indptr._version, int(n_src), int(col_mask))
     hit = _plans.get(key)
     if hit is not None:
-        return hit
+        return hit.get(indices.device)
     L = lib()
     L.yitu_plan_bytes.restype = c_size
     L.yitu_plan_workspace_bytes.restype = c_size
@@ -144,7 +183,7 @@ def row_plan(indptr, indices, n_src, col_mask):
                                c_i64(indptr.numel() - 1), c_i64(n_src), c_i64(nnz), c_int(col_mask),
                                ptr(ws), c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_plan_build")
-    _plans[key] = plan
+    _plans[key] = _Built(plan, dev)
     weakref.finalize(indices, _plans.pop, key, None)
     return plan
 

@@ -20,6 +20,8 @@
 #include "../../include/yitu_hip.h"
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace yitu {
 
 namespace {
@@ -172,6 +174,156 @@ __global__ __launch_bounds__(256) void transpose16_kernel(uint16_t *__restrict__
         if (n0 + r < N && k0 + tx < K) dst[(int64_t)(n0 + r) * ld_dst + k0 + tx] = tile[tx][r];
 }
 
+
+// ---- C[Ki, No] = A^T . B : the weight gradient dW = X^T . dY ------------------------
+// A [M, lda] and B [M, ldb] are row-major bf16, the sum runs over their (many) rows,
+// the output is small. The matrix instruction wants each lane to hold 8 consecutive
+// elements ALONG the summed index, which in memory are a row stride apart. A
+// workgroup therefore stages 32 rows x 128 columns of both operands in LDS as they
+// lie in memory (16-byte global loads, one stage ahead in registers); a lane then
+// reads one dword = two neighbouring columns from each of its 8 rows and splits them
+// with byte permutes into the operand of the even column and the operand of the odd
+// column. Output tile rows are thereby interleaved (even columns, then odd ones),
+// which only matters when the tile is written. Each wave owns 64 x 64 of the
+// workgroup's 128 x 128 tile. The rows are split over the grid; every workgroup
+// writes its partial tile and a second kernel adds the partials in chunk order
+// (bitwise reproducible).
+constexpr int TN_TILE = 128, TN_ROWS = 32, TN_LD = TN_TILE + 4;  // padded LDS row (bf16)
+
+struct TnParams {
+    const uint16_t *A, *B;
+    float *partial;  // [n_chunks, Ki, No]
+    int M, Ki, No;
+    int64_t lda, ldb;
+    int rows_per_chunk;  // multiple of TN_ROWS
+};
+
+__global__ __launch_bounds__(256) void hgemm_tn_kernel(TnParams p) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][TN_ROWS][TN_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][TN_ROWS][TN_LD];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int tiles_j = (p.No + TN_TILE - 1) / TN_TILE;
+    const int i0 = (blockIdx.y / tiles_j) * TN_TILE, j0 = (blockIdx.y % tiles_j) * TN_TILE;
+    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+    const int m_beg = blockIdx.x * p.rows_per_chunk;
+    const int m_end = min(p.M, m_beg + p.rows_per_chunk);
+    // loader: thread -> (row, 8 columns); 16 threads cover the 128 columns of a row
+    const int lrow = t >> 4, lcol = (t & 15) * 8;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[a][b][e] = 0.0f;
+
+    uint4 ra[2], rb[2];
+    auto gload = [&](int m0) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int row = m0 + lrow + 16 * h;
+            const bool in = row < m_end;
+            // Ki, No are multiples of 8: a column below the bound has its 8 elements
+            ra[h] = (in && i0 + lcol < p.Ki)
+                        ? *reinterpret_cast<const uint4 *>(p.A + (int64_t)row * p.lda + i0 + lcol)
+                        : make_uint4(0, 0, 0, 0);
+            rb[h] = (in && j0 + lcol < p.No)
+                        ? *reinterpret_cast<const uint4 *>(p.B + (int64_t)row * p.ldb + j0 + lcol)
+                        : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol]) = make_uint2(ra[h].x, ra[h].y);
+            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol + 4]) = make_uint2(ra[h].z, ra[h].w);
+            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol]) = make_uint2(rb[h].x, rb[h].y);
+            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol + 4]) = make_uint2(rb[h].z, rb[h].w);
+        }
+    };
+    // operand pair (even column, odd column) of the 8 rows kk + 8 * lk .. + 7
+    auto fragments = [&](const uint16_t (*tile)[TN_LD], int col0, int kk, bf16x8 &even, bf16x8 &odd) {
+        uint32_t raw[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            raw[k] = *reinterpret_cast<const uint32_t *>(&tile[kk + 8 * lk + k][col0 + 2 * l32]);
+        uint32_t e[4], o[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            e[q] = __builtin_amdgcn_perm(raw[2 * q + 1], raw[2 * q], 0x05040100u);
+            o[q] = __builtin_amdgcn_perm(raw[2 * q + 1], raw[2 * q], 0x07060302u);
+        }
+        even = __builtin_bit_cast(bf16x8, make_uint4(e[0], e[1], e[2], e[3]));
+        odd = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
+    };
+
+    if (m_beg < m_end) {
+        gload(m_beg);
+        lstore(0);
+        __syncthreads();
+        int buf = 0;
+        for (int m0 = m_beg; m0 < m_end; m0 += TN_ROWS) {
+            const bool more = m0 + TN_ROWS < m_end;
+            if (more) gload(m0 + TN_ROWS);
+#pragma unroll
+            for (int kk = 0; kk < TN_ROWS; kk += 16) {
+                bf16x8 a[2], b[2];
+                fragments(As[buf], wi, kk, a[0], a[1]);
+                fragments(Bs[buf], wj, kk, b[0], b[1]);
+#pragma unroll
+                for (int x = 0; x < 2; x++)
+#pragma unroll
+                    for (int y = 0; y < 2; y++)
+                        acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
+            }
+            if (more) lstore(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+    // accumulator element 4*jj + ii of tile (x, y) is row 8jj + 4lk + ii, column l32 of the
+    // MFMA tile; MFMA row r of parity x is output row wi + 2r + x, column c of parity y is
+    // output column wj + 2c + y
+    float *dst = p.partial + (int64_t)blockIdx.x * p.Ki * p.No;
+#pragma unroll
+    for (int x = 0; x < 2; x++)
+#pragma unroll
+        for (int y = 0; y < 2; y++) {
+            const int col = j0 + wj + 2 * l32 + y;
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+                for (int ii = 0; ii < 4; ii++) {
+                    const int row = i0 + wi + 2 * (8 * jj + 4 * lk + ii) + x;
+                    if (row < p.Ki && col < p.No) dst[(int64_t)row * p.No + col] = acc[x][y][4 * jj + ii];
+                }
+        }
+}
+
+// C[i] (+)= sum over chunks of partial[c][i], in chunk order
+__global__ __launch_bounds__(256) void hgemm_tn_reduce_kernel(float *__restrict__ c, int64_t ldc,
+                                                              const float *__restrict__ partial,
+                                                              int n_chunks, int Ki, int No,
+                                                              int accumulate) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)Ki * No) return;
+    float s = 0.0f;
+    for (int k = 0; k < n_chunks; k++) s += partial[(int64_t)k * Ki * No + idx];
+    float *out = c + (idx / No) * ldc + idx % No;
+    *out = accumulate ? *out + s : s;
+}
+
+// Row chunks of the A^T.B product: enough workgroups for about three per CU, chunks a
+// multiple of the stage height.
+inline int tn_chunk_rows(int64_t m, int64_t ki, int64_t no) {
+    const int64_t tiles = ceil_div(ki, TN_TILE) * ceil_div(no, TN_TILE);
+    const int64_t want_chunks = std::max<int64_t>(1, 768 / tiles);
+    int64_t rows = ceil_div(ceil_div(m, want_chunks), TN_ROWS) * TN_ROWS;
+    return (int)std::max<int64_t>(rows, 4 * TN_ROWS);
+}
+
 }  // namespace
 
 }  // namespace yitu
@@ -224,6 +376,48 @@ YITU_API int yitu_gemm_bf16(void *c, int c_is_bf16, const void *a, const void *b
         hgemm_mfma_kernel<true><<<grid, 256, 0, stream>>>(p);
     else
         hgemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+
+YITU_API size_t yitu_gemm_bf16_tn_workspace_bytes(int64_t m, int64_t ki, int64_t no) {
+    const int64_t chunks = ceil_div(std::max<int64_t>(m, 1), tn_chunk_rows(m, ki, no));
+    return align_up((size_t)(chunks * ki * no) * sizeof(float), 256) + 256;
+}
+
+YITU_API int yitu_gemm_bf16_tn(float *c, const void *a, const void *b, int64_t m, int64_t ki,
+                               int64_t no, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
+                               void *workspace, size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(m >= 0 && ki >= 0 && no >= 0, "negative size");
+    if (ki == 0 || no == 0) return 0;
+    YITU_REQUIRE(c && (m == 0 || (a && b)), "null operand");
+    YITU_REQUIRE(m < INT32_MAX && ki < (1 << 20) && no < (1 << 20) && ldc >= no, "size out of range");
+    YITU_REQUIRE(ki % 8 == 0 && no % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && lda >= ki &&
+                     ldb >= no && aligned16(a) && aligned16(b),
+                 "bf16 A^T.B needs both widths and leading dimensions to be multiples of 8 and "
+                 "16-byte aligned operands");
+    const int rows = tn_chunk_rows(m, ki, no);
+    const int64_t chunks = ceil_div(std::max<int64_t>(m, 1), rows);
+    const size_t need = (size_t)(chunks * ki * no) * sizeof(float);
+    YITU_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
+                 "workspace too small for the partial products: need %zu bytes", need);
+    TnParams p{};
+    p.A = static_cast<const uint16_t *>(a);
+    p.B = static_cast<const uint16_t *>(b);
+    p.partial = static_cast<float *>(workspace);
+    p.M = (int)m;
+    p.Ki = (int)ki;
+    p.No = (int)no;
+    p.lda = lda;
+    p.ldb = ldb;
+    p.rows_per_chunk = rows;
+    dim3 grid((unsigned)chunks, (unsigned)(ceil_div(ki, TN_TILE) * ceil_div(no, TN_TILE)));
+    hgemm_tn_kernel<<<grid, 256, 0, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    hgemm_tn_reduce_kernel<<<(unsigned)ceil_div(ki * no, 256), 256, 0, stream>>>(
+        c, ldc, p.partial, (int)chunks, (int)ki, (int)no, accumulate);
     YITU_LAUNCH_CHECK();
     return 0;
 }

@@ -60,7 +60,7 @@ def transposed(indptr, indices, n_src):
            indptr._version, int(n_src))
     hit = _transposed.get(key)
     if hit is not None:
-        return hit
+        return hit.get(indices.device)
     dev = indices.device
     n_rows = indptr.numel() - 1
     nnz = indices.numel()
@@ -78,9 +78,26 @@ def transposed(indptr, indices, n_src):
     check(rc, "yitu_csr_transpose")
     t.max_degree_t = _lib.max_degree(t.t_indptr)
     t.plan_t = _lib.row_plan(t.t_indptr, t.t_rows, n_rows, 0x7FFFFFFF)
-    _transposed[key] = t
+    _transposed[key] = _lib._Built(t, dev)
     weakref.finalize(indices, _transposed.pop, key, None)
     return t
+
+
+def forget(*tensors):
+    """Drops everything derived from the given index / weight tensors: widest row, row
+    plan, by-source view, by-source weight copies. Needed after a tensor was refilled in
+    place through its raw pointer (kernels of this library, DLPack consumers): torch's
+    version counter, which the caches key on, does not see such writes."""
+    idents = {id(t) for t in tensors if t is not None}
+    derived = []
+    for key in [k for k in _transposed if k[0] in idents or k[3] in idents]:
+        t = _transposed.pop(key).value
+        derived += [t.t_indptr, t.t_rows]
+    _lib.forget(*tensors, *derived)
+    for ident in list(_values_seen):
+        state = _values_seen[ident]
+        if ident in idents or state[2] in idents or state[4] in idents:
+            _forget_values(ident)
 
 
 # --------------------------------------------------------------------------- #
@@ -123,9 +140,12 @@ _values_seen = {}       # id(values) -> state of the tensor when it last came by
 _values_by_source = {}  # id(values) -> (that state, the copy in by-source order)
 
 
-def _by_source_values(values, indptr, indices, n_src):
+def _by_source_values(values, indptr, indices, n_src, force=False):
+    """The copy of ``values`` in by-source order once the same tensor has come by twice
+    (``force``: at once), else None."""
     ident = id(values)
-    state = (values.data_ptr(), values._version, id(indices), indices._version, int(n_src))
+    state = (values.data_ptr(), values._version, id(indices), indices._version, id(indptr),
+             indptr._version, int(n_src))
     hit = _values_by_source.get(ident)
     if hit is not None and hit[0] == state:
         return hit[1]
@@ -134,7 +154,8 @@ def _by_source_values(values, indptr, indices, n_src):
             weakref.finalize(values, _forget_values, ident)
         _values_seen[ident] = state
         _values_by_source.pop(ident, None)
-        return None
+        if not force:
+            return None
     tr = transposed(indptr, indices, n_src)
     copy = values.index_select(0, tr.t_perm)
     _values_by_source[ident] = (state, copy)
@@ -153,8 +174,20 @@ def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
     _check(values, torch.float32, "values", 2)
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
-    _check(features, torch.float32, "features", 3)
-    _check(grad_out, torch.float32, "grad_out", 3)
+    bf16 = grad_out.dtype == torch.bfloat16
+    if bf16:
+        # bf16 pipeline: gradient rows in bf16, fp32 sums and fp32 grad_x out. The edge
+        # weights of such a pipeline are constants of the graph (norms): grad_a is not
+        # offered, and the forward's features are not read at all.
+        if need_grad_a:
+            raise RuntimeError("spmm_backward with bf16 rows computes grad_x only "
+                               "(need_grad_a=False): the reference's op is fp32")
+        if features.dtype not in (torch.float32, torch.bfloat16) or features.dim() != 3:
+            raise RuntimeError("features must be a [n_src, H, F] tensor")
+        _check(grad_out, torch.bfloat16, "grad_out", 3)
+    else:
+        _check(features, torch.float32, "features", 3)
+        _check(grad_out, torch.float32, "grad_out", 3)
     dev = _lib.require_device(values, indptr, indices, features, grad_out)
     n_dst = indptr.numel() - 1
     n_src, h, f = features.shape
@@ -163,6 +196,14 @@ def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
         raise RuntimeError("grad_out must be [n_dst, n_heads, n_features]")
     if not (need_grad_a or need_grad_x):
         return [None, None]
+    if bf16:
+        if n_dst > COL_MASK:
+            raise RuntimeError("bf16 spmm_backward needs at most 2**24 destination rows")
+        # grad_x[c] = sum over the edges of source c of values[e] * grad_out[row_e]: the
+        # forward product over the by-source structure, weights copied into that order
+        tr = transposed(indptr, indices, n_src)
+        values_t = _by_source_values(values, indptr, indices, n_src, force=True)
+        return [None, spmm_forward(values_t, tr.t_indptr, tr.t_rows, grad_out)]
     if not need_grad_a and nnz > 0 and n_dst <= COL_MASK:
         values_t = _by_source_values(values, indptr, indices, n_src)
         if values_t is not None:
@@ -463,6 +504,36 @@ def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32, out=None):
                                        c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_gemm_bf16")
     return c
+
+
+def gemm_bf16_tn(a, b, out=None, accumulate=False):
+    """a^T . b for bf16 ``a`` [m, ki] and ``b`` [m, no] (rows may be strided slices of a
+    wider buffer), fp32 accumulation on the matrix cores, fp32 [ki, no] out: the weight
+    gradient X^T . dY of a bf16 layer. ``accumulate`` adds to ``out``."""
+    for t, name in ((a, "a"), (b, "b")):
+        if t.dtype != torch.bfloat16 or t.dim() != 2 or t.stride(1) != 1 or not t.is_cuda:
+            raise RuntimeError("%s must be a 2-D bf16 GPU tensor with contiguous rows" % name)
+    if a.device != b.device or a.size(0) != b.size(0):
+        raise RuntimeError("a and b must have the same number of rows on one device")
+    dev = a.device
+    m, ki = a.shape
+    no = b.size(1)
+    if out is None:
+        if accumulate:
+            raise RuntimeError("accumulate needs an output to add to")
+        out = torch.empty((ki, no), dtype=torch.float32, device=dev)
+    elif out.dtype != torch.float32 or tuple(out.shape) != (ki, no) or not out.is_contiguous() \
+            or out.device != dev:
+        raise RuntimeError("out must be a contiguous fp32 [%d, %d] tensor" % (ki, no))
+    ws = _lib.workspace(_size_fn("yitu_gemm_bf16_tn_workspace_bytes")(c_i64(m), c_i64(ki), c_i64(no)),
+                        dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gemm_bf16_tn(ptr(out), ptr(a), ptr(b), c_i64(m), c_i64(ki), c_i64(no),
+                                          c_i64(a.stride(0)), c_i64(b.stride(0)), c_i64(no),
+                                          c_int(int(accumulate)), ptr(ws), c_size(ws.numel()),
+                                          stream_ptr(dev))
+    check(rc, "yitu_gemm_bf16_tn")
+    return out
 
 
 # --------------------------------------------------------------------------- #
