@@ -361,6 +361,29 @@ int yitu_sgemm_typed(float *const *c_device_ptrs, const float *const *a_device_p
                      size_t workspace_bytes, void *stream);
 
 /*
+ * hfused_forward (entry.cpp:136-155; hfused_cuda.cu:5-45,96-137): the SpMM of
+ * graph A and the SDDMM + LeakyReLU + edge softmax of graph B (same number of
+ * rows, same head count) in ONE launch: the first workgroups of the grid run the
+ * SpMM row kernel on A, the others the SDDMM row kernel on B. That holds when
+ * both longest rows are known (max_degree_* >= 0) and below the long-row
+ * thresholds (A: 64 edges, B: 512), n_heads <= 16, n_features a multiple of 4
+ * and n_heads * n_features <= 1024; any other case runs yitu_spmm_forward and
+ * then yitu_sddmm_forward. spmm_out [n_rows,H,F], attn [nnz_b,H]; query
+ * [n_bid,n_rows,H], key [n_src_b,H]. Workspace (used by the two-op case only):
+ * yitu_hfused_forward_workspace_bytes.
+ */
+size_t yitu_hfused_forward_workspace_bytes(int64_t n_rows, int64_t nnz_a, int64_t row_len,
+                                           int64_t nnz_b, int64_t n_heads, int64_t n_bid);
+int yitu_hfused_forward(float *spmm_out_device, float *attn_device, const float *spmm_values_device,
+                        const int32_t *spmm_indptr_device, const int32_t *spmm_indices_device,
+                        const float *spmm_features_device, const int32_t *sddmm_indptr_device,
+                        const int32_t *sddmm_indices_device, const float *sddmm_query_device,
+                        const float *sddmm_key_device, int64_t n_rows, int64_t n_src_a,
+                        int64_t nnz_a, int64_t n_heads, int64_t n_features, int64_t n_src_b,
+                        int64_t nnz_b, int64_t n_bid, int64_t max_degree_a, int64_t max_degree_b,
+                        void *workspace_device, size_t workspace_bytes, void *stream);
+
+/*
  * b2gemm (entry.cpp:56-64; fc_cuda.cu:4-75): y_a = x . w_a^T, y_b = x . w_b^T
  * as one grouped launch. x [n,k], w_* [m,k], y_* [n,m], contiguous.
  */

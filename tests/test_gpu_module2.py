@@ -287,6 +287,36 @@ def test_check_hfuse(dev):
         assert torch.allclose(a, b.grad, atol=1e-3)
 
 
+@pytest.mark.parametrize("n_dst,n_src,h,f,n_bid,long_rows", [
+    (4096, 2048, 8, 4, 1, False), (300, 500, 1, 4, 1, False), (1000, 700, 3, 16, 2, False),
+    (513, 129, 16, 64, 5, False), (64, 64, 4, 256, 1, False), (2000, 900, 4, 8, 1, True),
+    (400, 300, 2, 6, 1, False), (400, 300, 20, 4, 1, False)])
+def test_hfused_forward_against_the_oracle_ops(dev, n_dst, n_src, h, f, n_bid, long_rows):
+    """The one-launch form (and its two-op fallback for long rows, unvectorised widths or
+    more than 16 heads) against the oracle's two functions, not against the ops it is
+    built from (hfused_cuda.cu:5-45)."""
+    hubs = dict(hub_rows=(3,), hub_degree=600) if long_rows else {}
+    a_ptr, a_idx = random_csr(n_dst, n_src, 0.02, n_dst + 1, **hubs)
+    blocks = [random_csr(n_dst, n_src, 0.03, 10 * n_dst + b, empty_rows=(b,), **hubs)
+              for b in range(n_bid)]
+    if n_bid == 1:
+        b_ptr, b_idx, n_cols = blocks[0][0].numpy(), blocks[0][1].numpy(), n_src
+    else:
+        b_ptr, b_idx, n_cols = oracle.stitch_csr([(p_, i_, n_src) for p_, i_ in blocks])
+    g = torch.Generator().manual_seed(h + f)
+    vals = torch.randn(a_idx.numel(), h, generator=g)
+    x = torch.randn(n_src, h, f, generator=g)
+    q = torch.randn(n_bid, n_dst, h, generator=g)
+    k = torch.randn(n_cols, h, generator=g)
+    b_ptr_t, b_idx_t = torch.as_tensor(b_ptr), torch.as_tensor(b_idx)
+    out, attn = graph_ext.hfused_forward(vals.to(dev), a_ptr.to(dev), a_idx.to(dev), x.to(dev),
+                                         b_ptr_t.to(dev), b_idx_t.to(dev), q.to(dev), k.to(dev))
+    want_out, want_attn = oracle.hfused_forward(vals, a_ptr, a_idx, x, b_ptr, b_idx, q.numpy(), k)
+    abs_out = oracle.mh_spmm_forward(vals.abs(), a_ptr, a_idx, x.abs())
+    assert_close(out, want_out, abs_sum=abs_out, what="spmm part")
+    assert_close(attn, want_attn, what="sddmm part")
+
+
 def test_dtype_and_device_checks(dev):
     indptr, indices = random_csr(10, 10, 0.3, 0)
     v = torch.randn(indices.numel(), 2)

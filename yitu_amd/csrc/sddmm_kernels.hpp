@@ -159,8 +159,8 @@ __device__ __forceinline__ void fwd_write(const SddmmParams &p, int e_beg, int e
 }
 
 template <int HP>
-__global__ __launch_bounds__(kBlock) void sddmm_fwd_rows_kernel(SddmmParams p) {
-    const int row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+__device__ __forceinline__ void sddmm_fwd_rows_body(const SddmmParams &p, int block) {
+    const int row = block * kWavesPerBlock + threadIdx.x / kWave;
     if (row >= p.n_dst) return;
     const int beg = p.indptr[row], end = p.indptr[row + 1];
     if (end == beg) return;
@@ -178,6 +178,11 @@ __global__ __launch_bounds__(kBlock) void sddmm_fwd_rows_kernel(SddmmParams p) {
             fwd_write<HP>(p, beg, end, b, h, act_h, qv, a.m, 1.0f / a.s);
         }
     }
+}
+
+template <int HP>
+__global__ __launch_bounds__(kBlock) void sddmm_fwd_rows_kernel(SddmmParams p) {
+    sddmm_fwd_rows_body<HP>(p, blockIdx.x);
 }
 
 // stats layout: [(item or hub row) * n_bid + b] * H + h, three floats each

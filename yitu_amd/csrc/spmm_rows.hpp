@@ -206,11 +206,11 @@ __host__ __device__ inline int rows_per_wave(int n_rows) {
 // short row costs one round of feature gathers and nothing else that waits on
 // memory. Rows that the plan covers are skipped.
 template <int VEC, int G, int KT, int WMODE, typename TIN>
-__global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
+__device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block) {
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
     const int rpw = rows_per_wave(p.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + wave) * rpw;
+    const int r0 = (block * kWavesPerBlock + wave) * rpw;
     if (r0 >= p.n_rows) return;
     const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
@@ -259,6 +259,11 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
             }
         }
     }
+}
+
+template <int VEC, int G, int KT, int WMODE, typename TIN>
+__global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
+    spmm_rows_body<VEC, G, KT, WMODE, TIN>(p, blockIdx.x);
 }
 
 constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave

@@ -334,18 +334,56 @@ def sddmm_backward(indptr, indices, query, key, attn_values, grad_out, determini
 def hfused_forward(spmm_values, spmm_indptr, spmm_indices, spmm_features, sddmm_indptr,
                    sddmm_indices, sddmm_query, sddmm_key):
     """An SpMM on graph A and an SDDMM+softmax on graph B with equal row counts
-    (entry.cpp:136-155; hfused_cuda.cu:96-137). Returns [spmm_out, attn]."""
+    (entry.cpp:136-155; hfused_cuda.cu:96-137) as one launch whose workgroups are split
+    between the two ops (when neither graph has long rows; otherwise the two ops one
+    after the other). Returns [spmm_out, attn]."""
     if spmm_indptr.numel() != sddmm_indptr.numel():
         raise RuntimeError("the two graphs must have the same number of rows")
-    out = spmm_forward(spmm_values, spmm_indptr, spmm_indices, spmm_features)
-    attn = sddmm_forward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key)
+    _check(spmm_values, torch.float32, "spmm_values", 2)
+    _check(spmm_features, torch.float32, "spmm_features", 3)
+    _check(sddmm_key, torch.float32, "sddmm_key", 2)
+    if sddmm_query.dtype != torch.float32 or sddmm_query.dim() not in (2, 3):
+        raise RuntimeError("sddmm_query must be float32 [n_dst, H] or [n_bid, n_dst, H]")
+    for t, name in ((spmm_indptr, "spmm_indptr"), (spmm_indices, "spmm_indices"),
+                    (sddmm_indptr, "sddmm_indptr"), (sddmm_indices, "sddmm_indices")):
+        _check(t, torch.int32, name, 1)
+    dev = _lib.require_device(spmm_values, spmm_indptr, spmm_indices, spmm_features, sddmm_indptr,
+                              sddmm_indices, sddmm_query, sddmm_key)
+    query = sddmm_query if sddmm_query.dim() == 3 else sddmm_query.unsqueeze(0)
+    n_rows = spmm_indptr.numel() - 1
+    n_src_a, h, f = spmm_features.shape
+    n_bid = query.size(0)
+    n_src_b = sddmm_key.size(0)
+    nnz_a, nnz_b = spmm_indices.numel(), sddmm_indices.numel()
+    if spmm_values.shape != (nnz_a, h):
+        raise RuntimeError("spmm_values must be [n_edges, n_heads]")
+    if query.size(1) != n_rows or query.size(2) != h or sddmm_key.size(1) != h:
+        raise RuntimeError("query must be [n_bid, n_dst, H] and key [n_src, H] with the SpMM's H")
+    if not 1 <= n_bid <= 16:
+        raise RuntimeError("at most 16 query blocks (4-bit block tag)")
+    out = torch.empty((n_rows, h, f), dtype=torch.float32, device=dev)
+    attn = torch.zeros((nnz_b, h), dtype=torch.float32, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_hfused_forward_workspace_bytes")(
+        c_i64(n_rows), c_i64(nnz_a), c_i64(h * f), c_i64(nnz_b), c_i64(h), c_i64(n_bid)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_hfused_forward(
+            ptr(out), ptr(attn), ptr(spmm_values), ptr(spmm_indptr), ptr(spmm_indices),
+            ptr(spmm_features), ptr(sddmm_indptr), ptr(sddmm_indices), ptr(query), ptr(sddmm_key),
+            c_i64(n_rows), c_i64(n_src_a), c_i64(nnz_a), c_i64(h), c_i64(f), c_i64(n_src_b),
+            c_i64(nnz_b), c_i64(n_bid), c_i64(_lib.max_degree(spmm_indptr)),
+            c_i64(_lib.max_degree(sddmm_indptr)), ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_hfused_forward")
     return [out, attn]
 
 
 def hfused_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad, sddmm_indptr,
                     sddmm_indices, sddmm_query, sddmm_key, sddmm_attn, sddmm_grad):
-    """Union of the two backward ops (entry.cpp:157-182) with the correct
-    arithmetic: returns [grad_a, grad_x, grad_query, grad_key]."""
+    """Union of the two backward ops (entry.cpp:157-182) with the correct arithmetic:
+    returns [grad_a, grad_x, grad_query, grad_key]. Not one launch: both gradients
+    with respect to per-source tensors are gathers over a by-source structure of
+    their own graph (no atomics), which follow the per-row passes. The reference's
+    fused backward kernel is unreachable (sparse.py:109-110) and indexes heads by
+    threadIdx.x although they lie on threadIdx.y (hfused_cuda.cu:59,186)."""
     grad_a, grad_x = spmm_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad)
     grad_q, grad_k = sddmm_backward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key, sddmm_attn,
                                     sddmm_grad)
