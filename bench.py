@@ -206,6 +206,8 @@ def run_spmm(args, dev, bf16):
                    "63M draws dedup + self loops, vertex ids renamed by the Rabbit-Order "
                    "reorder, CSR by destination", "reorder_host_s": info["reorder_s"], "n_nodes": n,
                    "n_edges": nnz, "max_in_degree": maxdeg, "feature_dim": dim,
+                   "short_row_edges_sampled_and_local": plan[264:272].view(torch.int32).tolist()[::-1]
+                   if plan is not None else None,
                    "step": "aggregate(X) + aggregate(dY), same CSR, W = I"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
@@ -792,6 +794,62 @@ def run_c3_orders(args, dev):
     res["random_then_rabbit_ids_ms"] = _event_ms(lambda: K._aggregate(x, rp_r, ci_r, deg_r, 1.0), args.steps,
                                      args.warmup)
     res["n_edges"] = int(ci.numel())
+    res["planted_partition"] = run_planted_orders(args, dev)
+    return res
+
+
+def planted_partition(n_comm, size, intra, inter, seed, dev):
+    """Planted-partition graph: n_comm communities of `size` vertices; every vertex draws
+    `intra` sources inside its community and `inter` anywhere. Ids as planted (a
+    community is a contiguous id block). Returns (src, dst) int64 on `dev`, self loops
+    included once per vertex."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    n = n_comm * size
+    dst = torch.arange(n, device=dev).repeat_interleave(intra)
+    base = dst // size * size
+    src = base + torch.randint(0, size, (n * intra,), generator=g, device=dev)
+    dst2 = torch.arange(n, device=dev).repeat_interleave(inter)
+    src2 = torch.randint(0, n, (n * inter,), generator=g, device=dev)
+    loop = torch.arange(n, device=dev)
+    return torch.cat([src, src2, loop]), torch.cat([dst, dst2, loop])
+
+
+def run_planted_orders(args, dev):
+    """The reorder on a graph it can help: a planted-partition graph of the third
+    configuration's size (2^21 vertices, about 30 sources per vertex, 28 of them inside
+    the vertex's community of 512) with shuffled vertex ids, the same passed through the
+    Rabbit-Order reorder (single-thread and all-thread aggregation), and the ids as
+    planted. fp32 aggregation with per-edge column scales, F = 128, one call each; the
+    L2-miss traffic of the three is in profiles/ (planted-partition summary)."""
+    from yitu_amd import YiTu_GNN_kernel as K, rabbit
+    from yitu_amd.data import graphgen
+    n_comm, size = 4096, 512
+    n = n_comm * size
+    src, dst = planted_partition(n_comm, size, 28, 2, 20244, dev)
+    g = torch.Generator(device=dev).manual_seed(20244)
+    x = torch.randn(n, 128, generator=g, device=dev)
+    res = {"n_nodes": n, "communities": n_comm, "community_size": size}
+
+    def measure(tag, s_ids, d_ids):
+        rp, ci = graphgen.csr_by_destination(s_ids, d_ids, n)
+        deg = graphgen.gcn_norm(rp)
+        es = K.edge_scale(ci, deg)
+        res[tag + "_ms"] = _event_ms(lambda: K._aggregate(x, rp, ci, deg, 1.0, es), args.steps,
+                                     args.warmup)
+        res.setdefault("n_edges", int(ci.numel()))
+
+    measure("planted_ids", src, dst)
+    perm = torch.randperm(n, generator=g, device=dev)
+    src_s, dst_s = perm[src], perm[dst]
+    del src, dst
+    measure("shuffled_ids", src_s, dst_s)
+    ei = torch.stack([src_s, dst_s]).to(torch.int32).cpu()
+    for tag, threads in (("rabbit_1_thread", 1), ("rabbit_all_threads", 0)):
+        t0 = time.perf_counter()
+        ei_r = rabbit.reorder(ei, threads=threads)
+        res[tag + "_host_s"] = time.perf_counter() - t0
+        ei_r = ei_r.to(dev)
+        measure(tag + "_ids", ei_r[0].long(), ei_r[1].long())
     return res
 
 
@@ -866,6 +924,8 @@ def main():
         res = run_c5(args, dev)
     elif args.workload == "c3_vertex_orders":
         res = run_c3_orders(args, dev)
+    elif args.workload == "planted_partition_orders":
+        res = run_planted_orders(args, dev)
     else:
         sys.exit("unknown workload %s" % args.workload)
     print(json.dumps(res))

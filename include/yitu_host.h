@@ -31,6 +31,17 @@ int yitu_rabbit_reorder(int32_t *out_edge_index, int32_t *perm_out, int64_t perm
                         int64_t *n_vertices, const int32_t *in_edge_index, int64_t n_edges);
 
 /*
+ * The same with the community aggregation on n_threads threads (<= 0: all the
+ * OpenMP runtime offers; 1: the reproducible order above), by the reference's
+ * protocol (rabbit_order.hpp:393-526, 554-621: lock by strength swap, merge by one
+ * compare-and-swap, per-thread retry list). Like the reference's, the result then
+ * depends on timing: a valid Rabbit-Order permutation, not the same one twice.
+ */
+int yitu_rabbit_reorder_threads(int32_t *out_edge_index, int32_t *perm_out,
+                                int64_t perm_capacity, int64_t *n_vertices,
+                                const int32_t *in_edge_index, int64_t n_edges, int n_threads);
+
+/*
  * Most-recent-neighbour temporal sampler: replaces sampler_core.ParallelSampler
  * (YiTu_GNN/YiTu_T/sampler_core.cpp:43-359, binding :374-402) in its
  * `recent = True`, `num_history = 1`, `window_duration = 0` mode.

@@ -292,3 +292,28 @@ def test_edge_scale_is_the_same_aggregation(dev):
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
     with pytest.raises(RuntimeError):
         K._aggregate(x, rp, ci, deg, 1.0, es[:-1].contiguous())
+
+
+@pytest.mark.parametrize("per_row,dim", [(20, 64), (50, 128)])
+def test_local_graph_rows_are_dealt_xcd_by_xcd(dev, per_row, dim):
+    """A graph whose row plan says "local" (sources near the row's own id) has its short
+    rows walked one eighth per XCD instead of round robin; the row count is no multiple of
+    the launch's rounding, so surplus workgroups must find nothing. Same results, bit for
+    bit on a second call, as for any graph; with 20 sources per row no row is long and the
+    plan exists for its header alone (2^20 edges or more)."""
+    from yitu_amd import _lib
+    n, size = 70001, 500
+    rng = np.random.default_rng(per_row)
+    dst = np.repeat(np.arange(n), per_row)
+    src = np.minimum(dst // size * size + rng.integers(0, size, dst.size), n - 1)
+    indptr, indices = graphgen.csr_from_edges(torch.from_numpy(dst), torch.from_numpy(src), n, n)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    plan = _lib.row_plan(rp, ci, n, 0x7FFFFFFF)
+    assert plan is not None
+    header = plan[:1024].cpu().numpy().view(np.int32)
+    assert 4 * int(header[66]) > 3 * int(header[67]) > 0
+    x = torch.randn(n, dim, generator=torch.Generator().manual_seed(2))
+    got = K._aggregate(x.to(dev), rp, ci, deg, 1.0)
+    want = oracle.row_agg(x.numpy(), indptr, indices, deg.cpu().numpy(), oracle.MODE_GCN)
+    assert_close(got, want)
+    assert torch.equal(got, K._aggregate(x.to(dev), rp, ci, deg, 1.0))

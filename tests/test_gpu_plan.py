@@ -28,12 +28,14 @@ def read_plan(plan, nnz):
     max_items = nnz // CHUNK + nnz // 16 + max_rows + 1
     n_items, n_rows, overflow = raw[0], raw[1], raw[2]
     band_shift, n_bands = int(raw[64]), int(raw[65])
+    local_rows, sampled_rows = int(raw[66]), int(raw[67])
     rows_off = 128
     rows = raw[rows_off:rows_off + 4 * max_rows].reshape(-1, 4)[:n_rows]
     rec_off = rows_off + ((16 * max_rows + 255) // 256 * 256) // 4
     records = raw[rec_off:rec_off + 4 * max_items].reshape(-1, 4)
     return dict(n_items=int(n_items), n_rows=int(n_rows), overflow=int(overflow),
-                band_shift=band_shift, n_bands=n_bands, rows=rows,
+                band_shift=band_shift, n_bands=n_bands, rows=rows, local=local_rows,
+                sampled=sampled_rows,
                 records=records[:n_items], tail=records[n_items:], max_items=max_items)
 
 
@@ -69,6 +71,19 @@ def check_plan(indptr, indices, n_src, col_mask, dev):
         assert b[sl][0] == ip[rr] and e[sl][-1] == ip[rr + 1]                # tiles the row ...
         assert np.array_equal(b[sl][1:], e[sl][:-1])                         # ... in item order
         assert np.all(s[sl] == (count == 1))
+    # locality: up to 4 evenly spaced edges of every row below 64 edges are sampled; local
+    # = source within 1/64 of the id space (at least 1,024 ids) of the row's own position
+    n_dst = deg.size
+    cols_all = (indices.numpy() & col_mask).astype(np.int64)
+    own = np.arange(n_dst, dtype=np.int64) * n_src // max(n_dst, 1)
+    n_sampled = n_local = 0
+    for k in range(4):
+        take = (deg < CHUNK) & (deg > k)
+        ns = np.minimum(deg[take], 4)
+        c = cols_all[ip[:-1][take] + deg[take] * k // ns]
+        n_sampled += int(take.sum())
+        n_local += int((np.abs(c - own[take]) <= max(n_src >> 6, 1024)).sum())
+    assert p["sampled"] == n_sampled and p["local"] == n_local
     # bands of 2^17 ids, wider only when that would give more than 64 of them
     assert p["band_shift"] >= BAND_SHIFT and 1 <= p["n_bands"] <= MAX_BANDS
     assert ((max(n_src, 1) - 1) >> p["band_shift"]) + 1 == p["n_bands"]
@@ -142,3 +157,22 @@ def test_more_sources_than_edges(dev):
 def test_no_long_rows(dev):
     indptr, indices = random_csr(500, 500, 0.01, 2)
     assert check_plan(indptr, indices, 500, 0x7fffffff, dev) is None
+
+
+def test_locality_of_a_planted_graph_and_of_its_shuffle(dev):
+    """Most rows of a graph with planted communities (contiguous ids) are local, few of the
+    same graph with shuffled ids are: the flag the row kernels deal their rows by."""
+    from yitu_amd.data import graphgen
+    n_comm, size = 256, 512
+    n = n_comm * size
+    rng = np.random.default_rng(3)
+    dst = np.repeat(np.arange(n), 40)
+    src = dst // size * size + rng.integers(0, size, dst.size)
+    indptr, indices = graphgen.csr_from_edges(torch.from_numpy(dst), torch.from_numpy(src), n, n)
+    p = check_plan(indptr, indices, n, 0x7fffffff, dev)
+    assert p["local"] == p["sampled"] == 4 * n
+    shuffle = rng.permutation(n)
+    indptr, indices = graphgen.csr_from_edges(torch.from_numpy(shuffle[dst]),
+                                              torch.from_numpy(shuffle[src]), n, n)
+    p = check_plan(indptr, indices, n, 0x7fffffff, dev)
+    assert p["local"] * 8 < p["sampled"]

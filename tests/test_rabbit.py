@@ -183,3 +183,63 @@ def test_input_checks():
         rabbit.reorder(torch.tensor([[0, -1], [1, 2]], dtype=torch.int32))
     empty = rabbit.reorder(torch.zeros(2, 0, dtype=torch.int32))
     assert empty.shape == (2, 0)
+
+
+def _planted(k, size, seed, links_per_community=2):
+    rng = np.random.default_rng(seed)
+    n = k * size
+    src, dst = [], []
+    for c in range(k):
+        ids = np.arange(c * size, (c + 1) * size)
+        a = rng.choice(ids, size * 6)
+        b = rng.choice(ids, size * 6)
+        src.append(a)
+        dst.append(b)
+    src.append(rng.integers(0, n, k * links_per_community))
+    dst.append(rng.integers(0, n, k * links_per_community))
+    shuffle = rng.permutation(n)
+    s, d = shuffle[np.concatenate(src)], shuffle[np.concatenate(dst)]
+    return n, shuffle, np.ascontiguousarray(np.stack([s, d]).astype(np.int32))
+
+
+@pytest.mark.parametrize("threads", [2, 8, 0])
+def test_parallel_aggregation_gives_a_valid_local_permutation(threads):
+    """Several threads follow the reference's lock-free protocol (rabbit_order.hpp:554-621);
+    the permutation then depends on timing, like the reference's, so what is checked is
+    what every valid outcome has: a bijection, the same edges under it, planted communities
+    contiguous, the reference's own locality metric (mean |src - dst|) far below the
+    shuffled ids' and close to the single-thread result's."""
+    k, size = 400, 30
+    n, shuffle, ei_np = _planted(k, size, seed=threads)
+    ei = torch.from_numpy(ei_np)
+    single = rabbit.reorder(ei)
+    for _ in range(3):
+        out, perm = rabbit.reorder_with_perm(ei, threads=threads)
+        p = perm.numpy()
+        assert sorted(p.tolist()) == list(range(n))
+        assert np.array_equal(out.numpy()[0], p[ei_np[0]]) and np.array_equal(out.numpy()[1], p[ei_np[1]])
+        before = np.abs(ei_np[0].astype(np.int64) - ei_np[1]).mean()
+        after = (out[0].long() - out[1].long()).abs().float().mean().item()
+        ref = (single[0].long() - single[1].long()).abs().float().mean().item()
+        assert after < before / 20 and after < 3 * ref + 10
+        spans = [np.ptp(p[shuffle[c * size:(c + 1) * size]]) + 1 for c in range(k)]
+        assert np.median(spans) <= size * 1.5
+
+
+def test_parallel_aggregation_on_a_power_law_graph():
+    """Hub vertices are where merges contend: the retry lists and the final serial pass
+    must leave every vertex numbered exactly once."""
+    from yitu_amd.data import graphgen
+    src, dst = graphgen.rmat(15, 400000, 5)
+    ei = torch.stack([src, dst]).to(torch.int32).contiguous()
+    n = int(ei.max()) + 1
+    for threads in (8, 8, 3):
+        out, perm = rabbit.reorder_with_perm(ei, threads=threads)
+        assert sorted(perm.tolist()) == list(range(n))
+        assert torch.equal(out, perm[ei.long()])
+
+
+def test_one_thread_through_the_threaded_entry_is_the_reproducible_order():
+    n, _, ei_np = _planted(50, 20, seed=1)
+    ei = torch.from_numpy(ei_np)
+    assert torch.equal(rabbit.reorder(ei, threads=1), rabbit.reorder(ei))

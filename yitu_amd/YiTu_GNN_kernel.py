@@ -74,7 +74,7 @@ def _aggregate(x, row_pointers, column_index, degrees, alpha, edge_scale=None):
     maxdeg = _lib.max_degree(row_pointers)
     plan = _lib.row_plan(row_pointers, column_index, n_src, 0x7FFFFFFF)
     need = _lib.size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(dim), c_int(1)) \
-        if plan is not None else 0
+        if plan is not None and maxdeg >= 64 else 0
     ws = _lib.workspace(need, x.device)
     with torch.cuda.device(x.device):
         rc = _lib.lib().yitu_agg_csr(

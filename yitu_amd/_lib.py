@@ -163,8 +163,10 @@ _plans = {}
 
 def row_plan(indptr, indices, n_src, col_mask):
     """Device buffer holding the row plan of (indptr, indices), or None when no
-    row reaches the planning threshold."""
-    if max_degree(indptr) < 64:
+    row reaches the planning threshold and the graph is small. A large graph without
+    long rows still gets one: its header tells the row kernels whether most sources of
+    a row lie near the row's own id, which decides how rows are dealt to the XCDs."""
+    if max_degree(indptr) < 64 and indices.numel() < (1 << 20):
         return None
     key = (id(indices), indices.data_ptr(), indices._version, id(indptr), indptr.data_ptr(),
            indptr._version, int(n_src), int(col_mask))

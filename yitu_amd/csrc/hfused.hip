@@ -21,14 +21,15 @@ template <int G, int KT, int HP>
 __global__ __launch_bounds__(kBlock) void hfused_rows_kernel(SpmmParams a, int a_blocks,
                                                              SddmmParams b) {
     if ((int)blockIdx.x < a_blocks)
-        spmm_rows_body<4, G, KT, W_EDGEHEAD, float>(a, blockIdx.x);
+        spmm_rows_body<4, G, KT, W_EDGEHEAD, float>(a, blockIdx.x, a_blocks);
     else
         sddmm_fwd_rows_body<HP>(b, blockIdx.x - a_blocks);
 }
 
 template <int G, int KT>
 int launch_heads(const SpmmParams &a, const SddmmParams &b, hipStream_t stream) {
-    const int ga = (int)ceil_div(a.n_rows, kWavesPerBlock * rows_per_wave(a.n_rows));
+    int ga = (int)ceil_div(a.n_rows, kWavesPerBlock * rows_per_wave(a.n_rows));
+    if (ga >= 64) ga = (ga + 7) / 8 * 8;  // as the SpMM launches its row kernel (row_block)
     const int gb = (int)ceil_div(b.n_dst, kWavesPerBlock);
 #define YITU_HF(HP)                                                              \
     hfused_rows_kernel<G, KT, HP><<<ga + gb, kBlock, 0, stream>>>(a, ga, b);     \

@@ -13,12 +13,19 @@
 //      merge dendrogram; communities are laid out in the order in which they
 //      became top-level (rabbit_order.hpp:623-673)
 //
-// The aggregation in step 2 runs on one thread: the reference's lock-free
-// parallel version gives a thread-count- and timing-dependent permutation, and
-// the single-thread order is the one that is reproducible. Edge weights are
+// Step 2 exists twice. On one thread it is a function of the graph alone (the
+// reproducible order, the default). With several threads it follows the
+// reference's protocol (rabbit_order.hpp:393-526, 554-621): threads take the
+// degree-sorted vertices in turn; a vertex is locked by swapping its strength for
+// -1, merged into its best neighbour with one compare-and-swap on that
+// neighbour's (strength, last child) word, and put on the thread's retry list
+// when the neighbour is locked or the swap loses a race. Which vertex wins such
+// a race depends on timing, so the permutation differs from run to run, as the
+// reference's does; every outcome is a valid merge dendrogram. Edge weights are
 // counts held in float (exact below 2^24), so the order in which duplicates are
 // summed does not change any comparison.
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -50,21 +57,27 @@ struct Adjacency {
 };
 
 Adjacency build_adjacency(const int32_t *src, const int32_t *dst, int64_t m, vint n) {
+    // counting sort by end point; the slots of a row are handed out with relaxed atomic
+    // adds (the rows are sorted afterwards, so the order of arrival does not matter)
     std::vector<int64_t> count(n + 1, 0);
+#pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < m; i++) {
         if (src[i] != dst[i]) {
-            count[(vint)src[i] + 1]++;
-            count[(vint)dst[i] + 1]++;
+            __atomic_fetch_add(&count[(vint)src[i] + 1], 1, __ATOMIC_RELAXED);
+            __atomic_fetch_add(&count[(vint)dst[i] + 1], 1, __ATOMIC_RELAXED);
         }
     }
     for (vint v = 0; v < n; v++) count[v + 1] += count[v];
     std::vector<vint> raw((size_t)count[n]);
     {
         std::vector<int64_t> fill(count.begin(), count.end() - 1);
+#pragma omp parallel for schedule(static)
         for (int64_t i = 0; i < m; i++) {
             if (src[i] != dst[i]) {
-                raw[(size_t)fill[(vint)src[i]]++] = (vint)dst[i];
-                raw[(size_t)fill[(vint)dst[i]]++] = (vint)src[i];
+                raw[(size_t)__atomic_fetch_add(&fill[(vint)src[i]], 1, __ATOMIC_RELAXED)] =
+                    (vint)dst[i];
+                raw[(size_t)__atomic_fetch_add(&fill[(vint)dst[i]], 1, __ATOMIC_RELAXED)] =
+                    (vint)src[i];
             }
         }
     }
@@ -217,6 +230,183 @@ Dendrogram aggregate(const Adjacency &adj, vint n) {
     return g;
 }
 
+// ---- parallel aggregation ---------------------------------------------------------
+// (strength, last merged child) of a vertex in one 64-bit word, so that a merge is
+// one compare-and-swap; strength < 0 = locked by the thread that is merging it away
+// (or merged for good).
+struct Atom {
+    float str;
+    vint child;
+};
+inline uint64_t pack(Atom a) {
+    uint32_t s;
+    std::memcpy(&s, &a.str, 4);
+    return (uint64_t)a.child << 32 | s;
+}
+inline Atom unpack(uint64_t x) {
+    Atom a;
+    const uint32_t s = (uint32_t)x;
+    std::memcpy(&a.str, &s, 4);
+    a.child = (vint)(x >> 32);
+    return a;
+}
+
+struct SharedGraph {
+    vint n = 0;
+    std::vector<std::atomic<uint64_t>> atom;
+    std::vector<vint> com;           // read and shortened by every thread (relaxed)
+    std::vector<vint> sibling;
+    std::vector<vint> united_child;  // touched only by the thread that merges the vertex
+    std::vector<std::vector<Edge>> es;
+    double total = 0.0;
+    explicit SharedGraph(vint n_) : n(n_), atom(n_), com(n_), sibling(n_, kNone),
+                                    united_child(n_, kNone), es(n_) {}
+};
+
+inline vint load_com(const SharedGraph &g, vint v) {
+    return __atomic_load_n(&g.com[v], __ATOMIC_RELAXED);
+}
+
+inline vint shared_root(SharedGraph &g, vint v) {
+    vint c = v;
+    for (vint next = load_com(g, c); next != c; next = load_com(g, c)) c = next;
+    if (v != c && load_com(g, v) != c) __atomic_store_n(&g.com[v], c, __ATOMIC_RELAXED);
+    return c;
+}
+
+// like gather_community_edges, on the shared structure; other threads may append
+// children to v meanwhile, the caller checks for that after locking v
+void unite_shared(SharedGraph &g, vint v, std::vector<Edge> &buf) {
+    buf.clear();
+    size_t combined = 0;
+    auto push = [&](vint u) {
+        for (const Edge &e : g.es[u]) {
+            const vint c = shared_root(g, e.to);
+            if (c != v) buf.push_back(Edge{c, e.w});
+        }
+        if (buf.size() - combined >= 2048) {
+            combined += combine(buf.data() + combined, buf.data() + buf.size());
+            buf.resize(combined);
+        }
+    };
+    push(v);
+    for (vint c = unpack(g.atom[v].load()).child; g.united_child[v] != c;
+         c = unpack(g.atom[v].load()).child) {
+        // the vertices on the sibling list are merged for good: nobody modifies them
+        for (vint w = c; w != kNone && w != g.united_child[v]; w = g.sibling[w]) push(w);
+        g.united_child[v] = c;
+    }
+    buf.resize(combine(buf.data(), buf.data() + buf.size()));
+    g.es[v].assign(buf.begin(), buf.end());
+}
+
+// v itself: top-level for good; kNone: lost a race, try again later; else: merged into it
+vint merge_shared(SharedGraph &g, vint v, std::vector<Edge> &buf) {
+    unite_shared(g, v, buf);
+    // lock v: strength -> -1, child kept
+    uint64_t cur = g.atom[v].load();
+    while (!g.atom[v].compare_exchange_weak(cur, pack(Atom{-1.0f, unpack(cur).child}))) {
+    }
+    const float vstr = unpack(cur).str;
+    if (unpack(g.atom[v].load()).child != g.united_child[v]) unite_shared(g, v, buf);
+    auto unlock = [&] {
+        uint64_t x = g.atom[v].load();
+        while (!g.atom[v].compare_exchange_weak(x, pack(Atom{vstr, unpack(x).child}))) {
+        }
+    };
+    double best_gain = 0.0;
+    vint best = v;
+    for (const Edge &e : g.es[v]) {
+        const double d =
+            (double)e.w - (double)vstr * (double)unpack(g.atom[e.to].load()).str / g.total;
+        if (best_gain < d) {
+            best_gain = d;
+            best = e.to;
+        }
+    }
+    if (best == v) {
+        unlock();
+        return v;
+    }
+    uint64_t target = g.atom[best].load();
+    const Atom ta = unpack(target);
+    if (ta.str < 0.0f) {  // the neighbour is being merged itself
+        unlock();
+        return kNone;
+    }
+    g.sibling[v] = ta.child;  // visible to whoever sees v as best's child
+    if (!g.atom[best].compare_exchange_strong(target, pack(Atom{ta.str + vstr, v}))) {
+        g.sibling[v] = kNone;
+        unlock();
+        return kNone;
+    }
+    __atomic_store_n(&g.com[v], best, __ATOMIC_RELAXED);
+    return best;
+}
+
+Dendrogram aggregate_parallel(const Adjacency &adj, vint n, int n_threads) {
+    SharedGraph g(n);
+    double total = 0.0;
+#pragma omp parallel for reduction(+ : total) schedule(static) num_threads(n_threads)
+    for (int64_t v = 0; v < (int64_t)n; v++) {
+        const Edge *b = adj.edges.data() + adj.ptr[v], *e = adj.edges.data() + adj.ptr[v + 1];
+        float s = 0.0f;
+        for (const Edge *p = b; p != e; ++p) s += p->w;
+        g.es[v].assign(b, e);
+        g.com[v] = (vint)v;
+        g.atom[v].store(pack(Atom{s, kNone}));
+        total += s;
+    }
+    g.total = total;
+    std::vector<std::pair<vint, vint>> order(n);
+    for (vint v = 0; v < n; v++) order[v] = {v, (vint)g.es[v].size()};
+    std::stable_sort(order.begin(), order.end(),
+                     [](const std::pair<vint, vint> &x, const std::pair<vint, vint> &y) {
+                         return x.second < y.second;
+                     });
+    std::vector<std::vector<vint>> tops_of(n_threads);
+#pragma omp parallel num_threads(n_threads)
+    {
+        const int tid = omp_get_thread_num();
+        std::vector<vint> tops, pending, still;
+        std::vector<Edge> buf;
+        buf.reserve(1 << 16);
+        auto attempt = [&](vint v) {
+            const vint u = merge_shared(g, v, buf);
+            if (u == v) tops.push_back(v);
+            return u != kNone;
+        };
+#pragma omp for schedule(static, 1)
+        for (int64_t i = 0; i < (int64_t)n; i++) {
+            if (!pending.empty()) {
+                still.clear();
+                for (const vint w : pending)
+                    if (!attempt(w)) still.push_back(w);
+                pending.swap(still);
+            }
+            const vint v = order[(size_t)i].first;
+            if (!attempt(v)) pending.push_back(v);
+        }
+        // (implicit barrier) what is still pending is merged one thread at a time:
+        // nothing is locked any more, so every attempt succeeds
+#pragma omp critical
+        {
+            for (const vint w : pending)
+                while (!attempt(w)) {
+                }
+            tops_of[tid] = std::move(tops);
+        }
+    }
+    Dendrogram d;
+    d.n = n;
+    d.child.resize(n);
+    d.sibling = std::move(g.sibling);
+    for (vint v = 0; v < n; v++) d.child[v] = unpack(g.atom[v].load()).child;
+    for (auto &t : tops_of) d.tops.insert(d.tops.end(), t.begin(), t.end());
+    d.total = total;
+    return d;
+}
+
 // new id of every vertex: depth-first over each top-level community's merge tree
 std::vector<vint> permutation(const Dendrogram &g) {
     std::vector<vint> perm(g.n, kNone);
@@ -243,9 +433,9 @@ extern "C" __attribute__((visibility("default"))) const char *yitu_host_last_err
     return g_err;
 }
 
-extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder(
+extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder_threads(
     int32_t *out_edge_index, int32_t *perm_out, int64_t perm_capacity, int64_t *n_vertices,
-    const int32_t *in_edge_index, int64_t n_edges) {
+    const int32_t *in_edge_index, int64_t n_edges, int n_threads) {
     if (n_edges < 0 || (n_edges > 0 && !in_edge_index)) {
         snprintf(g_err, sizeof(g_err), "bad edge list");
         return -1;
@@ -268,7 +458,8 @@ extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder(
     }
     if (n == 0) return 0;
     const Adjacency adj = build_adjacency(src, dst, n_edges, n);
-    const Dendrogram g = aggregate(adj, n);
+    if (n_threads <= 0) n_threads = omp_get_max_threads();
+    const Dendrogram g = n_threads == 1 ? aggregate(adj, n) : aggregate_parallel(adj, n, n_threads);
     const std::vector<vint> perm = permutation(g);
     for (vint v = 0; v < n; v++) {
         if (perm[v] == kNone) {
@@ -286,4 +477,11 @@ extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder(
         }
     }
     return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int yitu_rabbit_reorder(
+    int32_t *out_edge_index, int32_t *perm_out, int64_t perm_capacity, int64_t *n_vertices,
+    const int32_t *in_edge_index, int64_t n_edges) {
+    return yitu_rabbit_reorder_threads(out_edge_index, perm_out, perm_capacity, n_vertices,
+                                       in_edge_index, n_edges, 1);
 }

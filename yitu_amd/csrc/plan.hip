@@ -21,7 +21,7 @@ struct BuildBuffers {
     PlanCounters *counters;
     int4 *rows;
     int4 *records;
-    int *band_info;   // {log2 of the band width, number of bands}, in the plan header
+    int *band_info;   // {log2 of the band width, number of bands, local edges, sampled edges}, in the plan header
     int4 *items;      // {first edge, end edge, index into rows[], row} in queue order
     uint32_t *keys_in, *keys_out;
     int32_t *vals_in, *order;
@@ -45,6 +45,8 @@ __global__ __launch_bounds__(kBlock) void plan_init_kernel(BuildBuffers b) {
     if (i0 == 0) {
         b.band_info[0] = b.band_shift;
         b.band_info[1] = b.n_bands;
+        b.band_info[kPlanInfoLocal] = 0;
+        b.band_info[kPlanInfoSampled] = 0;
     }
     // slots that get no item sort behind every real key
     for (int64_t i = i0; i < b.max_items; i += stride) {
@@ -80,14 +82,50 @@ __device__ __forceinline__ int block_rank(bool flag, int *wave_sums, int *block_
     return slot;
 }
 
+// The same pass measures whether the graph is local, on the rows that the row
+// kernels walk (fewer than 64 edges): up to 4 edges of every such row, evenly
+// spaced, are sampled, and an edge counts as local when its source lies within
+// 1/64 of the id space (at least 1,024 ids) of the row's own relative position.
+// One add per workgroup and counter.
 __global__ __launch_bounds__(kBlock) void plan_queue_kernel(BuildBuffers b,
                                                             const int32_t *__restrict__ indptr,
-                                                            int n_rows) {
+                                                            const int32_t *__restrict__ indices,
+                                                            int n_rows, int n_src, int col_mask) {
     __shared__ int wave_sums[kWavesPerBlock];
     __shared__ int block_base;
     const int row = blockIdx.x * kBlock + threadIdx.x;
-    int deg = 0;
-    if (row < n_rows) deg = indptr[row + 1] - indptr[row];
+    int deg = 0, beg = 0;
+    if (row < n_rows) {
+        beg = indptr[row];
+        deg = indptr[row + 1] - beg;
+    }
+    int sampled = 0, local = 0;
+    if (deg < kPlanThreshold) {
+        sampled = min(deg, 4);
+        const long long own = (long long)row * n_src / n_rows;
+        const long long reach = max((long long)n_src >> 6, 1024ll);
+        for (int k = 0; k < sampled; k++) {
+            const long long c = indices[beg + deg * k / sampled] & col_mask;
+            local += c - own <= reach && own - c <= reach;
+        }
+    }
+    __shared__ int seen[2];  // sampled edges, local ones
+    if (threadIdx.x == 0) seen[0] = seen[1] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+        sampled += __shfl_xor(sampled, o, kWave);
+        local += __shfl_xor(local, o, kWave);
+    }
+    if (lane_id() == 0 && sampled) {
+        atomicAdd(&seen[0], sampled);
+        atomicAdd(&seen[1], local);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && seen[0]) {
+        atomicAdd(&b.band_info[kPlanInfoSampled], seen[0]);
+        if (seen[1]) atomicAdd(&b.band_info[kPlanInfoLocal], seen[1]);
+    }
     const bool longrow = deg >= kPlanThreshold;
     const int slot = block_rank(longrow, wave_sums, &block_base, &b.counters->n_rows);
     if (longrow) {
@@ -258,6 +296,7 @@ PlanView plan_view(const void *plan, int64_t nnz) {
     w += align_up(sizeof(int4) * (size_t)v.max_rows, 256);
     v.records = reinterpret_cast<const int4 *>(w);
     v.threshold = kPlanThreshold;
+    v.info = reinterpret_cast<const int *>(static_cast<const char *>(plan) + 256);
     return v;
 }
 
@@ -303,8 +342,8 @@ int plan_build(void *plan, size_t plan_size, const int32_t *indptr, const int32_
     plan_init_kernel<<<std::min(item_grid, 4096), kBlock, 0, stream>>>(b);
     YITU_LAUNCH_CHECK();
     if (n_rows > 0) {
-        plan_queue_kernel<<<(int)ceil_div(n_rows, kBlock), kBlock, 0, stream>>>(b, indptr,
-                                                                                (int)n_rows);
+        plan_queue_kernel<<<(int)ceil_div(n_rows, kBlock), kBlock, 0, stream>>>(
+            b, indptr, indices, (int)n_rows, (int)n_src, col_mask);
         YITU_LAUNCH_CHECK();
     }
     plan_items_kernel<<<(int)ceil_div(b.max_rows, kWavesPerBlock), kBlock, 0, stream>>>(
@@ -325,12 +364,12 @@ int plan_resolve(PlanView &view, bool &has_items, const void *plan, const int32_
     *rest = workspace;
     *rest_bytes = workspace_bytes;
     has_items = nnz >= kPlanThreshold && !(max_degree_hint >= 0 && max_degree_hint < kPlanThreshold);
-    if (!has_items) {
-        view = plan_none();
+    if (plan) {  // also without long rows: the header says whether the graph is local
+        view = plan_view(plan, nnz);
         return 0;
     }
-    if (plan) {
-        view = plan_view(plan, nnz);
+    if (!has_items) {
+        view = plan_none();
         return 0;
     }
     const size_t pb = plan_bytes(nnz), bw = plan_build_workspace_bytes(nnz);

@@ -54,7 +54,24 @@ struct PlanView {
     int max_rows;
     int max_items;
     int threshold;  // rows with >= threshold edges are left to the item kernels
+    const int *info;  // header words behind the counters (kPlanInfo*), or null
 };
+
+// Header words: {log2 of the band width, number of bands, local edges, sampled edges}.
+// The builder samples edges of the short rows; an edge is local when its source lies
+// near the row's own relative position in the id space. A graph three quarters of
+// whose sampled edges are local (community structure with ids to match, as planted
+// or as a reorder leaves them) has its short rows walked XCD by XCD. Measured on two
+// graphs of 2^21 vertices and 62 M edges, fp32 rows of 128 floats: planted
+// communities of 512 (97 % local) 4.43 ms round robin, 2.69 ms XCD by XCD; an R-MAT
+// graph after the Rabbit-Order reorder (51 % local: its rows of one or two edges sit
+// next to their source, its hot sources are everybody's) 2.70 and 2.94 ms.
+constexpr int kPlanInfoLocal = 2;
+constexpr int kPlanInfoSampled = 3;
+
+__device__ __forceinline__ bool plan_says_local(const PlanView &v) {
+    return v.info && 4ll * v.info[kPlanInfoLocal] > 3ll * v.info[kPlanInfoSampled];
+}
 
 inline int64_t plan_max_rows(int64_t nnz) { return nnz / kPlanThreshold + 1; }
 // A row of deg >= 64 edges gives at most deg / 64 + min(bands, deg / 16) items.

@@ -57,7 +57,8 @@ size_t spmm_workspace_bytes(int64_t nnz, int64_t L, bool with_plan) {
 
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 static int launch_variant(const SpmmParams &p, bool has_items, hipStream_t stream) {
-    const int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * rows_per_wave(p.n_rows));
+    int grid = (int)ceil_div(p.n_rows, kWavesPerBlock * rows_per_wave(p.n_rows));
+    if (grid >= 64) grid = (grid + 7) / 8 * 8;  // whole eighths for row_block
     spmm_rows_kernel<VEC, G, KT, WMODE, TIN><<<grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (has_items) {

@@ -201,16 +201,31 @@ __host__ __device__ inline int rows_per_wave(int n_rows) {
     return r < 1 ? 1 : (r > kRowsPerWave ? kRowsPerWave : r);
 }
 
+// Which block of rows a workgroup of the row kernel takes. The hardware deals
+// consecutive workgroups to the 8 XCDs round robin. Taken as they come, the
+// workgroups that run on one XCD at one time are spread over 8 times as many rows
+// as they cover: right for graphs without locality, whose hot sources every L2
+// holds anyway. When most sources of a row lie near the row's own id (community
+// structure, a reordered graph), XCD k instead walks the k-th eighth of the rows,
+// so that the rows in flight on an XCD are neighbours and share their sources in
+// that XCD's L2. Which of the two a graph is, its row plan says (measured when the
+// plan is built); launches of at least 64 workgroups come in multiples of 8, whose
+// surplus workgroups find no rows.
+__device__ __forceinline__ int row_block(const SpmmParams &p, int block, int n_blocks) {
+    if (n_blocks < 64 || (n_blocks & 7) || !plan_says_local(p.plan)) return block;
+    return (block & 7) * (n_blocks >> 3) + (block >> 3);
+}
+
 // Row kernel: a wave walks rows_per_wave consecutive rows. Their bounds come from
 // one coalesced indptr load, their edges from a sliding 64-edge window, so a
 // short row costs one round of feature gathers and nothing else that waits on
 // memory. Rows that the plan covers are skipped.
 template <int VEC, int G, int KT, int WMODE, typename TIN>
-__device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block) {
+__device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, int n_blocks) {
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
     const int rpw = rows_per_wave(p.n_rows);
-    const int r0 = (block * kWavesPerBlock + wave) * rpw;
+    const int r0 = (row_block(p, block, n_blocks) * kWavesPerBlock + wave) * rpw;
     if (r0 >= p.n_rows) return;
     const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
@@ -263,7 +278,7 @@ __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block) {
 
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
-    spmm_rows_body<VEC, G, KT, WMODE, TIN>(p, blockIdx.x);
+    spmm_rows_body<VEC, G, KT, WMODE, TIN>(p, blockIdx.x, gridDim.x);
 }
 
 constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave

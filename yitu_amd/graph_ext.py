@@ -121,7 +121,7 @@ def spmm_forward(values, indptr, indices, features):
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f), c_int(1)) \
-        if plan is not None else 0
+        if plan is not None and maxdeg >= 64 else 0
     ws = _lib.workspace(need, dev)
     entry = _lib.lib().yitu_spmm_forward_bf16 if bf16 else _lib.lib().yitu_spmm_forward
     with torch.cuda.device(dev):
