@@ -433,6 +433,85 @@ int yitu_gemm_bf16_tn(float *c_device, const void *a_bf16_device, const void *b_
                       int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Temporal neighbour attention                                                */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * TransfomerAttentionLayer.forward, non-combined branches
+ * (YiTu_GNN/YiTu_T/layers.py:75-142): for a sampled block of n_dst roots whose
+ * n_edges neighbour edges are grouped by root (indptr [n_dst+1]), with node
+ * features h [n_dst + n_edges, dim_node] (roots first, one row per edge after
+ * them), edge features f [n_edges, dim_edge] and time deltas dt [n_edges],
+ *   Q = w_q [h_root | cos(time_b)] + b_q
+ *   K, V = w_{k,v} [h_edge | f | cos(time_w dt + time_b)] + b_{k,v}      (layers.py:6-17, 109-125)
+ *   agg[r] = sum_e softmax_r(LeakyReLU_0.2(<Q[r], K[e]>_head)) V[e]      (layers.py:126-135)
+ *   out = LayerNorm(ReLU(w_out [agg | h_root] + b_out))                  (layers.py:136-142)
+ * The three products run on yitu_sgemm / yitu_sgemm_typed between these calls;
+ * every matrix they touch has rows of ld = yitu_tattn_row_length(...) floats
+ * whose last column carries the ones (inputs) or the bias (weights), so the
+ * products add the biases and their transposed forms return the bias gradients.
+ *
+ * yitu_tattn_prepare fills, in one launch: x_kv [n_edges, ld], x_q [n_dst, ld],
+ * columns dim_out.. of x_r [n_dst, ld] (h_root, ones), w_kv [2 dim_out, ld]
+ * (w_k above w_v), w_q2 [2 dim_out, ld] (w_q, then zero rows: its product has the
+ * width of the K|V product and shares its launch), w_r [dim_out, ld]. Weights are
+ * row-major [out, in] like nn.Linear.weight. Needs dim_node + dim_time > 0.
+ * Then: kv [n_edges, 2 dim_out] = x_kv . w_kv^T, q2 [n_dst, 2 dim_out] = x_q . w_q2^T.
+ *
+ * yitu_tattn_forward: attn [n_edges, n_heads] and x_r[:, 0..dim_out) = agg (zero
+ * for a root without edges), one wave per root. Then pre [n_dst, dim_out] =
+ * x_r . w_r^T and yitu_relu_layernorm_forward.
+ *
+ * Backward: yitu_relu_layernorm_backward (d_pre with a row stride, partial sums
+ * of the affine gradients: [yitu_tattn_partial_rows(n_rows), 2 n_cols], gamma's
+ * then beta's), dx_r = d_pre . w_r, yitu_tattn_backward (dq2 [n_dst, 2 dim_out]
+ * columns 0..dim_out-1, dkv [n_edges, 2 dim_out]; scratch [n_edges, n_heads, 2]),
+ * dx_kv = dkv . w_kv, dx_q = dq2 . w_q2, the weight gradients as transposed
+ * products, yitu_tattn_finalize (grad_h [n_dst + n_edges, dim_node], grad_f, either
+ * may be NULL; partial sums of the time encoder's gradients
+ * [yitu_tattn_partial_rows(n_dst + n_edges), 2 dim_time], frequency then phase) and
+ * yitu_partial_sums (column sums of two partial tables, rows added in ascending
+ * order). No atomics: bitwise reproducible. Limits: dim_out, dim_time <= 256,
+ * n_heads <= 8 and a divisor of dim_out.
+ */
+int64_t yitu_tattn_row_length(int64_t dim_node, int64_t dim_edge, int64_t dim_time,
+                              int64_t dim_out);
+int64_t yitu_tattn_partial_rows(int64_t n_rows);
+int yitu_tattn_prepare(float *x_kv_device, float *x_q_device, float *x_r_device,
+                       float *w_kv_device, float *w_q2_device, float *w_r_device,
+                       const float *h_device, const float *f_device, const float *dt_device,
+                       const float *time_w_device, const float *time_b_device,
+                       const float *w_q_device, const float *b_q_device, const float *w_k_device,
+                       const float *b_k_device, const float *w_v_device, const float *b_v_device,
+                       const float *w_out_device, const float *b_out_device, int64_t n_dst,
+                       int64_t n_edges, int64_t dim_node, int64_t dim_edge, int64_t dim_time,
+                       int64_t dim_out, int64_t ld, void *stream);
+int yitu_tattn_forward(float *x_r_device, float *attn_device, const float *q2_device,
+                       const float *kv_device, const int32_t *indptr_device, int64_t n_dst,
+                       int64_t n_edges, int64_t dim_out, int64_t n_heads, int64_t ld, void *stream);
+int yitu_tattn_backward(float *dq2_device, float *dkv_device, float *scratch_device,
+                        const float *dx_r_device, const float *q2_device, const float *kv_device,
+                        const float *attn_device, const int32_t *indptr_device, int64_t n_dst,
+                        int64_t n_edges, int64_t dim_out, int64_t n_heads, int64_t ld,
+                        void *stream);
+int yitu_relu_layernorm_forward(float *out_device, const float *pre_device,
+                                const float *gamma_device, const float *beta_device,
+                                int64_t n_rows, int64_t n_cols, float eps, void *stream);
+int yitu_relu_layernorm_backward(float *d_pre_device, float *partial_device,
+                                 const float *grad_out_device, const float *pre_device,
+                                 const float *gamma_device, int64_t n_rows, int64_t n_cols,
+                                 int64_t d_pre_row_stride, float eps, void *stream);
+int yitu_tattn_finalize(float *grad_h_device, float *grad_f_device, float *partial_device,
+                        const float *dx_kv_device, const float *dx_q_device,
+                        const float *dx_r_device, const float *dt_device,
+                        const float *time_w_device, const float *time_b_device, int64_t n_dst,
+                        int64_t n_edges, int64_t dim_node, int64_t dim_edge, int64_t dim_time,
+                        int64_t dim_out, int64_t ld, void *stream);
+int yitu_partial_sums(float *out_a_device, const float *partial_a_device, int64_t rows_a,
+                      int64_t cols_a, float *out_b_device, const float *partial_b_device,
+                      int64_t rows_b, int64_t cols_b, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Temporal most-recent-neighbour sampling on the device                       */
 /* ------------------------------------------------------------------------- */
 

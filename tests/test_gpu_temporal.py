@@ -72,3 +72,126 @@ def test_empty_block_returns_zeros(dev):
                         h=torch.randn(5, 8, device=dev), device=dev)
     out = layer(blk)
     assert out.shape == (5, 6) and torch.all(out == 0)
+
+
+def _reference_layer(layer, blk, dtype=torch.float64):
+    """The layer's arithmetic (layers.py:75-142) edge by edge in float64 torch ops, with
+    autograd: per-root softmax through index_reduce / index_add."""
+    import copy
+    ref = copy.deepcopy(layer).to(dtype)
+    n_dst, row = blk.n_dst, blk.row
+    E = row.numel()
+    h = blk.h.detach().to(dtype).requires_grad_() if layer.dim_node_feat > 0 else None
+    f = blk.f.detach().to(dtype).requires_grad_() if layer.dim_edge_feat > 0 else None
+    parts_q, parts_kv = [], []
+    if h is not None:
+        parts_q.append(h[:n_dst])
+        parts_kv.append(h[n_dst:])
+    if f is not None:
+        parts_kv.append(f)
+    if layer.dim_time > 0:
+        # the argument of the cosine as float32 rounds it (product, then bias); the
+        # reference rounds there as well (Linear(1, dim) in float32)
+        w32, b32 = layer.time_enc.w.weight.detach()[:, 0], layer.time_enc.w.bias.detach()
+        arg32 = (blk.dt[:, None] * w32[None, :] + b32).to(dtype)
+        w, b = ref.time_enc.w.weight[:, 0], ref.time_enc.w.bias
+        exact = blk.dt.to(dtype)[:, None] * w[None, :] + b
+        parts_kv.append(torch.cos(exact + (arg32 - exact).detach()))
+        parts_q.append(torch.cos(b)[None, :].expand(n_dst, -1))
+    q = ref.w_q(torch.cat(parts_q, 1))[row]
+    kv_in = torch.cat(parts_kv, 1)
+    k, v = ref.w_k(kv_in), ref.w_v(kv_in)
+    H, D = layer.num_head, layer.dim_out // layer.num_head
+    logits = torch.nn.functional.leaky_relu((q * k).view(E, H, D).sum(-1), 0.2)
+    top = torch.full((n_dst, H), -1e30, dtype=dtype, device=row.device)
+    top = top.index_reduce(0, row, logits.detach(), "amax")
+    p = torch.exp(logits - top[row])
+    s = torch.zeros(n_dst, H, dtype=dtype, device=row.device).index_add(0, row, p)
+    att = p / s[row]
+    agg = torch.zeros(n_dst, H, D, dtype=dtype, device=row.device).index_add(
+        0, row, v.view(E, H, D) * att[:, :, None]).reshape(n_dst, H * D)
+    rst = torch.cat([agg, h[:n_dst]], 1) if h is not None else agg
+    out = ref.layer_norm(torch.relu(ref.w_out(rst)))
+    return ref, out, h, f
+
+
+@pytest.mark.parametrize("dims", [
+    # dim_node, dim_edge, dim_time, num_head, dim_out
+    (172, 0, 100, 1, 100), (172, 0, 100, 4, 100), (16, 12, 8, 2, 32), (0, 5, 10, 1, 24),
+    (20, 0, 0, 2, 64), (33, 7, 100, 8, 256), (9, 0, 3, 1, 6)])
+def test_fused_layer_all_input_combinations(dev, dims):
+    """The layer as one autograd node (input assembly, products, attention per root, ReLU +
+    LayerNorm) for every combination of node / edge / time inputs the reference's branches
+    cover, with roots that have no neighbour, one, 64, 65 and 150 (more than one chunk of
+    the online softmax): output and every gradient against the float64 statement above,
+    rtol 1e-5 / atol 1e-4 (looser for the frequency gradients, see above)."""
+    dim_node, dim_edge, dim_time, num_head, dim_out = dims
+    torch.manual_seed(sum(dims))
+    counts = [0, 1, 64, 65, 150, 3, 0, 20, 20, 7] + [5] * 40
+    n_dst = len(counts)
+    row = np.repeat(np.arange(n_dst), counts)
+    E = row.size
+    dt = np.random.default_rng(0).uniform(0, 1e4, E).astype(np.float32)
+    h = torch.randn(n_dst + E, dim_node, device=dev) if dim_node else None
+    f = torch.randn(E, dim_edge, device=dev) if dim_edge else None
+    blk = TemporalBlock(row, n_dst, dt, h=h, f=f, device=dev)
+    layer = TransfomerAttentionLayer(dim_node, dim_edge, dim_time, num_head, 0.0, 0.0, dim_out).to(dev)
+    with torch.no_grad():   # biases and phases away from their zero initial values
+        for p in layer.parameters():
+            if p.dim() == 1:
+                p.add_(torch.randn_like(p) * 0.3)
+    if h is not None:
+        h.requires_grad_()
+    if f is not None:
+        f.requires_grad_()
+    out = layer(blk)
+    assert out.grad_fn.name().startswith("TemporalAttentionFunction")
+    w = torch.randn_like(out)
+    (out * w).sum().backward()
+    ref, want, h_ref, f_ref = _reference_layer(layer, blk)
+    (want * w.double()).sum().backward()
+    assert_close(out, want.float(), atol=1e-4, what="out")
+    pairs = [(n, p.grad, dict(ref.named_parameters())[n].grad) for n, p in layer.named_parameters()]
+    if h is not None:
+        pairs.append(("h", h.grad, h_ref.grad))
+    if f is not None:
+        pairs.append(("f", f.grad, f_ref.grad))
+    for name, got, ref_grad in pairs:
+        assert got is not None, name
+        scale = 1e4 if name == "time_enc.w.weight" else 1.0   # sums of products with dt <= 10^4
+        assert_close(got, ref_grad.float(), rtol=1e-4, atol=1e-4 * scale, what=name)
+    # same bits on a second run
+    layer.zero_grad()
+    out2 = layer(blk)
+    (out2 * w).sum().backward()
+    assert torch.equal(out, out2)
+    for name, got, _ in pairs[:len(list(layer.parameters()))]:
+        assert torch.equal(got, dict(layer.named_parameters())[name].grad), name
+
+
+def test_fused_layer_equals_the_composed_ops(dev, monkeypatch):
+    """The same block through the fused node and through the composition of graph_ext ops
+    that the layer used before (and still uses under dropout)."""
+    from yitu_amd.temporal import fused
+    torch.manual_seed(5)
+    counts = np.random.default_rng(5).integers(0, 21, 300)
+    row = np.repeat(np.arange(300), counts)
+    dt = np.random.default_rng(6).uniform(0, 1e6, row.size).astype(np.float32)
+    h = torch.randn(300 + row.size, 172, device=dev, requires_grad=True)
+    blk = TemporalBlock(row, 300, dt, h=h, device=dev)
+    layer = TransfomerAttentionLayer(172, 0, 100, 1, 0.0, 0.0, 100).to(dev)
+    w = torch.randn(300, 100, device=dev)
+    out = layer(blk)
+    (out * w).sum().backward()
+    got = [h.grad.clone()] + [p.grad.clone() for p in layer.parameters()]
+    h.grad = None
+    layer.zero_grad()
+    monkeypatch.setattr(fused, "supported", lambda *a: False)
+    out_c = layer(blk)
+    assert not out_c.grad_fn.name().startswith("TemporalAttentionFunction")
+    (out_c * w).sum().backward()
+    assert_close(out, out_c, atol=1e-4)
+    for g, r, name in zip(got, [h.grad] + [p.grad for p in layer.parameters()],
+                          ["h"] + [n for n, _ in layer.named_parameters()]):
+        rtol = 1e-3 if name == "time_enc.w.weight" else 1e-4
+        assert_close(g, r, rtol=rtol, atol=5e-4, what=name)

@@ -13,6 +13,7 @@ import numpy as np
 import torch
 
 from .. import graph_ext
+from . import fused
 from ..xgnn_h import block as xblock
 from ..xgnn_h import bundle, sparse
 
@@ -166,6 +167,19 @@ class TransfomerAttentionLayer(torch.nn.Module):
         n_dst = b.num_dst_nodes()
         if b.num_edges() == 0:
             return torch.zeros((n_dst, self.dim_out), device=dev)
+        drops = self.training and (self.dropout.p > 0 or self.att_dropout.p > 0)
+        if not drops and self.w_k.weight.is_cuda and self.w_k.weight.dtype == torch.float32 and \
+                fused.supported(self.dim_node_feat, self.dim_edge_feat, self.dim_time, self.dim_out,
+                                self.num_head):
+            # the whole layer as one autograd node of twelve launches
+            te = self.time_enc.w if self.dim_time > 0 else None
+            return fused.TemporalAttentionFunction.apply(
+                b.blk.adj_sparse[0], n_dst, self.num_head, self.layer_norm.eps,
+                b.h if self.dim_node_feat > 0 else None, b.f if self.dim_edge_feat > 0 else None,
+                b.dt, te.weight if te is not None else None, te.bias if te is not None else None,
+                self.w_q.weight, self.w_q.bias, self.w_k.weight, self.w_k.bias, self.w_v.weight,
+                self.w_v.bias, self.w_out.weight, self.w_out.bias, self.layer_norm.weight,
+                self.layer_norm.bias)
         parts_q, parts_kv = [], []
         if self.dim_node_feat > 0:
             parts_q.append(b.h[:n_dst])
