@@ -510,6 +510,21 @@ int yitu_tattn_finalize(float *grad_h_device, float *grad_f_device, float *parti
 int yitu_partial_sums(float *out_a_device, const float *partial_a_device, int64_t rows_a,
                       int64_t cols_a, float *out_b_device, const float *partial_b_device,
                       int64_t rows_b, int64_t cols_b, void *stream);
+/*
+ * The last launch of the layer's backward: both column sums (grad_ln [2 dim_out] =
+ * gamma's, beta's; grad_time [2 dim_time] = frequency, phase) and the parameter
+ * gradients out of the bias-augmented rows of dw_kv [2 dim_out, ld], dw_q, dw_r
+ * [dim_out, ld] into one contiguous tensor per parameter (shapes of the
+ * nn.Linear weights / biases of layers.py:63-68).
+ */
+int yitu_tattn_collect(float *grad_ln_device, float *grad_time_device, float *grad_w_q_device,
+                       float *grad_b_q_device, float *grad_w_k_device, float *grad_b_k_device,
+                       float *grad_w_v_device, float *grad_b_v_device, float *grad_w_out_device,
+                       float *grad_b_out_device, const float *partial_ln_device, int64_t rows_ln,
+                       const float *partial_time_device, int64_t rows_time,
+                       const float *dw_kv_device, const float *dw_q_device,
+                       const float *dw_r_device, int64_t dim_node, int64_t dim_edge,
+                       int64_t dim_time, int64_t dim_out, int64_t ld, void *stream);
 
 /* ------------------------------------------------------------------------- */
 /* Temporal most-recent-neighbour sampling on the device                       */

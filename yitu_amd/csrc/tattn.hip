@@ -35,6 +35,7 @@ namespace {
 constexpr int kTattnMaxOut = 256;            // dim_out (and dim_time) <= 4 elements per lane
 constexpr int kT = kTattnMaxOut / kWave;
 constexpr int kTattnMaxHeads = 8;
+constexpr int kEdgesInFlight = 4;            // neighbour rows a wave requests at a time
 constexpr int kRowsPerWaveReduce = 8;        // rows a wave folds before the per-workgroup partial
 
 struct TattnDims {
@@ -173,23 +174,30 @@ __global__ __launch_bounds__(kBlock) void tattn_forward_kernel(
         float mine[kTattnMaxHeads];  // logits of edge c0 + lane
 #pragma unroll
         for (int h = 0; h < kTattnMaxHeads; h++) mine[h] = -INFINITY;
-        for (int j = 0; j < n; j++) {
-            const float *krow = kv + (int64_t)(c0 + j) * 2 * O;
-            float prod[kT];
+        for (int j = 0; j < n; j += kEdgesInFlight) {
+            // the rows of several edges are requested before the first reduction waits
+            float prod[kEdgesInFlight][kT];
 #pragma unroll
-            for (int t = 0; t < kT; t++) {
-                const int i = lane + t * kWave;
-                prod[t] = i < O ? q[t] * krow[i] : 0.0f;
+            for (int u = 0; u < kEdgesInFlight; u++) {
+                const float *krow = kv + (int64_t)(c0 + min(j + u, n - 1)) * 2 * O;
+#pragma unroll
+                for (int t = 0; t < kT; t++) {
+                    const int i = lane + t * kWave;
+                    prod[u][t] = i < O ? q[t] * krow[i] : 0.0f;
+                }
             }
 #pragma unroll
             for (int h = 0; h < kTattnMaxHeads; h++) {
                 if (h < H) {
-                    float part = 0.0f;
 #pragma unroll
-                    for (int t = 0; t < kT; t++) part += head[t] == h ? prod[t] : 0.0f;
-                    float l = wave_sum(part);
-                    l = l > 0.0f ? l : 0.2f * l;
-                    if (lane == j) mine[h] = l;
+                    for (int u = 0; u < kEdgesInFlight; u++) {
+                        float part = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < kT; t++) part += head[t] == h ? prod[u][t] : 0.0f;
+                        float l = wave_sum(part);
+                        l = l > 0.0f ? l : 0.2f * l;
+                        if (j + u < n && lane == j + u) mine[h] = l;
+                    }
                 }
             }
         }
@@ -210,16 +218,26 @@ __global__ __launch_bounds__(kBlock) void tattn_forward_kernel(
                 if (lane < n) attn[(int64_t)(c0 + lane) * H + h] = mine[h];
             }
         }
-        for (int j = 0; j < n; j++) {
-            const float *vrow = kv + (int64_t)(c0 + j) * 2 * O + O;
+        for (int j = 0; j < n; j += kEdgesInFlight) {
+            float v[kEdgesInFlight][kT];
 #pragma unroll
-            for (int h = 0; h < kTattnMaxHeads; h++) {
-                if (h < H) {
-                    const float pj = __shfl(p[h], j, kWave);
+            for (int u = 0; u < kEdgesInFlight; u++) {
+                const float *vrow = kv + (int64_t)(c0 + min(j + u, n - 1)) * 2 * O + O;
 #pragma unroll
-                    for (int t = 0; t < kT; t++) {
-                        const int i = lane + t * kWave;
-                        if (head[t] == h) acc[t] += pj * vrow[i];
+                for (int t = 0; t < kT; t++) {
+                    const int i = lane + t * kWave;
+                    v[u][t] = i < O ? vrow[i] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kEdgesInFlight; u++) {
+#pragma unroll
+                for (int h = 0; h < kTattnMaxHeads; h++) {
+                    if (h < H) {
+                        const float pj = j + u < n ? __shfl(p[h], (j + u) & (kWave - 1), kWave) : 0.0f;
+#pragma unroll
+                        for (int t = 0; t < kT; t++)
+                            if (head[t] == h) acc[t] += pj * v[u][t];
                     }
                 }
             }
@@ -277,29 +295,35 @@ __global__ __launch_bounds__(kBlock) void tattn_backward_kernel(
         float d_att[kTattnMaxHeads], slope[kTattnMaxHeads];
 #pragma unroll
         for (int h = 0; h < kTattnMaxHeads; h++) d_att[h] = slope[h] = 0.0f;
-        for (int j = 0; j < n; j++) {
-            const float *row = kv + (int64_t)(c0 + j) * 2 * O;
-            float qk[kT], gv[kT];
+        for (int j = 0; j < n; j += kEdgesInFlight) {
+            float qk[kEdgesInFlight][kT], gv[kEdgesInFlight][kT];
 #pragma unroll
-            for (int t = 0; t < kT; t++) {
-                const int i = lane + t * kWave;
-                qk[t] = i < O ? q[t] * row[i] : 0.0f;
-                gv[t] = i < O ? g[t] * row[O + i] : 0.0f;
+            for (int u = 0; u < kEdgesInFlight; u++) {
+                const float *row = kv + (int64_t)(c0 + min(j + u, n - 1)) * 2 * O;
+#pragma unroll
+                for (int t = 0; t < kT; t++) {
+                    const int i = lane + t * kWave;
+                    qk[u][t] = i < O ? q[t] * row[i] : 0.0f;
+                    gv[u][t] = i < O ? g[t] * row[O + i] : 0.0f;
+                }
             }
 #pragma unroll
             for (int h = 0; h < kTattnMaxHeads; h++) {
                 if (h < H) {
-                    float a = 0.0f, b = 0.0f;
 #pragma unroll
-                    for (int t = 0; t < kT; t++) {
-                        a += head[t] == h ? qk[t] : 0.0f;
-                        b += head[t] == h ? gv[t] : 0.0f;
-                    }
-                    a = wave_sum(a);
-                    b = wave_sum(b);
-                    if (lane == j) {
-                        slope[h] = a > 0.0f ? 1.0f : 0.2f;
-                        d_att[h] = b;
+                    for (int u = 0; u < kEdgesInFlight; u++) {
+                        float a = 0.0f, b = 0.0f;
+#pragma unroll
+                        for (int t = 0; t < kT; t++) {
+                            a += head[t] == h ? qk[u][t] : 0.0f;
+                            b += head[t] == h ? gv[u][t] : 0.0f;
+                        }
+                        a = wave_sum(a);
+                        b = wave_sum(b);
+                        if (j + u < n && lane == j + u) {
+                            slope[h] = a > 0.0f ? 1.0f : 0.2f;
+                            d_att[h] = b;
+                        }
                     }
                 }
             }
@@ -329,6 +353,7 @@ __global__ __launch_bounds__(kBlock) void tattn_backward_kernel(
                 dl[h] = a[h] * (scratch[(e * H + h) * 2] - row_s[h]) * scratch[(e * H + h) * 2 + 1];
             }
         }
+#pragma unroll 2
         for (int j = 0; j < n; j++) {
             const float *row = kv + (int64_t)(c0 + j) * 2 * O;
             float *drow = dkv + (int64_t)(c0 + j) * 2 * O;
@@ -532,19 +557,97 @@ __global__ __launch_bounds__(kBlock) void tattn_finalize_kernel(
     }
 }
 
-// out_x[c] = sum over the n_x rows of partial_x[., c], rows in ascending order; two
-// tables in one launch (x = a for the first blocks_a workgroups).
+// Column sums of a table of partial rows, 64 columns per workgroup: wave w adds the rows
+// w, w + 4, ... (four independent chains, so the loads overlap), the four waves' sums are
+// added in wave order. The order of additions is fixed by the table's height alone.
+__device__ __forceinline__ void column_sums_block(float *__restrict__ out,
+                                                  const float *__restrict__ part, int n, int cols,
+                                                  int block) {
+    __shared__ float fold[kWavesPerBlock][kWave];
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int c = block * kWave + lane;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (c < cols) {
+        int r = wave;
+        for (; r + 3 * kWavesPerBlock < n; r += 4 * kWavesPerBlock) {
+            s0 += part[(int64_t)r * cols + c];
+            s1 += part[(int64_t)(r + kWavesPerBlock) * cols + c];
+            s2 += part[(int64_t)(r + 2 * kWavesPerBlock) * cols + c];
+            s3 += part[(int64_t)(r + 3 * kWavesPerBlock) * cols + c];
+        }
+        for (; r < n; r += kWavesPerBlock) s0 += part[(int64_t)r * cols + c];
+    }
+    fold[wave][lane] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (wave == 0 && c < cols) out[c] = (fold[0][lane] + fold[1][lane]) + (fold[2][lane] + fold[3][lane]);
+}
+
+// out_x[c] = sum over the n_x rows of partial_x[., c]; two tables in one launch (x = a for
+// the first blocks_a workgroups).
 __global__ __launch_bounds__(kBlock) void partial_sums_kernel(
     float *__restrict__ out_a, const float *__restrict__ part_a, int n_a, int cols_a, int blocks_a,
     float *__restrict__ out_b, const float *__restrict__ part_b, int n_b, int cols_b) {
-    const bool first = (int)blockIdx.x < blocks_a;
-    const int c = (first ? blockIdx.x : blockIdx.x - blocks_a) * kBlock + threadIdx.x;
-    const int cols = first ? cols_a : cols_b, n = first ? n_a : n_b;
-    const float *part = first ? part_a : part_b;
-    if (c >= cols) return;
-    float s = 0.0f;
-    for (int r = 0; r < n; r++) s += part[(int64_t)r * cols + c];
-    (first ? out_a : out_b)[c] = s;
+    if ((int)blockIdx.x < blocks_a)
+        column_sums_block(out_a, part_a, n_a, cols_a, blockIdx.x);
+    else
+        column_sums_block(out_b, part_b, n_b, cols_b, blockIdx.x - blocks_a);
+}
+
+struct CollectArgs {
+    float *out_ln, *out_time;
+    const float *part_ln, *part_t;
+    int rows_ln, rows_t;
+    float *g_wq, *g_bq, *g_wk, *g_bk, *g_wv, *g_bv, *g_wo, *g_bo;
+    const float *dw_kv, *dw_q, *dw_r;
+};
+
+// The last launch of the backward: the two tables of partial sums (LayerNorm affine,
+// time encoder) and the weight gradients out of their bias-augmented rows into one
+// contiguous tensor per parameter (one wave per row).
+__global__ __launch_bounds__(kBlock) void tattn_collect_kernel(TattnDims d, CollectArgs a,
+                                                               int blocks_ln, int blocks_t) {
+    int block = blockIdx.x;
+    if (block < blocks_ln) {
+        column_sums_block(a.out_ln, a.part_ln, a.rows_ln, 2 * d.O, block);
+        return;
+    }
+    block -= blocks_ln;
+    if (block < blocks_t) {
+        column_sums_block(a.out_time, a.part_t, a.rows_t, 2 * d.Dt, block);
+        return;
+    }
+    block -= blocks_t;
+    const int lane = lane_id();
+    const int O = d.O, LD = d.LD;
+    const int Dkv = d.Dn + d.De + d.Dt, Dq = d.Dn + d.Dt, Dr = O + d.Dn;
+    int r = block * kWavesPerBlock + threadIdx.x / kWave;
+    const float *src;
+    float *w, *bias;
+    int width;
+    if (r < 2 * O) {
+        const bool is_k = r < O;
+        src = a.dw_kv + (int64_t)r * LD;
+        r = is_k ? r : r - O;
+        w = (is_k ? a.g_wk : a.g_wv) + (int64_t)r * Dkv;
+        bias = (is_k ? a.g_bk : a.g_bv) + r;
+        width = Dkv;
+    } else if (r < 3 * O) {
+        r -= 2 * O;
+        src = a.dw_q + (int64_t)r * LD;
+        w = a.g_wq + (int64_t)r * Dq;
+        bias = a.g_bq + r;
+        width = Dq;
+    } else if (r < 4 * O) {
+        r -= 3 * O;
+        src = a.dw_r + (int64_t)r * LD;
+        w = a.g_wo + (int64_t)r * Dr;
+        bias = a.g_bo + r;
+        width = Dr;
+    } else {
+        return;
+    }
+    for (int c = lane; c < width; c += kWave) w[c] = src[c];
+    if (lane == 0) *bias = src[LD - 1];
 }
 
 int check_dims(TattnDims &d, int64_t n_dst, int64_t n_edges, int64_t dim_node, int64_t dim_edge,
@@ -696,11 +799,40 @@ YITU_API int yitu_partial_sums(float *out_a, const float *partial_a, int64_t row
     YITU_REQUIRE((cols_a == 0 || (out_a && (rows_a == 0 || partial_a))) &&
                      (cols_b == 0 || (out_b && (rows_b == 0 || partial_b))),
                  "null operand");
-    const int blocks_a = (int)ceil_div(cols_a, kBlock), blocks_b = (int)ceil_div(cols_b, kBlock);
+    const int blocks_a = (int)ceil_div(cols_a, kWave), blocks_b = (int)ceil_div(cols_b, kWave);
     if (blocks_a + blocks_b == 0) return 0;
     partial_sums_kernel<<<blocks_a + blocks_b, kBlock, 0, static_cast<hipStream_t>(stream)>>>(
         out_a, partial_a, (int)rows_a, (int)cols_a, blocks_a, out_b, partial_b, (int)rows_b,
         (int)cols_b);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+YITU_API int yitu_tattn_collect(float *grad_ln, float *grad_time, float *grad_w_q, float *grad_b_q,
+                                float *grad_w_k, float *grad_b_k, float *grad_w_v, float *grad_b_v,
+                                float *grad_w_out, float *grad_b_out, const float *partial_ln,
+                                int64_t rows_ln, const float *partial_time, int64_t rows_time,
+                                const float *dw_kv, const float *dw_q, const float *dw_r,
+                                int64_t dim_node, int64_t dim_edge, int64_t dim_time,
+                                int64_t dim_out, int64_t ld, void *stream) {
+    TattnDims d;
+    if (int rc = check_dims(d, 0, 0, dim_node, dim_edge, dim_time, dim_out, 1, ld)) return rc;
+    YITU_REQUIRE(rows_ln >= 0 && rows_time >= 0 && rows_ln < INT32_MAX && rows_time < INT32_MAX,
+                 "size out of range");
+    YITU_REQUIRE(grad_ln && (rows_ln == 0 || partial_ln) &&
+                     (dim_time == 0 || (grad_time && (rows_time == 0 || partial_time))),
+                 "null partial table");
+    YITU_REQUIRE(grad_w_q && grad_b_q && grad_w_k && grad_b_k && grad_w_v && grad_b_v &&
+                     grad_w_out && grad_b_out && dw_kv && dw_q && dw_r,
+                 "null gradient");
+    CollectArgs a{grad_ln, grad_time, partial_ln, partial_time, (int)rows_ln, (int)rows_time,
+                  grad_w_q, grad_b_q, grad_w_k, grad_b_k, grad_w_v, grad_b_v, grad_w_out,
+                  grad_b_out, dw_kv, dw_q, dw_r};
+    const int blocks_ln = (int)ceil_div(2 * dim_out, kWave);
+    const int blocks_t = (int)ceil_div(2 * dim_time, kWave);
+    const int blocks_w = (int)ceil_div(4 * dim_out, kWavesPerBlock);
+    tattn_collect_kernel<<<blocks_ln + blocks_t + blocks_w, kBlock, 0,
+                           static_cast<hipStream_t>(stream)>>>(d, a, blocks_ln, blocks_t);
     YITU_LAUNCH_CHECK();
     return 0;
 }

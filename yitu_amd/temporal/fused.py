@@ -126,14 +126,17 @@ class TemporalAttentionFunction(torch.autograd.Function):
         rows_t = int(L.yitu_tattn_partial_rows(c_i64(B + E)))
         grad_out = grad_out.contiguous()
         shapes = ((B, 2 * O), (B, LD), (B, 2 * O), (E, 2 * O), (E, H, 2), (E, LD), (B, LD),
-                  (rows_ln, 2 * O), (rows_t, 2 * max(Dt, 1)))
+                  (rows_ln, 2 * O), (rows_t, 2 * max(Dt, 1)), (2 * O, LD), (O, LD), (O, LD))
         buf = torch.empty(_room(*shapes), dtype=torch.float32, device=dev)
-        d_pre2, dx_r, dq2, dkv, scratch, dx_kv, dx_q, part_ln, part_t = _carve(buf, *shapes)
-        # parameter gradients: [w_k | b_k ; w_v | b_v], [w_q | b_q], [w_out | b_out], then the
-        # LayerNorm's (gamma, beta) and the time encoder's (frequency, phase)
-        gshapes = ((2 * O, LD), (O, LD), (O, LD), (2, O), (2, max(Dt, 1)))
+        (d_pre2, dx_r, dq2, dkv, scratch, dx_kv, dx_q, part_ln, part_t, dw_kv, dw_q,
+         dw_r) = _carve(buf, *shapes)
+        # weight gradients with the bias gradient as their last column: [w_k | b_k ; w_v | b_v],
+        # [w_q | b_q], [w_out | b_out]; the last launch unpacks them into one tensor per parameter
+        Dkv, Dq, Dr = Dn + De + Dt, Dn + Dt, O + Dn
+        gshapes = ((O, Dq), (O,), (O, Dkv), (O,), (O, Dkv), (O,), (O, Dr), (O,), (2, O),
+                   (2, max(Dt, 1)))
         gbuf = torch.empty(_room(*gshapes), dtype=torch.float32, device=dev)
-        dw_kv, dw_q, dw_r, d_ln, d_time = _carve(gbuf, *gshapes)
+        g_wq, g_bq, g_wk, g_bk, g_wv, g_bv, g_wo, g_bo, d_ln, d_time = _carve(gbuf, *gshapes)
         need_h = Dn > 0 and ctx.needs_input_grad[4]
         need_f = De > 0 and ctx.needs_input_grad[5]
         grad_h = torch.empty((B + E, Dn), dtype=torch.float32, device=dev) if need_h else None
@@ -164,13 +167,12 @@ class TemporalAttentionFunction(torch.autograd.Function):
                                         ptr(dx_r), ptr(dt), ptr(time_w), ptr(time_b), c_i64(B),
                                         c_i64(E), c_i64(Dn), c_i64(De), c_i64(Dt), c_i64(O),
                                         c_i64(LD), stream), "yitu_tattn_finalize")
-            check(L.yitu_partial_sums(ptr(d_ln), ptr(part_ln), c_i64(rows_ln), c_i64(2 * O),
-                                      ptr(d_time), ptr(part_t), c_i64(rows_t), c_i64(2 * Dt), stream),
-                  "yitu_partial_sums")
-        Dkv, Dq, Dr = Dn + De + Dt, Dn + Dt, O + Dn
+            check(L.yitu_tattn_collect(
+                ptr(d_ln), ptr(d_time), ptr(g_wq), ptr(g_bq), ptr(g_wk), ptr(g_bk), ptr(g_wv),
+                ptr(g_bv), ptr(g_wo), ptr(g_bo), ptr(part_ln), c_i64(rows_ln), ptr(part_t),
+                c_i64(rows_t), ptr(dw_kv), ptr(dw_q), ptr(dw_r), c_i64(Dn), c_i64(De), c_i64(Dt),
+                c_i64(O), c_i64(LD), stream), "yitu_tattn_collect")
         g_time_w = d_time[0, :Dt].reshape(Dt, 1) if Dt > 0 else None
         g_time_b = d_time[1, :Dt] if Dt > 0 else None
         return (None, None, None, None, grad_h, grad_f, None, g_time_w, g_time_b,
-                dw_q[:, :Dq], dw_q[:, LD - 1], dw_kv[:O, :Dkv], dw_kv[:O, LD - 1],
-                dw_kv[O:, :Dkv], dw_kv[O:, LD - 1], dw_r[:, :Dr], dw_r[:, LD - 1],
-                d_ln[0], d_ln[1])
+                g_wq, g_bq, g_wk, g_bk, g_wv, g_bv, g_wo, g_bo, d_ln[0], d_ln[1])
