@@ -384,6 +384,39 @@ int yitu_hfused_forward(float *spmm_out_device, float *attn_device, const float 
                         void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
+ * hfused_backward (entry.cpp:157-182; hfused_cuda.cu:47-94, unreachable in the
+ * reference: sparse.py:109-110, and indexing heads by the wrong thread
+ * coordinate, :59,186): the backward of both ops in TWO launches shared by the
+ * two graphs. First the per-row passes (per-edge dot products of A -> grad_values
+ * [nnz_a,H]; softmax backward of B -> grad_query [n_bid,n_rows,H] and the per-edge
+ * logit gradient grad_edge [nnz_b,H], a scratch output), then the two by-source
+ * gathers (grad_features [n_src_a,H,F] over A's by-source structure; grad_key
+ * [n_src_b,H] = sums of grad_edge over B's). No atomics. That holds when all four
+ * longest rows (A, A by source, B, B by source) are known and below the long-row
+ * thresholds (64; B by destination: 512), n_heads <= 16, n_features a multiple of
+ * 4, n_heads * n_features <= 1024; any other case runs yitu_spmm_backward and
+ * yitu_sddmm_backward. Both by-source structures come from yitu_csr_transpose.
+ */
+size_t yitu_hfused_backward_workspace_bytes(int64_t n_rows, int64_t n_src_a, int64_t nnz_a,
+                                            int64_t row_len, int64_t n_src_b, int64_t nnz_b,
+                                            int64_t n_heads, int64_t n_bid);
+int yitu_hfused_backward(float *grad_values_device, float *grad_features_device,
+                         float *grad_query_device, float *grad_key_device, float *grad_edge_device,
+                         const float *spmm_values_device, const int32_t *spmm_indptr_device,
+                         const int32_t *spmm_indices_device, const float *spmm_features_device,
+                         const float *spmm_grad_device, const int32_t *spmm_t_indptr_device,
+                         const int32_t *spmm_t_rows_device, const int32_t *spmm_t_perm_device,
+                         const int32_t *sddmm_indptr_device, const int32_t *sddmm_indices_device,
+                         const float *sddmm_query_device, const float *sddmm_key_device,
+                         const float *sddmm_attn_device, const float *sddmm_grad_device,
+                         const int32_t *sddmm_t_indptr_device, const int32_t *sddmm_t_perm_device,
+                         int64_t n_rows, int64_t n_src_a, int64_t nnz_a, int64_t n_heads,
+                         int64_t n_features, int64_t n_src_b, int64_t nnz_b, int64_t n_bid,
+                         int64_t max_degree_a, int64_t max_degree_a_t, int64_t max_degree_b,
+                         int64_t max_degree_b_t, void *workspace_device, size_t workspace_bytes,
+                         void *stream);
+
+/*
  * b2gemm (entry.cpp:56-64; fc_cuda.cu:4-75): y_a = x . w_a^T, y_b = x . w_b^T
  * as one grouped launch. x [n,k], w_* [m,k], y_* [n,m], contiguous.
  */

@@ -317,6 +317,45 @@ def test_hfused_forward_against_the_oracle_ops(dev, n_dst, n_src, h, f, n_bid, l
     assert_close(attn, want_attn, what="sddmm part")
 
 
+@pytest.mark.parametrize("n_dst,n_src,h,f,n_bid,long_rows", [
+    (4096, 2048, 8, 4, 1, False), (300, 500, 1, 4, 1, False), (1000, 700, 3, 16, 2, False),
+    (513, 129, 16, 64, 5, False), (64, 64, 4, 256, 1, False), (2000, 900, 4, 8, 1, True),
+    (400, 300, 2, 6, 1, False), (400, 300, 20, 4, 1, False)])
+def test_hfused_backward_against_the_oracle_ops(dev, n_dst, n_src, h, f, n_bid, long_rows):
+    """The backward of both ops in two shared launches (per-row passes, then by-source
+    gathers), and its fallback to the two ops, against the oracle's spmm / sddmm backward
+    functions (spmm_cuda.cu:27-38, sddmm_cuda.cu:36-66); same bits on a second call."""
+    hubs = dict(hub_rows=(3,), hub_degree=600) if long_rows else {}
+    a_ptr, a_idx = random_csr(n_dst, n_src, 0.02, n_dst + 1, **hubs)
+    blocks = [random_csr(n_dst, n_src, 0.03, 10 * n_dst + b, empty_rows=(b,), **hubs)
+              for b in range(n_bid)]
+    if n_bid == 1:
+        b_ptr, b_idx, n_cols = blocks[0][0].numpy(), blocks[0][1].numpy(), n_src
+    else:
+        b_ptr, b_idx, n_cols = oracle.stitch_csr([(p_, i_, n_src) for p_, i_ in blocks])
+    g = torch.Generator().manual_seed(h + f)
+    vals = torch.randn(a_idx.numel(), h, generator=g)
+    x = torch.randn(n_src, h, f, generator=g)
+    gy = torch.randn(n_dst, h, f, generator=g)
+    q = torch.randn(n_bid, n_dst, h, generator=g)
+    k = torch.randn(n_cols, h, generator=g)
+    b_ptr_t, b_idx_t = torch.as_tensor(b_ptr), torch.as_tensor(b_idx)
+    attn = oracle.sddmm_forward(b_ptr, b_idx, q.numpy(), k.numpy())
+    gattn = torch.randn(b_idx_t.numel(), h, generator=g)
+    args = (vals.to(dev), a_ptr.to(dev), a_idx.to(dev), x.to(dev), gy.to(dev), b_ptr_t.to(dev),
+            b_idx_t.to(dev), q.to(dev), k.to(dev), torch.as_tensor(attn).to(dev), gattn.to(dev))
+    got = graph_ext.hfused_backward(*args)
+    want_ga, want_gx = oracle.mh_spmm_backward(vals, a_ptr, a_idx, x.numpy(), gy.numpy())
+    want_gq, want_gk = oracle.sddmm_backward(b_ptr, b_idx, q.numpy(), k.numpy(), attn, gattn.numpy())
+    abs_ga = oracle.mh_spmm_backward(vals.abs(), a_ptr, a_idx, x.abs().numpy(), gy.abs().numpy())
+    assert_close(got[0], want_ga, abs_sum=abs_ga[0], what="grad of the SpMM's edge values")
+    assert_close(got[1], want_gx, abs_sum=abs_ga[1], what="grad of the SpMM's features")
+    assert_close(got[2], want_gq, atol=2e-4, what="grad_query")
+    assert_close(got[3], want_gk, atol=2e-4, what="grad_key")
+    again = graph_ext.hfused_backward(*args)
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+
+
 def test_dtype_and_device_checks(dev):
     indptr, indices = random_csr(10, 10, 0.3, 0)
     v = torch.randn(indices.numel(), 2)

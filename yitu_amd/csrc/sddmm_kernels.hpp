@@ -343,8 +343,8 @@ __device__ __forceinline__ void bwd_apply(const SddmmParams &p, int e_beg, int e
 }
 
 template <int HP>
-__global__ __launch_bounds__(kBlock) void sddmm_bwd_rows_kernel(SddmmParams p) {
-    const int row = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+__device__ __forceinline__ void sddmm_bwd_rows_body(const SddmmParams &p, int block) {
+    const int row = block * kWavesPerBlock + threadIdx.x / kWave;
     if (row >= p.n_dst) return;
     const int beg = p.indptr[row], end = p.indptr[row + 1];
     if (end - beg < p.skip_below) return;
@@ -367,6 +367,11 @@ __global__ __launch_bounds__(kBlock) void sddmm_bwd_rows_kernel(SddmmParams p) {
             bwd_apply<HP>(p, beg, end, b, h, act_h, qv, r.s);
         }
     }
+}
+
+template <int HP>
+__global__ __launch_bounds__(kBlock) void sddmm_bwd_rows_kernel(SddmmParams p) {
+    sddmm_bwd_rows_body<HP>(p, blockIdx.x);
 }
 
 template <int HP>

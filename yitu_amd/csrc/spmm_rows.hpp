@@ -496,10 +496,10 @@ __device__ __forceinline__ void tiny_sum(float (&acc)[VEC], const TinyWindow<VEC
 }
 
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
+__device__ __forceinline__ void tiny_rows_body(const SpmmParams &p, int block) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (block * kWavesPerBlock + threadIdx.x / kWave) * rpw;
     if (r0 >= p.n_rows) return;
     const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
@@ -526,6 +526,11 @@ __global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
             store_row<VEC>(p.out + (size_t)(r0 + i) * VEC, acc);
         }
     }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
+    tiny_rows_body<VEC>(p, blockIdx.x);
 }
 
 template <int VEC>

@@ -378,15 +378,53 @@ def hfused_forward(spmm_values, spmm_indptr, spmm_indices, spmm_features, sddmm_
 
 def hfused_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad, sddmm_indptr,
                     sddmm_indices, sddmm_query, sddmm_key, sddmm_attn, sddmm_grad):
-    """Union of the two backward ops (entry.cpp:157-182) with the correct arithmetic:
-    returns [grad_a, grad_x, grad_query, grad_key]. Not one launch: both gradients
-    with respect to per-source tensors are gathers over a by-source structure of
-    their own graph (no atomics), which follow the per-row passes. The reference's
-    fused backward kernel is unreachable (sparse.py:109-110) and indexes heads by
-    threadIdx.x although they lie on threadIdx.y (hfused_cuda.cu:59,186)."""
-    grad_a, grad_x = spmm_backward(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad)
-    grad_q, grad_k = sddmm_backward(sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key, sddmm_attn,
-                                    sddmm_grad)
+    """The two backward ops (entry.cpp:157-182) with the correct arithmetic, returning
+    [grad_a, grad_x, grad_query, grad_key], in two launches shared by the two graphs: the
+    per-row passes of both, then both by-source gathers (no atomics). Graphs with long rows
+    run the two ops one after the other. The reference's fused backward kernel is
+    unreachable (sparse.py:109-110) and indexes heads by threadIdx.x although they lie on
+    threadIdx.y (hfused_cuda.cu:59,186)."""
+    if spmm_indptr.numel() != sddmm_indptr.numel():
+        raise RuntimeError("the two graphs must have the same number of rows")
+    _check(spmm_values, torch.float32, "spmm_values", 2)
+    _check(spmm_features, torch.float32, "spmm_features", 3)
+    _check(spmm_grad, torch.float32, "spmm_grad", 3)
+    _check(sddmm_attn, torch.float32, "sddmm_attn", 2)
+    _check(sddmm_grad, torch.float32, "sddmm_grad", 2)
+    n_rows, n_src_b, nnz_b, h, n_bid = _sddmm_shapes(sddmm_indptr, sddmm_indices, sddmm_query,
+                                                     sddmm_key)
+    dev = _lib.require_device(spmm_values, spmm_indptr, spmm_indices, spmm_features, spmm_grad,
+                              sddmm_indptr, sddmm_indices, sddmm_query, sddmm_key, sddmm_attn,
+                              sddmm_grad)
+    n_src_a, h_a, f = spmm_features.shape
+    nnz_a = spmm_indices.numel()
+    if h_a != h or spmm_values.shape != (nnz_a, h) or spmm_grad.shape != (n_rows, h, f):
+        raise RuntimeError("spmm_values must be [n_edges, H], spmm_grad [n_rows, H, F], with the "
+                           "SDDMM's H")
+    if sddmm_attn.shape != (nnz_b, h) or sddmm_grad.shape != (nnz_b, h):
+        raise RuntimeError("sddmm_attn and sddmm_grad must be [n_edges, H]")
+    ta = transposed(spmm_indptr, spmm_indices, n_src_a)
+    tb = transposed(sddmm_indptr, sddmm_indices, n_src_b)
+    grad_a = torch.empty_like(spmm_values)
+    grad_x = torch.empty_like(spmm_features)
+    grad_q = torch.empty_like(sddmm_query)
+    grad_k = torch.empty_like(sddmm_key)
+    grad_e = torch.empty_like(sddmm_attn)
+    ws = _lib.workspace(_size_fn("yitu_hfused_backward_workspace_bytes")(
+        c_i64(n_rows), c_i64(n_src_a), c_i64(nnz_a), c_i64(h * f), c_i64(n_src_b), c_i64(nnz_b),
+        c_i64(h), c_i64(n_bid)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_hfused_backward(
+            ptr(grad_a), ptr(grad_x), ptr(grad_q), ptr(grad_k), ptr(grad_e), ptr(spmm_values),
+            ptr(spmm_indptr), ptr(spmm_indices), ptr(spmm_features), ptr(spmm_grad.contiguous()),
+            ptr(ta.t_indptr), ptr(ta.t_rows), ptr(ta.t_perm), ptr(sddmm_indptr), ptr(sddmm_indices),
+            ptr(sddmm_query), ptr(sddmm_key), ptr(sddmm_attn), ptr(sddmm_grad.contiguous()),
+            ptr(tb.t_indptr), ptr(tb.t_perm), c_i64(n_rows), c_i64(n_src_a), c_i64(nnz_a), c_i64(h),
+            c_i64(f), c_i64(n_src_b), c_i64(nnz_b), c_i64(n_bid),
+            c_i64(_lib.max_degree(spmm_indptr)), c_i64(ta.max_degree_t),
+            c_i64(_lib.max_degree(sddmm_indptr)), c_i64(tb.max_degree_t), ptr(ws),
+            c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_hfused_backward")
     return [grad_a, grad_x, grad_q, grad_k]
 
 
