@@ -14,7 +14,8 @@ the timed region.
 
 Prints ONE JSON line on stdout. Other workloads (also carried in ``extra`` of the
 default run): ``--workload c3_spmm_bf16``, ``c2_gat_f32``, ``c1_gcn_f32``,
-``c4_rgcn_f32``, ``c5_temporal_attention_f32``, ``c3_vertex_orders``.
+``c4_rgcn_f32``, ``c5_temporal_attention_f32``, ``c3_vertex_orders``,
+``planted_partition_orders``, ``small_hetero_models``.
 """
 import argparse
 import json
@@ -645,6 +646,65 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
     return res
 
 
+def run_small_hetero(args, dev):
+    """The scale the reference's own benchmark runs at (README.md:273-286, 344-353: AIFB,
+    7,262 nodes, 48,810 edges, 104 relations, d_hidden = 32; bench_macro.py:371-391:
+    throughput = edges / mean time of forward + backward): a synthetic heterogeneous graph
+    of that shape (7 node types, 104 uniform-random relations), the reference's 2-layer
+    RGCN and RGAT models captured and lowered, executed relation by relation and after the
+    stitcher has joined the relations of each destination type."""
+    from yitu_amd import xgnn_h
+    from yitu_amd.data import graphgen
+    from yitu_amd.xgnn_h import block as xblock, layers as xl, models, mp
+    counts = [2800, 1500, 1200, 800, 500, 300, 162]
+    ntypes = {"n%d" % i: c for i, c in enumerate(counts)}
+    names = list(ntypes)
+    gen = torch.Generator().manual_seed(20246)
+    blocks = {}
+    for r in range(104):
+        s_t, d_t = (int(v) for v in torch.randint(0, 7, (2,), generator=gen))
+        n_dst, n_src = counts[d_t], counts[s_t]
+        rp, ci = graphgen.bipartite_uniform(n_dst, n_src, 48810 / 104 / n_dst, 20246 + r)
+        b = xblock.Block([n_dst, n_src], [rp.to(dev), ci.to(dev)])
+        b.right_norm = xl.right_norm(b)
+        blocks[(names[s_t], "r%d" % r, names[d_t])] = b
+    n_edges = sum(b.num_edges() for b in blocks.values())
+    hg = mp.HeteroGraph.from_blocks(ntypes, blocks, device=dev)
+    xs = {n: torch.arange(c, device=dev) for n, c in ntypes.items()}
+    steps, warm = max(args.steps, 20), max(args.warmup, 3)
+    res = {"n_nodes": sum(counts), "n_edges": n_edges, "relations": len(blocks), "hidden": 32}
+    for tag, make, kwargs in (
+            ("rgcn", lambda: models.RGCNModel(hg, 32, 32, 32),
+             {"hgraph": hg, "xs": xs,
+              "norms": {str(rel): gr.right_norm() for rel, gr in hg.hetero_graph.items()}}),
+            ("rgat", lambda: models.RGATModel(hg, 32, 32, 32, n_heads=2), {"hgraph": hg, "xs": xs})):
+        torch.manual_seed(7)
+        model = make().to(dev)
+        lowered = xgnn_h.Optimizer().lower(xgnn_h.Module2IR().transform(model, kwargs), kwargs)
+        stitched = xgnn_h.Stitcher().transform(lowered, kwargs)
+        executor = xgnn_h.Executor()
+        executor.train()
+        gy = None
+
+        def step(flow):
+            def run():
+                nonlocal gy
+                out = executor.run(flow, kwargs)
+                if gy is None:
+                    gy = {n: torch.randn_like(t) for n, t in out.items()}
+                torch.autograd.backward([out[n] for n in out], [gy[n] for n in out])
+                model.zero_grad(set_to_none=True)
+            return run
+
+        for form, flow in (("lowered", lowered), ("stitched", stitched)):
+            ms = _event_ms(step(flow), steps, warm)
+            res["%s_%s_fwd_bwd_ms" % (tag, form)] = ms
+            res["%s_%s_edges_per_s" % (tag, form)] = n_edges / (ms * 1e-3)
+            res["%s_%s_sparse_ops" % (tag, form)] = sum(
+                1 for n in xgnn_h.ir.walk(flow) if n.op in ("spmm", "gat", "sddmm"))
+    return res
+
+
 def run_c5(args, dev):
     """Fifth configuration: temporal neighbour attention. 2^20 events over 2^17
     nodes (Zipf 1.2 endpoints, sorted uniform times), T-CSR with reverse edges;
@@ -924,6 +984,8 @@ def main():
         res = run_c5(args, dev)
     elif args.workload == "c3_vertex_orders":
         res = run_c3_orders(args, dev)
+    elif args.workload == "small_hetero_models":
+        res = run_small_hetero(args, dev)
     elif args.workload == "planted_partition_orders":
         res = run_planted_orders(args, dev)
     else:

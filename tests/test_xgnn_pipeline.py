@@ -184,6 +184,11 @@ def test_stitching_replaces_sums_of_relations(which):
     # layer 2 reads all three types of layer 1: one stitched term per destination type
     # with several relations (paper: 4 -> 1, author: 2 -> 1), venue keeps its single one
     assert ops["spmm"] + ops["gat"] == 1 + 3
+    if which == "rgat":
+        # without the fused op the stitched terms keep the two-op form
+        plain = xgnn_h.Optimizer(fuse_gat=False).lower(root, kwargs)
+        two_op = cases.ops_of(xgnn_h.Stitcher().transform(plain, dict(kwargs)))
+        assert two_op["gat"] == 0 and two_op["sddmm"] == two_op["spmm"] == 1 + 3
     if which == "rgcn":
         # the relations' Linears feed nothing else: one typed Linear per stitched term
         # writes the feature rows, nothing is concatenated
@@ -192,7 +197,9 @@ def test_stitching_replaces_sums_of_relations(which):
     else:
         # the transformed features are also read by the projections: they stay as they are
         assert ops["concat"] >= 3 and ops["typed_linear"] == 0
-        assert ops["sddmm"] == 3 and ops["stack"] == 3 and ops["gat"] == 1
+        # the relations ran the fused attention op, so do the stitched terms (one query
+        # block per relation)
+        assert ops["sddmm"] == 0 and ops["stack"] == 3 and ops["gat"] == 1 + 3
     new = kwargs["stitch"]
     assert isinstance(new, mp.HeteroGraph) and len(new.hetero_graph) == 2
     (sty, ety, dty), g = next(iter(new))

@@ -18,6 +18,30 @@ class Block:
             self.right_norm = self.right_norm.to(device)
         return self
 
+    def by_query_block(self, n_blocks: int):
+        """A stitched block seen as ``n_dst * n_blocks`` rows: row ``r * n_blocks + b`` holds
+        the edges of destination ``r`` that carry block tag ``b`` (they are contiguous: a
+        stitched row is sorted by tag, then column). Same ``indices`` tensor, so per-graph
+        state derived from it is shared. A softmax per (destination, block), which is what a
+        stitched attention term asks for, is a plain per-row softmax over this view. Built
+        once per block and kept."""
+        kept = getattr(self, "_by_query_block", None)
+        if kept is None or kept[0] != n_blocks or kept[2] is not self.adj_sparse[1]:
+            indptr, indices = self.adj_sparse
+            n_dst = indptr.numel() - 1
+            deg = (indptr[1:] - indptr[:-1]).to(torch.int64)
+            rows = torch.repeat_interleave(torch.arange(n_dst, device=indptr.device), deg)
+            key = rows * n_blocks + (indices.to(torch.int64) >> 24)
+            if key.numel() > 1:
+                assert bool((key[1:] >= key[:-1]).all()), "rows must be sorted by block tag"
+            counts = torch.bincount(key, minlength=n_dst * n_blocks)
+            v_indptr = torch.zeros(n_dst * n_blocks + 1, dtype=torch.int32, device=indptr.device)
+            v_indptr[1:] = torch.cumsum(counts, 0)
+            view = Block([n_dst * n_blocks, self.size[1]], [v_indptr, indices])
+            kept = (n_blocks, view, indices)
+            self._by_query_block = kept
+        return kept[1]
+
     def num_edges(self):
         indices = self.adj_sparse[1]
         assert indices.dim() == 1

@@ -141,9 +141,25 @@ class FusedGATFunction(autograd.Function):
 def fused_gat(block: block.Block, query: torch.Tensor, key: torch.Tensor, x: torch.Tensor,
               head_mean: bool = False):
     """query [n_dst, H], key [n_src, H], x [n_src, H, F] -> [n_dst, H, F], or
-    [n_dst, F] (the mean over heads) with ``head_mean``."""
-    assert x.dim() == 3 and query.dim() == 2 and key.dim() == 2
-    return FusedGATFunction.apply(block.adj_sparse, query, key, x, head_mean)
+    [n_dst, F] (the mean over heads) with ``head_mean``.
+
+    For a stitched block query is [n_blocks, n_dst, H] and the softmax runs per
+    (destination, block tag) like ``fused_gsddmm``'s (sddmm_cuda.cu:11-31): the block is
+    taken as ``n_dst * n_blocks`` rows, one per (destination, tag), the fused op runs on
+    that view, and the rows of a destination are added up. The tagged rows cost
+    ``n_blocks`` output rows per destination instead of one; the attention itself, one
+    pass over the edges forward and one backward, is the fused op's."""
+    assert x.dim() == 3 and key.dim() == 2
+    if query.dim() == 3 and query.size(0) == 1:
+        query = query[0]
+    if query.dim() == 2:
+        return FusedGATFunction.apply(block.adj_sparse, query, key, x, head_mean)
+    n_blocks, n_dst = query.size(0), query.size(1)
+    view = block.by_query_block(n_blocks)
+    per_tag = FusedGATFunction.apply(view.adj_sparse,
+                                     query.permute(1, 0, 2).reshape(n_dst * n_blocks, -1), key, x,
+                                     head_mean)
+    return per_tag.view(n_dst, n_blocks, *per_tag.shape[1:]).sum(dim=1)
 
 
 class GATHeadsFunction(autograd.Function):

@@ -175,6 +175,16 @@ class Stitcher:
                         size=[len(qs)] + qs[0].size)
             k = ir.Node("concat", {str(i): n for i, n in enumerate(ks)},
                         size=[new_blk.size[1]] + ks[0].size[1:])
+            if all(t.core.op == "gat" for t in terms):
+                # the relations ran the fused attention op: so does the stitched term, with
+                # one query block per relation (and the mean over heads inside, if they had it)
+                mean = terms[0].mean_inside
+                size = [new_blk.size[0]] + (xs[0].size[2:] if mean else xs[0].size[1:])
+                out = ir.Node("gat", {"g": g, "q": q, "k": k, "x": x}, {"head_mean": mean}, size)
+                if not mean and terms[0].post is not None:
+                    (slot,) = terms[0].post.inputs
+                    out = terms[0].post.with_inputs({slot: out})
+                return out
             inputs["e"] = ir.Node("sddmm", {"g": g, "q": q, "k": k}, size=[n_edges, ks[0].size[1]])
         elif terms[0].scale is not None:
             scales = {str(i): t.scale for i, t in enumerate(terms)}
