@@ -606,6 +606,22 @@ int yitu_coo_to_csr(int32_t *indptr_device, int32_t *indices_device, long long *
                     void *stream);
 
 /*
+ * build_part on the device (ccsrc/kernel/YiTu_GNN.cpp:203-245, which walks the rows on
+ * the host): neighbour group p covers edges [part_ptr[p], part_ptr[p+1]) of row
+ * part2node[p], at most part_size of them; row r has ceil(deg_r / part_size) groups.
+ * Same integers as the reference's arrays, including part_ptr[n_parts], which is the
+ * number of edges only when the last row has edges and 0 otherwise (cpp:240-241).
+ * part_ptr has room for capacity + 1 entries, part2node for capacity;
+ * capacity >= nnz / part_size + n_rows always suffices. *n_parts (device int64) receives
+ * the number of groups; entries beyond the capacity are not written.
+ */
+size_t yitu_build_part_workspace_bytes(int64_t n_rows);
+int yitu_build_part(int32_t *part_ptr_device, int32_t *part2node_device,
+                    long long *n_parts_device, const int32_t *indptr_device, int64_t n_rows,
+                    int64_t part_size, int64_t capacity, void *workspace_device,
+                    size_t workspace_bytes, void *stream);
+
+/*
  * By-source (transposed) view of a CSR, built once per graph on the device.
  * The reference has no such step: its backward kernels scatter with atomics
  * (spmm_cuda.cu:33-38, sddmm_cuda.cu:59-63); this turns those scatters into

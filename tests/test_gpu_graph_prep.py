@@ -105,3 +105,30 @@ def test_forget_after_a_raw_pointer_refill(dev):
     # the plan built on the side stream, used from the default stream
     got_b2 = graph_ext.spmm_forward(values.to(dev), indptr, indices, x.to(dev))
     assert torch.equal(got_b2, got_b)
+
+
+@pytest.mark.parametrize("ps", [1, 7, 32, 64, 1000])
+@pytest.mark.parametrize("last_empty", [False, True])
+def test_build_part_on_the_device(dev, ps, last_empty):
+    """build_part (YiTu_GNN.cpp:203-245) built on the GPU from a device indptr: the same
+    integers as the oracle's restatement of the reference loop, including the sentinel that
+    stays 0 behind an empty last row; hub rows of several waves' worth of groups, empty rows."""
+    import oracle
+    from helpers import random_csr
+    from yitu_amd import YiTu_GNN_kernel as K
+    indptr, _ = random_csr(3000, 3000, 0.004, ps, hub_rows=(5, 2998), hub_degree=2500,
+                           empty_rows=(0, 17) + ((2999,) if last_empty else ()))
+    if not last_empty:
+        assert indptr[-1] > indptr[-2]
+    pp, p2n = K.build_part(ps, indptr.to(dev))
+    want_pp, want_p2n = oracle.build_part(ps, indptr.numpy())
+    assert pp.is_cuda and pp.dtype == torch.int32 and p2n.dtype == torch.int32
+    assert np.array_equal(pp.cpu().numpy(), want_pp) and np.array_equal(p2n.cpu().numpy(), want_p2n)
+
+
+def test_build_part_on_the_device_empty_graph(dev):
+    from yitu_amd import YiTu_GNN_kernel as K
+    pp, p2n = K.build_part(8, torch.zeros(5, dtype=torch.int32, device=dev))
+    assert pp.tolist() == [0] and p2n.numel() == 0
+    pp, p2n = K.build_part(8, torch.zeros(1, dtype=torch.int32, device=dev))
+    assert pp.tolist() == [0] and p2n.numel() == 0

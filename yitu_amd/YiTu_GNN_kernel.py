@@ -145,14 +145,38 @@ def backward_gin(d_output, X, W, row_pointers, column_index, epsilon, part_point
     return [_aggregate(g, row_pointers, column_index, None, float(epsilon)), d_weight]
 
 
+def _build_part_device(part_size, indptr):
+    _lib.require_dtype(indptr, torch.int32, "indptr")
+    if part_size <= 0:
+        raise RuntimeError("partSize must be positive")
+    dev = indptr.device
+    indptr = indptr.contiguous()
+    n_rows = indptr.numel() - 1
+    nnz = int(indptr[-1].item()) if n_rows > 0 else 0
+    capacity = nnz // part_size + n_rows
+    part_ptr = torch.zeros(capacity + 1, dtype=torch.int32, device=dev)
+    part2node = torch.empty(capacity, dtype=torch.int32, device=dev)
+    n_parts = torch.zeros(1, dtype=torch.int64, device=dev)
+    ws = _lib.workspace(_lib.size_fn("yitu_build_part_workspace_bytes")(c_i64(n_rows)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_build_part(ptr(part_ptr), ptr(part2node), ptr(n_parts), ptr(indptr),
+                                        c_i64(n_rows), c_i64(part_size), c_i64(capacity), ptr(ws),
+                                        c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_build_part")
+    n = int(n_parts.item())
+    return [part_ptr[:n + 1], part2node[:n]]
+
+
 def build_part(partSize, indptr):
     """Neighbour-group partition of a CSR (YiTu_GNN.cpp:203-245): group p covers
     edges [partPtr[p], partPtr[p+1]) of row part2Node[p], at most partSize of
-    them. ``indptr`` is a CPU int32 tensor; returns [partPtr, part2Node] (int32,
-    CPU). As in the reference the sentinel partPtr[P] is only written when the
-    last row is non-empty, otherwise it stays 0."""
+    them. ``indptr`` is an int32 tensor: on the CPU like the reference's
+    (accessor<int,1>), or on the GPU, where the partition is built by
+    ``yitu_build_part`` and stays there; returns [partPtr, part2Node] (int32, on
+    indptr's device). As in the reference the sentinel partPtr[P] is only written
+    when the last row is non-empty, otherwise it stays 0."""
     if indptr.is_cuda:
-        raise RuntimeError("build_part expects a CPU tensor (the reference uses accessor<int,1>)")
+        return _build_part_device(int(partSize), indptr)
     _lib.require_dtype(indptr, torch.int32, "indptr")
     partSize = int(partSize)
     if partSize <= 0:

@@ -7,6 +7,7 @@
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 #include <rocprim/device/device_select.hpp>
 
 #include "../../include/yitu_hip.h"
@@ -129,6 +130,52 @@ static size_t sort_temp_bytes(int64_t nnz, int bits) {
 
 }  // namespace yitu
 
+namespace yitu {
+namespace {
+
+// groups of row r = ceil(deg / part_size)
+__global__ __launch_bounds__(kBlock) void part_count_kernel(int32_t *__restrict__ count,
+                                                            const int32_t *__restrict__ indptr,
+                                                            int n_rows, int part_size) {
+    const int r = blockIdx.x * kBlock + threadIdx.x;
+    if (r < n_rows) count[r] = (indptr[r + 1] - indptr[r] + part_size - 1) / part_size;
+}
+
+// One wave per row: group g of row r starts at edge indptr[r] + g part_size. The entry
+// behind the last group is the number of edges when the last row has edges and 0
+// otherwise, as the reference leaves it (YiTu_GNN.cpp:240-241).
+__global__ __launch_bounds__(kBlock) void part_fill_kernel(
+    int32_t *__restrict__ part_ptr, int32_t *__restrict__ part2node, long long *__restrict__ n_parts,
+    const int32_t *__restrict__ first, const int32_t *__restrict__ count,
+    const int32_t *__restrict__ indptr, int n_rows, int part_size, long long capacity) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    if (r >= n_rows) return;
+    const int base = first[r], n = count[r], beg = indptr[r];
+    for (int g = lane; g < n; g += kWave) {
+        if (base + g < capacity) {
+            part_ptr[base + g] = beg + g * part_size;
+            part2node[base + g] = r;
+        }
+    }
+    if (r == n_rows - 1 && lane == 0) {
+        const long long total = (long long)base + n;
+        *n_parts = total;
+        if (total < capacity + 1) part_ptr[total] = n > 0 ? indptr[n_rows] : 0;
+    }
+}
+
+size_t part_scan_bytes(int64_t n_rows) {
+    size_t bytes = 0;
+    int32_t *p = nullptr;
+    (void)rocprim::exclusive_scan(nullptr, bytes, p, p, 0, (size_t)std::max<int64_t>(n_rows, 1),
+                                  rocprim::plus<int32_t>());
+    return bytes;
+}
+
+}  // namespace
+}  // namespace yitu
+
 using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
@@ -230,6 +277,48 @@ YITU_API int yitu_coo_to_csr(int32_t *indptr, int32_t *indices, long long *nnz_o
     // after unique, `keys` holds the distinct (row, col) pairs in ascending order
     coo_finish_kernel<<<grid, kBlock, 0, stream>>>(keys, n_unique, bad, indptr, indices, nnz_out,
                                                    (int32_t)n_rows, n_edges);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+YITU_API size_t yitu_build_part_workspace_bytes(int64_t n_rows) {
+    return 2 * align_up(sizeof(int32_t) * (size_t)std::max<int64_t>(n_rows, 1), 256) +
+           align_up(part_scan_bytes(n_rows), 256);
+}
+
+YITU_API int yitu_build_part(int32_t *part_ptr, int32_t *part2node, long long *n_parts_out,
+                             const int32_t *indptr, int64_t n_rows, int64_t part_size,
+                             int64_t capacity, void *workspace, size_t workspace_bytes,
+                             void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_rows >= 0 && n_rows < INT32_MAX, "row count out of range");
+    YITU_REQUIRE(part_size > 0 && part_size < INT32_MAX, "partSize must be positive");
+    YITU_REQUIRE(capacity >= 0 && part_ptr && n_parts_out && (capacity == 0 || part2node),
+                 "null output");
+    YITU_REQUIRE(indptr, "null indptr");
+    YITU_REQUIRE(workspace && workspace_bytes >= yitu_build_part_workspace_bytes(n_rows) &&
+                     (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
+                 "workspace too small or misaligned: need %zu bytes, 256-byte aligned",
+                 yitu_build_part_workspace_bytes(n_rows));
+    if (n_rows == 0) {
+        YITU_HIP(hipMemsetAsync(n_parts_out, 0, sizeof(long long), stream));
+        YITU_HIP(hipMemsetAsync(part_ptr, 0, sizeof(int32_t), stream));
+        return 0;
+    }
+    char *w = static_cast<char *>(workspace);
+    const size_t arr = align_up(sizeof(int32_t) * (size_t)n_rows, 256);
+    int32_t *count = reinterpret_cast<int32_t *>(w);
+    int32_t *first = reinterpret_cast<int32_t *>(w + arr);
+    void *temp = w + 2 * arr;
+    size_t temp_bytes = part_scan_bytes(n_rows);
+    part_count_kernel<<<(int)ceil_div(n_rows, kBlock), kBlock, 0, stream>>>(count, indptr,
+                                                                           (int)n_rows, (int)part_size);
+    YITU_LAUNCH_CHECK();
+    YITU_HIP(rocprim::exclusive_scan(temp, temp_bytes, count, first, 0, (size_t)n_rows,
+                                     rocprim::plus<int32_t>(), stream));
+    part_fill_kernel<<<(int)ceil_div(n_rows, kWavesPerBlock), kBlock, 0, stream>>>(
+        part_ptr, part2node, n_parts_out, first, count, indptr, (int)n_rows, (int)part_size,
+        (long long)capacity);
     YITU_LAUNCH_CHECK();
     return 0;
 }
