@@ -5,7 +5,7 @@
 // aggregate) process the items in this order, one wave per item: at any moment
 // the waves read one narrow band of the feature table, whose hot rows stay in
 // L2. On a power-law graph the same gathers in CSR order run at about half the
-// speed. Short rows are not in the plan; a wave of the row kernels walks 16 of
+// speed. Short rows are not in the plan; a wave of the row kernels walks 4 of
 // them in a row.
 //
 // Bands: the source ids are cut into bands of 2^17 consecutive ids (wider when
@@ -63,9 +63,10 @@ struct PlanView {
 // whose sampled edges are local (community structure with ids to match, as planted
 // or as a reorder leaves them) has its short rows walked XCD by XCD. Measured on two
 // graphs of 2^21 vertices and 62 M edges, fp32 rows of 128 floats: planted
-// communities of 512 (97 % local) 4.43 ms round robin, 2.69 ms XCD by XCD; an R-MAT
-// graph after the Rabbit-Order reorder (51 % local: its rows of one or two edges sit
-// next to their source, its hot sources are everybody's) 2.70 and 2.94 ms.
+// communities of 512 (97 % local) 4.43 ms round robin, 2.69 ms XCD by XCD (16 rows
+// per wave; 2.07 ms with 4); an R-MAT graph after the Rabbit-Order reorder (51 %
+// local: its rows of one or two edges sit next to their source, its hot sources are
+// everybody's) 2.70 and 2.94 ms.
 constexpr int kPlanInfoLocal = 2;
 constexpr int kPlanInfoSampled = 3;
 

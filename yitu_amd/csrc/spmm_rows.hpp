@@ -12,7 +12,7 @@
 //     in flight per wave;
 //   * slots are folded with a fixed butterfly and a row is written once:
 //     no atomics, bitwise reproducible;
-//   * rows below the plan threshold (64 edges): a wave walks 16 consecutive rows
+//   * rows below the plan threshold (64 edges): a wave walks 4 consecutive rows
 //     through a sliding window; longer rows: the row plan's items of at most 64
 //     edges in band order, four per wave, whose partial rows a third kernel adds
 //     in a fixed order.
@@ -190,12 +190,19 @@ __device__ __forceinline__ void fold_slots(float (&acc)[KT][VEC]) {
             for (int i = 0; i < VEC; i++) acc[t][i] += __shfl_xor(acc[t][i], o, kWave);
 }
 
-constexpr int kRowsPerWave = 16;  // most consecutive rows one wave of a row kernel handles
+constexpr int kRowsPerWave = 4;  // most consecutive rows one wave of a row kernel handles
 
-// Rows per wave of the row kernels: 16 where that still leaves several thousand
+// Rows per wave of the row kernels: 4 where that still leaves several thousand
 // waves, fewer on small graphs (one root per wave at 2,048 sampled roots), so a
 // small problem is spread over the chip instead of walked by a few waves. Host
 // (grid size) and device (row range of a wave) both derive it from n_rows.
+// Why not more: the rows that the resident waves of an XCD cover together are its
+// working set. With 16 rows per wave 1,024 resident waves span 16 k rows, and on a
+// graph whose rows share sources with their neighbours (communities of 512) the
+// sources of 32 communities (8 MB) do not fit the 4 MB L2; with 4 rows they do.
+// 2^21 vertices, 63 M edges, fp32 rows of 128 floats, per call: 16 / 8 / 4 / 2 / 1
+// rows per wave = 2.69 / 2.15 / 2.07 / 2.06 / 2.09 ms on planted communities,
+// 2.70 / 2.69 / 2.71 / 2.79 / 2.94 ms on a power-law graph without locality.
 __host__ __device__ inline int rows_per_wave(int n_rows) {
     const int r = n_rows / 4096;
     return r < 1 ? 1 : (r > kRowsPerWave ? kRowsPerWave : r);
