@@ -166,16 +166,23 @@ __device__ __forceinline__ void accumulate_window(float (&acc)[KT][VEC], const S
 #pragma unroll
                 for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
     }
-    // remaining steps one at a time
-    for (; s < n; s += SLOTS) {
-        float v[KT][VEC];
-        float w[KT];
-        gather_step<VEC, G, KT, WMODE, TIN>(v, w, p, feat, win, first, s, n, tl.off, tl.head,
-                                            tl.live);
+    // the remaining steps (fewer than UNROLL) as one more group: their gathers go out
+    // together as well, and the sums are added in the same order as one step at a time
+    if (s < n) {
+        float v[UNROLL][KT][VEC];
+        float w[UNROLL][KT];
 #pragma unroll
-        for (int t = 0; t < KT; t++)
+        for (int u = 0; u < UNROLL; u++)
+            if (s + u * SLOTS < n)  // wave-uniform
+                gather_step<VEC, G, KT, WMODE, TIN>(v[u], w[u], p, feat, win, first, s + u * SLOTS,
+                                                    n, tl.off, tl.head, tl.live);
 #pragma unroll
-            for (int i = 0; i < VEC; i++) acc[t][i] += w[t] * v[t][i];
+        for (int u = 0; u < UNROLL; u++)
+            if (s + u * SLOTS < n)
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
     }
 }
 
