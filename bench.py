@@ -702,6 +702,28 @@ def run_small_hetero(args, dev):
             res["%s_%s_edges_per_s" % (tag, form)] = n_edges / (ms * 1e-3)
             res["%s_%s_sparse_ops" % (tag, form)] = sum(
                 1 for n in xgnn_h.ir.walk(flow) if n.op in ("spmm", "gat", "sddmm"))
+        # the stitched step recorded into a HIP graph and replayed (dropout off, so that
+        # every replay can be checked against the eager step)
+        from yitu_amd.utils.replay import ReplayedStep
+        still = xgnn_h.Executor()
+        still.eval()
+        params = list(model.parameters())
+
+        def graph_step():
+            for p in params:
+                p.grad = None
+            out = still.run(stitched, kwargs)
+            torch.autograd.backward([out[n] for n in out], [gy[n] for n in out])
+            return [out[n] for n in out] + [p.grad for p in params if p.grad is not None]
+
+        try:
+            replayed = ReplayedStep(graph_step, rtol=1e-4, atol=1e-5)
+            ms = _event_ms(replayed.replay, steps, warm)
+            res["%s_stitched_replayed_ms" % tag] = ms
+            res["%s_stitched_replayed_edges_per_s" % tag] = n_edges / (ms * 1e-3)
+        except Exception as exc:
+            sys.stderr.write("HIP graph replay of the %s step not reported: %s\n" % (tag, exc))
+            res["%s_stitched_replayed_ms" % tag] = None
     return res
 
 
@@ -780,46 +802,24 @@ def run_c5(args, dev):
 
 
 def _c5_graph_ms(layer, blk, gout, steps):
-    """The same forward + backward captured once into a HIP graph and replayed (the step is
-    some forty small launches). Every replay is checked against the eager gradients; None
-    when capture is not possible or a replay differs."""
+    """The same forward + backward captured once into a HIP graph and replayed
+    (yitu_amd.utils.replay: every replay is checked against the eager gradients); None when
+    capture is not possible or a replay differs."""
+    from yitu_amd.utils.replay import ReplayedStep
+    params = [blk.h] + list(layer.parameters())
+
+    def run():
+        for p in params:
+            p.grad = None
+        layer(blk).backward(gout)
+        return [p.grad for p in params]
+
     try:
-        params = [blk.h] + list(layer.parameters())
-
-        def run():
-            for p in params:
-                p.grad = None
-            layer(blk).backward(gout)
-            return [p.grad for p in params]
-
-        want = [g.clone() for g in run()]
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                run()
-        torch.cuda.current_stream().wait_stream(side)
-        _sync()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            grads = run()
-        for _ in range(3):
-            for g in grads:
-                g.fill_(float("nan"))
-            graph.replay()
-            _sync()
-            bad = [i for i, (g, w) in enumerate(zip(grads, want))
-                   if not torch.allclose(g, w, rtol=1e-5, atol=1e-6)]
-            if bad:
-                sys.stderr.write("HIP graph replay of the temporal step differs from eager in "
-                                 "gradients %s: not reported\n" % bad)
-                return None
-            run()  # eager work between replays
-            _sync()
-        return _event_ms(graph.replay, steps, 3)
-    except Exception as exc:  # capture refused by some op: report the eager time only
-        sys.stderr.write("HIP graph capture of the temporal step failed: %s\n" % exc)
+        replayed = ReplayedStep(run)
+    except Exception as exc:  # capture refused by some op, or a replay differs: eager time only
+        sys.stderr.write("HIP graph replay of the temporal step not reported: %s\n" % exc)
         return None
+    return _event_ms(replayed.replay, steps, 3)
 
 
 def run_c3_orders(args, dev):
