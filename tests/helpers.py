@@ -43,6 +43,40 @@ def assert_close(got, want, rtol=RTOL_F32, atol=ATOL_F32, what="", abs_sum=None,
                              (what, bad.sum(), bad.size, i, got[i], want[i]))
 
 
+def spmm_abs_sums(values, indptr, indices, x, gy=None):
+    """Sums of absolute terms of the multi-head SpMM's three reductions (``abs_sum`` of
+    ``assert_close``): out = sum a x, and with ``gy`` also grad_a = sum_f gy x and
+    grad_x = sum_e a gy, each evaluated by the oracle on the absolute inputs."""
+    import oracle
+    a, xa = np.abs(_np(values)), np.abs(_np(x))
+    out = oracle.mh_spmm_forward(a, indptr, indices, xa)
+    if gy is None:
+        return out
+    ga, gx = oracle.mh_spmm_backward(a, indptr, indices, xa, np.abs(_np(gy)))
+    return out, ga, gx
+
+
+def softmax_backward_abs_sums(indptr, indices, attn, grad_abs, n_src):
+    """Bounds on the absolute terms behind the edge-softmax backward (sddmm_cuda.cu:36-66):
+    with T[r,b,h] = sum_e a_e |g_e| over the edges of destination r that carry block tag b,
+    grad_query[b,r,h] = sum_e a_e (g_e - S) d_e has absolute terms below 2 T, and the
+    per-edge logit gradient is below a_e (|g_e| + T), summed per source for grad_key.
+    ``grad_abs``: |g| per edge and head, or a bound on it (for the fused op, whose g is
+    itself a dot product, the dot of the absolute operands). Returns (query, key) bounds
+    shaped [n_bid, n_dst, H] and [n_src, H]."""
+    indptr, indices = _np(indptr).astype(np.int64), _np(indices).astype(np.int64)
+    a, g = _np(attn).astype(np.float64), np.abs(_np(grad_abs)).astype(np.float64)
+    n_dst, h = indptr.size - 1, a.shape[1]
+    rows = np.repeat(np.arange(n_dst), np.diff(indptr))
+    bid, col = indices >> 24, indices & 0xffffff
+    n_bid = int(bid.max()) + 1 if bid.size else 1
+    t = np.zeros((n_bid * n_dst, h))
+    np.add.at(t, bid * n_dst + rows, a * g)
+    key_bound = np.zeros((n_src, h))
+    np.add.at(key_bound, col, a * (g + t[bid * n_dst + rows]))
+    return 2.0 * t.reshape(n_bid, n_dst, h), key_bound
+
+
 def random_csr(n_dst, n_src, density, seed, hub_rows=(), hub_degree=0, empty_rows=()):
     """Canonical CSR with a given density plus optional hub / empty rows."""
     rng = np.random.default_rng(seed)

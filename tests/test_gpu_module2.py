@@ -8,7 +8,7 @@ import torch
 from torch import nn
 
 import oracle
-from helpers import assert_close, powerlaw_graph, random_csr
+from helpers import softmax_backward_abs_sums, spmm_abs_sums, assert_close, powerlaw_graph, random_csr
 from yitu_amd import graph_ext
 from yitu_amd.xgnn_h import block as xblock
 from yitu_amd.xgnn_h import sparse
@@ -55,12 +55,13 @@ def test_spmm_random_shapes(dev, seed):
     gy = torch.randn(n_dst, h, f, generator=g)
     args = (values.to(dev), indptr.to(dev), indices.to(dev), x.to(dev))
     what = "n_dst=%d n_src=%d H=%d F=%d" % (n_dst, n_src, h, f)
+    abs_out, abs_ga, abs_gx = spmm_abs_sums(values, indptr, indices, x, gy)
     assert_close(graph_ext.spmm_forward(*args), oracle.mh_spmm_forward(values, indptr, indices, x),
-                 what=what)
+                 abs_sum=abs_out, what=what)
     ga, gx = graph_ext.spmm_backward(*args, gy.to(dev))
     want_ga, want_gx = oracle.mh_spmm_backward(values, indptr, indices, x, gy)
-    assert_close(ga, want_ga, atol=2e-4, what="grad_a " + what)
-    assert_close(gx, want_gx, atol=2e-4, what="grad_x " + what)
+    assert_close(ga, want_ga, abs_sum=abs_ga, what="grad_a " + what)
+    assert_close(gx, want_gx, abs_sum=abs_gx, what="grad_x " + what)
 
 
 @pytest.mark.parametrize("h,f", [(4, 64), (1, 128), (8, 8), (2, 600), (3, 5)])
@@ -73,12 +74,13 @@ def test_spmm_power_law_with_hub_rows_and_columns(dev, h, f):
     x = torch.randn(n, h, f, generator=g)
     gy = torch.randn(n, h, f, generator=g)
     args = (values.to(dev), indptr.to(dev), indices.to(dev), x.to(dev))
+    abs_out, abs_ga, abs_gx = spmm_abs_sums(values, indptr, indices, x, gy)
     assert_close(graph_ext.spmm_forward(*args), oracle.mh_spmm_forward(values, indptr, indices, x),
-                 atol=5e-4)
+                 abs_sum=abs_out)
     ga, gx = graph_ext.spmm_backward(*args, gy.to(dev))
     want_ga, want_gx = oracle.mh_spmm_backward(values, indptr, indices, x, gy)
-    assert_close(ga, want_ga, atol=5e-4)
-    assert_close(gx, want_gx, atol=5e-4)
+    assert_close(ga, want_ga, abs_sum=abs_ga)
+    assert_close(gx, want_gx, abs_sum=abs_gx)
     ga2, gx2 = graph_ext.spmm_backward(*args, gy.to(dev))
     assert torch.equal(ga, ga2) and torch.equal(gx, gx2)  # no atomics: reproducible
 
@@ -177,8 +179,9 @@ def test_sddmm_power_law_hub_rows(dev, h):
     for det in (True, False):
         gq, gk = graph_ext.sddmm_backward(*dargs, attn, ge.to(dev), deterministic=det)
         want_gq, want_gk = oracle.sddmm_backward(indptr, indices, q, k, want, ge)
-        assert_close(gq, want_gq, atol=2e-4)
-        assert_close(gk, want_gk, atol=2e-4)
+        abs_gq, abs_gk = softmax_backward_abs_sums(indptr, indices, want, ge, n)
+        assert_close(gq, want_gq, abs_sum=abs_gq)
+        assert_close(gk, want_gk, abs_sum=abs_gk)
 
 
 def test_sddmm_large_logits_do_not_overflow(dev):
@@ -252,20 +255,23 @@ def test_stitched_blocks_fused_attention(dev, n_blk, h, f, head_mean):
     g_out = torch.from_numpy(rng.standard_normal(out.shape).astype(np.float32))
     out.backward(g_out.to(dev))
     g_full = g_out.unsqueeze(1).expand(-1, h, -1) / h if head_mean else g_out
-    assert_close(out, want.mean(axis=1) if head_mean else want, atol=2e-4)
     g_full = np.ascontiguousarray(g_full.numpy())
+    abs_out, abs_ga, abs_gx = spmm_abs_sums(want_attn, sp, si, x, g_full)
+    assert_close(out, want.mean(axis=1) if head_mean else want,
+                 abs_sum=abs_out.mean(axis=1) if head_mean else abs_out)
     want_ga, want_gx = oracle.mh_spmm_backward(want_attn, sp, si, x.numpy(), g_full)
     want_gq, want_gk = oracle.sddmm_backward(sp, si, q.numpy(), k.numpy(), want_attn, want_ga)
-    assert_close(dx.grad, want_gx, atol=2e-4, what="grad_x")
-    assert_close(dq.grad, want_gq, atol=2e-4, what="grad_query")
-    assert_close(dk.grad, want_gk, atol=2e-4, what="grad_key")
+    abs_gq, abs_gk = softmax_backward_abs_sums(sp, si, want_attn, abs_ga, k.shape[0])
+    assert_close(dx.grad, want_gx, abs_sum=abs_gx, what="grad_x")
+    assert_close(dq.grad, want_gq, abs_sum=abs_gq, what="grad_query")
+    assert_close(dk.grad, want_gk, abs_sum=abs_gk, what="grad_key")
     # one query block: the same entry point, the plain block
     ip0, ix0 = blocks[0].adj_sparse
     want_one = oracle.mh_spmm_forward(oracle.sddmm_forward(ip0, ix0, qs[0].unsqueeze(0), ks[0]),
                                       ip0, ix0, xs[0])
     one = sparse.fused_gat(xblock.Block(blocks[0].size, [ip0.to(dev), ix0.to(dev)]),
                            qs[0].to(dev).unsqueeze(0), ks[0].to(dev), xs[0].to(dev))
-    assert_close(one, want_one, atol=2e-4)
+    assert_close(one, want_one)
 
 
 # ---- the reference's own checks, end to end through autograd -----------------------
@@ -395,8 +401,9 @@ def test_hfused_backward_against_the_oracle_ops(dev, n_dst, n_src, h, f, n_bid, 
     abs_ga = oracle.mh_spmm_backward(vals.abs(), a_ptr, a_idx, x.abs().numpy(), gy.abs().numpy())
     assert_close(got[0], want_ga, abs_sum=abs_ga[0], what="grad of the SpMM's edge values")
     assert_close(got[1], want_gx, abs_sum=abs_ga[1], what="grad of the SpMM's features")
-    assert_close(got[2], want_gq, atol=2e-4, what="grad_query")
-    assert_close(got[3], want_gk, atol=2e-4, what="grad_key")
+    abs_gq, abs_gk = softmax_backward_abs_sums(b_ptr, b_idx, attn, gattn, n_cols)
+    assert_close(got[2], want_gq, abs_sum=abs_gq, what="grad_query")
+    assert_close(got[3], want_gk, abs_sum=abs_gk, what="grad_key")
     again = graph_ext.hfused_backward(*args)
     assert all(torch.equal(a, b) for a, b in zip(got, again))
 
@@ -516,14 +523,15 @@ def test_spmm_backward_one_gather_shapes(dev, h, f):
     d = lambda t: t.to(dev)
     ga, gx = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
     want_ga, want_gx = oracle.mh_spmm_backward(values, indptr, indices, x, gy)
-    assert_close(ga, want_ga, atol=5e-4)
-    assert_close(gx, want_gx, atol=1e-3)
+    _, abs_ga, abs_gx = spmm_abs_sums(values, indptr, indices, x, gy)
+    assert_close(ga, want_ga, abs_sum=abs_ga)
+    assert_close(gx, want_gx, abs_sum=abs_gx)
     ga2, _ = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy),
                                      need_grad_x=False)
     _, gx2 = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy),
                                      need_grad_a=False)
-    assert_close(ga, ga2, atol=5e-4)
-    assert_close(gx, gx2, atol=1e-3)
+    assert_close(ga, ga2, abs_sum=abs_ga)
+    assert_close(gx, gx2, abs_sum=abs_gx)
     again = graph_ext.spmm_backward(d(values), d(indptr), d(indices), d(x), d(gy))
     assert torch.equal(again[0], ga) and torch.equal(again[1], gx)
 
@@ -540,10 +548,11 @@ def test_spmm_backward_constant_weights_take_the_by_source_copy(dev):
     gy = torch.randn(n, 2, 24, generator=g)
     ip, ix, xd, gyd = indptr.to(dev), indices.to(dev), x.to(dev), gy.to(dev)
     want = oracle.mh_spmm_backward(values.cpu(), indptr, indices, x, gy)[1]
+    abs_gx = spmm_abs_sums(values.cpu(), indptr, indices, x, gy)[2]
     for _ in range(3):  # first call: through the permutation; then: the kept copy
         got = graph_ext.spmm_backward(values, ip, ix, xd, gyd, need_grad_a=False)[1]
-        assert_close(got, want, atol=5e-4)
+        assert_close(got, want, abs_sum=abs_gx)
     values.mul_(2.0)
     for _ in range(3):
         got = graph_ext.spmm_backward(values, ip, ix, xd, gyd, need_grad_a=False)[1]
-        assert_close(got, 2 * torch.as_tensor(want), atol=1e-3)
+        assert_close(got, 2 * torch.as_tensor(want), abs_sum=2 * abs_gx)
