@@ -195,3 +195,85 @@ def test_fused_layer_equals_the_composed_ops(dev, monkeypatch):
                           ["h"] + [n for n, _ in layer.named_parameters()]):
         rtol = 1e-3 if name == "time_enc.w.weight" else 1e-4
         assert_close(g, r, rtol=rtol, atol=5e-4, what=name)
+
+
+def _reference_combined(layer, blk):
+    """layers.py:81-103 in float64: one Linear per input part, results added."""
+    import copy
+    ref = copy.deepcopy(layer).double()
+    n_dst, row = blk.n_dst, blk.row
+    E = row.numel()
+    dev = row.device
+    O = layer.dim_out
+    q = torch.zeros(E, O, dtype=torch.float64, device=dev)
+    k = torch.zeros(E, O, dtype=torch.float64, device=dev)
+    v = torch.zeros(E, O, dtype=torch.float64, device=dev)
+    h = blk.h.detach().double().requires_grad_() if layer.dim_node_feat > 0 else None
+    f = blk.f.detach().double().requires_grad_() if layer.dim_edge_feat > 0 else None
+    if h is not None:
+        q = q + ref.w_q_n(h[:n_dst])[row]
+        k = k + ref.w_k_n(h[n_dst:])
+        v = v + ref.w_v_n(h[n_dst:])
+    if f is not None:
+        k = k + ref.w_k_e(f)
+        v = v + ref.w_v_e(f)
+    if layer.dim_time > 0:
+        w32, b32 = layer.time_enc.w.weight.detach()[:, 0], layer.time_enc.w.bias.detach()
+        arg32 = (blk.dt[:, None] * w32[None, :] + b32).double()
+        w, b = ref.time_enc.w.weight[:, 0], ref.time_enc.w.bias
+        exact = blk.dt.double()[:, None] * w[None, :] + b
+        te = torch.cos(exact + (arg32 - exact).detach())
+        te0 = torch.cos(b)[None, :].expand(n_dst, -1)
+        q = q + ref.w_q_t(te0)[row]
+        k = k + ref.w_k_t(te)
+        v = v + ref.w_v_t(te)
+    H, D = layer.num_head, O // layer.num_head
+    logits = torch.nn.functional.leaky_relu((q * k).view(E, H, D).sum(-1), 0.2)
+    top = torch.full((n_dst, H), -1e300, dtype=torch.float64, device=dev)
+    top = top.index_reduce(0, row, logits.detach(), "amax")
+    p = torch.exp(logits - top[row])
+    s = torch.zeros(n_dst, H, dtype=torch.float64, device=dev).index_add(0, row, p)
+    att = p / s[row]
+    agg = torch.zeros(n_dst, H, D, dtype=torch.float64, device=dev).index_add(
+        0, row, v.view(E, H, D) * att[:, :, None]).reshape(n_dst, O)
+    rst = torch.cat([agg, h[:n_dst]], 1) if h is not None else agg
+    return ref, ref.layer_norm(torch.relu(ref.w_out(rst))), h, f
+
+
+@pytest.mark.parametrize("dims", [(24, 6, 10, 2, 32), (24, 0, 10, 1, 16), (0, 6, 0, 1, 8),
+                                  (12, 5, 0, 4, 32)])
+def test_combined_branch(dev, dims):
+    """combined=True (layers.py:53-66, 81-103): per-part Linears with the reference's
+    parameter names, added up; computed as one product over concatenated weights. Against
+    the part-by-part float64 statement, output and every gradient; (0, 6, 0): edge
+    features only, where the query stays zero and the attention is uniform."""
+    dim_node, dim_edge, dim_time, num_head, dim_out = dims
+    torch.manual_seed(sum(dims))
+    counts = [0, 1, 70, 3, 20] + [6] * 30
+    n_dst = len(counts)
+    row = np.repeat(np.arange(n_dst), counts)
+    E = row.size
+    dt = np.random.default_rng(1).uniform(0, 1e4, E).astype(np.float32)
+    h = torch.randn(n_dst + E, dim_node, device=dev).requires_grad_() if dim_node else None
+    f = torch.randn(E, dim_edge, device=dev).requires_grad_() if dim_edge else None
+    blk = TemporalBlock(row, n_dst, dt, h=h, f=f, device=dev)
+    layer = TransfomerAttentionLayer(dim_node, dim_edge, dim_time, num_head, 0.0, 0.0, dim_out,
+                                     combined=True).to(dev)
+    names = {n for n, _ in layer.named_parameters()}
+    assert ("w_k_e.weight" in names) == (dim_edge > 0) and ("w_q_t.bias" in names) == (dim_time > 0)
+    assert "w_q.weight" not in names and "w_k.weight" not in names
+    out = layer(blk)
+    w = torch.randn_like(out)
+    (out * w).sum().backward()
+    ref, want, h_ref, f_ref = _reference_combined(layer, blk)
+    (want * w.double()).sum().backward()
+    assert_close(out, want.float(), what="out")
+    pairs = [(n, p.grad, dict(ref.named_parameters())[n].grad) for n, p in layer.named_parameters()]
+    if h is not None:
+        pairs.append(("h", h.grad, h_ref.grad))
+    if f is not None:
+        pairs.append(("f", f.grad, f_ref.grad))
+    for name, got, ref_grad in pairs:
+        assert got is not None, name
+        scale = 1e4 if name == "time_enc.w.weight" else 1.0
+        assert_close(got, ref_grad.float(), rtol=1e-4, atol=1e-4 * scale, what=name)

@@ -136,14 +136,16 @@ class TemporalBlock:
 
 
 class TransfomerAttentionLayer(torch.nn.Module):
-    """layers.py:39-142, the non-``combined`` branches. Parameter names and shapes
-    are the reference's, so its state_dicts load unchanged."""
+    """layers.py:39-142. Parameter names and shapes are the reference's, so its
+    state_dicts load unchanged. ``combined=True`` (layers.py:53-66, 81-103) keeps one
+    Linear per input part (node / edge / time) and adds their results; that is the
+    product of the concatenated inputs with the concatenated weights, biases added up,
+    which is how it is computed here (same kernels as the other branch)."""
 
     def __init__(self, dim_node_feat, dim_edge_feat, dim_time, num_head, dropout, att_dropout,
                  dim_out, combined=False):
         super().__init__()
-        if combined:
-            raise NotImplementedError("combined=True is not built")
+        self.combined = combined
         self.num_head = num_head
         self.dim_node_feat = dim_node_feat
         self.dim_edge_feat = dim_edge_feat
@@ -154,21 +156,53 @@ class TransfomerAttentionLayer(torch.nn.Module):
         self.att_act = torch.nn.LeakyReLU(0.2)
         if dim_time > 0:
             self.time_enc = TimeEncode(dim_time)
-        if dim_node_feat + dim_time > 0:
-            self.w_q = torch.nn.Linear(dim_node_feat + dim_time, dim_out)
-        self.w_k = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
-        self.w_v = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
+        if combined:
+            if dim_node_feat > 0:
+                self.w_q_n = torch.nn.Linear(dim_node_feat, dim_out)
+                self.w_k_n = torch.nn.Linear(dim_node_feat, dim_out)
+                self.w_v_n = torch.nn.Linear(dim_node_feat, dim_out)
+            if dim_edge_feat > 0:
+                self.w_k_e = torch.nn.Linear(dim_edge_feat, dim_out)
+                self.w_v_e = torch.nn.Linear(dim_edge_feat, dim_out)
+            if dim_time > 0:
+                self.w_q_t = torch.nn.Linear(dim_time, dim_out)
+                self.w_k_t = torch.nn.Linear(dim_time, dim_out)
+                self.w_v_t = torch.nn.Linear(dim_time, dim_out)
+        else:
+            if dim_node_feat + dim_time > 0:
+                self.w_q = torch.nn.Linear(dim_node_feat + dim_time, dim_out)
+            self.w_k = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
+            self.w_v = torch.nn.Linear(dim_node_feat + dim_edge_feat + dim_time, dim_out)
         self.w_out = torch.nn.Linear(dim_node_feat + dim_out, dim_out)
         self.layer_norm = torch.nn.LayerNorm(dim_out)
 
+    def _projection(self, which):
+        """(weight, bias) of the q / k / v projection over the concatenated inputs
+        [node | edge | time] (q: [node | time]); None when q has no input."""
+        if not self.combined:
+            lin = getattr(self, "w_" + which, None)
+            return (lin.weight, lin.bias) if lin is not None else None
+        parts = [getattr(self, "w_%s_%s" % (which, tag), None)
+                 for tag, dim in (("n", self.dim_node_feat), ("e", self.dim_edge_feat),
+                                  ("t", self.dim_time)) if dim > 0 and not (which == "q" and tag == "e")]
+        parts = [p for p in parts if p is not None]
+        if not parts:
+            return None
+        weight = parts[0].weight if len(parts) == 1 else torch.cat([p.weight for p in parts], dim=1)
+        bias = parts[0].bias
+        for p in parts[1:]:
+            bias = bias + p.bias
+        return weight, bias
+
     def forward(self, b: TemporalBlock):
         assert self.dim_time + self.dim_node_feat + self.dim_edge_feat > 0
-        dev = self.w_k.weight.device
+        dev = self.w_out.weight.device
+        wq, wk, wv = self._projection("q"), self._projection("k"), self._projection("v")
         n_dst = b.num_dst_nodes()
         if b.num_edges() == 0:
             return torch.zeros((n_dst, self.dim_out), device=dev)
         drops = self.training and (self.dropout.p > 0 or self.att_dropout.p > 0)
-        if not drops and self.w_k.weight.is_cuda and self.w_k.weight.dtype == torch.float32 and \
+        if not drops and wk[0].is_cuda and wk[0].dtype == torch.float32 and \
                 fused.supported(self.dim_node_feat, self.dim_edge_feat, self.dim_time, self.dim_out,
                                 self.num_head):
             # the whole layer as one autograd node of twelve launches
@@ -177,9 +211,8 @@ class TransfomerAttentionLayer(torch.nn.Module):
                 b.blk.adj_sparse[0], n_dst, self.num_head, self.layer_norm.eps,
                 b.h if self.dim_node_feat > 0 else None, b.f if self.dim_edge_feat > 0 else None,
                 b.dt, te.weight if te is not None else None, te.bias if te is not None else None,
-                self.w_q.weight, self.w_q.bias, self.w_k.weight, self.w_k.bias, self.w_v.weight,
-                self.w_v.bias, self.w_out.weight, self.w_out.bias, self.layer_norm.weight,
-                self.layer_norm.bias)
+                wq[0], wq[1], wk[0], wk[1], wv[0], wv[1], self.w_out.weight, self.w_out.bias,
+                self.layer_norm.weight, self.layer_norm.bias)
         parts_q, parts_kv = [], []
         if self.dim_node_feat > 0:
             parts_q.append(b.h[:n_dst])
@@ -192,10 +225,12 @@ class TransfomerAttentionLayer(torch.nn.Module):
         kv_in = torch.cat(parts_kv, dim=1)
         head_dim = self.dim_out // self.num_head
         if parts_q:
-            Q = _linear(self.w_q, torch.cat(parts_q, dim=1))
+            Q = bundle.linear(torch.cat(parts_q, dim=1), wq[0], wq[1])
+        elif self.combined:  # nothing is added to the zeros Q starts from (layers.py:82)
+            Q = torch.zeros((n_dst, self.dim_out), device=dev)
         else:  # edge features only (layers.py:104-107)
             Q = torch.ones((n_dst, self.dim_out), device=dev)
-        K, V = bundle.linear_pair(kv_in, self.w_k, self.w_v)  # one grouped launch
+        K, V = bundle.bundled_linear(kv_in, wk[0], wv[0], wk[1], wv[1])  # one grouped launch
         K = K.reshape(-1, self.num_head, head_dim).contiguous()
         V = V.reshape(-1, self.num_head, head_dim).contiguous()
         Q = Q.reshape(n_dst, self.num_head, head_dim).contiguous()
