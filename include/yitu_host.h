@@ -42,20 +42,32 @@ int yitu_rabbit_reorder_threads(int32_t *out_edge_index, int32_t *perm_out,
                                 const int32_t *in_edge_index, int64_t n_edges, int n_threads);
 
 /*
- * Most-recent-neighbour temporal sampler: replaces sampler_core.ParallelSampler
- * (YiTu_GNN/YiTu_T/sampler_core.cpp:43-359, binding :374-402) in its
- * `recent = True`, `num_history = 1`, `window_duration = 0` mode.
+ * Temporal neighbour sampler: replaces sampler_core.ParallelSampler
+ * (YiTu_GNN/YiTu_T/sampler_core.cpp:43-359, binding :374-402).
  * T-CSR inputs: indptr [n_nodes+1], indices / eid [n_edges] int32, ts [n_edges]
  * float32 ascending inside every node. num_neighbors [num_layers] is the fan-out
- * per layer. Layer l > 0 expands every node of block l-1 at that block's
- * timestamps (the reference reads an uninitialised pointer there,
- * sampler_core.cpp:204-213, so only its single-layer behaviour is defined).
+ * per layer. yitu_sampler_create is the most-recent mode (recent = True,
+ * num_history = 1, window_duration = 0); yitu_sampler_create_modes takes the
+ * reference constructor's remaining arguments: recent = 0 draws num_neighbors
+ * edges uniformly from a root's window with the C library's rand_r, one generator
+ * per chunk of ceil(n_roots / num_threads) roots seeded with the chunk's index, as
+ * the reference's threads do (:238-253, 306-318), so the draws depend on the
+ * NOMINAL num_threads only; num_history > 1 yields one block per snapshot and
+ * layer, of windows window_duration wide (:216-226, 271-279), in the reference's
+ * block order. A layer after the first that uses cursors (recent or prop_time)
+ * advances them from the nodes of the previous layer's block (the reference reads
+ * an uninitialised pointer there, sampler_core.cpp:204-213).
  */
 typedef struct yitu_sampler yitu_sampler;
 yitu_sampler *yitu_sampler_create(const int32_t *indptr, const int32_t *indices, const int32_t *eid,
                                   const float *ts, int64_t n_nodes, int64_t n_edges,
                                   int num_threads, int num_layers, const int32_t *num_neighbors,
                                   int prop_time);
+yitu_sampler *yitu_sampler_create_modes(const int32_t *indptr, const int32_t *indices,
+                                        const int32_t *eid, const float *ts, int64_t n_nodes,
+                                        int64_t n_edges, int num_threads, int num_layers,
+                                        const int32_t *num_neighbors, int recent, int prop_time,
+                                        int num_history, float window_duration);
 void yitu_sampler_destroy(yitu_sampler *s);
 int yitu_sampler_reset(yitu_sampler *s);
 int yitu_sampler_sample(yitu_sampler *s, const int32_t *root_nodes, const float *root_ts,

@@ -1,4 +1,4 @@
-"""Writes tests/golden/sampler_recent.npz: input/output vectors of the
+"""Writes tests/golden/sampler_recent.npz and sampler_modes.npz: input/output vectors of the
 reference's own temporal sampler (YiTu_GNN/YiTu_T/sampler_core.cpp compiled
 as-is into oracle/_ref/ by oracle/Makefile) on small seeded event streams.
 
@@ -92,6 +92,57 @@ def main():
             out[bp + "nodes"] = np.asarray(blk.nodes(), np.int32)
             out[bp + "dims"] = np.asarray([blk.dim_in(), blk.dim_out()], np.int64)
     path = os.path.join(ROOT, "tests", "golden", "sampler_recent.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, os.path.getsize(path), "bytes")
+    write_modes(ref)
+
+
+# (seed, n_nodes, n_events, batch, n_batches, threads, layers, fans, recent, prop_time,
+#  num_history, window): uniform draws with 1 / 2 / 5 nominal threads, two layers by binary
+# search, prop_time cursors in the first layer, snapshots of a window (most recent and drawn)
+MODE_CASES = [
+    (11, 60, 3000, 24, 3, 1, 1, [5], False, False, 1, 0.0),
+    (12, 60, 3000, 24, 3, 2, 1, [5], False, False, 1, 0.0),
+    (13, 200, 8000, 40, 3, 5, 1, [10], False, False, 1, 0.0),
+    (14, 80, 4000, 16, 2, 3, 2, [6, 4], False, False, 1, 0.0),
+    (15, 80, 4000, 16, 2, 2, 1, [4], False, True, 1, 0.0),
+    (16, 50, 4000, 20, 3, 2, 1, [5], True, False, 3, 50000.0),
+    (17, 50, 4000, 20, 3, 4, 1, [3], False, False, 2, 100000.0),
+    (18, 50, 4000, 12, 2, 2, 2, [4, 3], False, False, 2, 100000.0),
+]
+
+
+def write_modes(ref):
+    out = {"n_cases": np.int64(len(MODE_CASES))}
+    for ci, (seed, n_nodes, n_events, batch, n_batches, threads, layers, fans, recent, prop_time,
+             hist, window) in enumerate(MODE_CASES):
+        c = make_case(seed, n_nodes, n_events, batch, fans[0], n_batches, prop_time)
+        s = ref.ParallelSampler(c["indptr"].tolist(), c["indices"].tolist(), c["eid"].tolist(),
+                                c["ts"].tolist(), threads, 1, layers, list(fans), recent, prop_time,
+                                hist, float(window))
+        pre = "c%d_" % ci
+        for k in ("indptr", "indices", "eid", "ts"):
+            out[pre + k] = c[k]
+        out[pre + "args"] = np.asarray([threads, layers, int(recent), int(prop_time), hist], np.int64)
+        out[pre + "fans"] = np.asarray(fans, np.int64)
+        out[pre + "window"] = np.float32(window)
+        out[pre + "n_batches"] = np.int64(n_batches)
+        for bi, (roots, rts) in enumerate(c["batches"]):
+            s.sample(roots.tolist(), rts.tolist())
+            ret = s.get_ret()
+            bp = pre + "b%d_" % bi
+            out[bp + "roots"], out[bp + "root_ts"] = roots, rts
+            out[bp + "n_blocks"] = np.int64(len(ret))
+            for ri, blk in enumerate(ret):
+                rp = bp + "r%d_" % ri
+                out[rp + "row"] = np.asarray(blk.row(), np.int32)
+                out[rp + "col"] = np.asarray(blk.col(), np.int32)
+                out[rp + "eid"] = np.asarray(blk.eid(), np.int32)
+                out[rp + "ts"] = np.asarray(blk.ts(), np.float32)
+                out[rp + "dts"] = np.asarray(blk.dts(), np.float32)
+                out[rp + "nodes"] = np.asarray(blk.nodes(), np.int32)
+                out[rp + "dims"] = np.asarray([blk.dim_in(), blk.dim_out()], np.int64)
+    path = os.path.join(ROOT, "tests", "golden", "sampler_modes.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")
 

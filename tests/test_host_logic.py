@@ -30,6 +30,16 @@ def test_library_exports_every_declared_symbol():
     assert lib.yitu_abi_version() >= 1
 
 
+def test_host_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "yitu_host.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = set(re.findall(r"\b(yitu_[a-z0-9_]+)\s*\(", header))
+    assert len(names) >= 10
+    lib = ctypes.CDLL(os.path.join(ROOT, "yitu_amd", "libyitu_host.so"))
+    missing = [n for n in sorted(names) if not hasattr(lib, n)]
+    assert not missing, "declared but not exported: %s" % missing
+
+
 @pytest.mark.parametrize("ps", [1, 4, 32])
 @pytest.mark.parametrize("last_empty", [False, True])
 def test_build_part_matches_oracle(ps, last_empty):

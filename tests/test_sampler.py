@@ -106,8 +106,8 @@ def test_edge_cases():
     assert blk.row().tolist() == [2, 2] and blk.eid().tolist() == [13, 12]
     with pytest.raises(RuntimeError):
         s.sample(np.asarray([3], np.int32), np.asarray([1.0], np.float32))
-    with pytest.raises(NotImplementedError):
-        sampler_core.ParallelSampler(indptr, indices, eid, ts, 1, 1, 1, [10], False, False, 1, 0.0)
+    with pytest.raises(ValueError):
+        sampler_core.ParallelSampler(indptr, indices, eid, ts, 1, 1, 1, [10], True, False, 0, 0.0)
 
 
 def test_two_layers_expand_previous_block():
@@ -164,6 +164,42 @@ def test_against_compiled_reference_live(seed):
         assert (g.dim_in(), g.dim_out()) == (w.dim_in(), w.dim_out())
 
 
+@pytest.mark.parametrize("threads,layers,fans,recent,prop_time,hist,window", [
+    (4, 1, [6], False, False, 1, 0.0),
+    (3, 2, [4, 3], False, False, 1, 0.0),
+    (2, 1, [5], True, False, 3, 5e4),
+    (7, 2, [3, 3], False, False, 2, 8e4),
+])
+def test_other_modes_against_compiled_reference_live(threads, layers, fans, recent, prop_time,
+                                                     hist, window):
+    ref = _load_ref()
+    if ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    rng = np.random.default_rng(7 * threads + layers)
+    n_nodes, n_edges = 300, 12000
+    owner = np.sort((rng.zipf(1.3, n_edges) - 1) % n_nodes)
+    indptr = np.searchsorted(owner, np.arange(n_nodes + 1)).astype(np.int32)
+    ts = np.concatenate([np.sort(rng.uniform(0, 1e6, indptr[v + 1] - indptr[v]))
+                         for v in range(n_nodes)]).astype(np.float32)
+    indices = rng.integers(0, n_nodes, n_edges).astype(np.int32)
+    eid = rng.permutation(n_edges).astype(np.int32)
+    mine = sampler_core.ParallelSampler(indptr, indices, eid, ts, threads, 1, layers, fans, recent,
+                                        prop_time, hist, window)
+    theirs = ref.ParallelSampler(indptr.tolist(), indices.tolist(), eid.tolist(), ts.tolist(),
+                                 threads, 1, layers, fans, recent, prop_time, hist, window)
+    for b in range(4):
+        roots = ((rng.zipf(1.3, 150) - 1) % n_nodes).astype(np.int32)
+        rts = np.sort(rng.uniform(b * 2e5, (b + 1) * 2e5 + 1e5, 150)).astype(np.float32)
+        mine.sample(roots, rts)
+        theirs.sample(roots.tolist(), rts.tolist())
+        got, want = mine.get_ret(), theirs.get_ret()
+        assert len(got) == len(want) == layers * hist
+        for r, (g, w) in enumerate(zip(got, want)):
+            for f in FIELDS:
+                assert np.array_equal(getattr(g, f)(), np.asarray(getattr(w, f)())), (b, r, f)
+            assert (g.dim_in(), g.dim_out()) == (w.dim_in(), w.dim_out())
+
+
 @pytest.mark.parametrize("add_reverse", [True, False])
 def test_build_tcsr_equals_per_node_lists_sorted_by_time(add_reverse):
     """gen_graph.py:40-95 restated with Python lists and a stable sort, on a stream whose
@@ -193,3 +229,53 @@ def test_build_tcsr_equals_per_node_lists_sorted_by_time(add_reverse):
     s = sampler_core.ParallelSampler(*[g.numpy() for g in got], 1, 1, 1, [5], True, False, 1, 0.0)
     s.sample(src[-20:], np.full(20, 60.0, np.float32))
     assert s.get_ret()[0].dim_out() == 20
+
+
+MODES = np.load(os.path.join(ROOT, "tests", "golden", "sampler_modes.npz"))
+
+
+@pytest.mark.parametrize("case", range(int(MODES["n_cases"])))
+def test_other_modes_match_reference_golden_vectors(case):
+    """Uniform draws (the reference's per-thread rand_r streams, for 1 / 2 / 5 nominal
+    threads), a second layer found by binary search, prop_time, and snapshots of a sliding
+    window (num_history 2 and 3), every block of every batch bit for bit against what the
+    compiled reference returned (tests/golden/make_sampler_golden.py: MODE_CASES)."""
+    pre = "c%d_" % case
+    threads, layers, recent, prop_time, hist = (int(v) for v in MODES[pre + "args"])
+    s = sampler_core.ParallelSampler(MODES[pre + "indptr"], MODES[pre + "indices"], MODES[pre + "eid"],
+                                     MODES[pre + "ts"], threads, 1, layers,
+                                     [int(v) for v in MODES[pre + "fans"]], bool(recent),
+                                     bool(prop_time), hist, float(MODES[pre + "window"]))
+    for b in range(int(MODES[pre + "n_batches"])):
+        bp = pre + "b%d_" % b
+        s.sample(MODES[bp + "roots"], MODES[bp + "root_ts"])
+        ret = s.get_ret()
+        assert len(ret) == int(MODES[bp + "n_blocks"]) == layers * hist
+        for r, blk in enumerate(ret):
+            got = _block_arrays(blk)
+            for f in FIELDS:
+                want = MODES[bp + "r%d_" % r + f]
+                assert got[f].dtype == want.dtype and got[f].shape == want.shape, (case, b, r, f)
+                assert np.array_equal(got[f], want), (case, b, r, f)
+            assert [blk.dim_in(), blk.dim_out()] == MODES[bp + "r%d_dims" % r].tolist()
+
+
+def test_uniform_draws_do_not_depend_on_the_real_thread_count(monkeypatch):
+    """The draws are a function of the nominal thread count; how many threads really run
+    (OMP_NUM_THREADS of the host) must not matter: same blocks for the same arguments from
+    two samplers, one of them built and run after the OpenMP pool was shrunk to one thread."""
+    pre = "c2_"
+    args = (MODES[pre + "indptr"], MODES[pre + "indices"], MODES[pre + "eid"], MODES[pre + "ts"],
+            5, 1, 1, [10], False, False, 1, 0.0)
+    a = sampler_core.ParallelSampler(*args)
+    a.sample(MODES[pre + "b0_roots"], MODES[pre + "b0_root_ts"])
+    import ctypes
+    omp = ctypes.CDLL("libgomp.so.1")
+    omp.omp_set_num_threads(1)
+    try:
+        b = sampler_core.ParallelSampler(*args)
+        b.sample(MODES[pre + "b0_roots"], MODES[pre + "b0_root_ts"])
+    finally:
+        omp.omp_set_num_threads(os.cpu_count() or 1)
+    for f in FIELDS:
+        assert np.array_equal(_block_arrays(a.get_ret()[0])[f], _block_arrays(b.get_ret()[0])[f])

@@ -16,6 +16,7 @@ def lib():
         l.yitu_host_last_error.restype = ctypes.c_char_p
         l.yitu_sampler_last_error.restype = ctypes.c_char_p
         l.yitu_sampler_create.restype = ctypes.c_void_p
+        l.yitu_sampler_create_modes.restype = ctypes.c_void_p
         l.yitu_sampler_num_blocks.restype = ctypes.c_int64
         _lib = l
     return _lib

@@ -1,9 +1,12 @@
 """Drop-in for the reference's ``sampler_core`` extension module
 (YiTu_GNN/YiTu_T/sampler_core.cpp:374-402): ``ParallelSampler`` with
 ``sample / reset / get_ret`` and ``TemporalGraphBlock`` accessors returning numpy
-arrays. Only the most-recent-neighbour mode the temporal attention path uses is
-implemented (``recent=True``, ``num_history=1``, ``window_duration=0``); other
-modes raise ``NotImplementedError``.
+arrays, in every mode of the reference's constructor: most recent or uniformly drawn
+neighbours (``recent``), cursors or binary search in later layers (``prop_time``),
+snapshots of a sliding window (``num_history``, ``window_duration``). The uniform draws
+are the reference's own (its per-thread ``rand_r`` streams are a function of
+``num_thread_per_worker * num_workers``). ``GpuParallelSampler`` is the most-recent mode
+with the T-CSR and the cursors on the device.
 """
 import ctypes
 
@@ -55,10 +58,8 @@ class TemporalGraphBlock:
 class ParallelSampler:
     def __init__(self, indptr, indices, eid, ts, num_thread_per_worker, num_workers, num_layers,
                  num_neighbors, recent, prop_time, num_history, window_duration):
-        if not recent:
-            raise NotImplementedError("only recent=True (most-recent-k neighbours) is built")
-        if num_history != 1 or abs(window_duration) > 1e-7:
-            raise NotImplementedError("only num_history=1, window_duration=0 is built")
+        if int(num_history) < 1:
+            raise ValueError("num_history must be at least 1")
         self._indptr = np.ascontiguousarray(indptr, dtype=np.int32)
         self._indices = np.ascontiguousarray(indices, dtype=np.int32)
         self._eid = np.ascontiguousarray(eid, dtype=np.int32)
@@ -67,11 +68,14 @@ class ParallelSampler:
         if fan.shape[0] < num_layers:
             raise ValueError("num_neighbors needs one entry per layer")
         p = lambda a: ctypes.c_void_p(a.ctypes.data)
-        self._h = _host.lib().yitu_sampler_create(
+        create = _host.lib().yitu_sampler_create_modes
+        create.restype = ctypes.c_void_p
+        self._h = create(
             p(self._indptr), p(self._indices), p(self._eid), p(self._ts),
             ctypes.c_int64(self._indptr.shape[0] - 1), ctypes.c_int64(self._indices.shape[0]),
             ctypes.c_int(int(num_thread_per_worker) * int(num_workers)), ctypes.c_int(num_layers),
-            p(fan), ctypes.c_int(int(bool(prop_time))))
+            p(fan), ctypes.c_int(int(bool(recent))), ctypes.c_int(int(bool(prop_time))),
+            ctypes.c_int(int(num_history)), ctypes.c_float(float(window_duration)))
         if not self._h:
             raise RuntimeError("invalid T-CSR passed to ParallelSampler")
         self._ret = []
