@@ -587,6 +587,39 @@ int yitu_tsample_recent(int32_t *row_device, int32_t *col_device, int32_t *eid_o
                         int fan, int prop_time, void *workspace_device, size_t workspace_bytes,
                         void *stream);
 
+/*
+ * The other modes of ParallelSampler (sampler_core.cpp:201-359), as the two pieces its
+ * sample() strings together per layer and snapshot.
+ * yitu_tsample_advance: update_ts_ptr (:103-127) for one cursor array [n_nodes]: the
+ * cursor of every root's node moves to the last edge with ts <= t + offset - 1e-7,
+ * never backwards.
+ * yitu_tsample_window: one snapshot of one layer (:216-333). The window [lo, hi] of a
+ * root is read from two cursor arrays, or, with both null, found by binary search:
+ * [first edge, last edge with ts <= t] (windowed = 0), or [last edge with ts <= t +
+ * offset - window, last edge with ts <= t + offset] (windowed = 1: num_history > 1).
+ * recent = 1 keeps the `fan` most recent edges of the window; recent = 0 makes `fan`
+ * draws lo + rand_r() % (hi - lo + 1) when the window holds at least `fan` edges
+ * (:306-318), from the generators of the reference's threads: thread c owns the roots
+ * [c chunk, (c + 1) chunk), chunk = ceil(n_roots / threads), and rand_r state c (the C
+ * library's rand_r, restated in the kernel; a root's state is reached by skipping
+ * ahead, so the result does not depend on how the device schedules the roots). Edges
+ * not older than t + offset - 1e-7 are dropped either way. Outputs as
+ * yitu_tsample_recent's. Same bits as the host library in every mode.
+ */
+int yitu_tsample_advance(int32_t *cursor_device, const int32_t *indptr_device,
+                         const float *ts_device, int64_t n_nodes, const int32_t *roots_device,
+                         const float *root_ts_device, int64_t n_roots, float offset, void *stream);
+size_t yitu_tsample_window_workspace_bytes(int64_t n_roots);
+int yitu_tsample_window(int32_t *row_device, int32_t *col_device, int32_t *eid_out_device,
+                        float *ts_out_device, float *dts_out_device, int32_t *nodes_out_device,
+                        long long *n_edges_device, const int32_t *lo_cursor_device,
+                        const int32_t *hi_cursor_device, const int32_t *indptr_device,
+                        const int32_t *indices_device, const int32_t *eid_device,
+                        const float *ts_device, int64_t n_nodes, const int32_t *roots_device,
+                        const float *root_ts_device, int64_t n_roots, int fan, int prop_time,
+                        int recent, int windowed, float offset, float window, int64_t chunk,
+                        void *workspace_device, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Graph preparation                                                           */
 /* ------------------------------------------------------------------------- */

@@ -117,3 +117,79 @@ def test_device_block_feeds_the_attention_layer(dev):
     a = layer(TemporalBlock.from_sampler(host.get_ret()[0], memory, device=dev))
     b = layer(TemporalBlock.from_device_block(gpu.get_ret()[0], memory))
     assert torch.equal(a, b)
+
+
+MODES = np.load(os.path.join(ROOT, "tests", "golden", "sampler_modes.npz"))
+
+
+@pytest.mark.parametrize("case", range(int(MODES["n_cases"])))
+def test_other_modes_match_reference_golden_vectors(dev, case):
+    """Uniform draws for 1 / 2 / 5 nominal threads, a second layer by binary search,
+    prop_time, 2 and 3 window snapshots: every block of every batch bit for bit against
+    what the compiled reference returned (tests/golden/make_sampler_golden.py)."""
+    pre = "c%d_" % case
+    threads, layers, recent, prop_time, hist = (int(v) for v in MODES[pre + "args"])
+    s = sampler_core.GpuParallelSampler(MODES[pre + "indptr"], MODES[pre + "indices"],
+                                        MODES[pre + "eid"], MODES[pre + "ts"], threads, 1, layers,
+                                        [int(v) for v in MODES[pre + "fans"]], bool(recent),
+                                        bool(prop_time), hist, float(MODES[pre + "window"]),
+                                        device=dev)
+    for b in range(int(MODES[pre + "n_batches"])):
+        bp = pre + "b%d_" % b
+        s.sample(MODES[bp + "roots"], MODES[bp + "root_ts"])
+        ret = s.get_ret()
+        assert len(ret) == int(MODES[bp + "n_blocks"]) == layers * hist
+        for r, blk in enumerate(ret):
+            got = blk.cpu_block()
+            for f in FIELDS:
+                want = MODES[bp + "r%d_" % r + f]
+                assert getattr(got, f)().dtype == want.dtype, (case, b, r, f)
+                assert np.array_equal(getattr(got, f)(), want), (case, b, r, f)
+            assert [got.dim_in(), got.dim_out()] == MODES[bp + "r%d_dims" % r].tolist()
+
+
+@pytest.mark.parametrize("threads,layers,fans,recent,prop,hist,window", [
+    (16, 1, [20], False, False, 1, 0.0),      # uniform draws, many roots per chunk
+    (3, 2, [6, 4], False, False, 1, 0.0),     # second layer by binary search
+    (1, 1, [5], False, True, 1, 0.0),
+    (4, 1, [8], True, False, 3, 40.0),        # most recent of three window snapshots
+    (5, 2, [4, 3], False, False, 2, 60.0),    # uniform draws inside window snapshots, two layers
+    (2, 2, [3, 3], True, False, 2, 50.0),     # cursors in both layers
+])
+def test_other_modes_equal_host_sampler_over_a_stream_of_batches(dev, threads, layers, fans, recent,
+                                                                prop, hist, window):
+    rng = np.random.default_rng(11 + threads)
+    indptr, indices, eid, tt, src, dst, ts = _tcsr(rng, 300, 8000)
+    args = (indptr, indices, eid, tt, threads, 1, layers, fans, recent, prop, hist, window)
+    host = sampler_core.ParallelSampler(*args)
+    gpu = sampler_core.GpuParallelSampler(*args, device=dev)
+    batches = [np.arange(i, i + 200) for i in range(0, 8000, 1600)]
+    batches += [rng.integers(0, 8000, 300), np.full(50, 4000), rng.integers(0, 500, 100),
+                np.arange(7)]
+    for bi, ev in enumerate(batches):
+        roots = np.concatenate([src[ev], dst[ev]])
+        rts = np.concatenate([ts[ev], ts[ev]])
+        host.sample(roots, rts)
+        gpu.sample(roots, rts)
+        hb, gb = host.get_ret(), gpu.get_ret()
+        assert len(hb) == len(gb) == layers * hist
+        for l in range(len(hb)):
+            _same(gb[l], hb[l], (bi, l))
+    host.reset()
+    gpu.reset()
+    ev = batches[-2]
+    host.sample(src[ev], ts[ev])
+    gpu.sample(src[ev], ts[ev])
+    for l in range(layers * hist):
+        _same(gpu.get_ret()[l], host.get_ret()[l], ("after reset", l))
+
+
+def test_uniform_mode_bad_root_and_empty_batch(dev):
+    rng = np.random.default_rng(1)
+    indptr, indices, eid, tt, *_ = _tcsr(rng, 50, 400)
+    gpu = sampler_core.GpuParallelSampler(indptr, indices, eid, tt, 2, 1, 1, [4], False, False, 2,
+                                          10.0, device=dev)
+    gpu.sample(np.zeros(0, np.int32), np.zeros(0, np.float32))
+    assert [b.dim_in() for b in gpu.get_ret()] == [0, 0]
+    with pytest.raises(RuntimeError, match="out of range"):
+        gpu.sample(np.array([3, 50]), np.array([10.0, 10.0]))

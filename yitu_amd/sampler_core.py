@@ -157,17 +157,19 @@ class DeviceTemporalGraphBlock:
 
 
 class GpuParallelSampler:
-    """ParallelSampler (recent = True, one snapshot) with the T-CSR and the cursors
-    in device memory (yitu_tsample_recent): same constructor arguments, same
-    results bit for bit, blocks returned as DeviceTemporalGraphBlock."""
+    """ParallelSampler with the T-CSR and the cursors in device memory: same constructor
+    arguments, same results bit for bit in every mode (the uniform draws included: a
+    root's generator state is reached by skipping ahead in its nominal thread's
+    sequence), blocks returned as DeviceTemporalGraphBlock. The most-recent,
+    single-snapshot mode runs as one call per layer (yitu_tsample_recent); the other
+    modes string yitu_tsample_advance / yitu_tsample_window together per layer and
+    snapshot the way the reference's sample() does (sampler_core.cpp:337-359)."""
 
     def __init__(self, indptr, indices, eid, ts, num_thread_per_worker, num_workers, num_layers,
                  num_neighbors, recent, prop_time, num_history, window_duration, device="cuda"):
         import torch
-        if not recent:
-            raise NotImplementedError("only recent=True (most-recent-k neighbours) is built")
-        if num_history != 1 or abs(window_duration) > 1e-7:
-            raise NotImplementedError("only num_history=1, window_duration=0 is built")
+        if int(num_history) < 1:
+            raise ValueError("num_history must be at least 1")
         if len(num_neighbors) < num_layers:
             raise ValueError("num_neighbors needs one entry per layer")
         self._dev = torch.device(device)
@@ -179,40 +181,90 @@ class GpuParallelSampler:
         self._n_nodes = self._indptr.numel() - 1
         self._fan = [int(x) for x in num_neighbors[:num_layers]]
         self._prop_time = bool(prop_time)
-        self._cursor = torch.empty(max(self._n_nodes, 1), dtype=torch.int32, device=self._dev)
+        self._recent = bool(recent)
+        self._hist = int(num_history)
+        self._window = float(np.float32(window_duration))
+        self._threads = max(1, int(num_thread_per_worker) * int(num_workers))
+        self._simple = self._recent and self._hist == 1 and abs(self._window) <= 1e-7
+        # cursor k of a node, k = 0 .. num_history (ts_ptr of the reference, :57-58)
+        self._cursors = torch.empty(self._hist + 1, max(self._n_nodes, 1), dtype=torch.int32,
+                                    device=self._dev)
+        self._cursor = self._cursors[self._hist]
         self._ret = []
         self.reset()
 
     def reset(self):
         from . import _lib
-        rc = _lib.lib().yitu_tsample_reset(_lib.ptr(self._cursor), _lib.ptr(self._indptr),
-                                           _lib.c_i64(self._n_nodes), _lib.stream_ptr(self._dev))
-        _lib.check(rc, "yitu_tsample_reset")
+        for k in range(self._hist + 1):
+            rc = _lib.lib().yitu_tsample_reset(_lib.ptr(self._cursors[k]), _lib.ptr(self._indptr),
+                                               _lib.c_i64(self._n_nodes),
+                                               _lib.stream_ptr(self._dev))
+            _lib.check(rc, "yitu_tsample_reset")
 
-    def _layer(self, roots, root_ts, fan):
+    def _outputs(self, n, fan):
         import torch
-        from . import _lib
-        n = roots.numel()
         i32 = lambda m: torch.empty(max(m, 1), dtype=torch.int32, device=self._dev)
         f32 = lambda m: torch.empty(max(m, 1), dtype=torch.float32, device=self._dev)
-        row, col, eid = i32(n * fan), i32(n * fan), i32(n * fan)
-        ts, dts, nodes = f32(n * (fan + 1)), f32(n * (fan + 1)), i32(n * (fan + 1))
-        count = torch.empty(1, dtype=torch.int64, device=self._dev)
-        ws = _lib.workspace(_lib.size_fn("yitu_tsample_workspace_bytes")(_lib.c_i64(n)), self._dev)
-        with torch.cuda.device(self._dev):
-            rc = _lib.lib().yitu_tsample_recent(
-                _lib.ptr(row), _lib.ptr(col), _lib.ptr(eid), _lib.ptr(ts), _lib.ptr(dts),
-                _lib.ptr(nodes), _lib.ptr(count), _lib.ptr(self._cursor), _lib.ptr(self._indptr),
-                _lib.ptr(self._indices), _lib.ptr(self._eid), _lib.ptr(self._ts),
-                _lib.c_i64(self._n_nodes), _lib.ptr(roots), _lib.ptr(root_ts), _lib.c_i64(n),
-                _lib.c_int(fan), _lib.c_int(int(self._prop_time)), _lib.ptr(ws),
-                _lib.c_size(ws.numel()), _lib.stream_ptr(self._dev))
-        _lib.check(rc, "yitu_tsample_recent")
+        return (i32(n * fan), i32(n * fan), i32(n * fan), f32(n * (fan + 1)), f32(n * (fan + 1)),
+                i32(n * (fan + 1)), torch.empty(1, dtype=torch.int64, device=self._dev))
+
+    def _block(self, outs, n):
+        row, col, eid, ts, dts, nodes, count = outs
         m = int(count.item())
         if m < 0:
             raise RuntimeError("sample failed: a root node id is out of range")
         return DeviceTemporalGraphBlock(row[:m], col[:m], eid[:m], ts[:n + m], dts[:n + m],
                                         nodes[:n + m], n + m, n)
+
+    def _layer(self, roots, root_ts, fan):
+        import torch
+        from . import _lib
+        n = roots.numel()
+        outs = self._outputs(n, fan)
+        ws = _lib.workspace(_lib.size_fn("yitu_tsample_workspace_bytes")(_lib.c_i64(n)), self._dev)
+        with torch.cuda.device(self._dev):
+            rc = _lib.lib().yitu_tsample_recent(
+                *[_lib.ptr(t) for t in outs], _lib.ptr(self._cursor), _lib.ptr(self._indptr),
+                _lib.ptr(self._indices), _lib.ptr(self._eid), _lib.ptr(self._ts),
+                _lib.c_i64(self._n_nodes), _lib.ptr(roots), _lib.ptr(root_ts), _lib.c_i64(n),
+                _lib.c_int(fan), _lib.c_int(int(self._prop_time)), _lib.ptr(ws),
+                _lib.c_size(ws.numel()), _lib.stream_ptr(self._dev))
+        _lib.check(rc, "yitu_tsample_recent")
+        return self._block(outs, n)
+
+    def _advance(self, k, roots, root_ts, offset):
+        import torch
+        from . import _lib
+        with torch.cuda.device(self._dev):
+            rc = _lib.lib().yitu_tsample_advance(
+                _lib.ptr(self._cursors[k]), _lib.ptr(self._indptr), _lib.ptr(self._ts),
+                _lib.c_i64(self._n_nodes), _lib.ptr(roots), _lib.ptr(root_ts),
+                _lib.c_i64(roots.numel()), _lib.c_f32(offset), _lib.stream_ptr(self._dev))
+        _lib.check(rc, "yitu_tsample_advance")
+
+    def _snapshot(self, roots, root_ts, fan, use_ptr, i):
+        import torch
+        from . import _lib
+        n = roots.numel()
+        outs = self._outputs(n, fan)
+        ws = _lib.workspace(_lib.size_fn("yitu_tsample_window_workspace_bytes")(_lib.c_i64(n)),
+                            self._dev)
+        offset = float(-np.float32(i) * np.float32(self._window))
+        # the reference's static chunk of roots per thread, computed in float as it does (:239)
+        chunk = int(np.ceil(np.float32(n) / np.float32(self._threads))) if n else 1
+        lo = self._cursors[self._hist - 1 - i] if use_ptr else None
+        hi = self._cursors[self._hist - i] if use_ptr else None
+        with torch.cuda.device(self._dev):
+            rc = _lib.lib().yitu_tsample_window(
+                *[_lib.ptr(t) for t in outs], _lib.ptr(lo), _lib.ptr(hi), _lib.ptr(self._indptr),
+                _lib.ptr(self._indices), _lib.ptr(self._eid), _lib.ptr(self._ts),
+                _lib.c_i64(self._n_nodes), _lib.ptr(roots), _lib.ptr(root_ts), _lib.c_i64(n),
+                _lib.c_int(fan), _lib.c_int(int(self._prop_time)), _lib.c_int(int(self._recent)),
+                _lib.c_int(int(self._hist > 1)), _lib.c_f32(offset), _lib.c_f32(self._window),
+                _lib.c_i64(chunk), _lib.ptr(ws), _lib.c_size(ws.numel()),
+                _lib.stream_ptr(self._dev))
+        _lib.check(rc, "yitu_tsample_window")
+        return self._block(outs, n)
 
     def sample(self, root_nodes, root_ts):
         import torch
@@ -221,11 +273,35 @@ class GpuParallelSampler:
         if roots.shape != ts.shape or roots.dim() != 1:
             raise ValueError("root_nodes and root_ts must be 1-D and equally long")
         self._ret = []
-        for fan in self._fan:
-            blk = self._layer(roots, ts, fan)
-            self._ret.append(blk)
-            # the next layer expands every node of this block (roots and neighbours)
-            roots, ts = blk.nodes(), blk.ts()
+        if self._simple:
+            for fan in self._fan:
+                blk = self._layer(roots, ts, fan)
+                self._ret.append(blk)
+                # the next layer expands every node of this block (roots and neighbours)
+                roots, ts = blk.nodes(), blk.ts()
+            return
+        H = self._hist
+        first_layer = True
+        for layer, fan in enumerate(self._fan):
+            self._ret.extend([None] * H)
+            n_blocks = len(self._ret)
+            use_ptr = first_layer or (self._prop_time and H == 1) or self._recent
+            first_layer = False
+
+            def layer_roots(i):
+                if layer == 0:
+                    return roots, ts
+                prev = self._ret[n_blocks - 1 - i - H]
+                return prev.nodes(), prev.ts()
+
+            if use_ptr:
+                self._advance(H, *layer_roots(0), 0.0)
+            for i in range(H):
+                r, t = layer_roots(i)
+                if use_ptr and abs(self._window) > 1e-7:
+                    off = np.float32(-np.float32(i) * np.float32(self._window)) - np.float32(self._window)
+                    self._advance(H - 1 - i, r, t, float(off))
+                self._ret[n_blocks - 1 - i] = self._snapshot(r, t, fan, use_ptr, i)
 
     def get_ret(self):
         return list(self._ret)
