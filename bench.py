@@ -413,11 +413,24 @@ def run_gat_c3(args, dev):
     alg_fwd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h + 8 * n * h * f
     alg_bwd = (2 * 4 * n * h * f + 4 * nnz * h + 8 * nnz + 8 * (n + 1) + 4 * nnz
                + 4 * n * h * f + 8 * n * h)
+    # the stand-alone SDDMM + LeakyReLU + edge softmax on the same graph (one query block)
+    q1 = q.unsqueeze(0).contiguous()
+    attn_sa = graph_ext.sddmm_forward(rp, ci, q1, k)
+    ga = torch.randn(nnz, h, generator=g, device=dev)
+    sd_fwd_ms = _event_ms(lambda: graph_ext.sddmm_forward(rp, ci, q1, k), args.steps, args.warmup)
+    sd_bwd_ms = _event_ms(lambda: graph_ext.sddmm_backward(rp, ci, q1, k, attn_sa, ga), args.steps,
+                          args.warmup)
+    alg_sd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h
     return {
         "metric": "GAT attention fwd+bwd (fused SDDMM+LeakyReLU+softmax+aggregate), edges/sec",
         "value": nnz / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "sddmm": {"fwd_ms": sd_fwd_ms, "bwd_ms": sd_bwd_ms,
+                  "edges_per_s_fwd_bwd": nnz / ((sd_fwd_ms + sd_bwd_ms) * 1e-3),
+                  "fwd_algorithmic_bytes": alg_sd,
+                  "fwd_GBps": alg_sd / (sd_fwd_ms * 1e-3) / 1e9,
+                  "fwd_hbm_frac": alg_sd / (sd_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "config": {"workload": "c3_gat_f32", "graph": "R-MAT scale 21, 63M draws dedup + self "
                    "loops, reordered, CSR by destination", "n_nodes": n, "n_edges": nnz, "heads": h,
                    "head_dim": f},

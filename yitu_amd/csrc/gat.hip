@@ -896,6 +896,12 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams
     }
 }
 
+}  // namespace yitu
+
+#include "attn_packed.hpp"
+
+namespace yitu {
+
 // ---- backward over the transposed structure: one gather for every gradient -------
 // Walking the edges by source c, the source's own row x[c] is local and the
 // gathered row is grad_out[row_e]. That single gather gives both
@@ -1555,6 +1561,13 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
 }
 
 // ---- attention only: host side ---------------------------------------------------
+// every pointer aligned to a vector of hv floats
+static bool vec_aligned(int hv, const void *a, const void *b, const void *c) {
+    const uintptr_t m = (uintptr_t)hv * sizeof(float) - 1;
+    return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+             reinterpret_cast<uintptr_t>(c)) & m) == 0;
+}
+
 size_t attn_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t H) {
     return align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * H), 256) +
            align_up(sizeof(float) * 2 * (size_t)(n_dst * H), 256);
@@ -1584,8 +1597,19 @@ int attn_forward_run(float *attn, const int32_t *indptr, const int32_t *indices,
                           max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
     if (rc) return rc;
     if (!has_items) p.sp.plan.threshold = 0x7fffffff;
-    attn_rows_kernel<<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
-                       kBlock, 0, stream>>>(p);
+    // one lane per edge whenever the heads of an edge are a few aligned vectors
+    const int hv = packed_head_vec(p.sp.H);
+    const bool packed = packed_heads_ok(p.sp.H) && vec_aligned(hv, query, key, attn);
+    if (packed) {
+        const int R = packed_rows_per_wave(p.sp.n_rows);
+        const int grid = (int)ceil_div(p.sp.n_rows, (int64_t)kWavesPerBlock * R);
+        if (hv == 4) attn_rows_packed_kernel<4><<<grid, kBlock, 0, stream>>>(p, R);
+        else if (hv == 2) attn_rows_packed_kernel<2><<<grid, kBlock, 0, stream>>>(p, R);
+        else attn_rows_packed_kernel<1><<<grid, kBlock, 0, stream>>>(p, R);
+    } else {
+        attn_rows_kernel<<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
+                           kBlock, 0, stream>>>(p);
+    }
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);
@@ -1596,13 +1620,20 @@ int attn_forward_run(float *attn, const int32_t *indptr, const int32_t *indices,
     p.row_stats = reinterpret_cast<float *>(w);
     const int item_grid = (int)std::min<int64_t>(
         ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
-    gat_item_stats_kernel<<<item_grid, kBlock, 0, stream>>>(p);
+    const int packed_grid = packed_item_grid(p.sp.plan.max_items);
+    if (packed && hv == 4) attn_item_stats_packed_kernel<4><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed && hv == 2) attn_item_stats_packed_kernel<2><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed) attn_item_stats_packed_kernel<1><<<packed_grid, kBlock, 0, stream>>>(p);
+    else gat_item_stats_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     gat_row_combine_kernel<<<(int)std::min<int64_t>(
                                  ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15),
                              kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    attn_item_write_kernel<<<item_grid, kBlock, 0, stream>>>(p);
+    if (packed && hv == 4) attn_item_write_packed_kernel<4><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed && hv == 2) attn_item_write_packed_kernel<2><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed) attn_item_write_packed_kernel<1><<<packed_grid, kBlock, 0, stream>>>(p);
+    else attn_item_write_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     return 0;
 }
@@ -1637,9 +1668,20 @@ int attn_backward_run(float *grad_query, float *grad_edge, const int32_t *indptr
                           max_degree, workspace, workspace_bytes, &rest, &rest_bytes, stream);
     if (rc) return rc;
     if (!has_items) p.sp.plan.threshold = 0x7fffffff;
-    attn_bwd_rows_kernel<<<(int)ceil_div(p.sp.n_rows,
-                                         kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
-                           kBlock, 0, stream>>>(p);
+    const int hv = packed_head_vec(p.sp.H);
+    const bool packed = packed_heads_ok(p.sp.H) && vec_aligned(hv, query, key, attn) &&
+                        vec_aligned(hv, grad_attn, grad_query, grad_edge);
+    if (packed) {
+        const int R = packed_rows_per_wave(p.sp.n_rows);
+        const int grid = (int)ceil_div(p.sp.n_rows, (int64_t)kWavesPerBlock * R);
+        if (hv == 4) attn_bwd_rows_packed_kernel<4><<<grid, kBlock, 0, stream>>>(p, R);
+        else if (hv == 2) attn_bwd_rows_packed_kernel<2><<<grid, kBlock, 0, stream>>>(p, R);
+        else attn_bwd_rows_packed_kernel<1><<<grid, kBlock, 0, stream>>>(p, R);
+    } else {
+        attn_bwd_rows_kernel<<<(int)ceil_div(p.sp.n_rows,
+                                             kWavesPerBlock * rows_per_wave(p.sp.n_rows)),
+                               kBlock, 0, stream>>>(p);
+    }
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const size_t need = attn_workspace_bytes(n_dst, nnz, n_heads);
@@ -1648,19 +1690,22 @@ int attn_backward_run(float *grad_query, float *grad_edge, const int32_t *indptr
     p.item_sums = reinterpret_cast<float *>(w);
     w += align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * n_heads), 256);
     p.row_sum = reinterpret_cast<float *>(w);
-    attn_bwd_item_sums_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
-                                                                kWavesPerBlock * kItemsPerWave),
-                                                       1 << 16),
-                                kBlock, 0, stream>>>(p);
+    const int item_grid = (int)std::min<int64_t>(
+        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+    const int packed_grid = packed_item_grid(p.sp.plan.max_items);
+    if (packed && hv == 4) attn_bwd_item_sums_packed_kernel<4><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed && hv == 2) attn_bwd_item_sums_packed_kernel<2><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed) attn_bwd_item_sums_packed_kernel<1><<<packed_grid, kBlock, 0, stream>>>(p);
+    else attn_bwd_item_sums_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     gat_bwd_combine_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock),
                                                     1 << 15),
                              kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
-    gat_bwd_apply_kernel<<<(int)std::min<int64_t>(ceil_div(p.sp.plan.max_items,
-                                                           kWavesPerBlock * kItemsPerWave),
-                                                  1 << 16),
-                           kBlock, 0, stream>>>(p);
+    if (packed && hv == 4) attn_bwd_apply_packed_kernel<4><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed && hv == 2) attn_bwd_apply_packed_kernel<2><<<packed_grid, kBlock, 0, stream>>>(p);
+    else if (packed) attn_bwd_apply_packed_kernel<1><<<packed_grid, kBlock, 0, stream>>>(p);
+    else gat_bwd_apply_kernel<<<item_grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     return 0;
 }

@@ -1,5 +1,5 @@
 // Instantiation table and host-side launch logic of the row-split SpMM.
-#include "spmm_rows.hpp"
+#include "packed_rows.hpp"
 
 #include <cstdarg>
 
@@ -96,8 +96,9 @@ static int dispatch_shape(const SpmmParams &p, bool with_hub, hipStream_t stream
 // Unweighted fp32 rows of 1, 2 or 4 floats: one lane per edge.
 template <int VEC>
 static int launch_tiny(const SpmmParams &p, bool has_items, hipStream_t stream) {
-    tiny_rows_kernel<VEC>
-        <<<(int)ceil_div(p.n_rows, kWavesPerBlock * rows_per_wave(p.n_rows)), kBlock, 0, stream>>>(p);
+    const int R = packed_rows_per_wave(p.n_rows);
+    tiny_rows_packed_kernel<VEC>
+        <<<(int)ceil_div(p.n_rows, (int64_t)kWavesPerBlock * R), kBlock, 0, stream>>>(p, R);
     YITU_LAUNCH_CHECK();
     if (has_items && p.cols_are_edges) {
         // a row's edges are contiguous: sum them in place, no items

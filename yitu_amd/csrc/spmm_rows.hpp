@@ -543,11 +543,6 @@ __device__ __forceinline__ void tiny_rows_body(const SpmmParams &p, int block) {
 }
 
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void tiny_rows_kernel(SpmmParams p) {
-    tiny_rows_body<VEC>(p, blockIdx.x);
-}
-
-template <int VEC>
 __global__ __launch_bounds__(kBlock) void tiny_items_kernel(SpmmParams p) {
     const int lane = lane_id();
     if (p.plan.counters->overflow) return;
