@@ -148,11 +148,25 @@ __device__ __forceinline__ float wave_max_strided(float v) {
     for (int o = 32; o >= STRIDE; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
     return v;
 }
-// Sum over aligned groups of WIDTH consecutive lanes.
+// One lane permutation inside rows of 16 lanes on the vector ALU's data-parallel
+// primitives: no LDS round trip, which is what __shfl_xor compiles to.
+template <int CTRL>
+__device__ __forceinline__ float dpp_permute(float v) {
+    return __int_as_float(
+        __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// Sum over aligned groups of WIDTH consecutive lanes, left in every lane of the group.
+// Up to 16 lanes: pairs, quads (quad permutes), halves of a row (mirror inside 8 lanes),
+// rows (mirror inside 16 lanes); beyond that, shuffles across rows. The order of the
+// additions is fixed.
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int o = WIDTH / 2; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
+    if constexpr (WIDTH >= 2) v += dpp_permute<0xb1>(v);   // quad_perm [1,0,3,2]
+    if constexpr (WIDTH >= 4) v += dpp_permute<0x4e>(v);   // quad_perm [2,3,0,1]
+    if constexpr (WIDTH >= 8) v += dpp_permute<0x141>(v);  // row_half_mirror
+    if constexpr (WIDTH >= 16) v += dpp_permute<0x140>(v); // row_mirror
+    if constexpr (WIDTH >= 32) v += __shfl_xor(v, 16, kWave);
+    if constexpr (WIDTH >= 64) v += __shfl_xor(v, 32, kWave);
     return v;
 }
 

@@ -969,8 +969,7 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float4 *__restrict_
 #pragma unroll
             for (int t = 0; t < KT; t++) {
                 float s = d[u][t];
-#pragma unroll
-                for (int o = LPH >> 1; o >= 1; o >>= 1) s += __shfl_xor(s, o, kWave);
+                s = group_sum<LPH>(s);
                 const int head = t * HPT + lane / LPH;
                 if (lane % LPH == 0 && r < n_rows) {
                     const size_t at = (size_t)r * H + head;
@@ -1048,8 +1047,7 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
                     for (int t = 0; t < KT; t++) {
                         float d = xt[t][0] * v[u][t][0] + xt[t][1] * v[u][t][1] +
                                   xt[t][2] * v[u][t][2] + xt[t][3] * v[u][t][3];
-#pragma unroll
-                        for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                        d = group_sum<LPH>(d);
                         if (sub == kk + u) keep[t] = d * g_scale;
 #pragma unroll
                         for (int i = 0; i < 4; i++) acc[t][i] += a[u][t] * v[u][t][i];
@@ -1104,8 +1102,7 @@ __device__ __forceinline__ void gat_src_end(float *x_dst, float *k_dst, const fl
         store_row<4>(x_dst + t * 256 + lane * 4, acc[t]);
         if constexpr (FULL) {
             float s = gk[t];
-#pragma unroll
-            for (int o = LPH >> 1; o >= 1; o >>= 1) s += __shfl_xor(s, o, kWave);
+            s = group_sum<LPH>(s);
             if (lane % LPH == 0) k_dst[t * (kWave / LPH) + lane / LPH] = s;
         }
     }
@@ -1275,8 +1272,7 @@ __device__ __forceinline__ void slot_window(SlotRow<LPH> &row, const GatSrcParam
             for (int h = 0; h < H; h++) {
                 float d = row.xh[h][0] * v[u][0] + row.xh[h][1] * v[u][1] + row.xh[h][2] * v[u][2] +
                           row.xh[h][3] * v[u][3];
-#pragma unroll
-                for (int o = LPH >> 1; o >= 1; o >>= 1) d += __shfl_xor(d, o, kWave);
+                d = group_sum<LPH>(d);
                 if (sub == h) mine = d;
                 const float w = valid[u] ? a[u][h] * p.g_scale : 0.0f;
 #pragma unroll
