@@ -78,7 +78,211 @@ __global__ __launch_bounds__(kBlock) void attn_rows_packed_kernel(GatParams p, i
                 }
             }
         },
-        [&](int row, int beg, int end) { attn_big_row<HV>(p, row, beg, end); }, [](int) {});
+        [&](int row, int beg, int end) { attn_big_row<HV>(p, row, beg, end); },
+        [](int, unsigned long long) {});
+}
+
+// ---- fused attention + aggregate on short rows, rows of 256 KT floats at most ------
+// Phase A is the packed softmax above, kept in registers: lane e ends up with the
+// probabilities of edge e for every head (H <= 4 HV). Phase B walks the rows of the chunk
+// one after the other: an edge is one wave-wide gather of its source's feature row (a lane
+// holds 4 floats of each of the KT tiles), weighted by the probability of the lane's head,
+// which reaches the lane as a scalar read of the edge's lane. The (edge, head)-per-lane
+// kernel did phase A row by row (a dependent load chain and several hundred instructions
+// per row, whatever its length) and was bound by instruction issue, not by the gathers.
+constexpr int kPackedGroups = 4;  // head groups of HV heads a lane can hold
+
+template <int HV, int KT>
+struct PackedGat {
+    const GatParams &p;
+    const float *__restrict__ feat;
+    TileLanes<4, kWave, KT, W_EDGEHEAD> tl;
+    int groups;
+
+    __device__ __forceinline__ PackedGat(const GatParams &p_)
+        : p(p_), feat(static_cast<const float *>(p_.sp.feat)), tl(p_.sp, 0),
+          groups(p_.sp.H / HV) {}
+
+    // acc += sum over the edges held by lanes [k, last] of prob[lane's head] * x[col]
+    __device__ __forceinline__ void apply(float (&acc)[KT][4], int col,
+                                          const float (&pr)[kPackedGroups][HV], int k,
+                                          int last) const {
+        constexpr int U = KT >= 4 ? 2 : 4;  // row gathers in flight
+        const int L = p.sp.L;
+        for (; k <= last; k += U) {
+            float v[U][KT][4], w[U][KT];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int ek = min(k + u, last);  // past the end: the last edge again, weight 0
+                const int c = __builtin_amdgcn_readlane(col, ek);
+#pragma unroll
+                for (int t = 0; t < KT; t++) {
+                    RowLoad<4, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                    w[u][t] = 0.0f;
+                }
+#pragma unroll
+                for (int g = 0; g < kPackedGroups; g++) {
+                    if (g >= groups) break;  // wave-uniform
+#pragma unroll
+                    for (int h = 0; h < HV; h++) {
+                        const float ph = __int_as_float(
+                            __builtin_amdgcn_readlane(__float_as_int(pr[g][h]), ek));
+#pragma unroll
+                        for (int t = 0; t < KT; t++)
+                            if (tl.head[t] == g * HV + h) w[u][t] = ph;
+                    }
+                }
+                if (k + u > last) {
+#pragma unroll
+                    for (int t = 0; t < KT; t++) w[u][t] = 0.0f;
+                }
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+                    if (!tl.live[t]) w[u][t] = 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[t][i] += w[u][t] * v[u][t][i];
+        }
+    }
+
+    __device__ __forceinline__ void store(int row, const float (&acc)[KT][4]) const {
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+            const int o = (t * kWave + lane_id()) * 4;
+            if (o < p.sp.L) store_row<4>(p.sp.out + (size_t)row * p.sp.L + o, acc[t]);
+        }
+    }
+};
+
+template <int HV, int KT>
+__global__ __launch_bounds__(kBlock) void gat_rows_packed_kernel(GatParams p, int R) {
+    const int lane = lane_id();
+    const int H = p.sp.H;
+    const PackedGat<HV, KT> pg(p);
+    packed_walk(
+        p.sp, R, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave,
+        [&](const PackedChunk &c) {
+            const bool act = lane < c.n;
+            const int e = c.base + min(lane, c.n - 1);
+            const int col = p.sp.indices[e] & kColMask;
+            float pr[kPackedGroups][HV];
+#pragma unroll
+            for (int g = 0; g < kPackedGroups; g++) {
+#pragma unroll
+                for (int h = 0; h < HV; h++) pr[g][h] = 0.0f;
+                if (g >= pg.groups) continue;  // wave-uniform
+                const int h0 = g * HV;
+                float l[HV], m[HV], s[HV], q[HV], k[HV];
+                RowLoad<HV, float>::ld(p.query + (size_t)(c.r0 + c.pos) * H + h0, q);
+                RowLoad<HV, float>::ld(p.key + (size_t)col * H + h0, k);
+#pragma unroll
+                for (int h = 0; h < HV; h++) m[h] = l[h] = act ? leaky(q[h] + k[h]) : -FLT_MAX;
+                seg_total<HV>(m, c, [](float a, float b) { return fmaxf(a, b); });
+#pragma unroll
+                for (int h = 0; h < HV; h++) l[h] = s[h] = act ? expf(l[h] - m[h]) : 0.0f;
+                seg_total<HV>(s, c, [](float a, float b) { return a + b; });
+                if (act) {
+#pragma unroll
+                    for (int h = 0; h < HV; h++) {
+                        s[h] = 1.0f / s[h];
+                        pr[g][h] = l[h] * s[h];
+                    }
+                    if (p.attn) store_row<HV>(p.attn + (size_t)e * H + h0, pr[g]);
+                    if (p.stats_out && lane == c.last) {
+#pragma unroll
+                        for (int h = 0; h < HV; h++) {
+                            p.stats_out[((size_t)(c.r0 + c.pos) * H + h0 + h) * 2] = m[h];
+                            p.stats_out[((size_t)(c.r0 + c.pos) * H + h0 + h) * 2 + 1] = s[h];
+                        }
+                    }
+                }
+            }
+            for (int k = 0; k < c.n;) {  // the rows of the chunk, one after the other
+                const int last = __builtin_amdgcn_readlane(c.last, k);
+                const int row = c.r0 + __builtin_amdgcn_readlane(c.pos, k);
+                float acc[KT][4];
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[t][i] = 0.0f;
+                pg.apply(acc, col, pr, k, last);
+                pg.store(row, acc);
+                k = last + 1;
+            }
+        },
+        [&](int row, int beg, int end) {  // more than 64 edges and no plan: two walks
+            MaxSum a[kPackedGroups][HV];
+#pragma unroll
+            for (int g = 0; g < kPackedGroups; g++) {
+#pragma unroll
+                for (int h = 0; h < HV; h++) a[g][h] = ms_init();
+                if (g >= pg.groups) continue;
+                float q[HV];
+                RowLoad<HV, float>::ld(p.query + (size_t)row * H + g * HV, q);
+                for (int e = beg + lane; e < end; e += kWave) {
+                    float k[HV];
+                    RowLoad<HV, float>::ld(
+                        p.key + (size_t)(p.sp.indices[e] & kColMask) * H + g * HV, k);
+#pragma unroll
+                    for (int h = 0; h < HV; h++) a[g][h] = ms_push(a[g][h], leaky(q[h] + k[h]));
+                }
+#pragma unroll
+                for (int h = 0; h < HV; h++) {
+                    a[g][h] = ms_wave<1>(a[g][h]);
+                    a[g][h].s = 1.0f / a[g][h].s;
+                    if (p.stats_out && lane == 0) {
+                        p.stats_out[((size_t)row * H + g * HV + h) * 2] = a[g][h].m;
+                        p.stats_out[((size_t)row * H + g * HV + h) * 2 + 1] = a[g][h].s;
+                    }
+                }
+            }
+            float acc[KT][4];
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[t][i] = 0.0f;
+            for (int b = beg; b < end; b += kWave) {
+                const int n = min(kWave, end - b);
+                const int e = b + min(lane, n - 1);
+                const int col = p.sp.indices[e] & kColMask;
+                float pr[kPackedGroups][HV];
+#pragma unroll
+                for (int g = 0; g < kPackedGroups; g++) {
+#pragma unroll
+                    for (int h = 0; h < HV; h++) pr[g][h] = 0.0f;
+                    if (g >= pg.groups) continue;
+                    float q[HV], k[HV];
+                    RowLoad<HV, float>::ld(p.query + (size_t)row * H + g * HV, q);
+                    RowLoad<HV, float>::ld(p.key + (size_t)col * H + g * HV, k);
+#pragma unroll
+                    for (int h = 0; h < HV; h++)
+                        pr[g][h] = expf(leaky(q[h] + k[h]) - a[g][h].m) * a[g][h].s;
+                    if (p.attn && lane < n) store_row<HV>(p.attn + (size_t)e * H + g * HV, pr[g]);
+                }
+                pg.apply(acc, col, pr, 0, n - 1);
+            }
+            pg.store(row, acc);
+        },
+        [&](int r0, unsigned long long empty) {
+            float z[KT][4];
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) z[t][i] = 0.0f;
+            while (empty) {  // wave-uniform: the whole wave clears one row per turn
+                const int i = __ffsll((long long)empty) - 1;
+                empty &= empty - 1;
+                pg.store(r0 + i, z);
+                if (p.stats_out && lane < H) {
+                    p.stats_out[((size_t)(r0 + i) * H + lane) * 2] = 0.0f;
+                    p.stats_out[((size_t)(r0 + i) * H + lane) * 2 + 1] = 0.0f;
+                }
+            }
+        });
 }
 
 // ---- planned rows: a software-pipelined walk over the plan's items ---------------
@@ -337,8 +541,9 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_rows_packed_kernel(GatBwdPara
             }
         },
         [&](int row, int beg, int end) { attn_bwd_big_row<HV>(p, row, beg, end); },
-        [&](int row) {
-            for (int h = 0; h < H; h++) p.grad_q[(size_t)row * H + h] = 0.0f;
+        [&](int r0, unsigned long long empty) {
+            if ((empty >> lane) & 1ull)
+                for (int h = 0; h < H; h++) p.grad_q[(size_t)(r0 + lane) * H + h] = 0.0f;
         });
 }
 

@@ -1523,11 +1523,29 @@ static size_t gat_own_bytes(int64_t n_dst, int64_t nnz, int64_t H, int64_t L) {
            align_up(sizeof(float) * (size_t)(plan_max_items(nnz) * L), 256);
 }
 
+// every pointer aligned to a vector of hv floats
+static bool vec_aligned(int hv, const void *a, const void *b, const void *c) {
+    const uintptr_t m = (uintptr_t)hv * sizeof(float) - 1;
+    return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+             reinterpret_cast<uintptr_t>(c)) & m) == 0;
+}
+
 template <int VEC, int G, int KT>
 static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
-    gat_rows_kernel<VEC, G, KT>
-        <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)), kBlock, 0,
-           stream>>>(p);
+    const int hv = packed_head_vec(p.sp.H);
+    if (G == kWave && VEC == 4 && p.sp.L <= 4 * kWave * KT && packed_heads_ok(p.sp.H) &&
+        vec_aligned(hv, p.query, p.key, p.attn)) {
+        // whole-wave rows: the short rows in the packed layout
+        const int R = packed_rows_per_wave(p.sp.n_rows);
+        const int grid = (int)ceil_div(p.sp.n_rows, (int64_t)kWavesPerBlock * R);
+        if (hv == 4) gat_rows_packed_kernel<4, KT><<<grid, kBlock, 0, stream>>>(p, R);
+        else if (hv == 2) gat_rows_packed_kernel<2, KT><<<grid, kBlock, 0, stream>>>(p, R);
+        else gat_rows_packed_kernel<1, KT><<<grid, kBlock, 0, stream>>>(p, R);
+    } else {
+        gat_rows_kernel<VEC, G, KT>
+            <<<(int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows)), kBlock, 0,
+               stream>>>(p);
+    }
     YITU_LAUNCH_CHECK();
     if (!has_items) return 0;
     const int item_grid = (int)std::min<int64_t>(
@@ -1557,13 +1575,6 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
 }
 
 // ---- attention only: host side ---------------------------------------------------
-// every pointer aligned to a vector of hv floats
-static bool vec_aligned(int hv, const void *a, const void *b, const void *c) {
-    const uintptr_t m = (uintptr_t)hv * sizeof(float) - 1;
-    return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
-             reinterpret_cast<uintptr_t>(c)) & m) == 0;
-}
-
 size_t attn_workspace_bytes(int64_t n_dst, int64_t nnz, int64_t H) {
     return align_up(sizeof(float) * 3 * (size_t)(plan_max_items(nnz) * H), 256) +
            align_up(sizeof(float) * 2 * (size_t)(n_dst * H), 256);

@@ -19,8 +19,9 @@ namespace yitu {
 
 constexpr int kPackedRows = 63;  // rows of a wave: bounds [0, 63] fill the 64 lanes
 
+// Enough waves to fill the chip several times over before a wave takes more rows.
 __host__ __device__ inline int packed_rows_per_wave(int n_rows) {
-    const int r = n_rows / 2048;
+    const int r = n_rows / 16384;
     return r < 1 ? 1 : (r > kPackedRows ? kPackedRows : r);
 }
 
@@ -86,9 +87,9 @@ __device__ __forceinline__ void wave_sum(float (&v)[HV]) {
 
 // Walks the short rows of wave `wave_id`: chunk(c) for every chunk of whole rows,
 // big(row, beg, end) for a row of more than 64 edges that no plan covers (a caller's
-// max-degree hint that was too small), empty(row) for rows without edges. Rows that the
-// plan covers are skipped. chunk and big are called by the whole wave, empty by the lane
-// that holds the row.
+// max-degree hint that was too small), empties(r0, mask) once with the mask of the rows
+// r0 + i that have no edges. Rows that the plan covers are skipped. Every call is made by
+// the whole wave.
 template <typename Chunk, typename Big, typename Empty>
 __device__ __forceinline__ void packed_walk(const SpmmParams &sp, int R, int wave_id, Chunk chunk,
                                             Big big, Empty empty) {
@@ -105,7 +106,7 @@ __device__ __forceinline__ void packed_walk(const SpmmParams &sp, int R, int wav
     const unsigned long long planned_mask = __ballot(planned);
     const unsigned long long stop =
         planned_mask | __ballot(!planned && deg > kWave) | (1ull << n_here);
-    if (is_row && deg == 0) empty(r0 + lane);
+    empty(r0, __ballot(is_row && deg == 0));
     int cur = 0;
     while (cur < n_here) {
         const int base = __shfl(my_ptr, cur, kWave);
@@ -185,11 +186,13 @@ __global__ __launch_bounds__(kBlock) void tiny_rows_packed_kernel(SpmmParams p, 
                 store_row<VEC>(p.out + (size_t)row * VEC, v);
             }
         },
-        [&](int row) {
-            float z[VEC];
+        [&](int r0, unsigned long long empty) {
+            if ((empty >> lane) & 1ull) {
+                float z[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; i++) z[i] = 0.0f;
-            store_row<VEC>(p.out + (size_t)row * VEC, z);
+                for (int i = 0; i < VEC; i++) z[i] = 0.0f;
+                store_row<VEC>(p.out + (size_t)(r0 + lane) * VEC, z);
+            }
         });
 }
 
