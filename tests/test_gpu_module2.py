@@ -421,7 +421,8 @@ def test_dtype_and_device_checks(dev):
                                 torch.randn(10, 2, device=dev))  # query rows != n_dst
 
 
-def test_too_small_max_degree_hint_costs_speed_not_correctness(dev, monkeypatch):
+@pytest.mark.parametrize("f", [16, 64])
+def test_too_small_max_degree_hint_costs_speed_not_correctness(dev, monkeypatch, f):
     """The widest-row argument of the entry points is a hint: told (wrongly) that no row is
     long, the library builds no row plan and its row kernels walk the long rows themselves.
     Every op must still give the right answer."""
@@ -429,7 +430,7 @@ def test_too_small_max_degree_hint_costs_speed_not_correctness(dev, monkeypatch)
     indptr, indices = powerlaw_graph(11, 40000, 77)
     n = indptr.numel() - 1
     assert int((indptr[1:] - indptr[:-1]).max()) > 500
-    h, f = 4, 16
+    h = 4  # f = 64: rows of 256 floats, the fused forward's whole-wave layout
     g = torch.Generator().manual_seed(9)
     q, k = torch.randn(1, n, h, generator=g), torch.randn(n, h, generator=g)
     x, gy = torch.randn(n, h, f, generator=g), torch.randn(n, h, f, generator=g)
@@ -456,6 +457,38 @@ def test_too_small_max_degree_hint_costs_speed_not_correctness(dev, monkeypatch)
     got = run()
     for i, (a, b) in enumerate(zip(got, want)):
         assert_close(a, b, rtol=1e-4, atol=5e-4, what="result %d" % i)
+
+
+def test_operands_that_are_not_vector_aligned(dev):
+    """query / key / attn that start 4 bytes off a 16-byte boundary (views into a larger
+    buffer): the one-lane-per-edge kernels read them as 16-byte vectors and must step aside
+    for the scalar kernels; same results as with aligned operands."""
+    indptr, indices = powerlaw_graph(10, 20000, 5)
+    n, h, f = indptr.numel() - 1, 4, 64
+    g = torch.Generator().manual_seed(4)
+    q, k = torch.randn(n, h, generator=g).to(dev), torch.randn(n, h, generator=g).to(dev)
+    x = torch.randn(n, h, f, generator=g).to(dev)
+    ga = torch.randn(indices.numel(), h, generator=g).to(dev)
+    ip, ix = indptr.to(dev), indices.to(dev)
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=dev)
+        v = buf[1:].view(t.shape)
+        v.copy_(t)
+        assert v.data_ptr() % 16 == 4 and v.is_contiguous()
+        return v
+
+    attn = graph_ext.sddmm_forward(ip, ix, q[None], k)
+    gq, gk = graph_ext.sddmm_backward(ip, ix, q[None], k, attn, ga)
+    out, _ = graph_ext.gat_forward(ip, ix, q, k, x)
+    qs, ks = shifted(q), shifted(k)
+    attn_s = graph_ext.sddmm_forward(ip, ix, qs[None], ks)
+    gq_s, gk_s = graph_ext.sddmm_backward(ip, ix, qs[None], ks, shifted(attn), shifted(ga))
+    out_s, _ = graph_ext.gat_forward(ip, ix, qs, ks, x)
+    assert_close(attn_s, attn, rtol=1e-5, atol=1e-6, what="attn")
+    assert_close(gq_s, gq, rtol=1e-4, atol=1e-5, what="grad_q")
+    assert_close(gk_s, gk, rtol=1e-4, atol=2e-4, what="grad_k")
+    assert_close(out_s, out, rtol=1e-5, atol=1e-4, what="out")
 
 
 def test_max_degree_cache_does_not_outlive_its_tensor(dev):
