@@ -999,9 +999,24 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
     // What is needed per (edge, head) is fetched once, before the row gathers, in the
     // layout of the epilogue: lane (h, sub) owns edge j * LPH + sub. The attention
     // weight reaches the accumulate loop by a lane shuffle.
+    // The first rows are asked for before anything else: they depend on the window only,
+    // while the per-edge values below wait for a gather of their own.
+    float v0[U][KT][4];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (u < n) {  // wave-uniform
+            const int r = __builtin_amdgcn_readlane(win.col, first + u);
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+                RowLoad<4, float>::ld(g + (size_t)r * p.g_ld + t * g_tile + g_lane, v0[u][t]);
+        }
+    }
     float ea[NS][KT], eS[NS][KT], eq[NS][KT];
 #pragma unroll
     for (int j = 0; j < NS; j++) {
+#pragma unroll
+        for (int t = 0; t < KT; t++) ea[j][t] = eS[j][t] = eq[j][t] = 0.0f;
+        if (j * LPH >= n) continue;  // wave-uniform: most short rows fill one group only
         const int k = min(j * LPH + sub, n - 1);
         const int vr = __shfl(win.vrow, first + k, kWave);
         const int r = __shfl(win.col, first + k, kWave);
@@ -1034,7 +1049,13 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
                     const int r = __builtin_amdgcn_readlane(win.col, first + k);
 #pragma unroll
                     for (int t = 0; t < KT; t++) {
-                        RowLoad<4, float>::ld(g + (size_t)r * p.g_ld + t * g_tile + g_lane, v[u][t]);
+                        if (j == 0 && kk == 0) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) v[u][t][i] = v0[u][t][i];
+                        } else {
+                            RowLoad<4, float>::ld(g + (size_t)r * p.g_ld + t * g_tile + g_lane,
+                                                  v[u][t]);
+                        }
                         a[u][t] = __shfl(ea[j][t], (lane - sub) + kk + u, kWave) * g_scale;
                     }
                 }
