@@ -362,7 +362,7 @@ def run_gat(args, dev):
                      "traffic": measured_traffic("c2_gat_f32")[0],
                      "traffic_source": measured_traffic("c2_gat_f32")[1],
                      "kernel": "yitu_gat_forward (row statistics out, no stored probabilities) = "
-                               "gat_rows_kernel + gat_item_local_kernel + gat_row_combine_kernel "
+                               "gat_rows_packed_kernel + gat_item_local_kernel + gat_row_combine_kernel "
                                "+ gat_scaled_reduce_kernel",
                      "kernel_ms": fwd_ms, "algorithmic_bytes": alg_fwd,
                      "bwd_achieved": alg_bwd / (bwd_ms * 1e-3) / 1e9,
@@ -437,7 +437,9 @@ def run_gat_c3(args, dev):
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
         "roofline": {"bound": "hbm", "achieved": alg_fwd / (fwd_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "frac": alg_fwd / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": measured_traffic("c3_gat_f32")[0],
+                     "traffic_source": measured_traffic("c3_gat_f32")[1],
                      "kernel": "yitu_gat_forward (row statistics out, no stored probabilities)",
                      "kernel_ms": fwd_ms, "algorithmic_bytes": alg_fwd,
                      "bwd_achieved": alg_bwd / (bwd_ms * 1e-3) / 1e9,
