@@ -226,19 +226,51 @@ __global__ __launch_bounds__(256) void sgemm_mfma_kernel(GemmParams p) {
         }
 }
 
-// C (+)= sum over splits of the partial slabs, in split order (reproducible)
+// C (+)= sum over splits of the partial slabs, in a fixed order (reproducible). A
+// workgroup takes 64 consecutive outputs; its four 64-thread groups each add a quarter of
+// the splits with four independent running sums (the loads of a thread do not wait for
+// each other), and the quarters are combined through LDS. One thread per output walking
+// all splits left a 256 x 256 product with 256 splits at one workgroup per CU and 256
+// dependent steps: 88 us.
+constexpr int kSplitReduceCols = 64;
+constexpr int kSplitReduceGroups = 256 / kSplitReduceCols;
+
 __global__ __launch_bounds__(256) void sgemm_splitk_reduce_kernel(GemmParams p) {
+    __shared__ float red[kSplitReduceGroups][kSplitReduceCols];
     const GemmProblem pr = p.prob[blockIdx.y];
     if (pr.n_split <= 1) return;  // written in place by the product kernel
     const int64_t total = (int64_t)pr.M * p.N;
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total;
-         e += (int64_t)gridDim.x * 256) {
-        const int row = (int)(e / p.N), col = (int)(e % p.N);
-        float s = 0.0f;
-        for (int z = 0; z < pr.n_split; z++)
-            s += p.partial[((size_t)(pr.z0 + z) * p.max_m + row) * p.N + col];
-        float *c = pr.C + (int64_t)row * p.ldc + col;
-        *c = p.accumulate ? *c + s : s;
+    const int lane_e = threadIdx.x % kSplitReduceCols, zg = threadIdx.x / kSplitReduceCols;
+    const int chunk = (pr.n_split + kSplitReduceGroups - 1) / kSplitReduceGroups;
+    const int zb = min(zg * chunk, pr.n_split), ze = min(zb + chunk, pr.n_split);
+    const size_t slab = (size_t)p.max_m * p.N;
+    for (int64_t e0 = (int64_t)blockIdx.x * kSplitReduceCols; e0 < total;
+         e0 += (int64_t)gridDim.x * kSplitReduceCols) {
+        const int64_t e = e0 + lane_e;
+        const bool live = e < total;
+        const int row = live ? (int)(e / p.N) : 0, col = live ? (int)(e % p.N) : 0;
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+        if (live) {
+            const float *src = p.partial + (size_t)pr.z0 * slab + (size_t)row * p.N + col;
+            int z = zb;
+            for (; z + 4 <= ze; z += 4) {
+                a0 += src[(size_t)z * slab];
+                a1 += src[(size_t)(z + 1) * slab];
+                a2 += src[(size_t)(z + 2) * slab];
+                a3 += src[(size_t)(z + 3) * slab];
+            }
+            for (; z < ze; z++) a0 += src[(size_t)z * slab];
+        }
+        red[zg][lane_e] = (a0 + a1) + (a2 + a3);
+        __syncthreads();
+        if (zg == 0 && live) {
+            float s = red[0][lane_e];
+#pragma unroll
+            for (int g = 1; g < kSplitReduceGroups; g++) s += red[g][lane_e];
+            float *c = pr.C + (int64_t)row * p.ldc + col;
+            *c = p.accumulate ? *c + s : s;
+        }
+        __syncthreads();
     }
 }
 
@@ -317,7 +349,7 @@ static int sgemm_launch_tile(const GemmParams &p, int max_m, int n_z, hipStream_
     }
     YITU_LAUNCH_CHECK();
     if (any_split) {
-        dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)max_m * p.N, 256), 2048),
+        dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)max_m * p.N, kSplitReduceCols), 4096),
                 (unsigned)p.n_prob);
         sgemm_splitk_reduce_kernel<<<rg, 256, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
