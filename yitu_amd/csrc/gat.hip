@@ -405,6 +405,139 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_kernel(GatParams p) {
     }
 }
 
+// The same with the head count (rounded up to a power of two) known at compile time:
+// the HP sub-batches of 64 / HP edges that an item can hold stay in registers, so every
+// (edge, head) logit is made once. The statistics are a maximum, then one exponential per
+// logit, then a sum (the running (max, sum) pair costs two exponentials per element and
+// per butterfly step), each reduced over the lanes that share a head in log2(64 / HP)
+// steps, and the exponentials are the weights of the aggregate: no second key gather.
+// Per item about 700 vector instructions against 1,250; the kernel above was bound by
+// instruction issue wherever most of its gathers hit L2.
+template <int VEC, int G, int KT, int HP>
+__global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) {
+    constexpr int EPS = kWave / HP;  // edges per sub-batch
+    constexpr int SLOTS = kWave / G;
+    constexpr int UNROLL = KT >= 4 ? 2 : (KT == 2 ? 4 : 8);  // row gathers in flight (KT = 1: 4 / 8 / 16 measured 811 / 767 / 822 us)
+    const int lane = lane_id();
+    const int sub = lane % G, slot = lane / G;
+    if (p.sp.plan.counters->overflow) return;
+    const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
+    const int n_waves = gridDim.x * kWavesPerBlock;
+    const int hl = lane & (HP - 1), esub = lane / HP;
+    const int H = p.sp.H, L = p.sp.L;
+    const float *__restrict__ feat = static_cast<const float *>(p.sp.feat);
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
+        const int n_here = min(kItemsPerWave, n_items - pos0);
+        const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
+        int col[kItemsPerWave], n_edges[kItemsPerWave], item_id[kItemsPerWave],
+            row_tag[kItemsPerWave];
+        float qv[kItemsPerWave];
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            const int beg = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item_id[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            row_tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
+            n_edges[j] = j < n_here ? end - beg : 0;
+            // lane e holds the source of the item's edge e (the last one again past the end)
+            col[j] = p.sp.indices[beg + min(lane, max(n_edges[j], 1) - 1)] & kColMask;
+            qv[j] = hl < H ? p.query[(size_t)(row_tag[j] & 0x7fffffff) * H + hl] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < kItemsPerWave; j++) {
+            if (n_edges[j] <= 0) continue;  // wave-uniform
+            const int n = n_edges[j];
+            // (edge, head) layout: sub-batch r, lane (esub, hl) = edge r EPS + esub, head hl
+            float pv[HP];
+            int cr[HP];
+#pragma unroll
+            for (int r = 0; r < HP; r++) {
+                const int k = r * EPS + esub;
+                cr[r] = __shfl(col[j], min(k, n - 1), kWave);
+                const float kv = hl < H ? p.key[(size_t)cr[r] * H + hl] : 0.0f;
+                pv[r] = (k < n && hl < H) ? leaky(qv[j] + kv) : -FLT_MAX;
+            }
+            float m = pv[0];
+#pragma unroll
+            for (int r = 1; r < HP; r++) m = fmaxf(m, pv[r]);
+            m = wave_max_strided<HP>(m);
+            float ssum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < HP; r++) {
+                pv[r] = (r * EPS + esub < n && hl < H) ? expf(pv[r] - m) : 0.0f;
+                ssum += pv[r];
+            }
+            ssum = wave_sum_strided<HP>(ssum);
+            const bool single = row_tag[j] < 0;
+            const int row = row_tag[j] & 0x7fffffff;
+            if (lane < HP && lane < H) {
+                p.item_stats[((size_t)item_id[j] * H + lane) * 2] = m;
+                p.item_stats[((size_t)item_id[j] * H + lane) * 2 + 1] = ssum;
+            }
+            if (single) {
+                const float inv = 1.0f / ssum;
+#pragma unroll
+                for (int r = 0; r < HP; r++) pv[r] *= inv;
+            }
+            float *dst = single ? p.sp.out + (size_t)row * L
+                                : p.sp.partial + (size_t)item_id[j] * L;
+            for (int c0 = 0; c0 < L; c0 += G * VEC * KT) {
+                const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);
+                float acc[KT][VEC];
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) acc[t][k] = 0.0f;
+#pragma unroll
+                for (int r = 0; r < HP; r++) {
+                    if (r * EPS >= n) break;  // wave-uniform
+                    const int nb = min(EPS, n - r * EPS);
+                    for (int j0 = 0; j0 < nb; j0 += SLOTS * UNROLL) {
+                        float v[UNROLL][KT][VEC], w[UNROLL][KT];
+#pragma unroll
+                        for (int u = 0; u < UNROLL; u++) {
+                            const int ej = j0 + u * SLOTS + slot;
+                            const bool valid = ej < nb;
+                            const int src = valid ? ej * HP : 0;  // lane of (edge ej, head 0)
+                            const int c = __shfl(cr[r], src, kWave);
+#pragma unroll
+                            for (int t = 0; t < KT; t++) {
+                                const float wt = __shfl(pv[r], src + tl.head[t], kWave);
+                                w[u][t] = (valid && tl.live[t]) ? wt : 0.0f;
+                            }
+                            if (j0 + u * SLOTS < nb) {  // wave-uniform
+#pragma unroll
+                                for (int t = 0; t < KT; t++)
+                                    RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                            } else {
+#pragma unroll
+                                for (int t = 0; t < KT; t++)
+#pragma unroll
+                                    for (int i = 0; i < VEC; i++) v[u][t][i] = 0.0f;
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                            for (int t = 0; t < KT; t++)
+#pragma unroll
+                                for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
+                    }
+                }
+                fold_slots<VEC, G, KT>(acc);
+                if (slot == 0) {
+#pragma unroll
+                    for (int t = 0; t < KT; t++) {
+                        const int o = c0 + (t * G + sub) * VEC;
+                        if (o < L) store_row<VEC>(dst + o, acc[t]);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // s += exp(max_c - m_row) * src[c * L] for c = first, first + step, ... < n, in
 // that order; st points at the first item's (max, sum) of this lane's head.
 __device__ __forceinline__ void sum_scaled_partials(float (&s)[4], const float *src,
@@ -1575,7 +1708,13 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
         (int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15);
     const int reduce_grid = (int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16);
     if (!p.attn && p.sp.F % 4 == 0) {
-        gat_item_local_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
+        switch (p.HP) {
+            case 1: gat_item_local_hp_kernel<VEC, G, KT, 1><<<item_grid, kBlock, 0, stream>>>(p); break;
+            case 2: gat_item_local_hp_kernel<VEC, G, KT, 2><<<item_grid, kBlock, 0, stream>>>(p); break;
+            case 4: gat_item_local_hp_kernel<VEC, G, KT, 4><<<item_grid, kBlock, 0, stream>>>(p); break;
+            case 8: gat_item_local_hp_kernel<VEC, G, KT, 8><<<item_grid, kBlock, 0, stream>>>(p); break;
+            default: gat_item_local_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
+        }
         YITU_LAUNCH_CHECK();
         gat_row_combine_kernel<<<combine_grid, kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
