@@ -144,7 +144,7 @@ struct TileLanes {
 // UNROLL: load instructions in flight per wave. With 4 slots (G = 16) an instruction
 // already fetches four rows and two of them measured best; wide rows keep registers low.
 template <int VEC, int G, int KT, int WMODE, typename TIN,
-          int UNROLL = ((KT >= 4 || G <= 16) ? 2 : 4)>
+          int UNROLL = ((KT >= 4 || G <= 16) ? 2 : ((G == kWave && KT == 1) ? 8 : 4))>
 __device__ __forceinline__ void accumulate_window(float (&acc)[KT][VEC], const SpmmParams &p,
                                                   const EdgeWindow &win, int first, int n,
                                                   const TileLanes<VEC, G, KT, WMODE> &tl) {
