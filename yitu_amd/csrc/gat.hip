@@ -500,7 +500,11 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
                             const int ej = j0 + u * SLOTS + slot;
                             const bool valid = ej < nb;
                             const int src = valid ? ej * HP : 0;  // lane of (edge ej, head 0)
-                            const int c = __shfl(cr[r], src, kWave);
+                            int c;
+                            if constexpr (SLOTS == 1)  // one edge for the whole wave: a scalar
+                                c = __builtin_amdgcn_readlane(cr[r], src);
+                            else
+                                c = __shfl(cr[r], src, kWave);
 #pragma unroll
                             for (int t = 0; t < KT; t++) {
                                 const float wt = __shfl(pv[r], src + tl.head[t], kWave);
