@@ -164,6 +164,59 @@ def test_sddmm_head_counts(dev, h, deterministic):
     assert torch.all(gq[0, 0] == 0) and torch.all(gq[0, 210] == 0)  # empty rows
 
 
+@pytest.mark.parametrize("pattern", ["boundaries", "tiny", "mixed", "sparse"])
+@pytest.mark.parametrize("h", [1, 2, 4, 8, 3])
+def test_packed_rows_at_chunk_boundaries(dev, pattern, h):
+    """Row lengths chosen against the one-lane-per-edge kernels: a wave packs whole rows
+    into chunks of at most 64 edges and owns up to 63 rows, so rows of 63 / 64 / 65 edges
+    next to each other, runs of empty rows, rows of one edge and rows that the plan takes
+    (64 and more) between short ones all have to land in the right chunk. Attention forward
+    and backward, the fused forward with row statistics, and grad_key's segmented sum."""
+    g = torch.Generator().manual_seed(len(pattern) * 10 + h)
+    n_dst, n_src = 20000, 3000  # more than 16,384 rows: several rows per wave
+    if pattern == "boundaries":
+        choice = torch.tensor([0, 1, 62, 63, 64, 65, 31, 32, 33, 2, 127, 128, 129])
+    elif pattern == "tiny":
+        choice = torch.tensor([0, 0, 0, 1, 1, 2, 3])
+    elif pattern == "mixed":
+        choice = torch.tensor([0, 5, 9, 17, 40, 63, 64, 200, 1, 1, 700])
+    else:
+        choice = torch.tensor([0] * 30 + [7, 63])
+    deg = choice[torch.randint(0, choice.numel(), (n_dst,), generator=g)]
+    indptr = torch.zeros(n_dst + 1, dtype=torch.int32)
+    indptr[1:] = torch.cumsum(deg, 0)
+    nnz = int(indptr[-1])
+    indices = torch.randint(0, n_src, (nnz,), generator=g, dtype=torch.int32)
+    q = torch.randn(1, n_dst, h, generator=g)
+    k = torch.randn(n_src, h, generator=g)
+    ge = torch.randn(nnz, h, generator=g)
+    dargs = (indptr.to(dev), indices.to(dev), q.to(dev), k.to(dev))
+    attn = graph_ext.sddmm_forward(*dargs)
+    want = oracle.sddmm_forward(indptr, indices, q, k)
+    assert_close(attn, want, what="attn")
+    gq, gk = graph_ext.sddmm_backward(*dargs, attn, ge.to(dev))
+    want_gq, want_gk = oracle.sddmm_backward(indptr, indices, q, k, want, ge)
+    abs_gq, abs_gk = softmax_backward_abs_sums(indptr, indices, want, ge.abs(), n_src)
+    assert_close(gq, want_gq, abs_sum=abs_gq, what="grad_q")
+    assert_close(gk, want_gk, abs_sum=abs_gk, what="grad_k")
+    assert torch.all(gq[0][deg == 0] == 0)
+    if h in (1, 2, 4):  # rows of 256 floats: the fused forward's whole-wave layout
+        f = 256 // h
+        x = torch.randn(n_src, h, f, generator=g)
+        out, _, stats = graph_ext.gat_forward(indptr.to(dev), indices.to(dev), q[0].to(dev),
+                                              k.to(dev), x.to(dev), stats_only=True)
+        want_out = oracle.mh_spmm_forward(want, indptr, indices, x)
+        assert_close(out, want_out, abs_sum=spmm_abs_sums(want, indptr, indices, x),
+                     what="fused out")
+        assert torch.all(out[deg == 0] == 0)
+        # (max, 1 / sum) of every non-empty row reproduce the probabilities
+        rows = torch.repeat_interleave(torch.arange(n_dst), deg.long())
+        logit = torch.nn.functional.leaky_relu(q[0][rows] + k[indices.long()], 0.2)
+        st = stats.cpu()
+        again = torch.exp(logit - st[rows, :, 0]) * st[rows, :, 1]
+        assert_close(again, want, rtol=1e-4, atol=1e-6, what="row statistics")
+
+
 @pytest.mark.parametrize("h", [4, 8, 5])
 def test_sddmm_power_law_hub_rows(dev, h):
     indptr, indices = powerlaw_graph(13, 150000, 40 + h)
