@@ -416,6 +416,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_kernel(GatParams p) {
 template <int VEC, int G, int KT, int HP>
 __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) {
     constexpr int EPS = kWave / HP;  // edges per sub-batch
+    constexpr int kLocalItems = 1;   // items of a group
     constexpr int SLOTS = kWave / G;
     constexpr int UNROLL = KT >= 4 ? 2 : (KT == 2 ? 4 : 8);  // row gathers in flight (KT = 1: 4 / 8 / 16 measured 811 / 767 / 822 us)
     const int lane = lane_id();
@@ -426,15 +427,15 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
     const int hl = lane & (HP - 1), esub = lane / HP;
     const int H = p.sp.H, L = p.sp.L;
     const float *__restrict__ feat = static_cast<const float *>(p.sp.feat);
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
-         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
-        const int n_here = min(kItemsPerWave, n_items - pos0);
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kLocalItems;
+         pos0 < n_items; pos0 += n_waves * kLocalItems) {
+        const int n_here = min(kLocalItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
-        int col[kItemsPerWave], n_edges[kItemsPerWave], item_id[kItemsPerWave],
-            row_tag[kItemsPerWave];
-        float qv[kItemsPerWave];
+        int col[kLocalItems], n_edges[kLocalItems], item_id[kLocalItems],
+            row_tag[kLocalItems];
+        float qv[kLocalItems];
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kLocalItems; j++) {
             const int beg = __builtin_amdgcn_readlane(my_rec.x, j);
             const int end = __builtin_amdgcn_readlane(my_rec.y, j);
             item_id[j] = __builtin_amdgcn_readlane(my_rec.z, j);
@@ -445,7 +446,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
             qv[j] = hl < H ? p.query[(size_t)(row_tag[j] & 0x7fffffff) * H + hl] : 0.0f;
         }
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kLocalItems; j++) {
             if (n_edges[j] <= 0) continue;  // wave-uniform
             const int n = n_edges[j];
             // (edge, head) layout: sub-batch r, lane (esub, hl) = edge r EPS + esub, head hl
@@ -1712,11 +1713,14 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
         (int)std::min<int64_t>(ceil_div(p.sp.plan.max_rows, kWavesPerBlock), 1 << 15);
     const int reduce_grid = (int)std::min<int64_t>(p.sp.plan.max_rows, 1 << 16);
     if (!p.attn && p.sp.F % 4 == 0) {
+        // two items per wave and turn of the grid-stride loop: twice the workgroups
+        const int hp_grid = (int)std::min<int64_t>(
+            ceil_div(p.sp.plan.max_items, kWavesPerBlock * 1), 1 << 19);
         switch (p.HP) {
-            case 1: gat_item_local_hp_kernel<VEC, G, KT, 1><<<item_grid, kBlock, 0, stream>>>(p); break;
-            case 2: gat_item_local_hp_kernel<VEC, G, KT, 2><<<item_grid, kBlock, 0, stream>>>(p); break;
-            case 4: gat_item_local_hp_kernel<VEC, G, KT, 4><<<item_grid, kBlock, 0, stream>>>(p); break;
-            case 8: gat_item_local_hp_kernel<VEC, G, KT, 8><<<item_grid, kBlock, 0, stream>>>(p); break;
+            case 1: gat_item_local_hp_kernel<VEC, G, KT, 1><<<hp_grid, kBlock, 0, stream>>>(p); break;
+            case 2: gat_item_local_hp_kernel<VEC, G, KT, 2><<<hp_grid, kBlock, 0, stream>>>(p); break;
+            case 4: gat_item_local_hp_kernel<VEC, G, KT, 4><<<hp_grid, kBlock, 0, stream>>>(p); break;
+            case 8: gat_item_local_hp_kernel<VEC, G, KT, 8><<<hp_grid, kBlock, 0, stream>>>(p); break;
             default: gat_item_local_kernel<VEC, G, KT><<<item_grid, kBlock, 0, stream>>>(p);
         }
         YITU_LAUNCH_CHECK();
