@@ -668,6 +668,8 @@ struct GatBwdParams {
 };
 
 constexpr int kDotUnroll = 4;  // gathers in flight per wave in the backward dots
+constexpr int kSrcItems = 2;   // plan items a wave of the by-source item kernels takes per turn (1 / 2 / 4:
+                               // 974 / 953 / 1004 us on a 2^18-node graph, 5.57 / 5.47 / 5.37 ms on a 2^21-node one)
 
 // One wave per planned row adds its items' sums (lane = (item slot, head),
 // fixed butterfly), writes S of the row and grad_q = A1 - S A2.
@@ -1305,14 +1307,14 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int L = p.sp.L, H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
-         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
-        const int n_here = min(kItemsPerWave, n_items - pos0);
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kSrcItems;
+         pos0 < n_items; pos0 += n_waves * kSrcItems) {
+        const int n_here = min(kSrcItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
-        EdgeWindow win[kItemsPerWave];
-        int n_edges[kItemsPerWave], tag[kItemsPerWave], item[kItemsPerWave];
+        EdgeWindow win[kSrcItems];
+        int n_edges[kSrcItems], tag[kSrcItems], item[kSrcItems];
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kSrcItems; j++) {
             const int beg = __shfl(my_rec.x, j, kWave);
             const int end = __shfl(my_rec.y, j, kWave);
             item[j] = __shfl(my_rec.z, j, kWave);
@@ -1321,7 +1323,7 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
             if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
         }
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kSrcItems; j++) {
             if (n_edges[j] <= 0) continue;
             const int row = tag[j] & 0x7fffffff;
             float xt[KT][4], acc[KT][4], kc[KT], gk[KT];
@@ -1509,14 +1511,14 @@ __global__ __launch_bounds__(kBlock) void gat_slot_items_kernel(GatSrcParams p) 
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
-         pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
-        const int n_here = min(kItemsPerWave, n_items - pos0);
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kSrcItems;
+         pos0 < n_items; pos0 += n_waves * kSrcItems) {
+        const int n_here = min(kSrcItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
-        EdgeWindow win[kItemsPerWave];
-        int n_edges[kItemsPerWave], tag[kItemsPerWave], item[kItemsPerWave];
+        EdgeWindow win[kSrcItems];
+        int n_edges[kSrcItems], tag[kSrcItems], item[kSrcItems];
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kSrcItems; j++) {
             const int beg = __shfl(my_rec.x, j, kWave);
             const int end = __shfl(my_rec.y, j, kWave);
             item[j] = __shfl(my_rec.z, j, kWave);
@@ -1525,7 +1527,7 @@ __global__ __launch_bounds__(kBlock) void gat_slot_items_kernel(GatSrcParams p) 
             if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
         }
 #pragma unroll
-        for (int j = 0; j < kItemsPerWave; j++) {
+        for (int j = 0; j < kSrcItems; j++) {
             if (n_edges[j] <= 0) continue;
             const int row = tag[j] & 0x7fffffff;
             SlotRow<LPH> acc;
@@ -1551,8 +1553,9 @@ static int gat_src_launch_shape(const GatSrcParams &p, bool has_items, const flo
         YITU_LAUNCH_CHECK();
     }
     const int row_grid = (int)ceil_div(p.sp.n_rows, kWavesPerBlock * rows_per_wave(p.sp.n_rows));
+    // enough workgroups to walk the item list once (a second turn would mix source bands)
     const int item_grid = (int)std::min<int64_t>(
-        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
+        ceil_div(p.sp.plan.max_items, kWavesPerBlock * kSrcItems), 1 << 20);
     // a head-mean gradient of F < 256 floats per row: the several-edges-per-load kernels
     constexpr bool kSlots = FULL && KT == 1 && LPH < kWave;
     bool slots = false;
