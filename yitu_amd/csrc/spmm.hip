@@ -62,9 +62,12 @@ static int launch_variant(const SpmmParams &p, bool has_items, hipStream_t strea
     spmm_rows_kernel<VEC, G, KT, WMODE, TIN><<<grid, kBlock, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
     if (has_items) {
+        // whole-wave rows (1 KB and more per gather): one item per wave and a grid that walks
+        // the list once; narrower rows: four items per wave, the grid capped
+        constexpr int IPW = (G == kWave && KT == 1) ? 1 : kItemsPerWave;
         const int item_grid = (int)std::min<int64_t>(
-            ceil_div(p.plan.max_items, kWavesPerBlock * kItemsPerWave), 1 << 16);
-        spmm_items_kernel<VEC, G, KT, WMODE, TIN><<<item_grid, kBlock, 0, stream>>>(p);
+            ceil_div(p.plan.max_items, kWavesPerBlock * IPW), IPW == 1 ? 1 << 20 : 1 << 16);
+        spmm_items_kernel<VEC, G, KT, WMODE, TIN, IPW><<<item_grid, kBlock, 0, stream>>>(p);
         YITU_LAUNCH_CHECK();
         const int red_grid = (int)std::min<int64_t>(p.plan.max_rows, 1 << 16);
         constexpr int RV = VEC >= 4 ? 4 : VEC;  // VEC | L whenever this variant is chosen

@@ -297,20 +297,20 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(SpmmParams p) {
 
 constexpr int kItemsPerWave = 4;  // band-sorted items handled by one wave
 
-// One group of up to kItemsPerWave consecutive records [pos0, pos0 + n_here):
+// One group of up to IPW (items per wave) consecutive records [pos0, pos0 + n_here):
 // the records come from one load, their edge windows are all fetched before the
 // first feature gather, so the only waits per item are its own gathers. The
 // unscaled partial row goes to partial[item id].
-template <int VEC, int G, int KT, int WMODE, typename TIN>
+template <int VEC, int G, int KT, int WMODE, typename TIN, int IPW>
 __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, int n_here) {
     const int lane = lane_id();
     const int sub = lane % G;
     const int slot = lane / G;
     const int4 my_rec = p.plan.records[pos0 + min(lane, n_here - 1)];
-    EdgeWindow win[kItemsPerWave];
-    int item_id[kItemsPerWave], n_edges[kItemsPerWave], row_tag[kItemsPerWave];
+    EdgeWindow win[IPW];
+    int item_id[IPW], n_edges[IPW], row_tag[IPW];
 #pragma unroll
-    for (int j = 0; j < kItemsPerWave; j++) {
+    for (int j = 0; j < IPW; j++) {
         const int beg = __shfl(my_rec.x, j, kWave);
         const int end = __shfl(my_rec.y, j, kWave);
         item_id[j] = __shfl(my_rec.z, j, kWave);
@@ -319,7 +319,7 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
         if (n_edges[j] > 0) load_window<WMODE>(win[j], p, beg, end);
     }
 #pragma unroll
-    for (int j = 0; j < kItemsPerWave; j++) {
+    for (int j = 0; j < IPW; j++) {
         if (n_edges[j] <= 0) continue;
         for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
             const TileLanes<VEC, G, KT, WMODE> tl(p, c0);
@@ -351,18 +351,18 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
     }
 }
 
-// Items of the plan in band order, kItemsPerWave per wave. The order only
+// Items of the plan in band order, IPW per wave. The order only
 // affects cache behaviour: every item writes its own row.
-template <int VEC, int G, int KT, int WMODE, typename TIN>
+template <int VEC, int G, int KT, int WMODE, typename TIN, int IPW = kItemsPerWave>
 __global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
     static_assert(kPlanChunk <= kWave, "an item must fit one edge window");
     if (p.plan.counters->overflow) return;
     const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
-    const int n_groups = (n_items + kItemsPerWave - 1) / kItemsPerWave;
+    const int n_groups = (n_items + IPW - 1) / IPW;
     const int stride = gridDim.x * kWavesPerBlock;
     for (int grp = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; grp < n_groups; grp += stride)
-        spmm_item_group<VEC, G, KT, WMODE, TIN>(p, grp * kItemsPerWave,
-                                                min(kItemsPerWave, n_items - grp * kItemsPerWave));
+        spmm_item_group<VEC, G, KT, WMODE, TIN, IPW>(p, grp * IPW,
+                                                min(IPW, n_items - grp * IPW));
 }
 
 // Adds the item partials of every planned row with more than one item and
