@@ -1698,7 +1698,10 @@ static int gat_fwd_launch(GatParams &p, bool has_items, hipStream_t stream) {
     if (G == kWave && VEC == 4 && p.sp.L <= 4 * kWave * KT && packed_heads_ok(p.sp.H) &&
         vec_aligned(hv, p.query, p.key, p.attn)) {
         // whole-wave rows: the short rows in the packed layout
-        const int R = packed_rows_per_wave(p.sp.n_rows);
+        // fewer rows per wave than the attention-only kernels take (63): with a wave-wide
+        // gather per edge, more waves in flight are worth more than longer chunk runs
+        // (24 / 63 rows: 1.94 / 2.05 ms on a 2^21-node graph)
+        const int R = std::min(packed_rows_per_wave(p.sp.n_rows), 24);
         const int grid = (int)ceil_div(p.sp.n_rows, (int64_t)kWavesPerBlock * R);
         if (hv == 4) gat_rows_packed_kernel<4, KT><<<grid, kBlock, 0, stream>>>(p, R);
         else if (hv == 2) gat_rows_packed_kernel<2, KT><<<grid, kBlock, 0, stream>>>(p, R);
