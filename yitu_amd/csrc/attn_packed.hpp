@@ -153,7 +153,7 @@ struct PackedGat {
 #pragma unroll
         for (int t = 0; t < KT; t++) {
             const int o = (t * kWave + lane_id()) * 4;
-            if (o < p.sp.L) store_row<4>(p.sp.out + (size_t)row * p.sp.L + o, acc[t]);
+            if (o < p.sp.L) store_row_streaming<4>(p.sp.out + (size_t)row * p.sp.L + o, acc[t]);
         }
     }
 };

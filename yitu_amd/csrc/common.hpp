@@ -131,6 +131,23 @@ __device__ __forceinline__ void store_row(float *p, const float (&v)[VEC]) {
     }
 }
 
+// The same for rows that are written once and not read again by this kernel: the store
+// does not claim a place in the caches.
+template <int VEC>
+__device__ __forceinline__ void store_row_streaming(float *p, const float (&v)[VEC]) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    if constexpr (VEC % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            f4 t = {v[i], v[i + 1], v[i + 2], v[i + 3]};
+            __builtin_nontemporal_store(t, reinterpret_cast<f4 *>(p + i));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) __builtin_nontemporal_store(v[i], p + i);
+    }
+}
+
 // ---- wave64 helpers ---------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 

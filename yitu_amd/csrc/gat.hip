@@ -535,7 +535,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
 #pragma unroll
                     for (int t = 0; t < KT; t++) {
                         const int o = c0 + (t * G + sub) * VEC;
-                        if (o < L) store_row<VEC>(dst + o, acc[t]);
+                        if (o < L) store_row_streaming<VEC>(dst + o, acc[t]);
                     }
                 }
             }
