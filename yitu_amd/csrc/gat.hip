@@ -611,7 +611,7 @@ __global__ __launch_bounds__(kBlock) void gat_scaled_reduce_kernel(GatParams p) 
                 if (live && slot == 0) {
 #pragma unroll
                     for (int i = 0; i < 4; i++) s[i] *= inv;
-                    store_row<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + sub) * 4, s);
+                    store_row_streaming<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + sub) * 4, s);
                 }
             }
         }
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(kBlock) void gat_scaled_reduce_kernel(GatParams p) 
                     for (int i = 0; i < 4; i++) s[i] += red[(gg * lanes + l) * 4 + i];
 #pragma unroll
                 for (int i = 0; i < 4; i++) s[i] *= inv;
-                store_row<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + l) * 4, s);
+                store_row_streaming<4>(p.sp.out + (size_t)r.x * L + (size_t)(l0 + l) * 4, s);
             }
         }
     }
@@ -1260,7 +1260,7 @@ __device__ __forceinline__ void gat_src_end(float *x_dst, float *k_dst, const fl
     const int lane = lane_id();
 #pragma unroll
     for (int t = 0; t < KT; t++) {
-        store_row<4>(x_dst + t * 256 + lane * 4, acc[t]);
+        store_row_streaming<4>(x_dst + t * 256 + lane * 4, acc[t]);
         if constexpr (FULL) {
             float s = gk[t];
             s = group_sum<LPH>(s);
@@ -1468,7 +1468,7 @@ __device__ __forceinline__ void slot_end(SlotRow<LPH> &row, float *x_dst, float 
     }
     if (s == 0) {
 #pragma unroll
-        for (int h = 0; h < H; h++) store_row<4>(x_dst + h * (4 * LPH) + sub * 4, row.acc[h]);
+        for (int h = 0; h < H; h++) store_row_streaming<4>(x_dst + h * (4 * LPH) + sub * 4, row.acc[h]);
         if (sub < H) k_dst[sub] = row.gk;
     }
 }

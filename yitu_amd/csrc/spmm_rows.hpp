@@ -282,7 +282,7 @@ __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, i
                         float r[VEC];
 #pragma unroll
                         for (int k = 0; k < VEC; k++) r[k] = acc[t][k] * sr;
-                        store_row<VEC>(p.out + (size_t)row * p.L + o, r);
+                        store_row_streaming<VEC>(p.out + (size_t)row * p.L + o, r);
                     }
                 }
             }
@@ -343,7 +343,7 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
                         float r[VEC];
 #pragma unroll
                         for (int i = 0; i < VEC; i++) r[i] = acc[t][i] * sr;
-                        store_row<VEC>(dst + o, r);
+                        store_row_streaming<VEC>(dst + o, r);
                     }
                 }
             }
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
                 if (live && slot == 0) {
 #pragma unroll
                     for (int i = 0; i < VEC; i++) s[i] *= sr;
-                    store_row<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + sub) * VEC, s);
+                    store_row_streaming<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + sub) * VEC, s);
                 }
             }
         }
@@ -464,7 +464,7 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
                     for (int i = 0; i < VEC; i++) s[i] += red[(gg * lanes + l) * VEC + i];
 #pragma unroll
                 for (int i = 0; i < VEC; i++) s[i] *= sr;
-                store_row<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + l) * VEC, s);
+                store_row_streaming<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + l) * VEC, s);
             }
         }
     }
