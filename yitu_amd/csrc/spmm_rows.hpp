@@ -70,12 +70,13 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
                                             int limit) {
     const int e = min(base + lane_id(), limit - 1);
     win.base = base;
-    win.col = p.cols_are_edges ? e : (p.indices[e] & p.col_mask);
+    // the edge arrays are read once per call: streaming loads leave the caches to the rows
+    win.col = p.cols_are_edges ? e : (__builtin_nontemporal_load(p.indices + e) & p.col_mask);
     win.w = 1.0f;
     win.vrow = 0;
     if constexpr (WMODE == W_DEGPROD)
-        win.w = p.edge_scale ? p.edge_scale[e] : p.scale_col[win.col];
-    if constexpr (WMODE == W_EDGEHEAD) win.vrow = p.eperm ? p.eperm[e] : e;
+        win.w = p.edge_scale ? __builtin_nontemporal_load(p.edge_scale + e) : p.scale_col[win.col];
+    if constexpr (WMODE == W_EDGEHEAD) win.vrow = p.eperm ? __builtin_nontemporal_load(p.eperm + e) : e;
 }
 
 // One step of the edge loop: every slot of the wave picks its edge
