@@ -593,9 +593,10 @@ def run_c4(args, dev):
 
     h_all16 = torch.empty(n_all, dim, device=dev, dtype=torch.bfloat16)
 
+    h_parts16 = [h_all16[off[t]:off[t + 1]] for t in range(4)]
+
     def gemm16():
-        for t in range(4):
-            graph_ext.gemm_bf16(xs16[t], wts16[t], out=h_all16[off[t]:off[t + 1]])
+        graph_ext.gemm_bf16_typed(xs16, wts16, out_list=h_parts16)
 
     def agg16():
         return graph_ext.spmm_forward(values, indptr, indices, h_all16.view(n_all, 1, dim))
@@ -611,8 +612,7 @@ def run_c4(args, dev):
         dh16 = dh.view(n_all, dim).to(torch.bfloat16)  # one rounding pass over the gradient rows
         parts = [dh16[off[t]:off[t + 1]] for t in range(4)]
         dws = [graph_ext.gemm_bf16_tn(xs16[t], parts[t]) for t in range(4)]
-        dxs = [graph_ext.gemm_bf16(parts[t], wts16[t], trans_b=True, out_dtype=torch.bfloat16)
-               for t in range(4)]
+        dxs = graph_ext.gemm_bf16_typed(parts, wts16, trans_b=True, out_dtype=torch.bfloat16)
         return dws, dxs
 
     gemm16()

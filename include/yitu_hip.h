@@ -452,6 +452,24 @@ int yitu_gemm_bf16(void *c_device, int c_is_bf16, const void *a_bf16_device,
                    size_t workspace_bytes, void *stream);
 
 /*
+ * The same product for a list of operand pairs of one width, one launch per 8 pairs: C_i[m_i,n] = A_i[m_i,k] . op(B_i), shared n, k, trans_b and leading
+ * dimensions; c, a, b are HOST arrays of device pointers, m a HOST array of row
+ * counts. The bf16 form of yitu_sgemm_typed's forward and input-gradient products
+ * (the loop of per-type / per-relation Linear layers, test/common/model.py:137-171
+ * over :7-30). With k = 64, 128 or 256 and at least 4,096 rows in all, the row tiles
+ * of every pair share one grid whose workgroups keep the pair's weight in registers;
+ * other shapes run as one yitu_gemm_bf16 per pair.
+ * Workspace: yitu_gemm_bf16_typed_workspace_bytes(n_problems, n, k, trans_b).
+ */
+size_t yitu_gemm_bf16_typed_workspace_bytes(int64_t n_problems, int64_t n, int64_t k, int trans_b);
+int yitu_gemm_bf16_typed(void *const *c_device_ptrs, int c_is_bf16,
+                         const void *const *a_bf16_device_ptrs,
+                         const void *const *b_bf16_device_ptrs, const int64_t *m,
+                         int64_t n_problems, int64_t n, int64_t k, int trans_b, int64_t lda,
+                         int64_t ldb, int64_t ldc, void *workspace_device, size_t workspace_bytes,
+                         void *stream);
+
+/*
  * C[ki, no] (+)= A^T . B with bf16 operands A [m, lda], B [m, ldb] (row-major,
  * summed over their m rows) and fp32 accumulation on the matrix cores; C fp32
  * [ki, ldc]. The weight gradient dW = X^T . dY of a bf16 layer (fc_cuda.cu:77-215,

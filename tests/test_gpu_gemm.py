@@ -158,6 +158,54 @@ def test_gemm_bf16_against_double(dev, tb, out_dtype, m, n, k):
                      atol=1e-4 * max(1.0, np.sqrt(k) / 4))
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(4100, 256, 256), (5000, 300, 64), (70001, 256, 48),
+                                   (4096, 250, 128), (20000, 520, 256), (40000, 64, 16)])
+def test_gemm_bf16_many_rows_short_inner_dimension(dev, out_dtype, m, n, k):
+    """Inner dimensions of at most 256 with thousands of rows run with the weight held in
+    registers and whole-row tiles: ragged last tile, column counts that are not multiples
+    of 4 / 64 / 256, several column blocks, short inner dimensions."""
+    g = torch.Generator().manual_seed(m + 3 * n + 5 * k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    b = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    got = graph_ext.gemm_bf16(a.to(dev), b.to(dev), trans_b=True, out_dtype=out_dtype)
+    want = (a.double() @ b.double().t()).float()
+    if out_dtype == torch.float32:
+        assert_close(got, want, atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+    else:
+        assert_close(got.float(), want, rtol=2.0 ** -8, atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+    assert torch.equal(got, graph_ext.gemm_bf16(a.to(dev), b.to(dev), trans_b=True,
+                                                out_dtype=out_dtype))
+
+
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ms,n,k", [([5000, 0, 4097, 300], 256, 256),
+                                    ([700] * 10, 192, 128),      # two launches of 8 and 2
+                                    ([33, 64, 1], 256, 64),      # few rows: one product each
+                                    ([3000, 2000], 72, 40)])     # not one of the grouped widths
+def test_gemm_bf16_typed_against_double(dev, tb, out_dtype, ms, n, k):
+    """Products of several node types in one call: row tiles of every type in one grid,
+    a type's ragged last tile next to the first tile of the next, an empty type."""
+    g = torch.Generator().manual_seed(sum(ms) + 3 * n + 5 * k)
+    a = [torch.randn(m, k, generator=g).to(torch.bfloat16) for m in ms]
+    b = [torch.randn((n, k) if tb else (k, n), generator=g).to(torch.bfloat16) for _ in ms]
+    rows = torch.zeros(sum(ms), n, dtype=out_dtype, device=dev)
+    outs = list(rows.split(ms))  # row slices of one buffer
+    got = graph_ext.gemm_bf16_typed([x.to(dev) for x in a], [w.to(dev) for w in b], trans_b=tb,
+                                    out_list=outs)
+    for x, w, c, m in zip(a, b, got, ms):
+        want = (x.double() @ (w.double().t() if tb else w.double())).float()
+        assert c.dtype == out_dtype and c.shape == (m, n)
+        if out_dtype == torch.float32:
+            assert_close(c, want, atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+        else:
+            assert_close(c.float(), want, rtol=2.0 ** -8, atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+    again = graph_ext.gemm_bf16_typed([x.to(dev) for x in a], [w.to(dev) for w in b], trans_b=tb,
+                                      out_dtype=out_dtype)
+    assert all(torch.equal(c, d) for c, d in zip(got, again))
+
+
 @pytest.mark.parametrize("m,ki,no", [(1, 8, 8), (33, 8, 16), (100, 72, 40), (4096, 256, 256),
                                      (5000, 128, 264), (70000, 256, 256), (0, 16, 8)])
 def test_gemm_bf16_tn_against_double(dev, m, ki, no):

@@ -160,11 +160,230 @@ __global__ __launch_bounds__(256, 2) void hgemm_mfma_kernel(HGemmParams p) {
         }
 }
 
+// Inner dimension of at most 256 and many rows: the weight stays in registers. A
+// workgroup of 4 waves holds all of Bt[n0 .. n0 + 256, 0 .. K) as MFMA operands (wave w
+// keeps 64 columns: 16 K-steps x 2 column tiles x 4 registers), walks row tiles of 32
+// rows and reads every one as whole rows: the tile is one contiguous piece of memory when
+// lda = K, requested RPF tiles ahead through a ring of registers and passed through a
+// double-buffered LDS tile, one barrier per tile. The kernel above asks for 64 bytes of
+// every row per K-step and writes its outputs two bytes at a time. Rows of the LDS tile
+// are padded to 528 bytes: the 16-byte operand reads of 16 consecutive lanes (16 rows, one
+// piece) then cover every bank once, at one address register and an immediate offset per
+// K-step. The inner dimension is a template parameter (64, 128 or 256), so the K loop has
+// no branch. The weight is the first MFMA operand, so a lane ends up with four consecutive columns of one row;
+// a wave passes them through an LDS area of its own and stores 128-byte row segments:
+// stores of 8 or 16 bytes per row cost the L2 one request each and ran at half the rate.
+constexpr int RM = 32, RPF = 2, RA_LD = 264;
+constexpr int RC_LD = 144;  // staged output row: 128 bytes + 16 of padding
+constexpr int kRowsProblems = 8;
+
+// Up to 8 products of one width (node types: C_q = A_q . Bt_q^T) share the launch. Their
+// row tiles form one list, tile_start[q] is the first tile of problem q; a workgroup
+// takes every gridDim.x-th tile and reloads the weight when the problem changes.
+struct HRowsParams {
+    const uint16_t *A[kRowsProblems];   // [M_q, lda]
+    const uint16_t *Bt[kRowsProblems];  // [N, ldbt]
+    void *C[kRowsProblems];             // [M_q, ldc] fp32 or bf16
+    int M[kRowsProblems];
+    int tile_start[kRowsProblems + 1];
+    int n_problems, N;
+    int64_t lda, ldbt, ldc;
+};
+
+template <bool OUT_BF16, int KS>
+__global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
+    constexpr int K = 16 * KS;        // inner dimension: KS steps of 16
+    constexpr int TPR = K / 8;        // threads that cover one row with 16 bytes each
+    constexpr int RPS = 256 / TPR;    // rows the workgroup covers at a time
+    constexpr int LR = RM / RPS;      // 16-byte pieces of the tile per thread
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][RM][RA_LD];
+    __shared__ __attribute__((aligned(16))) unsigned char Cs[4][RM * RC_LD];
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int wn = blockIdx.y * HN + wave * 64;
+    unsigned char *stage = Cs[wave];
+    const int stride = gridDim.x;
+    const bool whole_cols = blockIdx.y * HN + HN <= p.N;
+    // loader: TPR threads cover one row, the workgroup RPS rows at a time. Rows past the
+    // end are read from the last row (their outputs are never stored) and tiles past the
+    // end from the last tile: no load of the ring is conditional.
+    const int lrow = t / TPR, lk_ld = (t % TPR) * 8;
+
+    for (int q = 0; q < p.n_problems; q++) {
+    const int lo = p.tile_start[q], hi = p.tile_start[q + 1];
+    // this workgroup's tiles of the problem: lo <= tile < hi, tile = blockIdx.x (mod stride)
+    const int tile0 = lo + (int)(((int64_t)blockIdx.x - lo % stride + stride) % stride);
+    if (tile0 >= hi) continue;  // same for the whole workgroup
+    const uint16_t *a_q = p.A[q], *bt = p.Bt[q];
+    void *c_q = p.C[q];
+    const int m_q = p.M[q];
+    bf16x8 b[KS][2];
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = min(wn + 32 * j + l32, p.N - 1);  // columns past N: never stored
+            b[s][j] = __builtin_bit_cast(
+                bf16x8,
+                *reinterpret_cast<const uint4 *>(bt + (int64_t)col * p.ldbt + 16 * s + 8 * lk));
+        }
+    u32x4 ra[RPF][LR];
+    auto gload = [&](int slot, int64_t tile64) {
+        const int tile = (int)std::min<int64_t>(tile64, hi - 1);
+        const int r0 = (tile - lo) * RM + lrow;
+#pragma unroll
+        for (int i = 0; i < LR; i++) {
+            const int64_t row = min(r0 + RPS * i, m_q - 1);
+            ra[slot][i] = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x4 *>(a_q + row * p.lda + lk_ld));
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < RPF; u++) {
+        gload(u, tile0 + (int64_t)u * stride);
+        __builtin_amdgcn_sched_barrier(0);  // oldest first
+    }
+    for (int it0 = 0; tile0 + (int64_t)it0 * stride < hi; it0 += RPF) {
+#pragma unroll
+        for (int u = 0; u < RPF; u++) {
+            const int it = it0 + u;
+            const int64_t tile64 = tile0 + (int64_t)it * stride;
+            if (tile64 >= hi) break;  // same for the whole workgroup
+            const int tile = (int)tile64, buf = it & 1;
+            // this buffer was last read two tiles ago, before the previous barrier
+#pragma unroll
+            for (int i = 0; i < LR; i++)
+                *reinterpret_cast<u32x4 *>(&As[buf][lrow + RPS * i][lk_ld]) = ra[u][i];
+            __syncthreads();
+            gload(u, tile64 + (int64_t)RPF * stride);
+            f32x16 acc[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[j][e] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const bf16x8 a =
+                    *reinterpret_cast<const bf16x8 *>(&As[buf][l32][16 * s + 8 * lk]);
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[s][j], a, acc[j], 0, 0, 0);
+                // operand reads stay at most four steps ahead of their products: hoisted
+                // all the way they would not fit beside the weight
+                if (s % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+            }
+            // accumulator element 4 jj + ii of column tile j is
+            // C[32 tile + lane % 32][wn + 32 j + 8 jj + 4 (lane / 32) + ii]
+            const int row0 = (tile - lo) * RM;
+            if (whole_cols && row0 + RM <= m_q) {  // same for the whole workgroup
+                if constexpr (OUT_BF16) {
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+#pragma unroll
+                        for (int jj = 0; jj < 4; jj++) {
+                            u32x2 w;
+                            w[0] = (unsigned)f32_to_bf16_rne(acc[j][4 * jj]) |
+                                   ((unsigned)f32_to_bf16_rne(acc[j][4 * jj + 1]) << 16);
+                            w[1] = (unsigned)f32_to_bf16_rne(acc[j][4 * jj + 2]) |
+                                   ((unsigned)f32_to_bf16_rne(acc[j][4 * jj + 3]) << 16);
+                            *reinterpret_cast<u32x2 *>(stage + l32 * RC_LD + 64 * j + 16 * jj +
+                                                       8 * lk) = w;
+                        }
+#pragma unroll
+                    for (int r = 0; r < RM / 8; r++) {
+                        const int row = 8 * r + (lane >> 3);
+                        const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + row * RC_LD +
+                                                                         16 * (lane & 7));
+                        __builtin_nontemporal_store(
+                            w, reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(c_q) +
+                                                         (int64_t)(row0 + row) * p.ldc + wn +
+                                                         8 * (lane & 7)));
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+#pragma unroll
+                        for (int jj = 0; jj < 4; jj++) {
+                            const f4 w = {acc[j][4 * jj], acc[j][4 * jj + 1], acc[j][4 * jj + 2],
+                                          acc[j][4 * jj + 3]};
+                            *reinterpret_cast<f4 *>(stage + l32 * RC_LD + 32 * jj + 16 * lk) = w;
+                        }
+#pragma unroll
+                        for (int r = 0; r < RM / 8; r++) {
+                            const int row = 8 * r + (lane >> 3);
+                            const f4 w = *reinterpret_cast<const f4 *>(stage + row * RC_LD +
+                                                                       16 * (lane & 7));
+                            *reinterpret_cast<f4 *>(static_cast<float *>(c_q) +
+                                                    (int64_t)(row0 + row) * p.ldc + wn + 32 * j +
+                                                    4 * (lane & 7)) = w;
+                        }
+                    }
+                }
+            } else if (row0 + l32 < m_q) {
+                const int64_t row = row0 + l32;
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int col = wn + 32 * j + 8 * (e / 4) + 4 * lk + e % 4;
+                        if (col < p.N) {
+                            if constexpr (OUT_BF16)
+                                static_cast<uint16_t *>(c_q)[row * p.ldc + col] =
+                                    f32_to_bf16_rne(acc[j][e]);
+                            else
+                                static_cast<float *>(c_q)[row * p.ldc + col] = acc[j][e];
+                        }
+                    }
+            }
+        }
+    }
+    __syncthreads();  // the next problem starts over with the first LDS buffer
+    }
+}
+
+// Launches the kernel above for problems of one width; false when the shape is not one
+// of its own (the caller then takes the general kernel per problem).
+bool rows_kernel_takes(int64_t total_rows, int64_t k, const void *const *c, int n_problems,
+                       int c_is_bf16, int64_t ldc) {
+    if (!(k == 64 || k == 128 || k == 256) || total_rows < 4096) return false;
+    // the staged stores write 16 bytes at a time: C rows must keep them aligned
+    if (ldc % (c_is_bf16 ? 8 : 4) != 0) return false;
+    for (int q = 0; q < n_problems; q++)
+        if (!aligned16(c[q])) return false;
+    return true;
+}
+
+int rows_kernel_launch(const HRowsParams &p, int k, int c_is_bf16, hipStream_t stream) {
+    const int n_tiles = p.tile_start[p.n_problems];
+    dim3 grid((unsigned)std::min(n_tiles, 512), (unsigned)ceil_div(p.N, HN));
+    if (k == 256) {
+        if (c_is_bf16) hgemm_rows_kernel<true, 16><<<grid, 256, 0, stream>>>(p);
+        else hgemm_rows_kernel<false, 16><<<grid, 256, 0, stream>>>(p);
+    } else if (k == 128) {
+        if (c_is_bf16) hgemm_rows_kernel<true, 8><<<grid, 256, 0, stream>>>(p);
+        else hgemm_rows_kernel<false, 8><<<grid, 256, 0, stream>>>(p);
+    } else {
+        if (c_is_bf16) hgemm_rows_kernel<true, 4><<<grid, 256, 0, stream>>>(p);
+        else hgemm_rows_kernel<false, 4><<<grid, 256, 0, stream>>>(p);
+    }
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
 // dst[n][k] = src[k][n] for a [K, N] matrix of 16-bit elements (32 x 32 tiles through LDS)
-__global__ __launch_bounds__(256) void transpose16_kernel(uint16_t *__restrict__ dst,
-                                                          const uint16_t *__restrict__ src, int K,
-                                                          int N, int64_t ld_src, int64_t ld_dst) {
+struct Transpose16Params {
+    uint16_t *dst[kRowsProblems];        // [N, ld_dst]
+    const uint16_t *src[kRowsProblems];  // [K, ld_src]
+};
+
+__global__ __launch_bounds__(256) void transpose16_kernel(Transpose16Params tp, int K, int N,
+                                                          int64_t ld_src, int64_t ld_dst) {
     __shared__ uint16_t tile[32][33];
+    uint16_t *__restrict__ dst = tp.dst[blockIdx.z];
+    const uint16_t *__restrict__ src = tp.src[blockIdx.z];
     const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
     for (int r = ty; r < 32; r += 8)
@@ -364,12 +583,27 @@ YITU_API int yitu_gemm_bf16(void *c, int c_is_bf16, const void *a, const void *b
         YITU_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
                      "workspace too small for the transposed weight: need %zu bytes", need);
         dim3 tg((unsigned)ceil_div(n, 32), (unsigned)ceil_div(k, 32));
-        transpose16_kernel<<<tg, 256, 0, stream>>>(static_cast<uint16_t *>(workspace),
-                                                   static_cast<const uint16_t *>(b), (int)k, (int)n,
-                                                   ldb, k);
+        Transpose16Params tp{};
+        tp.dst[0] = static_cast<uint16_t *>(workspace);
+        tp.src[0] = static_cast<const uint16_t *>(b);
+        transpose16_kernel<<<tg, 256, 0, stream>>>(tp, (int)k, (int)n, ldb, k);
         YITU_LAUNCH_CHECK();
         p.Bt = static_cast<const uint16_t *>(workspace);
         p.ldbt = k;
+    }
+    if (rows_kernel_takes(m, k, &c, 1, c_is_bf16, ldc)) {
+        HRowsParams r{};
+        r.A[0] = p.A;
+        r.Bt[0] = p.Bt;
+        r.C[0] = c;
+        r.M[0] = (int)m;
+        r.tile_start[1] = (int)ceil_div(m, RM);
+        r.n_problems = 1;
+        r.N = (int)n;
+        r.lda = lda;
+        r.ldbt = p.ldbt;
+        r.ldc = ldc;
+        return rows_kernel_launch(r, (int)k, c_is_bf16, stream);
     }
     dim3 grid((unsigned)ceil_div(m, HM), (unsigned)ceil_div(n, HN));
     if (c_is_bf16)
@@ -377,6 +611,82 @@ YITU_API int yitu_gemm_bf16(void *c, int c_is_bf16, const void *a, const void *b
     else
         hgemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+
+YITU_API size_t yitu_gemm_bf16_typed_workspace_bytes(int64_t n_problems, int64_t n, int64_t k,
+                                                     int trans_b) {
+    if (trans_b) return 256;
+    const int64_t group = std::min<int64_t>(std::max<int64_t>(n_problems, 1), kRowsProblems);
+    return (size_t)group * align_up((size_t)(n * k) * sizeof(uint16_t), 256) + 256;
+}
+
+YITU_API int yitu_gemm_bf16_typed(void *const *c, int c_is_bf16, const void *const *a,
+                                  const void *const *b, const int64_t *m, int64_t n_problems,
+                                  int64_t n, int64_t k, int trans_b, int64_t lda, int64_t ldb,
+                                  int64_t ldc, void *workspace, size_t workspace_bytes,
+                                  void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_problems >= 0 && n >= 0 && k >= 0, "negative size");
+    if (n_problems == 0 || n == 0) return 0;
+    YITU_REQUIRE(c && a && b && m, "null pointer list");
+    YITU_REQUIRE(n < INT32_MAX && k < INT32_MAX && ldc >= n, "size out of range");
+    YITU_REQUIRE(k % 8 == 0 && lda % 8 == 0 && lda >= k,
+                 "bf16 GEMM needs K and lda to be multiples of 8");
+    YITU_REQUIRE(ldb >= (trans_b ? k : n), "leading dimension of B too small");
+    int64_t total = 0;
+    bool aligned = trans_b ? ldb % 8 == 0 : true;
+    for (int64_t q = 0; q < n_problems; q++) {
+        YITU_REQUIRE(m[q] >= 0 && m[q] < INT32_MAX, "row count out of range");
+        YITU_REQUIRE(m[q] == 0 || (c[q] && (k == 0 || (a[q] && b[q]))), "null operand");
+        total += m[q];
+        aligned = aligned && aligned16(a[q]) && (!trans_b || aligned16(b[q]));
+    }
+    const size_t slot = align_up((size_t)(n * k) * sizeof(uint16_t), 256);
+    const bool fits = trans_b || (workspace && aligned16(workspace) &&
+                                  workspace_bytes >= yitu_gemm_bf16_typed_workspace_bytes(
+                                                         n_problems, n, k, trans_b));
+    if (!(aligned && fits && total < INT32_MAX &&
+          rows_kernel_takes(total, k, c, (int)n_problems, c_is_bf16, ldc))) {
+        for (int64_t q = 0; q < n_problems; q++) {
+            const int rc = yitu_gemm_bf16(c[q], c_is_bf16, a[q], b[q], m[q], n, k, trans_b, lda,
+                                          ldb, ldc, workspace, workspace_bytes, stream_);
+            if (rc) return rc;
+        }
+        return 0;
+    }
+    for (int64_t g0 = 0; g0 < n_problems; g0 += kRowsProblems) {
+        const int cnt = (int)std::min<int64_t>(kRowsProblems, n_problems - g0);
+        HRowsParams r{};
+        Transpose16Params tp{};
+        for (int q = 0; q < cnt; q++) {
+            r.A[q] = static_cast<const uint16_t *>(a[g0 + q]);
+            r.C[q] = c[g0 + q];
+            r.M[q] = (int)m[g0 + q];
+            r.tile_start[q + 1] = r.tile_start[q] + (int)ceil_div(m[g0 + q], RM);
+            if (trans_b) {
+                r.Bt[q] = static_cast<const uint16_t *>(b[g0 + q]);
+            } else {
+                tp.dst[q] = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + q * slot);
+                tp.src[q] = static_cast<const uint16_t *>(b[g0 + q]);
+                r.Bt[q] = tp.dst[q];
+            }
+        }
+        r.n_problems = cnt;
+        r.N = (int)n;
+        r.lda = lda;
+        r.ldbt = trans_b ? ldb : k;
+        r.ldc = ldc;
+        if (r.tile_start[cnt] == 0) continue;
+        if (!trans_b) {
+            dim3 tg((unsigned)ceil_div(n, 32), (unsigned)ceil_div(k, 32), (unsigned)cnt);
+            transpose16_kernel<<<tg, 256, 0, stream>>>(tp, (int)k, (int)n, ldb, k);
+            YITU_LAUNCH_CHECK();
+        }
+        const int rc = rows_kernel_launch(r, (int)k, c_is_bf16, stream);
+        if (rc) return rc;
+    }
     return 0;
 }
 

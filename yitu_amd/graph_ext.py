@@ -582,6 +582,50 @@ def gemm_bf16(a, b, trans_b=False, out_dtype=torch.float32, out=None):
     return c
 
 
+def gemm_bf16_typed(a_list, b_list, trans_b=False, out_dtype=torch.float32, out_list=None):
+    """[a_i . op(b_i)] with bf16 operands for pairs that share the widths (the per-type
+    Linear layers of a heterogeneous model in bf16), eight products per launch.
+    ``out_list``: contiguous [m_i, n] fp32 or bf16 tensors to write (e.g. row slices of
+    one buffer; sets ``out_dtype``)."""
+    import ctypes
+    if len(a_list) != len(b_list) or not a_list:
+        raise RuntimeError("gemm_bf16_typed needs as many a as b operands, at least one")
+    for a, b in zip(a_list, b_list):
+        _check(a, torch.bfloat16, "a", 2)
+        _check(b, torch.bfloat16, "b", 2)
+    dev = _lib.require_device(*a_list, *b_list)
+    k = a_list[0].size(1)
+    n = b_list[0].size(0) if trans_b else b_list[0].size(1)
+    for a, b in zip(a_list, b_list):
+        if a.size(1) != k or tuple(b.shape) != ((n, k) if trans_b else (k, n)):
+            raise RuntimeError("gemm_bf16_typed: every pair must be [m_i, %d] x %s"
+                               % (k, "[%d, %d]" % ((n, k) if trans_b else (k, n))))
+    ms = [a.size(0) for a in a_list]
+    if out_list is None:
+        if out_dtype not in (torch.float32, torch.bfloat16):
+            raise RuntimeError("out_dtype must be float32 or bfloat16")
+        out_list = [torch.empty((m, n), dtype=out_dtype, device=dev) for m in ms]
+    else:
+        out_dtype = out_list[0].dtype
+        for c, m in zip(out_list, ms):
+            if c.dtype != out_dtype or out_dtype not in (torch.float32, torch.bfloat16) \
+                    or tuple(c.shape) != (m, n) or c.device != dev or not c.is_contiguous():
+                raise RuntimeError("out must be contiguous [%d, %d] fp32 or bf16 tensors of one "
+                                   "type" % (m, n))
+    count = len(a_list)
+    ws = _lib.workspace(_size_fn("yitu_gemm_bf16_typed_workspace_bytes")(
+        c_i64(count), c_i64(n), c_i64(k), c_int(int(trans_b))), dev)
+    pointers = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() or None for t in ts])
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gemm_bf16_typed(
+            pointers(out_list), c_int(int(out_dtype == torch.bfloat16)), pointers(a_list),
+            pointers(b_list), (ctypes.c_int64 * count)(*ms), c_i64(count), c_i64(n), c_i64(k),
+            c_int(int(trans_b)), c_i64(k), c_i64(b_list[0].size(1)), c_i64(n), ptr(ws),
+            c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_gemm_bf16_typed")
+    return list(out_list)
+
+
 def gemm_bf16_tn(a, b, out=None, accumulate=False):
     """a^T . b for bf16 ``a`` [m, ki] and ``b`` [m, no] (rows may be strided slices of a
     wider buffer), fp32 accumulation on the matrix cores, fp32 [ki, no] out: the weight
