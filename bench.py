@@ -611,7 +611,7 @@ def run_c4(args, dev):
     def gemm_bwd16(dh):
         dh16 = dh.view(n_all, dim).to(torch.bfloat16)  # one rounding pass over the gradient rows
         parts = [dh16[off[t]:off[t + 1]] for t in range(4)]
-        dws = [graph_ext.gemm_bf16_tn(xs16[t], parts[t]) for t in range(4)]
+        dws = graph_ext.gemm_bf16_tn_typed(xs16, parts)
         dxs = graph_ext.gemm_bf16_typed(parts, wts16, trans_b=True, out_dtype=torch.bfloat16)
         return dws, dxs
 

@@ -483,6 +483,22 @@ int yitu_gemm_bf16_tn(float *c_device, const void *a_bf16_device, const void *b_
                       int64_t m, int64_t ki, int64_t no, int64_t lda, int64_t ldb, int64_t ldc,
                       int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
 
+/*
+ * The same for a list of operand pairs of one shape [m_i, ki], [m_i, no] (the weight
+ * gradients of the per-type / per-relation Linear layers, test/common/model.py:137-171
+ * over :7-30, backward), one launch pair per 8 problems: the row chunks of every pair
+ * share one grid. c, a, b are HOST arrays of device pointers, m a HOST array of row
+ * counts; a pair without rows writes zeros (or leaves C_i as it is with accumulate).
+ * Workspace: yitu_gemm_bf16_tn_typed_workspace_bytes(m, n_problems, ki, no).
+ */
+size_t yitu_gemm_bf16_tn_typed_workspace_bytes(const int64_t *m, int64_t n_problems, int64_t ki,
+                                               int64_t no);
+int yitu_gemm_bf16_tn_typed(float *const *c_device_ptrs, const void *const *a_bf16_device_ptrs,
+                            const void *const *b_bf16_device_ptrs, const int64_t *m,
+                            int64_t n_problems, int64_t ki, int64_t no, int64_t lda, int64_t ldb,
+                            int64_t ldc, int accumulate, void *workspace_device,
+                            size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* Temporal neighbour attention                                                */
 /* ------------------------------------------------------------------------- */

@@ -231,6 +231,27 @@ def test_gemm_bf16_tn_against_double(dev, m, ki, no):
         assert_close(acc, want2.float(), abs_sum=abs2.float())
 
 
+@pytest.mark.parametrize("ms,ki,no", [([70000, 0, 4097, 300], 256, 256), ([900] * 10, 72, 136),
+                                      ([1, 31, 33], 8, 16)])
+def test_gemm_bf16_tn_typed_against_double(dev, ms, ki, no):
+    """Weight gradients of several node types in one call: the types' row chunks share a
+    grid, a type without rows gives zeros; reproducible; `accumulate` adds."""
+    g = torch.Generator().manual_seed(sum(ms) + ki + no)
+    a = [torch.randn(m, ki, generator=g).to(torch.bfloat16) for m in ms]
+    b = [torch.randn(m, no, generator=g).to(torch.bfloat16) for m in ms]
+    da, db = [x.to(dev) for x in a], [x.to(dev) for x in b]
+    got = graph_ext.gemm_bf16_tn_typed(da, db)
+    for x, y, c, m in zip(a, b, got, ms):
+        want = (x.double().t() @ y.double()).float()
+        assert_close(c, want, atol=1e-4 * max(1.0, np.sqrt(max(m, 1))))
+    again = graph_ext.gemm_bf16_tn_typed(da, db)
+    assert all(torch.equal(c, d) for c, d in zip(got, again))
+    acc = [torch.ones(ki, no, device=dev) for _ in ms]
+    graph_ext.gemm_bf16_tn_typed(da, db, out_list=acc, accumulate=True)
+    for c, d in zip(got, acc):
+        assert_close(d, c + 1.0, atol=1e-4 * max(1.0, np.sqrt(max(max(ms), 1))))
+
+
 def test_gemm_bf16_tn_rejects_unaligned_width(dev):
     a = torch.zeros(16, 12, dtype=torch.bfloat16, device=dev)
     b = torch.zeros(16, 8, dtype=torch.bfloat16, device=dev)

@@ -409,24 +409,46 @@ __global__ __launch_bounds__(256) void transpose16_kernel(Transpose16Params tp, 
 // (bitwise reproducible).
 constexpr int TN_TILE = 128, TN_ROWS = 32, TN_LD = TN_TILE + 4;  // padded LDS row (bf16)
 
+// Up to 8 products of one shape share the launch: their row chunks form one list,
+// chunk_start[q] is the first chunk of problem q.
 struct TnParams {
-    const uint16_t *A, *B;
-    float *partial;  // [n_chunks, Ki, No]
-    int M, Ki, No;
-    int64_t lda, ldb;
+    const uint16_t *A[kRowsProblems], *B[kRowsProblems];
+    float *C[kRowsProblems];  // [Ki, ldc]
+    int M[kRowsProblems];
+    int chunk_start[kRowsProblems + 1];
+    int n_problems;
+    float *partial;  // [chunks of all problems, Ki, No]
+    int Ki, No;
+    int64_t lda, ldb, ldc;
     int rows_per_chunk;  // multiple of TN_ROWS
+    int accumulate;
 };
 
-__global__ __launch_bounds__(256) void hgemm_tn_kernel(TnParams p) {
+constexpr int TN_DEPTH = 3;  // row stages requested ahead of the products
+
+__global__ __launch_bounds__(256, 3) void hgemm_tn_kernel(TnParams p) {
     __shared__ __attribute__((aligned(16))) uint16_t As[2][TN_ROWS][TN_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[2][TN_ROWS][TN_LD];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, lk = lane >> 5;
+    // Workgroups go to the 8 XCDs in turn. The output tiles of one row chunk read the same
+    // rows, so they are given ids that differ by multiples of 8: they run on one XCD, close
+    // in time, and all but the first find the rows in that XCD's L2. Spread over the XCDs
+    // every row crossed the fabric once per tile that reads it.
     const int tiles_j = (p.No + TN_TILE - 1) / TN_TILE;
-    const int i0 = (blockIdx.y / tiles_j) * TN_TILE, j0 = (blockIdx.y % tiles_j) * TN_TILE;
+    const int n_tiles = tiles_j * ((p.Ki + TN_TILE - 1) / TN_TILE);
+    const int tile = (blockIdx.x / 8) % n_tiles;
+    const int chunk = (blockIdx.x / 8 / n_tiles) * 8 + blockIdx.x % 8;
+    if (chunk >= p.chunk_start[p.n_problems]) return;  // same for the whole workgroup
+    const int i0 = (tile / tiles_j) * TN_TILE, j0 = (tile % tiles_j) * TN_TILE;
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
-    const int m_beg = blockIdx.x * p.rows_per_chunk;
-    const int m_end = min(p.M, m_beg + p.rows_per_chunk);
+    int q = 0;  // the chunk's problem (same for the whole workgroup)
+#pragma unroll
+    for (int k = 1; k < kRowsProblems; k++)
+        q += (k < p.n_problems && chunk >= p.chunk_start[k]) ? 1 : 0;
+    const uint16_t *__restrict__ A = p.A[q], *__restrict__ B = p.B[q];
+    const int m_beg = (chunk - p.chunk_start[q]) * p.rows_per_chunk;
+    const int m_end = min(p.M[q], m_beg + p.rows_per_chunk);
     // loader: thread -> (row, 8 columns); 16 threads cover the 128 columns of a row
     const int lrow = t >> 4, lcol = (t & 15) * 8;
 
@@ -438,28 +460,35 @@ __global__ __launch_bounds__(256) void hgemm_tn_kernel(TnParams p) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[a][b][e] = 0.0f;
 
-    uint4 ra[2], rb[2];
-    auto gload = [&](int m0) {
+    // Rows are requested TN_DEPTH stages ahead through a ring of registers: one stage
+    // ahead left 16 KB per workgroup in flight, too little to cover the memory latency.
+    uint4 ra[TN_DEPTH][2], rb[TN_DEPTH][2];
+    const bool a_cols = i0 + lcol < p.Ki, b_cols = j0 + lcol < p.No;
+    auto gload = [&](int slot, int m0) {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const int row = m0 + lrow + 16 * h;
             const bool in = row < m_end;
             // Ki, No are multiples of 8: a column below the bound has its 8 elements
-            ra[h] = (in && i0 + lcol < p.Ki)
-                        ? *reinterpret_cast<const uint4 *>(p.A + (int64_t)row * p.lda + i0 + lcol)
-                        : make_uint4(0, 0, 0, 0);
-            rb[h] = (in && j0 + lcol < p.No)
-                        ? *reinterpret_cast<const uint4 *>(p.B + (int64_t)row * p.ldb + j0 + lcol)
-                        : make_uint4(0, 0, 0, 0);
+            ra[slot][h] = (in && a_cols)
+                              ? *reinterpret_cast<const uint4 *>(A + (int64_t)row * p.lda + i0 + lcol)
+                              : make_uint4(0, 0, 0, 0);
+            rb[slot][h] = (in && b_cols)
+                              ? *reinterpret_cast<const uint4 *>(B + (int64_t)row * p.ldb + j0 + lcol)
+                              : make_uint4(0, 0, 0, 0);
         }
     };
-    auto lstore = [&](int buf) {
+    auto lstore = [&](int slot, int buf) {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol]) = make_uint2(ra[h].x, ra[h].y);
-            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol + 4]) = make_uint2(ra[h].z, ra[h].w);
-            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol]) = make_uint2(rb[h].x, rb[h].y);
-            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol + 4]) = make_uint2(rb[h].z, rb[h].w);
+            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol]) =
+                make_uint2(ra[slot][h].x, ra[slot][h].y);
+            *reinterpret_cast<uint2 *>(&As[buf][lrow + 16 * h][lcol + 4]) =
+                make_uint2(ra[slot][h].z, ra[slot][h].w);
+            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol]) =
+                make_uint2(rb[slot][h].x, rb[slot][h].y);
+            *reinterpret_cast<uint2 *>(&Bs[buf][lrow + 16 * h][lcol + 4]) =
+                make_uint2(rb[slot][h].z, rb[slot][h].w);
         }
     };
     // operand pair (even column, odd column) of the 8 rows kk + 8 * lk .. + 7
@@ -479,33 +508,40 @@ __global__ __launch_bounds__(256) void hgemm_tn_kernel(TnParams p) {
     };
 
     if (m_beg < m_end) {
-        gload(m_beg);
-        lstore(0);
+        const int n_steps = (m_end - m_beg + TN_ROWS - 1) / TN_ROWS;
+#pragma unroll
+        for (int u = 0; u < TN_DEPTH; u++) gload(u, m_beg + u * TN_ROWS);  // past the end: zeros
+        lstore(0, 0);
         __syncthreads();
-        int buf = 0;
-        for (int m0 = m_beg; m0 < m_end; m0 += TN_ROWS) {
-            const bool more = m0 + TN_ROWS < m_end;
-            if (more) gload(m0 + TN_ROWS);
+        for (int s0 = 0; s0 < n_steps; s0 += TN_DEPTH) {
 #pragma unroll
-            for (int kk = 0; kk < TN_ROWS; kk += 16) {
-                bf16x8 a[2], b[2];
-                fragments(As[buf], wi, kk, a[0], a[1]);
-                fragments(Bs[buf], wj, kk, b[0], b[1]);
+            for (int u = 0; u < TN_DEPTH; u++) {
+                const int st = s0 + u;
+                if (st >= n_steps) break;  // same for the whole workgroup
+                const int buf = st & 1;
+                // stage st went to LDS during stage st - 1: its slot takes stage st + TN_DEPTH
+                gload(u, m_beg + (st + TN_DEPTH) * TN_ROWS);
 #pragma unroll
-                for (int x = 0; x < 2; x++)
+                for (int kk = 0; kk < TN_ROWS; kk += 16) {
+                    bf16x8 a[2], b[2];
+                    fragments(As[buf], wi, kk, a[0], a[1]);
+                    fragments(Bs[buf], wj, kk, b[0], b[1]);
 #pragma unroll
-                    for (int y = 0; y < 2; y++)
-                        acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
+                    for (int x = 0; x < 2; x++)
+#pragma unroll
+                        for (int y = 0; y < 2; y++)
+                            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y],
+                                                                               0, 0, 0);
+                }
+                if (st + 1 < n_steps) lstore((u + 1) % TN_DEPTH, buf ^ 1);
+                __syncthreads();
             }
-            if (more) lstore(buf ^ 1);
-            __syncthreads();
-            buf ^= 1;
         }
     }
     // accumulator element 4*jj + ii of tile (x, y) is row 8jj + 4lk + ii, column l32 of the
     // MFMA tile; MFMA row r of parity x is output row wi + 2r + x, column c of parity y is
     // output column wj + 2c + y
-    float *dst = p.partial + (int64_t)blockIdx.x * p.Ki * p.No;
+    float *dst = p.partial + (int64_t)chunk * p.Ki * p.No;
 #pragma unroll
     for (int x = 0; x < 2; x++)
 #pragma unroll
@@ -521,26 +557,69 @@ __global__ __launch_bounds__(256) void hgemm_tn_kernel(TnParams p) {
         }
 }
 
-// C[i] (+)= sum over chunks of partial[c][i], in chunk order
-__global__ __launch_bounds__(256) void hgemm_tn_reduce_kernel(float *__restrict__ c, int64_t ldc,
-                                                              const float *__restrict__ partial,
-                                                              int n_chunks, int Ki, int No,
-                                                              int accumulate) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)Ki * No) return;
-    float s = 0.0f;
-    for (int k = 0; k < n_chunks; k++) s += partial[(int64_t)k * Ki * No + idx];
-    float *out = c + (idx / No) * ldc + idx % No;
-    *out = accumulate ? *out + s : s;
+// C_q (+)= sum over the problem's chunks of its partial products, in a fixed order. A
+// workgroup takes 64 consecutive outputs; its four 64-thread groups each add a quarter of
+// the chunks with four independent running sums and the quarters are combined through
+// LDS (one thread per output walking every chunk is a chain of dependent loads).
+__global__ __launch_bounds__(256) void hgemm_tn_reduce_kernel(TnParams p) {
+    __shared__ float red[4][64];
+    const int q = blockIdx.y;
+    const int c0 = p.chunk_start[q], n_chunks = p.chunk_start[q + 1] - c0;
+    if (p.M[q] == 0 && p.accumulate) return;
+    const int64_t total = (int64_t)p.Ki * p.No;
+    const int e_lane = threadIdx.x & 63, zg = threadIdx.x >> 6;
+    const int per = (n_chunks + 3) / 4;
+    const int zb = min(zg * per, n_chunks), ze = min(zb + per, n_chunks);
+    float *__restrict__ c = p.C[q];
+    for (int64_t e0 = (int64_t)blockIdx.x * 64; e0 < total; e0 += (int64_t)gridDim.x * 64) {
+        const int64_t e = e0 + e_lane;
+        const bool live = e < total;
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+        if (live) {
+            const float *src = p.partial + (size_t)c0 * total + e;
+            int z = zb;
+            for (; z + 4 <= ze; z += 4) {
+                a0 += src[(size_t)z * total];
+                a1 += src[(size_t)(z + 1) * total];
+                a2 += src[(size_t)(z + 2) * total];
+                a3 += src[(size_t)(z + 3) * total];
+            }
+            for (; z < ze; z++) a0 += src[(size_t)z * total];
+        }
+        red[zg][e_lane] = (a0 + a1) + (a2 + a3);
+        __syncthreads();
+        if (zg == 0 && live) {
+            const float sum = ((red[0][e_lane] + red[1][e_lane]) + red[2][e_lane]) + red[3][e_lane];
+            float *out = c + (e / p.No) * p.ldc + e % p.No;
+            *out = p.accumulate ? *out + sum : sum;
+        }
+        __syncthreads();
+    }
 }
 
-// Row chunks of the A^T.B product: enough workgroups for about three per CU, chunks a
-// multiple of the stage height.
-inline int tn_chunk_rows(int64_t m, int64_t ki, int64_t no) {
+// Row chunks of the A^T.B products: as many workgroups as the chip holds at once (three
+// per CU) over all the problems of a launch and no more, since a few left over would run
+// alone for as long again; chunks a multiple of the stage height. Every problem may add a
+// chunk by rounding, and the chunk count is rounded up to a multiple of 8.
+inline int tn_chunk_rows(int64_t total_rows, int64_t ki, int64_t no, int count) {
     const int64_t tiles = ceil_div(ki, TN_TILE) * ceil_div(no, TN_TILE);
-    const int64_t want_chunks = std::max<int64_t>(1, 768 / tiles);
-    int64_t rows = ceil_div(ceil_div(m, want_chunks), TN_ROWS) * TN_ROWS;
+    const int64_t want_chunks = std::max<int64_t>(1, 768 / tiles - count - 7);
+    int64_t rows = ceil_div(ceil_div(total_rows, want_chunks), TN_ROWS) * TN_ROWS;
     return (int)std::max<int64_t>(rows, 4 * TN_ROWS);
+}
+
+// chunks of a group of problems that share one launch (an empty problem keeps one chunk
+// of zeros, so that its output is written)
+inline int64_t tn_group_chunks(const int64_t *m, int count, int rows) {
+    int64_t chunks = 0;
+    for (int q = 0; q < count; q++) chunks += std::max<int64_t>(1, ceil_div(m[q], rows));
+    return chunks;
+}
+
+inline int64_t tn_group_rows(const int64_t *m, int count) {
+    int64_t total = 0;
+    for (int q = 0; q < count; q++) total += m[q];
+    return total;
 }
 
 }  // namespace
@@ -691,43 +770,79 @@ YITU_API int yitu_gemm_bf16_typed(void *const *c, int c_is_bf16, const void *con
 }
 
 
+YITU_API size_t yitu_gemm_bf16_tn_typed_workspace_bytes(const int64_t *m, int64_t n_problems,
+                                                        int64_t ki, int64_t no) {
+    int64_t most = 1;
+    for (int64_t g0 = 0; m && g0 < n_problems; g0 += kRowsProblems) {
+        const int cnt = (int)std::min<int64_t>(kRowsProblems, n_problems - g0);
+        const int rows = tn_chunk_rows(tn_group_rows(m + g0, cnt), ki, no, cnt);
+        most = std::max(most, tn_group_chunks(m + g0, cnt, rows));
+    }
+    return align_up((size_t)(most * ki * no) * sizeof(float), 256) + 256;
+}
+
+YITU_API int yitu_gemm_bf16_tn_typed(float *const *c, const void *const *a, const void *const *b,
+                                     const int64_t *m, int64_t n_problems, int64_t ki, int64_t no,
+                                     int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
+                                     void *workspace, size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_problems >= 0 && ki >= 0 && no >= 0, "negative size");
+    if (n_problems == 0 || ki == 0 || no == 0) return 0;
+    YITU_REQUIRE(c && a && b && m, "null pointer list");
+    YITU_REQUIRE(ki < (1 << 20) && no < (1 << 20) && ldc >= no, "size out of range");
+    YITU_REQUIRE(ki % 8 == 0 && no % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && lda >= ki &&
+                     ldb >= no,
+                 "bf16 A^T.B needs both widths and leading dimensions to be multiples of 8");
+    for (int64_t q = 0; q < n_problems; q++) {
+        YITU_REQUIRE(m[q] >= 0 && m[q] < INT32_MAX, "row count out of range");
+        YITU_REQUIRE(c[q] && (m[q] == 0 || (a[q] && b[q])), "null operand");
+        YITU_REQUIRE(aligned16(a[q]) && aligned16(b[q]), "bf16 A^T.B needs 16-byte aligned operands");
+    }
+    const size_t need = yitu_gemm_bf16_tn_typed_workspace_bytes(m, n_problems, ki, no) - 256;
+    YITU_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
+                 "workspace too small for the partial products: need %zu bytes", need);
+    for (int64_t g0 = 0; g0 < n_problems; g0 += kRowsProblems) {
+        const int cnt = (int)std::min<int64_t>(kRowsProblems, n_problems - g0);
+        TnParams p{};
+        p.rows_per_chunk = tn_chunk_rows(tn_group_rows(m + g0, cnt), ki, no, cnt);
+        for (int q = 0; q < cnt; q++) {
+            p.A[q] = static_cast<const uint16_t *>(a[g0 + q]);
+            p.B[q] = static_cast<const uint16_t *>(b[g0 + q]);
+            p.C[q] = c[g0 + q];
+            p.M[q] = (int)m[g0 + q];
+            p.chunk_start[q + 1] =
+                p.chunk_start[q] +
+                (int)std::max<int64_t>(1, ceil_div(m[g0 + q], (int64_t)p.rows_per_chunk));
+        }
+        p.n_problems = cnt;
+        p.partial = static_cast<float *>(workspace);
+        p.Ki = (int)ki;
+        p.No = (int)no;
+        p.lda = lda;
+        p.ldb = ldb;
+        p.ldc = ldc;
+        p.accumulate = accumulate;
+        const int64_t wgs = ceil_div((int64_t)p.chunk_start[cnt], 8) * 8 * ceil_div(ki, TN_TILE) *
+                            ceil_div(no, TN_TILE);
+        hgemm_tn_kernel<<<(unsigned)wgs, 256, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+        dim3 rgrid((unsigned)std::min<int64_t>(ceil_div(ki * no, 64), 4096), (unsigned)cnt);
+        hgemm_tn_reduce_kernel<<<rgrid, 256, 0, stream>>>(p);
+        YITU_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 YITU_API size_t yitu_gemm_bf16_tn_workspace_bytes(int64_t m, int64_t ki, int64_t no) {
-    const int64_t chunks = ceil_div(std::max<int64_t>(m, 1), tn_chunk_rows(m, ki, no));
-    return align_up((size_t)(chunks * ki * no) * sizeof(float), 256) + 256;
+    return yitu_gemm_bf16_tn_typed_workspace_bytes(&m, 1, ki, no);
 }
 
 YITU_API int yitu_gemm_bf16_tn(float *c, const void *a, const void *b, int64_t m, int64_t ki,
                                int64_t no, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
                                void *workspace, size_t workspace_bytes, void *stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    YITU_REQUIRE(m >= 0 && ki >= 0 && no >= 0, "negative size");
+    YITU_REQUIRE(m >= 0, "negative size");
     if (ki == 0 || no == 0) return 0;
     YITU_REQUIRE(c && (m == 0 || (a && b)), "null operand");
-    YITU_REQUIRE(m < INT32_MAX && ki < (1 << 20) && no < (1 << 20) && ldc >= no, "size out of range");
-    YITU_REQUIRE(ki % 8 == 0 && no % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && lda >= ki &&
-                     ldb >= no && aligned16(a) && aligned16(b),
-                 "bf16 A^T.B needs both widths and leading dimensions to be multiples of 8 and "
-                 "16-byte aligned operands");
-    const int rows = tn_chunk_rows(m, ki, no);
-    const int64_t chunks = ceil_div(std::max<int64_t>(m, 1), rows);
-    const size_t need = (size_t)(chunks * ki * no) * sizeof(float);
-    YITU_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
-                 "workspace too small for the partial products: need %zu bytes", need);
-    TnParams p{};
-    p.A = static_cast<const uint16_t *>(a);
-    p.B = static_cast<const uint16_t *>(b);
-    p.partial = static_cast<float *>(workspace);
-    p.M = (int)m;
-    p.Ki = (int)ki;
-    p.No = (int)no;
-    p.lda = lda;
-    p.ldb = ldb;
-    p.rows_per_chunk = rows;
-    dim3 grid((unsigned)chunks, (unsigned)(ceil_div(ki, TN_TILE) * ceil_div(no, TN_TILE)));
-    hgemm_tn_kernel<<<grid, 256, 0, stream>>>(p);
-    YITU_LAUNCH_CHECK();
-    hgemm_tn_reduce_kernel<<<(unsigned)ceil_div(ki * no, 256), 256, 0, stream>>>(
-        c, ldc, p.partial, (int)chunks, (int)ki, (int)no, accumulate);
-    YITU_LAUNCH_CHECK();
-    return 0;
+    return yitu_gemm_bf16_tn_typed(&c, &a, &b, &m, 1, ki, no, lda, ldb, ldc, accumulate, workspace,
+                                   workspace_bytes, stream_);
 }

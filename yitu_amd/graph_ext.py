@@ -656,6 +656,49 @@ def gemm_bf16_tn(a, b, out=None, accumulate=False):
     return out
 
 
+def gemm_bf16_tn_typed(a_list, b_list, out_list=None, accumulate=False):
+    """[a_i^T . b_i] for bf16 pairs [m_i, ki], [m_i, no] of one shape (rows may be strided
+    slices of wider buffers with a common row stride): the weight gradients of a
+    heterogeneous bf16 layer, eight products per launch. fp32 [ki, no] outputs."""
+    import ctypes
+    if len(a_list) != len(b_list) or not a_list:
+        raise RuntimeError("gemm_bf16_tn_typed needs as many a as b operands, at least one")
+    for t in list(a_list) + list(b_list):
+        if t.dtype != torch.bfloat16 or t.dim() != 2 or t.stride(1) != 1 or not t.is_cuda:
+            raise RuntimeError("operands must be 2-D bf16 GPU tensors with contiguous rows")
+    dev = a_list[0].device
+    ki, no = a_list[0].size(1), b_list[0].size(1)
+    lda, ldb = a_list[0].stride(0), b_list[0].stride(0)
+    for a, b in zip(a_list, b_list):
+        if a.device != dev or b.device != dev or a.size(0) != b.size(0) or a.size(1) != ki \
+                or b.size(1) != no or (a.size(0) > 1 and a.stride(0) != lda) \
+                or (b.size(0) > 1 and b.stride(0) != ldb):
+            raise RuntimeError("gemm_bf16_tn_typed: every pair must be [m_i, %d], [m_i, %d] with "
+                               "common row strides on one device" % (ki, no))
+    ms = [a.size(0) for a in a_list]
+    if out_list is None:
+        if accumulate:
+            raise RuntimeError("accumulate needs outputs to add to")
+        out_list = [torch.empty((ki, no), dtype=torch.float32, device=dev) for _ in ms]
+    else:
+        for c in out_list:
+            if c.dtype != torch.float32 or tuple(c.shape) != (ki, no) or not c.is_contiguous() \
+                    or c.device != dev:
+                raise RuntimeError("out must be contiguous fp32 [%d, %d] tensors" % (ki, no))
+    count = len(a_list)
+    m_arr = (ctypes.c_int64 * count)(*ms)
+    ws = _lib.workspace(_size_fn("yitu_gemm_bf16_tn_typed_workspace_bytes")(
+        m_arr, c_i64(count), c_i64(ki), c_i64(no)), dev)
+    pointers = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() or None for t in ts])
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_gemm_bf16_tn_typed(
+            pointers(out_list), pointers(a_list), pointers(b_list), m_arr, c_i64(count), c_i64(ki),
+            c_i64(no), c_i64(max(lda, ki)), c_i64(max(ldb, no)), c_i64(no), c_int(int(accumulate)),
+            ptr(ws), c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_gemm_bf16_tn_typed")
+    return list(out_list)
+
+
 # --------------------------------------------------------------------------- #
 # fused GAT attention (extension: the composition sddmm_forward -> spmm_forward)
 # --------------------------------------------------------------------------- #
