@@ -1057,6 +1057,7 @@ struct GatSrcParams {
                      // feat = grad_out, out = grad_x, plan = its row plan, partial
     const float *x;  // [n_src, L]
     float *grad_a;   // [nnz, H], CSR order: d_attn (FULL = false) or the logit gradient (FULL)
+    int grad_a_vec;  // grad_a is 16-byte aligned and H a multiple of 4: vector stores
     // FULL: the forward output is at hand, so the softmax row sum S[r,h] = sum_e a d_attn
     // = <grad_out[r,h,:], out[r,h,:]> is known before the pass and the whole
     // softmax + LeakyReLU backward happens per edge, here
@@ -1218,17 +1219,37 @@ __device__ __forceinline__ void gat_src_window(const GatSrcParams &p, const Edge
         }
         const int k = j * LPH + sub;
         const int vr = __shfl(win.vrow, first + min(k, n - 1), kWave);
-        if (k < n) {
+        // The per-(edge, head) results go to grad_a through the edge permutation: scattered
+        // stores. The W heads of an edge that sit in lanes LPH apart are collected by the
+        // first of them and leave as one 8- or 16-byte store: a store of 4 bytes costs the
+        // L2 a request of its own, four per edge.
+        constexpr int W = NS >= 4 ? 4 : NS;
 #pragma unroll
-            for (int t = 0; t < KT; t++) {
-                float *dst = p.grad_a + (size_t)vr * H + t * NS + h;
-                if constexpr (FULL) {
-                    const float gl = ea[j][t] * (keep[t] - eS[j][t]) *
-                                     (eq[j][t] + kc[t] < 0.0f ? kSlope : 1.0f);
-                    *dst = gl;
-                    gk[t] += gl;
-                } else {
-                    *dst = keep[t];
+        for (int t = 0; t < KT; t++) {
+            float val = keep[t];
+            if constexpr (FULL) {
+                val = ea[j][t] * (keep[t] - eS[j][t]) * (eq[j][t] + kc[t] < 0.0f ? kSlope : 1.0f);
+                if (k < n) gk[t] += val;
+            }
+            if constexpr (W == 1) {
+                if (k < n) p.grad_a[(size_t)vr * H + t * NS + h] = val;
+            } else {
+                float w[W];
+                w[0] = val;
+#pragma unroll
+                for (int i = 1; i < W; i++) w[i] = __shfl(val, lane + i * LPH, kWave);
+                if (k < n && h % W == 0) {
+                    float *dst = p.grad_a + (size_t)vr * H + t * NS + h;
+                    if (p.grad_a_vec) {
+                        typedef float fw __attribute__((ext_vector_type(W)));
+                        fw v;
+#pragma unroll
+                        for (int i = 0; i < W; i++) v[i] = w[i];
+                        *reinterpret_cast<fw *>(dst) = v;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < W; i++) dst[i] = w[i];
+                    }
                 }
             }
         }
@@ -1660,6 +1681,7 @@ int spmm_backward_one_gather(float *grad_a, float *grad_x, const float *values,
     p.sp.alpha = 1.0f;
     p.x = features;
     p.grad_a = grad_a;
+    p.grad_a_vec = aligned16(grad_a) ? 1 : 0;
     p.g_ld = (int)L;
     p.g_scale = 1.0f;
     bool has_items = false;
@@ -2031,6 +2053,7 @@ YITU_API int yitu_gat_backward(float *grad_query, float *grad_key, float *grad_f
         p.sp.alpha = 1.0f;
         p.x = features;
         p.grad_a = grad_attn_scratch;
+        p.grad_a_vec = aligned16(grad_attn_scratch) ? 1 : 0;
         p.g_ld = grad_out_is_head_mean ? (int)n_features : (int)L;
         p.head_mean = grad_out_is_head_mean ? 1 : 0;
         p.g_scale = grad_out_is_head_mean ? 1.0f / (float)n_heads : 1.0f;
