@@ -604,12 +604,13 @@ def run_c4(args, dev):
     d_out16 = d_out.to(torch.bfloat16)
 
     def agg_bwd16():
-        # bf16 gradient rows in, fp32 sums, fp32 rows out
+        # bf16 gradient rows in, fp32 sums, bf16 rows out (one rounding per output)
         return graph_ext.spmm_backward(values, indptr, indices, h_all16.view(n_all, 1, dim),
-                                       d_out16.view(n_all, 1, dim), need_grad_a=False)[1]
+                                       d_out16.view(n_all, 1, dim), need_grad_a=False,
+                                       grad_x_dtype=torch.bfloat16)[1]
 
     def gemm_bwd16(dh):
-        dh16 = dh.view(n_all, dim).to(torch.bfloat16)  # one rounding pass over the gradient rows
+        dh16 = dh.view(n_all, dim)
         parts = [dh16[off[t]:off[t + 1]] for t in range(4)]
         dws = graph_ext.gemm_bf16_tn_typed(xs16, parts)
         dxs = graph_ext.gemm_bf16_typed(parts, wts16, trans_b=True, out_dtype=torch.bfloat16)

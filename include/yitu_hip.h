@@ -148,6 +148,19 @@ int yitu_spmm_forward_bf16(float *out_device, const float *values_device,
                            void *stream);
 
 /*
+ * The same with bf16 rows out as well (fp32 sums, one rounding to nearest even per
+ * output): the gradient rows of a bf16 pipeline, which the next bf16 product reads
+ * without a conversion pass. n_features must be a multiple of 8 and both row buffers
+ * 16-byte aligned.
+ */
+int yitu_spmm_forward_bf16_rows(void *out_bf16_device, const float *values_device,
+                                const int32_t *indptr_device, const int32_t *indices_device,
+                                const void *features_bf16_device, int64_t n_dst, int64_t n_src,
+                                int64_t nnz, int64_t n_heads, int64_t n_features,
+                                int64_t max_degree, const void *plan_device,
+                                void *workspace_device, size_t workspace_bytes, void *stream);
+
+/*
  * spmm_backward (entry.cpp:92-104; spmm_cuda.cu:24-42,64-86):
  *   grad_a[i,h]   = sum_k grad_out[row_i,h,k] * features[col_i,h,k]
  *   grad_x[c,h,k] = sum_{i: col_i = c} grad_out[row_i,h,k] * values[i,h]

@@ -127,6 +127,41 @@ def test_spmm_backward_bf16_rows(dev, h, f):
         graph_ext.spmm_backward(*args, x.to(dev), gy16.to(dev))
 
 
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24), (1, 8)])
+def test_spmm_bf16_rows_in_and_out(dev, h, f):
+    """bf16 rows out: exactly the fp32-out result of the same call rounded once to nearest
+    even (short rows, single-item rows and reduced rows all take the same store), forward
+    and as the grad_x of the backward."""
+    indptr, indices = powerlaw_graph(12, 50000, 5 * h + f)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(3 * h + f)
+    values = torch.rand(indices.numel(), h, generator=g).to(dev)
+    x16 = torch.randn(n, h, f, generator=g).to(torch.bfloat16).to(dev)
+    args = (values, indptr.to(dev), indices.to(dev))
+    full = graph_ext.spmm_forward(*args, x16)
+    got = graph_ext.spmm_forward(*args, x16, out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got, full.to(torch.bfloat16))
+    gx32 = graph_ext.spmm_backward(*args, x16, x16, need_grad_a=False)[1]
+    gx16 = graph_ext.spmm_backward(*args, x16, x16, need_grad_a=False,
+                                   grad_x_dtype=torch.bfloat16)[1]
+    assert gx16.dtype == torch.bfloat16 and torch.equal(gx16, gx32.to(torch.bfloat16))
+    with pytest.raises(RuntimeError, match="out_dtype"):
+        graph_ext.spmm_forward(*args, x16.float(), out_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="grad_x_dtype"):
+        graph_ext.spmm_backward(*args, x16.float(), x16.float(), need_grad_a=False,
+                                grad_x_dtype=torch.bfloat16)
+
+
+def test_spmm_bf16_rows_out_rejects_odd_head_width(dev):
+    indptr, indices = powerlaw_graph(8, 2000, 1)
+    n = indptr.numel() - 1
+    x16 = torch.zeros(n, 3, 5, dtype=torch.bfloat16, device=dev)
+    values = torch.ones(indices.numel(), 3, device=dev)
+    with pytest.raises(RuntimeError, match="out_dtype"):
+        graph_ext.spmm_forward(values, indptr.to(dev), indices.to(dev), x16,
+                               out_dtype=torch.bfloat16)
+
+
 def test_spmm_more_than_65535_rows(dev):
     """The reference's dim3(n_heads, n_nodes) launch is invalid above 65,535 rows."""
     n_dst, n_src, h, f = 70000, 1000, 2, 8

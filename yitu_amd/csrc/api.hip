@@ -103,7 +103,7 @@ YITU_API int yitu_agg_csr_noalloc(float *out, const void *x, int x_is_bf16,
                         dim, alpha, max_degree, nullptr, nullptr, ws, kStaticScratchBytes, stream);
 }
 
-static int spmm_forward_any(float *out, const float *values, const int32_t *indptr,
+static int spmm_forward_any(void *out, bool bf16_out, const float *values, const int32_t *indptr,
                             const int32_t *indices, const void *features, bool bf16_in,
                             int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
                             int64_t n_features, int64_t max_degree, const void *plan,
@@ -115,11 +115,16 @@ static int spmm_forward_any(float *out, const float *values, const int32_t *indp
     YITU_REQUIRE(nnz == 0 || (values && indices && features), "null input with nnz > 0");
     YITU_REQUIRE(n_dst < INT32_MAX && n_src <= (1 << 24) && n_heads * n_features < (1 << 20),
                  "size out of range (columns are 24-bit)");
+    YITU_REQUIRE(!bf16_out || (bf16_in && n_features % 8 == 0 && aligned16(features) &&
+                               aligned16(out)),
+                 "bf16 output rows need bf16 feature rows, a head width that is a multiple of 8 "
+                 "and 16-byte aligned buffers");
     SpmmParams p{};
     p.indptr = indptr;
     p.indices = indices;
     p.feat = features;
-    p.out = out;
+    p.out = static_cast<float *>(out);
+    p.out_bf16 = bf16_out ? 1 : 0;
     p.values = values;
     p.n_rows = (int)n_dst;
     p.n_src = (int)n_src;
@@ -137,7 +142,7 @@ YITU_API int yitu_spmm_forward(float *out, const float *values, const int32_t *i
                                int64_t n_src, int64_t nnz, int64_t n_heads, int64_t n_features,
                                int64_t max_degree, const void *plan, void *workspace,
                                size_t workspace_bytes, void *stream) {
-    return spmm_forward_any(out, values, indptr, indices, features, false, n_dst, n_src, nnz,
+    return spmm_forward_any(out, false, values, indptr, indices, features, false, n_dst, n_src, nnz,
                             n_heads, n_features, max_degree, plan, workspace, workspace_bytes,
                             stream);
 }
@@ -147,9 +152,19 @@ YITU_API int yitu_spmm_forward_bf16(float *out, const float *values, const int32
                                     int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
                                     int64_t n_features, int64_t max_degree, const void *plan,
                                     void *workspace, size_t workspace_bytes, void *stream) {
-    return spmm_forward_any(out, values, indptr, indices, features_bf16, true, n_dst, n_src, nnz,
-                            n_heads, n_features, max_degree, plan, workspace, workspace_bytes,
+    return spmm_forward_any(out, false, values, indptr, indices, features_bf16, true, n_dst, n_src,
+                            nnz, n_heads, n_features, max_degree, plan, workspace, workspace_bytes,
                             stream);
+}
+
+YITU_API int yitu_spmm_forward_bf16_rows(void *out_bf16, const float *values, const int32_t *indptr,
+                                         const int32_t *indices, const void *features_bf16,
+                                         int64_t n_dst, int64_t n_src, int64_t nnz, int64_t n_heads,
+                                         int64_t n_features, int64_t max_degree, const void *plan,
+                                         void *workspace, size_t workspace_bytes, void *stream) {
+    return spmm_forward_any(out_bf16, true, values, indptr, indices, features_bf16, true, n_dst,
+                            n_src, nnz, n_heads, n_features, max_degree, plan, workspace,
+                            workspace_bytes, stream);
 }
 
 

@@ -32,7 +32,7 @@ struct SpmmParams {
     const int32_t *indptr;   // [n_rows + 1]
     const int32_t *indices;  // [nnz], column in the low bits selected by col_mask
     const void *feat;        // [n_src, L] fp32 or bf16
-    float *out;              // [n_rows, L]
+    float *out;              // [n_rows, L] fp32, or bf16 (see out_bf16)
     const float *scale_row;  // W_DEGPROD: s[n_rows]; otherwise unused
     const float *scale_col;  // W_DEGPROD: s[n_src]
     const float *edge_scale; // W_DEGPROD, optional: [nnz] = s[col of the edge], read in edge
@@ -47,9 +47,38 @@ struct SpmmParams {
     int col_mask;
     int cols_are_edges;  // nonzero: edge e reads feat row e (a segmented sum of per-edge rows)
     float alpha;   // output scale
+    int out_bf16;  // nonzero: the output rows are bf16 (round to nearest even); partial rows
+                   // stay fp32. Taken by the row / item / reduce kernels of this file.
     PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
     float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
 };
+
+// Stores VEC consecutive elements of an output row, `elem` elements into the output:
+// fp32 as they are, or rounded to bf16 when the caller asked for bf16 rows (a pipeline
+// whose next product reads bf16 then needs no conversion pass of its own).
+template <int VEC>
+__device__ __forceinline__ void store_out(const SpmmParams &p, size_t elem, const float (&v)[VEC]) {
+    if (!p.out_bf16) {  // same for the whole launch
+        store_row_streaming<VEC>(p.out + elem, v);
+        return;
+    }
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + elem;
+    if constexpr (VEC % 2 == 0) {
+        typedef unsigned int uv __attribute__((ext_vector_type(VEC / 2)));
+        uv w;
+#pragma unroll
+        for (int i = 0; i < VEC / 2; i++) {
+            const __bf16 lo = static_cast<__bf16>(v[2 * i]), hi = static_cast<__bf16>(v[2 * i + 1]);
+            w[i] = (unsigned)__builtin_bit_cast(uint16_t, lo) |
+                   ((unsigned)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        __builtin_nontemporal_store(w, reinterpret_cast<uv *>(dst));
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            dst[i] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v[i]));
+    }
+}
 
 // A window is up to 64 consecutive CSR edges held one per lane: column id,
 // per-edge scalar weight (W_NONE / W_DEGPROD) or the row of `values` to read
@@ -283,7 +312,7 @@ __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, i
                         float r[VEC];
 #pragma unroll
                         for (int k = 0; k < VEC; k++) r[k] = acc[t][k] * sr;
-                        store_row_streaming<VEC>(p.out + (size_t)row * p.L + o, r);
+                        store_out<VEC>(p, (size_t)row * p.L + o, r);
                     }
                 }
             }
@@ -333,7 +362,7 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
             fold_slots<VEC, G, KT>(acc);
             const bool single = row_tag[j] < 0;
             const int row = row_tag[j] & 0x7fffffff;
-            float *dst = single ? p.out + (size_t)row * p.L : p.partial + (size_t)item_id[j] * p.L;
+            float *dst = p.partial + (size_t)item_id[j] * p.L;  // not for single items
             const float sr =
                 single ? (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha : 1.0f;
             if (slot == 0) {
@@ -344,7 +373,8 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
                         float r[VEC];
 #pragma unroll
                         for (int i = 0; i < VEC; i++) r[i] = acc[t][i] * sr;
-                        store_row_streaming<VEC>(dst + o, r);
+                        if (single) store_out<VEC>(p, (size_t)row * p.L + o, r);
+                        else store_row_streaming<VEC>(dst + o, r);
                     }
                 }
             }
@@ -434,7 +464,7 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
                 if (live && slot == 0) {
 #pragma unroll
                     for (int i = 0; i < VEC; i++) s[i] *= sr;
-                    store_row_streaming<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + sub) * VEC, s);
+                    store_out<VEC>(p, (size_t)r.x * p.L + (size_t)(l0 + sub) * VEC, s);
                 }
             }
         }
@@ -465,7 +495,7 @@ __global__ __launch_bounds__(kBlock) void spmm_reduce_kernel(SpmmParams p) {
                     for (int i = 0; i < VEC; i++) s[i] += red[(gg * lanes + l) * VEC + i];
 #pragma unroll
                 for (int i = 0; i < VEC; i++) s[i] *= sr;
-                store_row_streaming<VEC>(p.out + (size_t)r.x * p.L + (size_t)(l0 + l) * VEC, s);
+                store_out<VEC>(p, (size_t)r.x * p.L + (size_t)(l0 + l) * VEC, s);
             }
         }
     }

@@ -103,9 +103,10 @@ def forget(*tensors):
 # --------------------------------------------------------------------------- #
 # SpMM
 # --------------------------------------------------------------------------- #
-def spmm_forward(values, indptr, indices, features):
+def spmm_forward(values, indptr, indices, features, out_dtype=torch.float32):
     """out[r,h,k] = sum_i values[i,h] * features[col_i,h,k] (entry.cpp:80-90).
-    ``features`` fp32 like the reference, or bf16 (fp32 accumulate, fp32 out)."""
+    ``features`` fp32 like the reference, or bf16 (fp32 accumulate; fp32 out, or bf16 rows
+    with ``out_dtype=torch.bfloat16``: one rounding per output)."""
     _check(values, torch.float32, "values", 2)
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
@@ -117,13 +118,20 @@ def spmm_forward(values, indptr, indices, features):
     nnz = indices.numel()
     if values.shape[0] != nnz or values.shape[1] != h:
         raise RuntimeError("values must be [n_edges, n_heads]")
-    out = torch.empty((n_dst, h, f), dtype=torch.float32, device=dev)
+    if out_dtype not in (torch.float32, torch.bfloat16) or (out_dtype == torch.bfloat16
+                                                            and not (bf16 and f % 8 == 0)):
+        raise RuntimeError("out_dtype is float32, or bfloat16 for bf16 features whose head "
+                           "width is a multiple of 8")
+    out = torch.empty((n_dst, h, f), dtype=out_dtype, device=dev)
     maxdeg = _lib.max_degree(indptr)
     plan = _lib.row_plan(indptr, indices, n_src, COL_MASK)
     need = _size_fn("yitu_spmm_workspace_bytes")(c_i64(nnz), c_i64(h * f), c_int(1)) \
         if plan is not None and maxdeg >= 64 else 0
     ws = _lib.workspace(need, dev)
-    entry = _lib.lib().yitu_spmm_forward_bf16 if bf16 else _lib.lib().yitu_spmm_forward
+    entry = _lib.lib().yitu_spmm_forward
+    if bf16:
+        entry = _lib.lib().yitu_spmm_forward_bf16_rows if out_dtype == torch.bfloat16 \
+            else _lib.lib().yitu_spmm_forward_bf16
     with torch.cuda.device(dev):
         rc = entry(ptr(out), ptr(values), ptr(indptr), ptr(indices), ptr(features), c_i64(n_dst),
                    c_i64(n_src), c_i64(nnz), c_i64(h), c_i64(f), c_i64(maxdeg), ptr(plan), ptr(ws),
@@ -168,9 +176,10 @@ def _forget_values(ident):
 
 
 def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
-                  need_grad_x=True):
+                  need_grad_x=True, grad_x_dtype=torch.float32):
     """Returns [grad_a [E,H], grad_x [Ns,H,F]] (entry.cpp:92-104). A gradient
-    that the caller does not need is skipped and returned as None."""
+    that the caller does not need is skipped and returned as None. ``grad_x_dtype``:
+    bfloat16 with bf16 ``grad_out`` rows writes grad_x as bf16 rows (fp32 sums)."""
     _check(values, torch.float32, "values", 2)
     _check(indptr, torch.int32, "indptr", 1)
     _check(indices, torch.int32, "indices", 1)
@@ -203,7 +212,10 @@ def spmm_backward(values, indptr, indices, features, grad_out, need_grad_a=True,
         # forward product over the by-source structure, weights copied into that order
         tr = transposed(indptr, indices, n_src)
         values_t = _by_source_values(values, indptr, indices, n_src, force=True)
-        return [None, spmm_forward(values_t, tr.t_indptr, tr.t_rows, grad_out)]
+        return [None, spmm_forward(values_t, tr.t_indptr, tr.t_rows, grad_out,
+                                   out_dtype=grad_x_dtype)]
+    if grad_x_dtype != torch.float32:
+        raise RuntimeError("grad_x_dtype other than float32 needs bf16 grad_out rows")
     if not need_grad_a and nnz > 0 and n_dst <= COL_MASK:
         values_t = _by_source_values(values, indptr, indices, n_src)
         if values_t is not None:
