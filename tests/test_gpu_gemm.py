@@ -50,6 +50,30 @@ def test_sgemm_typed_gemm_shape(dev):
     assert_close(graph_ext.sgemm(x.to(dev), w.to(dev)), _ref(x, w, False, False))
 
 
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("ms,n,k", [([4100], 256, 256), ([5000], 300, 64), ([70001], 256, 128),
+                                    ([4096], 250, 128), ([20000], 520, 256),
+                                    ([5000, 0, 4097, 300], 256, 256), ([700] * 10, 192, 128)])
+def test_sgemm_many_rows_short_inner_dimension(dev, tb, ms, n, k):
+    """Inner dimensions of 64 / 128 / 256 with thousands of rows run with the weight held
+    in registers and whole-row tiles: ragged last tiles, column counts that are not
+    multiples of 4 / 32 / 256, several column blocks, several node types in one launch
+    (an empty one among them, more than 8), both weight layouts."""
+    g = torch.Generator().manual_seed(sum(ms) + 3 * n + 5 * k + tb)
+    a = [torch.randn(m, k, generator=g) for m in ms]
+    b = [torch.randn((n, k) if tb else (k, n), generator=g) for _ in ms]
+    da, db = [x.to(dev) for x in a], [w.to(dev) for w in b]
+    got = graph_ext.sgemm_typed(da, db, False, tb) if len(ms) > 1 \
+        else [graph_ext.sgemm(da[0], db[0], False, tb)]
+    for x, w, c, m in zip(a, b, got, ms):
+        assert tuple(c.shape) == (m, n)
+        assert_close(c, _ref(x, w, False, tb), atol=1e-4 * max(1.0, np.sqrt(k) / 4),
+                     what="m=%d n=%d k=%d tb=%s" % (m, n, k, tb))
+    again = graph_ext.sgemm_typed(da, db, False, tb) if len(ms) > 1 \
+        else [graph_ext.sgemm(da[0], db[0], False, tb)]
+    assert all(torch.equal(c, d) for c, d in zip(got, again))
+
+
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
 @pytest.mark.parametrize("sizes", [[(300, 64), (1, 64), (0, 64), (129, 64)],
                                    [(1024, 256), (512, 256), (256, 256)],

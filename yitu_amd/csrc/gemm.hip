@@ -363,6 +363,209 @@ static int sgemm_launch(const GemmParams &p, int tile, int max_m, int n_z, hipSt
     return sgemm_launch_tile<1, A_KCONT, B_KCONT>(p, max_m, n_z, stream);
 }
 
+// ---- many rows, inner dimension 64 / 128 / 256: the weight stays in registers -------
+// C_q[M_q, N] = A_q[M_q, K] . B_q for up to 8 problems (node types). The 8 waves of a
+// workgroup hold all of B_q[0 .. K, n0 .. n0 + 256) as MFMA operands (wave w keeps 32
+// columns: K / 2 steps x 1 register), the workgroup walks 32-row tiles of A and reads each
+// as whole rows, two tiles ahead through a ring of registers into a double-buffered LDS
+// tile, one barrier per tile; no operand of the inner loop comes from memory. The MFMA
+// step s of lane (i, half) takes k = half * K / 2 + s, so a lane's A operands of four
+// consecutive steps are 16 contiguous bytes of its row (the weight registers are loaded in
+// the same order, once). LDS rows are padded by 16 bytes: 16 consecutive lanes read 16
+// different banks groups. The weight is the first MFMA operand, so a lane ends up with
+// four consecutive columns of one row; a wave passes its 32 x 32 outputs through an LDS
+// area of its own and stores whole 128-byte row segments.
+constexpr int SR_M = 32;      // rows of a tile
+constexpr int SR_C_LD = 144;  // staged output row: 128 bytes + 16 of padding
+constexpr int SR_PF = 2;      // tiles requested ahead
+
+struct SRowsParams {
+    const float *A[kMaxGroup];
+    const float *B[kMaxGroup];
+    float *C[kMaxGroup];
+    int M[kMaxGroup];
+    int tile_start[kMaxGroup + 1];
+    int n_problems, N;
+    int64_t lda, ldb, ldc;
+};
+
+template <int K>
+constexpr size_t sgemm_rows_lds_bytes() {
+    return (size_t)2 * SR_M * (K + 4) * sizeof(float) + (size_t)8 * SR_M * SR_C_LD;
+}
+
+template <int K, bool B_KCONT>
+__global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
+    constexpr int KS = K / 2;        // MFMA steps of 2
+    constexpr int A_LD = K + 4;      // padded LDS row, floats
+    constexpr int TPR = K / 4;       // threads that cover one row with 16 bytes each
+    constexpr int RPS = 512 / TPR;   // rows the workgroup covers at a time
+    constexpr int LR = SR_M / RPS;   // 16-byte pieces of the tile per thread
+    static_assert(LR >= 1, "a pass of the loader must not exceed the tile");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int wn = blockIdx.y * 256 + wave * 32;
+    float *As = reinterpret_cast<float *>(smem);  // [2][SR_M][A_LD]
+    unsigned char *stage = smem + (size_t)2 * SR_M * A_LD * sizeof(float) + wave * (SR_M * SR_C_LD);
+    const int stride = gridDim.x;
+    const bool whole_cols = blockIdx.y * 256 + 256 <= p.N;
+    const int lrow = t / TPR, lcol = (t % TPR) * 4;
+
+    for (int q = 0; q < p.n_problems; q++) {
+        const int lo = p.tile_start[q], hi = p.tile_start[q + 1];
+        // this workgroup's tiles of the problem: lo <= tile < hi, tile = blockIdx.x (mod stride)
+        const int tile0 = lo + (int)(((int64_t)blockIdx.x - lo % stride + stride) % stride);
+        if (tile0 >= hi) continue;  // same for the whole workgroup
+        const float *__restrict__ a_q = p.A[q];
+        const float *__restrict__ b_q = p.B[q];
+        float *__restrict__ c_q = p.C[q];
+        const int m_q = p.M[q];
+        float b[KS];
+        {
+            const int col = min(wn + l32, p.N - 1);  // columns past N: never stored
+            const float *bp = B_KCONT ? b_q + (int64_t)col * p.ldb + KS * lk
+                                      : b_q + (int64_t)(KS * lk) * p.ldb + col;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                b[s] = *bp;
+                bp += B_KCONT ? 1 : p.ldb;
+                // (addresses made as they are needed: all at once they crowd out the weight)
+                if (s % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        f4 ra[SR_PF][LR];
+        auto gload = [&](int slot, int64_t tile64) {
+            const int tile = (int)min(tile64, (int64_t)hi - 1);
+            const int r0 = (tile - lo) * SR_M + lrow;
+#pragma unroll
+            for (int i = 0; i < LR; i++) {
+                const int64_t row = min(r0 + RPS * i, m_q - 1);
+                ra[slot][i] = __builtin_nontemporal_load(
+                    reinterpret_cast<const f4 *>(a_q + row * p.lda + lcol));
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < SR_PF; u++) {
+            gload(u, tile0 + (int64_t)u * stride);
+            __builtin_amdgcn_sched_barrier(0);  // oldest first
+        }
+        for (int it0 = 0; tile0 + (int64_t)it0 * stride < hi; it0 += SR_PF) {
+#pragma unroll
+            for (int u = 0; u < SR_PF; u++) {
+                const int it = it0 + u;
+                const int64_t tile64 = tile0 + (int64_t)it * stride;
+                if (tile64 >= hi) break;  // same for the whole workgroup
+                const int tile = (int)tile64;
+                float *At = As + (size_t)(it & 1) * SR_M * A_LD;
+                // this buffer was last read two tiles ago, before the previous barrier
+#pragma unroll
+                for (int i = 0; i < LR; i++)
+                    *reinterpret_cast<f4 *>(At + (lrow + RPS * i) * A_LD + lcol) = ra[u][i];
+                __syncthreads();
+                gload(u, tile64 + (int64_t)SR_PF * stride);
+                float16v acc;
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+                const float *arow = At + l32 * A_LD + KS * lk;
+#pragma unroll
+                for (int s4 = 0; s4 < KS; s4 += 4) {
+                    const f4 a = *reinterpret_cast<const f4 *>(arow + s4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b[s4 + e], a[e], acc, 0, 0, 0);
+                    // operand reads stay a few steps ahead of their products: hoisted all the
+                    // way they would not fit beside the weight
+                    if (s4 % 16 == 12) __builtin_amdgcn_sched_barrier(0);
+                }
+                // accumulator element 4 jj + ii is C[32 tile + lane % 32][wn + 8 jj + 4 (lane / 32) + ii]
+                const int row0 = (tile - lo) * SR_M;
+                if (whole_cols && row0 + SR_M <= m_q) {  // same for the whole workgroup
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) {
+                        const f4 w = {acc[4 * jj], acc[4 * jj + 1], acc[4 * jj + 2], acc[4 * jj + 3]};
+                        *reinterpret_cast<f4 *>(stage + l32 * SR_C_LD + 32 * jj + 16 * lk) = w;
+                    }
+#pragma unroll
+                    for (int r = 0; r < SR_M / 8; r++) {
+                        const int row = 8 * r + (lane >> 3);
+                        const f4 w = *reinterpret_cast<const f4 *>(stage + row * SR_C_LD +
+                                                                   16 * (lane & 7));
+                        *reinterpret_cast<f4 *>(c_q + (int64_t)(row0 + row) * p.ldc + wn +
+                                                4 * (lane & 7)) = w;
+                    }
+                } else if (row0 + l32 < m_q) {
+                    const int64_t row = row0 + l32;
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int col = wn + 8 * (e / 4) + 4 * lk + e % 4;
+                        if (col < p.N) c_q[row * p.ldc + col] = acc[e];
+                    }
+                }
+            }
+        }
+        __syncthreads();  // the next problem starts over with the first LDS buffer
+    }
+}
+
+template <int K, bool B_KCONT>
+static int sgemm_rows_launch_k(const SRowsParams &r, hipStream_t stream) {
+    constexpr size_t lds = sgemm_rows_lds_bytes<K>();
+    static bool prepared = false;  // more LDS than the default limit: asked for once
+    if (!prepared) {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&sgemm_rows_kernel<K, B_KCONT>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            set_error("hipFuncSetAttribute(dynamic LDS %zu): %s", lds, hipGetErrorString(e));
+            return -1;
+        }
+        prepared = true;
+    }
+    const int n_tiles = r.tile_start[r.n_problems];
+    dim3 grid((unsigned)std::min(n_tiles, 256), (unsigned)ceil_div(r.N, 256));
+    sgemm_rows_kernel<K, B_KCONT><<<grid, 512, lds, stream>>>(r);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+// Takes the group when it is one of the kernel's shapes; *taken says whether it did.
+static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb,
+                          hipStream_t stream, bool *taken) {
+    *taken = false;
+    if (trans_a || p.accumulate || p.n_prob < 1 || p.ldc % 4 != 0 || lda % 4 != 0) return 0;
+    const int k = p.prob[0].K;
+    if (!(k == 64 || k == 128 || k == 256)) return 0;
+    int64_t total = 0;
+    SRowsParams r{};
+    for (int i = 0; i < p.n_prob; i++) {
+        const GemmProblem &pr = p.prob[i];
+        if (pr.K != k || !aligned16(pr.A) || !aligned16(pr.C) || pr.M < 0) return 0;
+        r.A[i] = pr.A;
+        r.B[i] = pr.B;
+        r.C[i] = pr.C;
+        r.M[i] = pr.M;
+        r.tile_start[i + 1] = r.tile_start[i] + (int)ceil_div(pr.M, SR_M);
+        total += pr.M;
+    }
+    if (total < 4096) return 0;
+    r.n_problems = p.n_prob;
+    r.N = p.N;
+    r.lda = lda;
+    r.ldb = ldb;
+    r.ldc = p.ldc;
+    *taken = true;
+    if (trans_b) {
+        if (k == 256) return sgemm_rows_launch_k<256, true>(r, stream);
+        if (k == 128) return sgemm_rows_launch_k<128, true>(r, stream);
+        return sgemm_rows_launch_k<64, true>(r, stream);
+    }
+    if (k == 256) return sgemm_rows_launch_k<256, false>(r, stream);
+    if (k == 128) return sgemm_rows_launch_k<128, false>(r, stream);
+    return sgemm_rows_launch_k<64, false>(r, stream);
+}
+
 // trans_a: A is given as [K, M] row-major (else [M, K]); trans_b: B is given as
 // [N, K] row-major (else [K, N]).
 int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, void *workspace,
@@ -388,6 +591,11 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
         }
     }
     p.n_prob = kept;
+    {
+        bool taken = false;
+        const int rc = sgemm_rows_try(p, trans_a, trans_b, lda, ldb, stream, &taken);
+        if (taken) return rc;
+    }
     int max_m = 0;
     for (int i = 0; i < p.n_prob; i++) max_m = std::max(max_m, p.prob[i].M);
     if (max_m == 0 || p.N == 0) return 0;
