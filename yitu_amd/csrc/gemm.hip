@@ -432,7 +432,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
                 b[s] = *bp;
                 bp += B_KCONT ? 1 : p.ldb;
                 // (addresses made as they are needed: all at once they crowd out the weight)
-                if (s % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+                if (s % 32 == 31) __builtin_amdgcn_sched_barrier(0);
             }
         }
         f4 ra[SR_PF][LR];
@@ -530,9 +530,39 @@ static int sgemm_rows_launch_k(const SRowsParams &r, hipStream_t stream) {
     return 0;
 }
 
+// dst_q[n][k] = src_q[k][n] for the weights of a group (blockIdx.z = problem): a weight
+// stored [K, N] is read by the kernel above with one 4-byte load per element and lane,
+// and a load of 4 bytes takes the address path as long as one of 16; from the [N, K]
+// copy the same registers are filled with a quarter of the loads.
+struct TransposeParams {
+    float *dst[kMaxGroup];
+    const float *src[kMaxGroup];
+};
+
+__global__ __launch_bounds__(256) void transpose32_kernel(TransposeParams tp, int K, int N,
+                                                          int64_t ld_src) {
+    __shared__ float tile[32][33];
+    float *__restrict__ dst = tp.dst[blockIdx.z];
+    const float *__restrict__ src = tp.src[blockIdx.z];
+    const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8)
+        tile[r][tx] = (k0 + r < K && n0 + tx < N) ? src[(int64_t)(k0 + r) * ld_src + n0 + tx] : 0.0f;
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8)
+        if (n0 + r < N && k0 + tx < K) dst[(int64_t)(n0 + r) * K + k0 + tx] = tile[tx][r];
+}
+
+static size_t sgemm_rows_workspace_bytes(int64_t n, int64_t k, int64_t n_problems) {
+    if (!(k == 64 || k == 128 || k == 256)) return 0;
+    return (size_t)std::min<int64_t>(std::max<int64_t>(n_problems, 1), kMaxGroup) *
+           align_up((size_t)(n * k) * sizeof(float), 256);
+}
+
 // Takes the group when it is one of the kernel's shapes; *taken says whether it did.
 static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb,
-                          hipStream_t stream, bool *taken) {
+                          void *workspace, size_t workspace_bytes, hipStream_t stream,
+                          bool *taken) {
     *taken = false;
     if (trans_a || p.accumulate || p.n_prob < 1 || p.ldc % 4 != 0 || lda % 4 != 0) return 0;
     const int k = p.prob[0].K;
@@ -556,6 +586,22 @@ static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int l
     r.ldb = ldb;
     r.ldc = p.ldc;
     *taken = true;
+    if (!trans_b && workspace && aligned16(workspace) &&
+        workspace_bytes >= sgemm_rows_workspace_bytes(p.N, k, p.n_prob)) {
+        // (weights are small: the copies cost a few microseconds for the whole group)
+        TransposeParams tp{};
+        const size_t slot = align_up((size_t)p.N * k * sizeof(float), 256);
+        for (int i = 0; i < p.n_prob; i++) {
+            tp.src[i] = r.B[i];
+            tp.dst[i] = reinterpret_cast<float *>(static_cast<char *>(workspace) + i * slot);
+            r.B[i] = tp.dst[i];
+        }
+        dim3 tg((unsigned)ceil_div(p.N, 32), (unsigned)ceil_div(k, 32), (unsigned)p.n_prob);
+        transpose32_kernel<<<tg, 256, 0, stream>>>(tp, k, p.N, ldb);
+        YITU_LAUNCH_CHECK();
+        r.ldb = k;
+        trans_b = true;
+    }
     if (trans_b) {
         if (k == 256) return sgemm_rows_launch_k<256, true>(r, stream);
         if (k == 128) return sgemm_rows_launch_k<128, true>(r, stream);
@@ -593,7 +639,8 @@ int sgemm_grouped(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb, v
     p.n_prob = kept;
     {
         bool taken = false;
-        const int rc = sgemm_rows_try(p, trans_a, trans_b, lda, ldb, stream, &taken);
+        const int rc = sgemm_rows_try(p, trans_a, trans_b, lda, ldb, workspace, workspace_bytes,
+                                      stream, &taken);
         if (taken) return rc;
     }
     int max_m = 0;
@@ -638,9 +685,11 @@ using namespace yitu;
 YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems) {
     const int tile = pick_tile(n, nullptr, (int)std::min<int64_t>(n_problems, kMaxGroup), m, k);
     const int64_t tiles = ceil_div(n, tile) * ceil_div(m, tile) * n_problems;
-    if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return 256;
+    // (or room for the [N, K] copies of the weights that the many-rows kernel reads)
+    const size_t rows_ws = std::max<size_t>(sgemm_rows_workspace_bytes(n, k, n_problems), 256);
+    if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return rows_ws;
     const int64_t splits = std::min<int64_t>(ceil_div(k, kMinSplitK), ceil_div(1024, tiles));
-    return align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256);
+    return std::max(rows_ws, align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256));
 }
 
 YITU_API int yitu_sgemm(float *c, const float *a, const float *b, int64_t m, int64_t n, int64_t k,
