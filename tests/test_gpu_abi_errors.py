@@ -74,3 +74,47 @@ def test_bad_arguments_are_reported_not_launched(dev):
     rc = L.yitu_column_sum(P(colsum), P(c), I64(16), I64(24), none, SZ(0), st)
     _fails(rc, "workspace too small")
     assert torch.equal(graph_ext.column_sum(c), graph_ext.column_sum(c))
+
+
+def test_typed_bf16_products_report_bad_arguments(dev):
+    """The typed bf16 entry points take host arrays of device pointers: null lists, null
+    operands of a problem that has rows, unaligned widths and a short workspace are all
+    reported; an empty list and a problem without rows are not errors."""
+    L = _lib.lib()
+    st = _lib.stream_ptr(dev)
+    none = P(None)
+    a = torch.randn(64, 64, device=dev).to(torch.bfloat16)
+    w = torch.randn(32, 64, device=dev).to(torch.bfloat16)
+    c = torch.empty(64, 32, device=dev)
+    ws = _lib.workspace(1 << 20, dev)
+    ptrs = lambda *ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() if t is not None else None
+                                                      for t in ts])
+    rows = lambda *v: (ctypes.c_int64 * len(v))(*v)
+
+    def typed(cs=ptrs(c), as_=ptrs(a), bs=ptrs(w), m=rows(64), count=1, k=64, lda=64):
+        return L.yitu_gemm_bf16_typed(cs, I32(0), as_, bs, m, I64(count), I64(32), I64(k), I32(1),
+                                      I64(lda), I64(64), I64(32), P(ws), SZ(ws.numel()), st)
+
+    assert typed() == 0
+    assert typed(count=0) == 0
+    _fails(typed(cs=None), "null pointer list")
+    _fails(typed(as_=ptrs(None)), "null operand")
+    _fails(typed(k=60, lda=60), "multiples of 8")
+    _fails(typed(m=rows(-1)), "row count out of range")
+    assert typed(as_=ptrs(None), m=rows(0)) == 0  # nothing to read for a type without rows
+
+    g = torch.randn(64, 32, device=dev).to(torch.bfloat16)
+    dw = torch.empty(64, 32, device=dev)
+
+    def tn(cs=ptrs(dw), as_=ptrs(a), bs=ptrs(g), m=rows(64), ki=64, ws_bytes=ws.numel()):
+        return L.yitu_gemm_bf16_tn_typed(cs, as_, bs, m, I64(1), I64(ki), I64(32), I64(64), I64(32),
+                                         I64(32), I32(0), P(ws), SZ(ws_bytes), st)
+
+    assert tn() == 0
+    _fails(tn(ws_bytes=16), "workspace too small")
+    _fails(tn(cs=ptrs(None)), "null operand")
+    _fails(tn(ki=60), "multiples of 8")
+    assert tn() == 0  # and a good call still works
+    torch.cuda.synchronize()
+    want = a.float().t() @ g.float()
+    assert torch.allclose(dw, want, rtol=1e-4, atol=1e-3)
