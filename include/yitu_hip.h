@@ -349,8 +349,9 @@ int yitu_column_sum(float *out_device, const float *x_device, int64_t n_rows, in
  * G.W^T and X^T.G (cu:471-472,715-716). Products with few output tiles and a long
  * inner dimension (X^T.G) are split along k over the chip; the slabs go to the
  * workspace (yitu_sgemm_workspace_bytes; NULL = no split) and are summed in a
- * fixed order. With k = 64, 128 or 256, at least 4,096 rows and no transposed A, the
- * product runs with the weight held in registers; a weight stored [k,n] is first
+ * fixed order. With k = 64, 128 or 256, at least 49,152 rows, at least 192 columns in
+ * the last block of 256 and no transposed A, the product runs with the weight held in
+ * registers; a weight stored [k,n] is first
  * copied as [n,k] into the workspace when that is large enough.
  */
 size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems);

@@ -51,14 +51,15 @@ def test_sgemm_typed_gemm_shape(dev):
 
 
 @pytest.mark.parametrize("tb", [False, True])
-@pytest.mark.parametrize("ms,n,k", [([4100], 256, 256), ([5000], 300, 64), ([70001], 256, 128),
-                                    ([4096], 250, 128), ([20000], 520, 256),
-                                    ([5000, 0, 4097, 300], 256, 256), ([700] * 10, 192, 128)])
+@pytest.mark.parametrize("ms,n,k", [([50000], 256, 256), ([60000], 448, 64), ([70001], 256, 128),
+                                    ([49157], 250, 128), ([20000], 520, 256), ([5000], 300, 64),
+                                    ([30000, 0, 20001, 300], 256, 256), ([7000] * 10, 192, 128)])
 def test_sgemm_many_rows_short_inner_dimension(dev, tb, ms, n, k):
-    """Inner dimensions of 64 / 128 / 256 with thousands of rows run with the weight held
-    in registers and whole-row tiles: ragged last tiles, column counts that are not
+    """Inner dimensions of 64 / 128 / 256 with tens of thousands of rows run with the weight
+    held in registers and whole-row tiles: ragged last tiles, column counts that are not
     multiples of 4 / 32 / 256, several column blocks, several node types in one launch
-    (an empty one among them, more than 8), both weight layouts."""
+    (an empty one among them, more than 8), both weight layouts; two shapes just outside
+    (few rows, a narrow last column block) take the tiled kernel."""
     g = torch.Generator().manual_seed(sum(ms) + 3 * n + 5 * k + tb)
     a = [torch.randn(m, k, generator=g) for m in ms]
     b = [torch.randn((n, k) if tb else (k, n), generator=g) for _ in ms]

@@ -309,6 +309,7 @@ static int pick_tile(int64_t n, const int64_t *m, int n_prob, int64_t same_m, in
     int64_t tiles = 0;
     for (int i = 0; i < n_prob; i++) tiles += ceil_div(n, 128) * ceil_div(m ? m[i] : same_m, 128);
     if (tiles <= 0) return 64;
+    if (n <= 64) return 64;  // half of every 128-column tile would be empty
     int64_t splits = 1;
     if (k_max >= 2 * kMinSplitK)
         splits = std::max<int64_t>(1, std::min<int64_t>(ceil_div(k_max, kMinSplitK),
@@ -579,7 +580,12 @@ static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int l
         r.tile_start[i + 1] = r.tile_start[i] + (int)ceil_div(pr.M, SR_M);
         total += pr.M;
     }
-    if (total < 4096) return 0;
+    // Eight waves side by side cover 256 columns: with fewer than 192 in the last block most
+    // of them would idle (N = 64: 279 us against 154 us for the tiled kernel at 2^18 rows),
+    // and a workgroup has to walk a few dozen tiles to pay for loading the weight
+    // (2^15 rows: 46 against 44 us).
+    const int last = p.N % 256;
+    if (total < 49152 || (last != 0 && last < 192)) return 0;
     r.n_problems = p.n_prob;
     r.N = p.N;
     r.lda = lda;
