@@ -410,14 +410,20 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
     const int wn = blockIdx.y * 256 + wave * 32;
     float *As = reinterpret_cast<float *>(smem);  // [2][SR_M][A_LD]
     unsigned char *stage = smem + (size_t)2 * SR_M * A_LD * sizeof(float) + wave * (SR_M * SR_C_LD);
-    const int stride = gridDim.x;
+    // A workgroup takes a run of consecutive tiles of the list of all problems: it then
+    // crosses from one problem into the next once at most (and loads a weight once or
+    // twice), where every gridDim.x-th tile took it through all of them.
+    constexpr int stride = 1;
+    const int n_all = p.tile_start[p.n_problems];
+    const int per_wg = (n_all + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int my_lo = blockIdx.x * per_wg, my_hi = min(my_lo + per_wg, n_all);
     const bool whole_cols = blockIdx.y * 256 + 256 <= p.N;
     const int lrow = t / TPR, lcol = (t % TPR) * 4;
 
     for (int q = 0; q < p.n_problems; q++) {
-        const int lo = p.tile_start[q], hi = p.tile_start[q + 1];
-        // this workgroup's tiles of the problem: lo <= tile < hi, tile = blockIdx.x (mod stride)
-        const int tile0 = lo + (int)(((int64_t)blockIdx.x - lo % stride + stride) % stride);
+        const int lo = p.tile_start[q];
+        // this workgroup's tiles of the problem
+        const int tile0 = max(lo, my_lo), hi = min(p.tile_start[q + 1], my_hi);
         if (tile0 >= hi) continue;  // same for the whole workgroup
         const float *__restrict__ a_q = p.A[q];
         const float *__restrict__ b_q = p.B[q];

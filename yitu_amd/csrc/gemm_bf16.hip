@@ -205,7 +205,13 @@ __global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
     const int l32 = lane & 31, lk = lane >> 5;
     const int wn = blockIdx.y * HN + wave * 64;
     unsigned char *stage = Cs[wave];
-    const int stride = gridDim.x;
+    // A workgroup takes a run of consecutive tiles of the list of all problems: it then
+    // crosses from one problem into the next once at most (and loads a weight once or
+    // twice), where every gridDim.x-th tile took it through all of them.
+    constexpr int stride = 1;
+    const int n_all = p.tile_start[p.n_problems];
+    const int per_wg = (n_all + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int my_lo = blockIdx.x * per_wg, my_hi = min(my_lo + per_wg, n_all);
     const bool whole_cols = blockIdx.y * HN + HN <= p.N;
     // loader: TPR threads cover one row, the workgroup RPS rows at a time. Rows past the
     // end are read from the last row (their outputs are never stored) and tiles past the
@@ -213,9 +219,9 @@ __global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
     const int lrow = t / TPR, lk_ld = (t % TPR) * 8;
 
     for (int q = 0; q < p.n_problems; q++) {
-    const int lo = p.tile_start[q], hi = p.tile_start[q + 1];
-    // this workgroup's tiles of the problem: lo <= tile < hi, tile = blockIdx.x (mod stride)
-    const int tile0 = lo + (int)(((int64_t)blockIdx.x - lo % stride + stride) % stride);
+    const int lo = p.tile_start[q];
+    // this workgroup's tiles of the problem
+    const int tile0 = max(lo, my_lo), hi = min(p.tile_start[q + 1], my_hi);
     if (tile0 >= hi) continue;  // same for the whole workgroup
     const uint16_t *a_q = p.A[q], *bt = p.Bt[q];
     void *c_q = p.C[q];
