@@ -42,6 +42,24 @@ def test_sgemm_split_k_long_inner_dimension(dev):
     assert torch.equal(got, again)
 
 
+@pytest.mark.parametrize("ks", [[70001], [49152], [30000, 10, 20001, 300], [7000] * 10])
+def test_sgemm_weight_gradient_many_rows(dev, ks):
+    """dW = X^T G for [rows, 256] operands and tens of thousands of rows: every chunk of
+    rows keeps the whole 256 x 256 product in registers; several node types in one launch
+    (one with fewer rows than a stage, more than 8), a fixed order of additions, and the
+    accumulating form."""
+    g = torch.Generator().manual_seed(sum(ks))
+    xs = [torch.randn(k, 256, generator=g) for k in ks]
+    gs = [torch.randn(k, 256, generator=g) for k in ks]
+    dx, dg = [x.to(dev) for x in xs], [x.to(dev) for x in gs]
+    run = lambda: graph_ext.sgemm_typed(dx, dg, True, False) if len(ks) > 1 \
+        else [graph_ext.sgemm(dx[0], dg[0], True, False)]
+    got = run()
+    for x, y, c, k in zip(xs, gs, got, ks):
+        assert_close(c, _ref(x, y, True, False), atol=1e-4 * np.sqrt(k), what="k=%d" % k)
+    assert all(torch.equal(c, d) for c, d in zip(got, run()))
+
+
 def test_sgemm_typed_gemm_shape(dev):
     """[n_t, 256] x [256, 256] of the heterogeneous configuration (fast path)."""
     g = torch.Generator().manual_seed(1)
