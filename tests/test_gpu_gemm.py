@@ -42,15 +42,17 @@ def test_sgemm_split_k_long_inner_dimension(dev):
     assert torch.equal(got, again)
 
 
+@pytest.mark.parametrize("ki,no", [(256, 256), (64, 256), (256, 64), (128, 256), (256, 128),
+                                   (128, 128), (128, 64), (64, 128), (64, 64)])
 @pytest.mark.parametrize("ks", [[70001], [49152], [30000, 10, 20001, 300], [7000] * 10])
-def test_sgemm_weight_gradient_many_rows(dev, ks):
-    """dW = X^T G for [rows, 256] operands and tens of thousands of rows: every chunk of
-    rows keeps the whole 256 x 256 product in registers; several node types in one launch
+def test_sgemm_weight_gradient_many_rows(dev, ks, ki, no):
+    """dW = X^T G for operands of 64 / 128 / 256 columns and tens of thousands of rows: every
+    chunk of rows keeps the whole product in registers (64 x 64 takes the tiled kernel); several node types in one launch
     (one with fewer rows than a stage, more than 8), a fixed order of additions, and the
     accumulating form."""
     g = torch.Generator().manual_seed(sum(ks))
-    xs = [torch.randn(k, 256, generator=g) for k in ks]
-    gs = [torch.randn(k, 256, generator=g) for k in ks]
+    xs = [torch.randn(k, ki, generator=g) for k in ks]
+    gs = [torch.randn(k, no, generator=g) for k in ks]
     dx, dg = [x.to(dev) for x in xs], [x.to(dev) for x in gs]
     run = lambda: graph_ext.sgemm_typed(dx, dg, True, False) if len(ks) > 1 \
         else [graph_ext.sgemm(dx[0], dg[0], True, False)]

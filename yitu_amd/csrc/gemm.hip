@@ -628,55 +628,72 @@ static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int l
     return sgemm_rows_launch_k<64, false>(r, stream);
 }
 
-// ---- weight gradients C_q[256, 256] = A_q^T . B_q over many rows: the output stays in
-// registers. A workgroup of 8 waves owns a chunk of the rows of one problem and the whole
-// 256 x 256 product of that chunk (wave (wi, wj) the block of rows 64 wi, columns 128 wj:
-// 2 x 4 MFMA tiles, 128 accumulator registers), so every row of A and B is read once,
-// whole, two 16-row stages ahead through a ring of registers into a double-buffered LDS
-// stage, one barrier per stage. Both MFMA operands are columns of the row-major stage
-// (lane = column, the two halves of the wave take the two rows of the step), with stage
-// rows padded by 128 bytes so that the halves fall into different banks. The chunk
-// products go to the slabs of `partial` and are added by sgemm_splitk_reduce_kernel.
-constexpr int TR_STAGE = 16;        // rows per stage
-constexpr int TR_LD = 256 + 32;     // padded stage row, floats
-constexpr size_t kTnRowsLds = (size_t)2 * 2 * TR_STAGE * TR_LD * sizeof(float);
+// ---- weight gradients C_q[KI, NO] = A_q^T . B_q over many rows (KI, NO = 64, 128 or 256):
+// the output stays in registers. A workgroup of 8 waves owns a chunk of the rows of one
+// problem and the whole KI x NO product of that chunk (256 x 256: wave (wi, wj) the block
+// of rows 64 wi, columns 128 wj, 2 x 4 MFMA tiles, 128 accumulator registers), so every
+// row of A and B is read once, whole, two 16-row stages ahead through a ring of registers
+// into a double-buffered LDS stage, one barrier per stage. Both MFMA operands are columns
+// of the row-major stage (lane = column, the two halves of the wave take the two rows of
+// the step), with stage rows padded by 128 bytes so that the halves fall into different
+// banks. The chunk products go to the slabs of `partial` and are added by
+// sgemm_splitk_reduce_kernel in a fixed order.
+constexpr int TR_STAGE = 16;  // rows per stage
 
+// KI x NO = (32 TX WI) x (32 TY WJ): WI x WJ = 8 waves, each TX x TY MFMA tiles.
+template <int WI, int WJ, int TX, int TY>
+struct TnRowsGeom {
+    static_assert(WI * WJ == 8 && TX * TY <= 8, "8 waves, at most 128 accumulator registers");
+    static constexpr int KI = 32 * TX * WI, NO = 32 * TY * WJ;
+    static constexpr int LDA = KI + 32, LDB = NO + 32;  // padded stage rows, floats
+    static constexpr size_t kLds = (size_t)2 * TR_STAGE * (LDA + LDB) * sizeof(float);
+};
+
+template <int WI, int WJ, int TX, int TY>
 __global__ __launch_bounds__(512, 1) void sgemm_tn_rows_kernel(GemmParams p) {
+    using G = TnRowsGeom<WI, WJ, TX, TY>;
+    constexpr int KI = G::KI, NO = G::NO, LDA = G::LDA, LDB = G::LDB;
+    constexpr int PA = (TR_STAGE * KI / 4 + 511) / 512, PB = (TR_STAGE * NO / 4 + 511) / 512;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef float f4 __attribute__((ext_vector_type(4)));
-    float *stage_mem = reinterpret_cast<float *>(smem);  // [2 buffers][A, B][TR_STAGE][TR_LD]
+    float *stage_mem = reinterpret_cast<float *>(smem);  // [2 buffers][A stage, B stage]
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, lk = lane >> 5;
-    const int i0 = (wave >> 1) * 64, j0 = (wave & 1) * 128;
+    const int i0 = (wave / WJ) * 32 * TX, j0 = (wave % WJ) * 32 * TY;
     const GemmProblem pr = p.prob[problem_of(p, blockIdx.x)];
     const int split = blockIdx.x - pr.z0;
     const int m_beg = split * pr.k_chunk, m_end = min(pr.K, m_beg + pr.k_chunk);
     const int n_stages = (m_end - m_beg + TR_STAGE - 1) / TR_STAGE;
-    // loader: 64 threads cover one row of 256 floats, the workgroup 8 rows at a time
-    const int lrow = t >> 6, lcol = (t & 63) * 4;
 
-    float16v acc[2][4];
+    float16v acc[TX][TY];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < TX; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < TY; b++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[a][b][e] = 0.0f;
 
-    f4 ra[2][2], rb[2][2];
+    // loader: thread t takes the 16-byte pieces t, t + 512, ... of a stage of A and of B
+    f4 ra[2][PA], rb[2][PB];
     auto gload = [&](int slot, int st) {
+        const int r0 = m_beg + st * TR_STAGE;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int row = m_beg + st * TR_STAGE + lrow + 8 * h;
-            f4 va = {0.0f, 0.0f, 0.0f, 0.0f}, vb = va;
-            if (row < m_end) {  // rows past the chunk add nothing
-                va = __builtin_nontemporal_load(
-                    reinterpret_cast<const f4 *>(pr.A + (int64_t)row * p.a_sk + lcol));
-                vb = __builtin_nontemporal_load(
-                    reinterpret_cast<const f4 *>(pr.B + (int64_t)row * p.b_sk + lcol));
-            }
-            ra[slot][h] = va;
-            rb[slot][h] = vb;
+        for (int h = 0; h < PA; h++) {
+            const int piece = t + 512 * h, row = r0 + piece / (KI / 4);
+            f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (piece < TR_STAGE * KI / 4 && row < m_end)  // rows past the chunk add nothing
+                v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(
+                    pr.A + (int64_t)row * p.a_sk + (piece % (KI / 4)) * 4));
+            ra[slot][h] = v;
+        }
+#pragma unroll
+        for (int h = 0; h < PB; h++) {
+            const int piece = t + 512 * h, row = r0 + piece / (NO / 4);
+            f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (piece < TR_STAGE * NO / 4 && row < m_end)
+                v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(
+                    pr.B + (int64_t)row * p.b_sk + (piece % (NO / 4)) * 4));
+            rb[slot][h] = v;
         }
     };
     gload(0, 0);
@@ -687,27 +704,36 @@ __global__ __launch_bounds__(512, 1) void sgemm_tn_rows_kernel(GemmParams p) {
         for (int u = 0; u < 2; u++) {
             const int st = s0 + u;
             if (st >= n_stages) break;  // same for the whole workgroup
-            float *As = stage_mem + (size_t)(st & 1) * 2 * TR_STAGE * TR_LD;
-            float *Bs = As + TR_STAGE * TR_LD;
+            float *As = stage_mem + (size_t)(st & 1) * TR_STAGE * (LDA + LDB);
+            float *Bs = As + TR_STAGE * LDA;
             // this buffer was last read two stages ago, before the previous barrier
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                *reinterpret_cast<f4 *>(As + (lrow + 8 * h) * TR_LD + lcol) = ra[u][h];
-                *reinterpret_cast<f4 *>(Bs + (lrow + 8 * h) * TR_LD + lcol) = rb[u][h];
+            for (int h = 0; h < PA; h++) {
+                const int piece = t + 512 * h;
+                if (piece < TR_STAGE * KI / 4)
+                    *reinterpret_cast<f4 *>(As + (piece / (KI / 4)) * LDA + (piece % (KI / 4)) * 4) =
+                        ra[u][h];
+            }
+#pragma unroll
+            for (int h = 0; h < PB; h++) {
+                const int piece = t + 512 * h;
+                if (piece < TR_STAGE * NO / 4)
+                    *reinterpret_cast<f4 *>(Bs + (piece / (NO / 4)) * LDB + (piece % (NO / 4)) * 4) =
+                        rb[u][h];
             }
             __syncthreads();
             gload(u, st + 2);
 #pragma unroll
             for (int k2 = 0; k2 < TR_STAGE; k2 += 2) {
-                float a[2], b[4];
+                float a[TX], b[TY];
 #pragma unroll
-                for (int x = 0; x < 2; x++) a[x] = As[(k2 + lk) * TR_LD + i0 + 32 * x + l32];
+                for (int x = 0; x < TX; x++) a[x] = As[(k2 + lk) * LDA + i0 + 32 * x + l32];
 #pragma unroll
-                for (int y = 0; y < 4; y++) b[y] = Bs[(k2 + lk) * TR_LD + j0 + 32 * y + l32];
+                for (int y = 0; y < TY; y++) b[y] = Bs[(k2 + lk) * LDB + j0 + 32 * y + l32];
 #pragma unroll
-                for (int x = 0; x < 2; x++)
+                for (int x = 0; x < TX; x++)
 #pragma unroll
-                    for (int y = 0; y < 4; y++)
+                    for (int y = 0; y < TY; y++)
                         acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x], b[y], acc[x][y], 0, 0, 0);
             }
         }
@@ -716,9 +742,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_tn_rows_kernel(GemmParams p) {
     // column j0 + 32 y + lane % 32 of this chunk's slab
     float *dst = p.partial + (size_t)blockIdx.x * p.max_m * p.N;
 #pragma unroll
-    for (int x = 0; x < 2; x++)
+    for (int x = 0; x < TX; x++)
 #pragma unroll
-        for (int y = 0; y < 4; y++)
+        for (int y = 0; y < TY; y++)
 #pragma unroll
             for (int jj = 0; jj < 4; jj++)
 #pragma unroll
@@ -729,57 +755,91 @@ __global__ __launch_bounds__(512, 1) void sgemm_tn_rows_kernel(GemmParams p) {
                 }
 }
 
-// Takes a group of weight-gradient products when every one is [rows, 256]^T . [rows, 256]
-// with many rows in all; *taken says whether it did.
+template <int WI, int WJ, int TX, int TY>
+static int sgemm_tn_rows_launch(const GemmParams &p, int z, hipStream_t stream) {
+    constexpr size_t lds = TnRowsGeom<WI, WJ, TX, TY>::kLds;
+    static bool prepared_on[64] = {};  // more LDS than the default limit: once per device
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) device = 0;
+    if (lds > 65536 && !prepared_on[device]) {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&sgemm_tn_rows_kernel<WI, WJ, TX, TY>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            set_error("hipFuncSetAttribute(dynamic LDS %zu): %s", lds, hipGetErrorString(e));
+            return -1;
+        }
+        prepared_on[device] = true;
+    }
+    sgemm_tn_rows_kernel<WI, WJ, TX, TY><<<z, 512, lds, stream>>>(p);
+    YITU_LAUNCH_CHECK();
+    return 0;
+}
+
+// widths the kernel is built for: 64, 128 or 256 on either side, at least 8 MFMA tiles
+static bool tn_rows_shape(int64_t ki, int64_t no) {
+    const bool ok_i = ki == 64 || ki == 128 || ki == 256, ok_j = no == 64 || no == 128 || no == 256;
+    return ok_i && ok_j && ki * no >= 64 * 128;
+}
+
+// chunks of all problems together: a workgroup per CU when the products keep the matrix
+// pipes busy (256 x 256), two when the rows are narrow and the kernel waits for memory
+static int tn_rows_chunks(int64_t ki, int64_t no) { return ki * no >= 256 * 256 ? 256 : 512; }
+
+// Takes a group of weight-gradient products [rows, KI]^T . [rows, NO] with many rows in
+// all; *taken says whether it did.
 static int sgemm_tn_rows_try(GemmParams &p, bool trans_a, bool trans_b, int lda, int ldb,
                              void *workspace, size_t workspace_bytes, hipStream_t stream,
                              bool *taken) {
     *taken = false;
-    if (!trans_a || trans_b || p.N != 256 || lda % 4 != 0 || ldb % 4 != 0 || !workspace) return 0;
+    if (!trans_a || trans_b || p.n_prob < 1 || lda % 4 != 0 || ldb % 4 != 0 || !workspace) return 0;
+    const int ki = p.prob[0].M, no = p.N;
+    if (!tn_rows_shape(ki, no)) return 0;
     int64_t total = 0;
     for (int i = 0; i < p.n_prob; i++) {
         const GemmProblem &pr = p.prob[i];
-        if (pr.M != 256 || !aligned16(pr.A) || !aligned16(pr.B)) return 0;
+        if (pr.M != ki || !aligned16(pr.A) || !aligned16(pr.B)) return 0;
         total += pr.K;
     }
     if (total < 49152) return 0;
-    // one workgroup per CU holds the chip: about 256 chunks over all problems, every
-    // problem at least two (its slabs are then always summed by the reduce kernel)
-    const size_t slab = (size_t)256 * 256 * sizeof(float);
+    // every problem gets at least two chunks (its slabs are then always summed by the
+    // reduce kernel)
+    const size_t slab = (size_t)ki * no * sizeof(float);
+    const int64_t chunks = tn_rows_chunks(ki, no);
     int z = 0;
+    GemmProblem saved[kMaxGroup];
+    for (int i = 0; i < p.n_prob; i++) saved[i] = p.prob[i];
     for (int i = 0; i < p.n_prob; i++) {
         GemmProblem &pr = p.prob[i];
-        int64_t want = std::max<int64_t>(2, (256 * (int64_t)pr.K + total / 2) / total);
+        int64_t want = std::max<int64_t>(2, (chunks * (int64_t)pr.K + total / 2) / total);
         want = std::min<int64_t>(want, std::max<int64_t>(2, ceil_div(pr.K, TR_STAGE)));
         pr.k_chunk = (int)(ceil_div(ceil_div(pr.K, want), TR_STAGE) * TR_STAGE);
         pr.n_split = (int)std::max<int64_t>(2, ceil_div(pr.K, pr.k_chunk));
         pr.z0 = z;
         z += pr.n_split;
     }
-    if ((size_t)z * slab > workspace_bytes || !aligned16(workspace)) return 0;
+    if ((size_t)z * slab > workspace_bytes || !aligned16(workspace)) {
+        for (int i = 0; i < p.n_prob; i++) p.prob[i] = saved[i];
+        return 0;
+    }
     *taken = true;
-    p.max_m = 256;
+    p.max_m = ki;
     p.partial = static_cast<float *>(workspace);
     p.a_sk = lda;
     p.a_si = 1;
     p.b_sk = ldb;
     p.b_sj = 1;
-    static bool prepared_on[64] = {};  // more LDS than the default limit: once per device
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) device = 0;
-    if (!prepared_on[device]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&sgemm_tn_rows_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)kTnRowsLds);
-        if (e != hipSuccess) {
-            set_error("hipFuncSetAttribute(dynamic LDS %zu): %s", kTnRowsLds, hipGetErrorString(e));
-            return -1;
-        }
-        prepared_on[device] = true;
-    }
-    sgemm_tn_rows_kernel<<<z, 512, kTnRowsLds, stream>>>(p);
-    YITU_LAUNCH_CHECK();
-    dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)256 * 256, kSplitReduceCols), 4096),
+    int rc = -1;
+    if (ki == 256 && no == 256) rc = sgemm_tn_rows_launch<4, 2, 2, 4>(p, z, stream);
+    else if (ki == 256 && no == 128) rc = sgemm_tn_rows_launch<4, 2, 2, 2>(p, z, stream);
+    else if (ki == 128 && no == 256) rc = sgemm_tn_rows_launch<2, 4, 2, 2>(p, z, stream);
+    else if (ki == 256 && no == 64) rc = sgemm_tn_rows_launch<8, 1, 1, 2>(p, z, stream);
+    else if (ki == 64 && no == 256) rc = sgemm_tn_rows_launch<1, 8, 2, 1>(p, z, stream);
+    else if (ki == 128 && no == 128) rc = sgemm_tn_rows_launch<2, 4, 2, 1>(p, z, stream);
+    else if (ki == 128 && no == 64) rc = sgemm_tn_rows_launch<4, 2, 1, 1>(p, z, stream);
+    else if (ki == 64 && no == 128) rc = sgemm_tn_rows_launch<2, 4, 1, 1>(p, z, stream);
+    if (rc) return rc;
+    dim3 rg((unsigned)std::min<int64_t>(ceil_div((int64_t)ki * no, kSplitReduceCols), 4096),
             (unsigned)p.n_prob);
     sgemm_splitk_reduce_kernel<<<rg, 256, 0, stream>>>(p);
     YITU_LAUNCH_CHECK();
@@ -865,8 +925,9 @@ YITU_API size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int6
     // (or room for the [N, K] copies of the weights that the many-rows kernel reads, or for
     // the chunk products of the weight-gradient kernel: a chunk per CU and two per problem)
     size_t rows_ws = std::max<size_t>(sgemm_rows_workspace_bytes(n, k, n_problems), 256);
-    if (m == 256 && n == 256)
-        rows_ws = std::max(rows_ws, (size_t)(256 + 2 * kMaxGroup) * 256 * 256 * sizeof(float));
+    if (tn_rows_shape(m, n))
+        rows_ws = std::max(rows_ws, (size_t)(tn_rows_chunks(m, n) + 2 * kMaxGroup) * m * n *
+                                        sizeof(float));
     if (tiles <= 0 || tiles >= 256 || k < 2 * kMinSplitK) return rows_ws;
     const int64_t splits = std::min<int64_t>(ceil_div(k, kMinSplitK), ceil_div(1024, tiles));
     return std::max(rows_ws, align_up((size_t)(splits * m * n * n_problems) * sizeof(float), 256));
