@@ -27,6 +27,8 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdint>
+#include <cstdlib>
+#include <new>
 #include <cstdio>
 #include <cstring>
 #include <numeric>
@@ -51,33 +53,75 @@ thread_local char g_err[256] = "";
 
 // Symmetric weighted adjacency in CSR form: row v = distinct neighbours of v
 // (ascending id) with the number of input edges between them in either direction.
+// Storage that is not cleared when it is made: the arrays of the adjacency are written in
+// full by the threads that fill them, and clearing 400 MB from one thread first (which is
+// what a vector does) took longer than everything else in the build.
+template <typename T>
+struct RawArray {
+    T *p = nullptr;
+    explicit RawArray(size_t n) : p(static_cast<T *>(std::malloc(std::max<size_t>(n, 1) * sizeof(T)))) {
+        if (!p) throw std::bad_alloc();
+    }
+    RawArray() = default;
+    RawArray(RawArray &&o) noexcept : p(o.p) { o.p = nullptr; }
+    RawArray &operator=(RawArray &&o) noexcept {
+        std::swap(p, o.p);
+        return *this;
+    }
+    RawArray(const RawArray &) = delete;
+    RawArray &operator=(const RawArray &) = delete;
+    ~RawArray() { std::free(p); }
+    T *data() const { return p; }
+    T &operator[](size_t i) const { return p[i]; }
+};
+
 struct Adjacency {
     std::vector<int64_t> ptr;
-    std::vector<Edge> edges;
+    RawArray<Edge> edges;
 };
 
 Adjacency build_adjacency(const int32_t *src, const int32_t *dst, int64_t m, vint n) {
-    // counting sort by end point; the slots of a row are handed out with relaxed atomic
-    // adds (the rows are sorted afterwards, so the order of arrival does not matter)
+    // counting sort by end point. Every thread reads the whole edge list and keeps the end
+    // points that fall into its own range of vertices: no counter is shared, where atomic
+    // adds from all threads met on the few vertices that hold most edges of a power-law
+    // graph (and took most of the reorder's time). The rows are sorted afterwards, so the
+    // order of arrival does not matter.
     std::vector<int64_t> count(n + 1, 0);
-#pragma omp parallel for schedule(static)
-    for (int64_t i = 0; i < m; i++) {
-        if (src[i] != dst[i]) {
-            __atomic_fetch_add(&count[(vint)src[i] + 1], 1, __ATOMIC_RELAXED);
-            __atomic_fetch_add(&count[(vint)dst[i] + 1], 1, __ATOMIC_RELAXED);
+    const int n_threads = omp_get_max_threads();
+#pragma omp parallel num_threads(n_threads)
+    {
+        const int tid = omp_get_thread_num(), nt = omp_get_num_threads();
+        const vint lo = (vint)((uint64_t)n * tid / nt), hi = (vint)((uint64_t)n * (tid + 1) / nt);
+        for (int64_t i = 0; i < m; i++) {
+            const vint s = (vint)src[i], d = (vint)dst[i];
+            if (s == d) continue;
+            if (s >= lo && s < hi) count[s + 1]++;
+            if (d >= lo && d < hi) count[d + 1]++;
         }
     }
     for (vint v = 0; v < n; v++) count[v + 1] += count[v];
-    std::vector<vint> raw((size_t)count[n]);
+    RawArray<vint> raw((size_t)count[n]);
     {
         std::vector<int64_t> fill(count.begin(), count.end() - 1);
-#pragma omp parallel for schedule(static)
-        for (int64_t i = 0; i < m; i++) {
-            if (src[i] != dst[i]) {
-                raw[(size_t)__atomic_fetch_add(&fill[(vint)src[i]], 1, __ATOMIC_RELAXED)] =
-                    (vint)dst[i];
-                raw[(size_t)__atomic_fetch_add(&fill[(vint)dst[i]], 1, __ATOMIC_RELAXED)] =
-                    (vint)src[i];
+        // ranges of about equal numbers of end points this time (the low ids of a
+        // power-law graph hold far more than their share)
+        std::vector<vint> cut(n_threads + 1, n);
+        cut[0] = 0;
+        for (int t = 1; t < n_threads; t++) {
+            const int64_t want = count[n] / n_threads * t;
+            cut[t] = (vint)(std::lower_bound(count.begin(), count.end(), want) - count.begin());
+            if (cut[t] > n) cut[t] = n;
+        }
+#pragma omp parallel num_threads(n_threads)
+        {
+            const int tid = omp_get_thread_num(), nt = omp_get_num_threads();
+            // (fewer threads than asked for: the last one takes the rest)
+            const vint lo = cut[tid], hi = tid + 1 == nt ? n : cut[tid + 1];
+            for (int64_t i = 0; i < m; i++) {
+                const vint s = (vint)src[i], d = (vint)dst[i];
+                if (s == d) continue;
+                if (s >= lo && s < hi) raw[(size_t)fill[s]++] = d;
+                if (d >= lo && d < hi) raw[(size_t)fill[d]++] = s;
             }
         }
     }
@@ -93,8 +137,7 @@ Adjacency build_adjacency(const int32_t *src, const int32_t *dst, int64_t m, vin
     }
     for (vint v = 0; v < n; v++) uniq[v + 1] += uniq[v];
     Adjacency adj;
-    adj.ptr = uniq;
-    adj.edges.resize((size_t)uniq[n]);
+    adj.edges = RawArray<Edge>((size_t)uniq[n]);
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int64_t v = 0; v < (int64_t)n; v++) {
         const vint *b = raw.data() + count[v], *e = raw.data() + count[v + 1];
@@ -109,6 +152,7 @@ Adjacency build_adjacency(const int32_t *src, const int32_t *dst, int64_t m, vin
             *out++ = Edge{t, w};
         }
     }
+    adj.ptr = std::move(uniq);
     return adj;
 }
 
