@@ -417,7 +417,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
     const int n_all = p.tile_start[p.n_problems];
     const int per_wg = (n_all + (int)gridDim.x - 1) / (int)gridDim.x;
     const int my_lo = blockIdx.x * per_wg, my_hi = min(my_lo + per_wg, n_all);
-    const bool whole_cols = blockIdx.y * 256 + 256 <= p.N;
+    // per wave: its 32 columns lie wholly inside the output (vector stores through the
+    // staging area), partly (element by element), or not at all (nothing to compute)
+    const bool whole_cols = wn + 32 <= p.N, no_cols = wn >= p.N;
     const int lrow = t / TPR, lcol = (t % TPR) * 4;
 
     for (int q = 0; q < p.n_problems; q++) {
@@ -475,6 +477,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
                 float16v acc;
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+                if (no_cols) continue;  // (after the barrier and the loads that every wave shares)
                 const float *arow = At + l32 * A_LD + KS * lk;
 #pragma unroll
                 for (int s4 = 0; s4 < KS; s4 += 4) {
@@ -488,7 +491,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
                 }
                 // accumulator element 4 jj + ii is C[32 tile + lane % 32][wn + 8 jj + 4 (lane / 32) + ii]
                 const int row0 = (tile - lo) * SR_M;
-                if (whole_cols && row0 + SR_M <= m_q) {  // same for the whole workgroup
+                if (whole_cols && row0 + SR_M <= m_q) {  // same for the whole wave
 #pragma unroll
                     for (int jj = 0; jj < 4; jj++) {
                         const f4 w = {acc[4 * jj], acc[4 * jj + 1], acc[4 * jj + 2], acc[4 * jj + 3]};

@@ -212,7 +212,9 @@ __global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
     const int n_all = p.tile_start[p.n_problems];
     const int per_wg = (n_all + (int)gridDim.x - 1) / (int)gridDim.x;
     const int my_lo = blockIdx.x * per_wg, my_hi = min(my_lo + per_wg, n_all);
-    const bool whole_cols = blockIdx.y * HN + HN <= p.N;
+    // per wave: its 64 columns lie wholly inside the output (vector stores through the
+    // staging area), partly (element by element), or not at all (nothing to compute)
+    const bool whole_cols = wn + 64 <= p.N, no_cols = wn >= p.N;
     // loader: TPR threads cover one row, the workgroup RPS rows at a time. Rows past the
     // end are read from the last row (their outputs are never stored) and tiles past the
     // end from the last tile: no load of the ring is conditional.
@@ -270,6 +272,7 @@ __global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[j][e] = 0.0f;
+            if (no_cols) continue;  // (after the barrier and the loads that every wave shares)
 #pragma unroll
             for (int s = 0; s < KS; s++) {
                 const bf16x8 a =
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(256, 2) void hgemm_rows_kernel(HRowsParams p) {
             // accumulator element 4 jj + ii of column tile j is
             // C[32 tile + lane % 32][wn + 32 j + 8 jj + 4 (lane / 32) + ii]
             const int row0 = (tile - lo) * RM;
-            if (whole_cols && row0 + RM <= m_q) {  // same for the whole workgroup
+            if (whole_cols && row0 + RM <= m_q) {  // same for the whole wave
                 if constexpr (OUT_BF16) {
 #pragma unroll
                     for (int j = 0; j < 2; j++)
