@@ -360,6 +360,16 @@ int yitu_sgemm(float *c_device, const float *a_device, const float *b_device, in
                int accumulate, void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
+ * y[m,n] = x[m,k] . w^T + bias, w stored [n,k] like nn.Linear.weight, bias [n] or NULL:
+ * the forward of the Linear layers of the models (test/common/model.py:25-29, 86-88).
+ * On the many-rows kernel (see yitu_sgemm) the bias is added before the rows are stored;
+ * otherwise by a pass of its own. Workspace as for yitu_sgemm(m, n, k).
+ */
+int yitu_linear_forward(float *y_device, const float *x_device, const float *w_device,
+                        const float *bias_device, int64_t m, int64_t n, int64_t k,
+                        void *workspace_device, size_t workspace_bytes, void *stream);
+
+/*
  * Typed products in one launch per 8 problems: C_i[m_i,n] (+)= op(A_i)[m_i,k_i] .
  * op(B_i)[k_i,n] for i < n_problems, with shared n, transposes and leading
  * dimensions. c, a, b, m, k are HOST arrays (of device pointers and sizes).

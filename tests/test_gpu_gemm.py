@@ -62,6 +62,22 @@ def test_sgemm_weight_gradient_many_rows(dev, ks, ki, no):
     assert all(torch.equal(c, d) for c, d in zip(got, run()))
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("m,n,k", [(70001, 256, 256), (50000, 250, 128), (60000, 448, 64),
+                                   (5000, 256, 256), (300, 40, 24), (1, 7, 3)])
+def test_linear_forward_with_bias(dev, with_bias, m, n, k):
+    """y = x w^T + bias: the bias is added inside the many-rows kernel (whole and ragged
+    tiles and column blocks) or by a pass of its own after the tiled kernel."""
+    g = torch.Generator().manual_seed(m + n + k)
+    x, w = torch.randn(m, k, generator=g), torch.randn(n, k, generator=g)
+    b = torch.randn(n, generator=g) if with_bias else None
+    got = graph_ext.linear_forward(x.to(dev), w.to(dev), None if b is None else b.to(dev))
+    want = x.double() @ w.double().t()
+    if b is not None:
+        want = want + b.double()
+    assert_close(got, want.float(), atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+
+
 def test_sgemm_typed_gemm_shape(dev):
     """[n_t, 256] x [256, 256] of the heterogeneous configuration (fast path)."""
     g = torch.Generator().manual_seed(1)

@@ -35,6 +35,7 @@ struct GemmProblem {
     // the K range [s * k_chunk, min(K, (s+1) * k_chunk)) and, when n_split > 1,
     // writes its own [M, N] slab of `partial` (slab index = blockIdx.z)
     int z0, n_split, k_chunk;
+    const float *bias = nullptr;  // [N], added to every row (the many-rows kernel only)
 };
 
 struct GemmParams {
@@ -384,6 +385,7 @@ struct SRowsParams {
     const float *A[kMaxGroup];
     const float *B[kMaxGroup];
     float *C[kMaxGroup];
+    const float *bias[kMaxGroup];  // [N] added to every row of the problem, or null
     int M[kMaxGroup];
     int tile_start[kMaxGroup + 1];
     int n_problems, N;
@@ -430,6 +432,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
         const float *__restrict__ a_q = p.A[q];
         const float *__restrict__ b_q = p.B[q];
         float *__restrict__ c_q = p.C[q];
+        const float *__restrict__ bias_q = p.bias[q];
         const int m_q = p.M[q];
         float b[KS];
         {
@@ -494,7 +497,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
                 if (whole_cols && row0 + SR_M <= m_q) {  // same for the whole wave
 #pragma unroll
                     for (int jj = 0; jj < 4; jj++) {
-                        const f4 w = {acc[4 * jj], acc[4 * jj + 1], acc[4 * jj + 2], acc[4 * jj + 3]};
+                        f4 w = {acc[4 * jj], acc[4 * jj + 1], acc[4 * jj + 2], acc[4 * jj + 3]};
+                        if (bias_q)  // same for the whole launch of the problem
+                            w += *reinterpret_cast<const f4 *>(bias_q + wn + 8 * jj + 4 * lk);
                         *reinterpret_cast<f4 *>(stage + l32 * SR_C_LD + 32 * jj + 16 * lk) = w;
                     }
 #pragma unroll
@@ -510,7 +515,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_rows_kernel(SRowsParams p) {
 #pragma unroll
                     for (int e = 0; e < 16; e++) {
                         const int col = wn + 8 * (e / 4) + 4 * lk + e % 4;
-                        if (col < p.N) c_q[row * p.ldc + col] = acc[e];
+                        if (col < p.N) c_q[row * p.ldc + col] = acc[e] + (bias_q ? bias_q[col] : 0.0f);
                     }
                 }
             }
@@ -585,7 +590,9 @@ static int sgemm_rows_try(const GemmParams &p, bool trans_a, bool trans_b, int l
     SRowsParams r{};
     for (int i = 0; i < p.n_prob; i++) {
         const GemmProblem &pr = p.prob[i];
-        if (pr.K != k || !aligned16(pr.A) || !aligned16(pr.C) || pr.M < 0) return 0;
+        if (pr.K != k || !aligned16(pr.A) || !aligned16(pr.C) || !aligned16(pr.bias) || pr.M < 0)
+            return 0;
+        r.bias[i] = pr.bias;
         r.A[i] = pr.A;
         r.B[i] = pr.B;
         r.C[i] = pr.C;
@@ -952,6 +959,46 @@ YITU_API int yitu_sgemm(float *c, const float *a, const float *b, int64_t m, int
     p.accumulate = accumulate;
     return sgemm_grouped(p, trans_a != 0, trans_b != 0, (int)lda, (int)ldb, workspace,
                          workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+namespace yitu {
+// y[i, j] += bias[j]: the bias of a Linear whose product did not run on the kernel that adds it
+__global__ __launch_bounds__(256) void bias_add_kernel(float *__restrict__ y,
+                                                       const float *__restrict__ bias, int64_t m,
+                                                       int n, int64_t ldy) {
+    const int64_t total = m * n, stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+        y[(i / n) * ldy + i % n] += bias[i % n];
+}
+}  // namespace yitu
+
+YITU_API int yitu_linear_forward(float *y, const float *x, const float *w, const float *bias,
+                                 int64_t m, int64_t n, int64_t k, void *workspace,
+                                 size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(m >= 0 && n >= 0 && k >= 0, "negative size");
+    if (m == 0 || n == 0) return 0;
+    YITU_REQUIRE(y && (k == 0 || (x && w)), "null operand");
+    YITU_REQUIRE(m < INT32_MAX && n < INT32_MAX && k < INT32_MAX, "size out of range");
+    GemmParams p{};
+    p.prob[0] = GemmProblem{x, w, y, (int)m, (int)k};
+    p.prob[0].bias = bias;
+    p.n_prob = 1;
+    p.N = (int)n;
+    p.ldc = (int)n;
+    if (k > 0) {
+        bool taken = false;
+        const int rc = sgemm_rows_try(p, false, true, (int)k, (int)k, workspace, workspace_bytes,
+                                      stream, &taken);
+        if (taken) return rc;
+    }
+    p.prob[0].bias = nullptr;
+    const int rc = sgemm_grouped(p, false, true, (int)k, (int)k, workspace, workspace_bytes, stream);
+    if (rc || !bias) return rc;
+    const int grid = (int)std::min<int64_t>(ceil_div(m * n, 256), 16384);
+    bias_add_kernel<<<grid, 256, 0, stream>>>(y, bias, m, (int)n, n);
+    YITU_LAUNCH_CHECK();
+    return 0;
 }
 
 YITU_API int yitu_sgemm_typed(float *const *c, const float *const *a, const float *const *b,

@@ -486,6 +486,29 @@ def b2gemm_backward(x, w_a, w_b, grad_a, grad_b):
     return [dx, dw_a, dw_b]
 
 
+def linear_forward(x, weight, bias=None):
+    """x . weight^T + bias in fp32 on the matrix cores (``weight`` [n, k] as nn.Linear keeps
+    it, ``bias`` [n] or None), the bias added inside the product where the kernel allows."""
+    _check(x, torch.float32, "x", 2)
+    _check(weight, torch.float32, "weight", 2)
+    if bias is not None:
+        _check(bias, torch.float32, "bias", 1)
+    dev = _lib.require_device(x, weight) if bias is None else _lib.require_device(x, weight, bias)
+    m, k = x.shape
+    n = weight.size(0)
+    if weight.size(1) != k or (bias is not None and bias.numel() != n):
+        raise RuntimeError("linear_forward: x [m, k], weight [n, k], bias [n]")
+    y = torch.empty((m, n), dtype=torch.float32, device=dev)
+    ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(c_i64(m), c_i64(n), c_i64(k),
+                                                               c_i64(1)), dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_linear_forward(ptr(y), ptr(x), ptr(weight), ptr(bias), c_i64(m),
+                                            c_i64(n), c_i64(k), ptr(ws), c_size(ws.numel()),
+                                            stream_ptr(dev))
+    check(rc, "yitu_linear_forward")
+    return y
+
+
 def sgemm(a, b, trans_a=False, trans_b=False, out=None):
     """op(a) . op(b) in fp32 on the matrix cores; a, b contiguous 2-D. ``out``:
     a contiguous [m, n] tensor (e.g. a row slice of a larger buffer) to write."""

@@ -107,8 +107,7 @@ class MfmaLinearFunction(autograd.Function):
     def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
-        y = graph_ext.sgemm(x, weight, trans_b=True)
-        return y if bias is None else y.add_(bias)
+        return graph_ext.linear_forward(x, weight, None if bias is None else bias.contiguous())
 
     @staticmethod
     @once_differentiable
