@@ -370,6 +370,19 @@ int yitu_linear_forward(float *y_device, const float *x_device, const float *w_d
                         void *workspace_device, size_t workspace_bytes, void *stream);
 
 /*
+ * The same for the Linear layers of several node or edge types at once (the
+ * per-relation loop of HeteroGraphConv, test/common/model.py:137-171, over layers
+ * of model.py:25-29): y_i[m_i,n] = x_i[m_i,k] . w_i^T + bias_i for i < n_problems, eight
+ * layers per launch. y, x, w, bias, m are HOST arrays (of device pointers and sizes); the
+ * bias table or single entries of it may be NULL. All y_i are contiguous (row stride n).
+ * Workspace as for yitu_sgemm(max m_i, n, k, min(n_problems, 8)).
+ */
+int yitu_linear_forward_typed(float *const *y, const float *const *x, const float *const *w,
+                              const float *const *bias, const int64_t *m, int64_t n_problems,
+                              int64_t n, int64_t k, void *workspace_device,
+                              size_t workspace_bytes, void *stream);
+
+/*
  * Typed products in one launch per 8 problems: C_i[m_i,n] (+)= op(A_i)[m_i,k_i] .
  * op(B_i)[k_i,n] for i < n_problems, with shared n, transposes and leading
  * dimensions. c, a, b, m, k are HOST arrays (of device pointers and sizes).

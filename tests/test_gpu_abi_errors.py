@@ -118,3 +118,37 @@ def test_typed_bf16_products_report_bad_arguments(dev):
     torch.cuda.synchronize()
     want = a.float().t() @ g.float()
     assert torch.allclose(dw, want, rtol=1e-4, atol=1e-3)
+
+
+def test_typed_linear_forward_reports_bad_arguments(dev):
+    """Host tables of device pointers: a null table, a null operand of a type that has rows
+    and sizes out of range are reported; no types, a type without rows, a null bias table
+    and null bias entries are not errors."""
+    L = _lib.lib()
+    st = _lib.stream_ptr(dev)
+    x = torch.randn(64, 48, device=dev)
+    w = torch.randn(32, 48, device=dev)
+    b = torch.randn(32, device=dev)
+    y = torch.empty(64, 32, device=dev)
+    ws = _lib.workspace(1 << 20, dev)
+    ptrs = lambda *ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() if t is not None else None
+                                                      for t in ts])
+    rows = lambda *v: (ctypes.c_int64 * len(v))(*v)
+
+    def call(ys=ptrs(y), xs=ptrs(x), wts=ptrs(w), bs=ptrs(b), m=rows(64), count=1, n=32, k=48):
+        return L.yitu_linear_forward_typed(ys, xs, wts, bs, m, I64(count), I64(n), I64(k), P(ws),
+                                           SZ(ws.numel()), st)
+
+    assert call() == 0
+    torch.cuda.synchronize()
+    assert torch.allclose(y, x @ w.t() + b, rtol=1e-4, atol=1e-4)
+    assert call(count=0) == 0
+    assert call(bs=None) == 0
+    assert call(bs=ptrs(None)) == 0
+    torch.cuda.synchronize()
+    assert torch.allclose(y, x @ w.t(), rtol=1e-4, atol=1e-4)
+    _fails(call(ys=None), "null problem table")
+    _fails(call(xs=ptrs(None)), "null operand")
+    _fails(call(m=rows(-1)), "size out of range")
+    _fails(call(n=-1), "negative size")
+    assert call(xs=ptrs(None), m=rows(0)) == 0

@@ -78,6 +78,35 @@ def test_linear_forward_with_bias(dev, with_bias, m, n, k):
     assert_close(got, want.float(), atol=1e-4 * max(1.0, np.sqrt(k) / 4))
 
 
+@pytest.mark.parametrize("ms,n,k", [([30000, 0, 20001, 300], 256, 256), ([7000] * 10, 192, 128),
+                                    ([900, 1, 77], 96, 40), ([40000, 30000], 250, 64)])
+def test_linear_forward_typed(dev, ms, n, k):
+    """Per-type Linear layers written as row slices of one buffer, some with and some without
+    a bias: on the many-rows kernel (bias inside), on the tiled kernel (bias pass after it),
+    with an empty type, with more than eight types, and against the layer-at-a-time call."""
+    g = torch.Generator().manual_seed(sum(ms) + n + k)
+    xs = [torch.randn(m, k, generator=g) for m in ms]
+    ws = [torch.randn(n, k, generator=g) for _ in ms]
+    bs = [torch.randn(n, generator=g) if i % 3 != 1 else None for i in range(len(ms))]
+    y = torch.full((sum(ms), n), float("nan"), device=dev)
+    parts, off = [], 0
+    for m in ms:
+        parts.append(y[off:off + m])
+        off += m
+    to = lambda t: None if t is None else t.to(dev)
+    got = graph_ext.linear_forward_typed([to(x) for x in xs], [to(w) for w in ws],
+                                         [to(b) for b in bs], out_list=parts)
+    for x, w, b, c, part in zip(xs, ws, bs, got, parts):
+        assert c.data_ptr() == part.data_ptr()
+        want = x.double() @ w.double().t()
+        if b is not None:
+            want = want + b.double()
+        assert_close(c, want.float(), atol=1e-4 * max(1.0, np.sqrt(k) / 4))
+        if x.size(0):
+            single = graph_ext.linear_forward(to(x), to(w), to(b))
+            assert_close(c, single.cpu())
+
+
 def test_sgemm_typed_gemm_shape(dev):
     """[n_t, 256] x [256, 256] of the heterogeneous configuration (fast path)."""
     g = torch.Generator().manual_seed(1)

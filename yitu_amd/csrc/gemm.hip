@@ -1001,6 +1001,56 @@ YITU_API int yitu_linear_forward(float *y, const float *x, const float *w, const
     return 0;
 }
 
+YITU_API int yitu_linear_forward_typed(float *const *y, const float *const *x,
+                                       const float *const *w, const float *const *bias,
+                                       const int64_t *m, int64_t n_problems, int64_t n, int64_t k,
+                                       void *workspace, size_t workspace_bytes, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_problems >= 0 && n >= 0 && k >= 0, "negative size");
+    if (n_problems == 0 || n == 0) return 0;
+    YITU_REQUIRE(y && x && w && m, "null problem table");
+    YITU_REQUIRE(n < INT32_MAX && k < INT32_MAX, "size out of range");
+    for (int64_t first = 0; first < n_problems; first += kMaxGroup) {
+        GemmParams p{};
+        p.N = (int)n;
+        p.ldc = (int)n;
+        const int count = (int)std::min<int64_t>(kMaxGroup, n_problems - first);
+        for (int i = 0; i < count; i++) {
+            const int64_t mi = m[first + i];
+            YITU_REQUIRE(mi >= 0 && mi < INT32_MAX, "problem %d: size out of range",
+                         (int)(first + i));
+            if (mi == 0) continue;
+            YITU_REQUIRE(y[first + i] && (k == 0 || (x[first + i] && w[first + i])),
+                         "problem %d: null operand", (int)(first + i));
+            GemmProblem pr{x[first + i], w[first + i], y[first + i], (int)mi, (int)k};
+            pr.bias = bias ? bias[first + i] : nullptr;
+            p.prob[p.n_prob++] = pr;
+        }
+        if (p.n_prob == 0) continue;
+        if (k > 0) {
+            bool taken = false;
+            const int rc = sgemm_rows_try(p, false, true, (int)k, (int)k, workspace,
+                                          workspace_bytes, stream, &taken);
+            if (rc) return rc;
+            if (taken) continue;
+        }
+        // (the grouped call drops problems from its table: keep what the bias pass needs)
+        const GemmParams all = p;
+        for (int i = 0; i < p.n_prob; i++) p.prob[i].bias = nullptr;
+        const int rc = sgemm_grouped(p, false, true, (int)k, (int)k, workspace, workspace_bytes,
+                                     stream);
+        if (rc) return rc;
+        for (int i = 0; i < all.n_prob; i++) {
+            const GemmProblem &pr = all.prob[i];
+            if (!pr.bias) continue;
+            const int grid = (int)std::min<int64_t>(ceil_div((int64_t)pr.M * n, 256), 16384);
+            bias_add_kernel<<<grid, 256, 0, stream>>>(pr.C, pr.bias, pr.M, (int)n, n);
+            YITU_LAUNCH_CHECK();
+        }
+    }
+    return 0;
+}
+
 YITU_API int yitu_sgemm_typed(float *const *c, const float *const *a, const float *const *b,
                               const int64_t *m, const int64_t *k, int64_t n_problems, int64_t n,
                               int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldc,

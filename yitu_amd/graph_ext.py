@@ -509,6 +509,46 @@ def linear_forward(x, weight, bias=None):
     return y
 
 
+def linear_forward_typed(x_list, weight_list, bias_list, out_list=None):
+    """[x_i . weight_i^T + bias_i] for Linear layers that share both widths (the per-type
+    layers of a heterogeneous model), eight layers per launch. ``bias_list`` entries may be
+    None. ``out_list``: contiguous [m_i, n] tensors to write (e.g. row slices of one buffer)."""
+    import ctypes
+    count = len(x_list)
+    if count == 0 or len(weight_list) != count or len(bias_list) != count:
+        raise RuntimeError("linear_forward_typed needs as many weights and biases as inputs")
+    n, k = weight_list[0].shape
+    for x, w, b in zip(x_list, weight_list, bias_list):
+        _check(x, torch.float32, "x", 2)
+        _check(w, torch.float32, "weight", 2)
+        if tuple(w.shape) != (n, k) or x.size(1) != k:
+            raise RuntimeError("linear_forward_typed: x_i [m_i, k], weight_i [n, k]")
+        if b is not None:
+            _check(b, torch.float32, "bias", 1)
+            if b.numel() != n:
+                raise RuntimeError("linear_forward_typed: bias_i [n]")
+    dev = _lib.require_device(*x_list, *weight_list, *[b for b in bias_list if b is not None])
+    ms = [x.size(0) for x in x_list]
+    if out_list is None:
+        out_list = [torch.empty((m, n), dtype=torch.float32, device=dev) for m in ms]
+    else:
+        for c, m in zip(out_list, ms):
+            _check(c, torch.float32, "out", 2)
+            if tuple(c.shape) != (m, n) or c.device != dev:
+                raise RuntimeError("out must be [%d, %d] on the operands' device" % (m, n))
+    ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(
+        c_i64(max(ms)), c_i64(n), c_i64(k), c_i64(min(count, 8))), dev)
+    pointers = lambda ts: (ctypes.c_void_p * count)(
+        *[(t.data_ptr() or None) if t is not None else None for t in ts])
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_linear_forward_typed(
+            pointers(out_list), pointers(x_list), pointers(weight_list), pointers(bias_list),
+            (ctypes.c_int64 * count)(*ms), c_i64(count), c_i64(n), c_i64(k), ptr(ws),
+            c_size(ws.numel()), stream_ptr(dev))
+    check(rc, "yitu_linear_forward_typed")
+    return list(out_list)
+
+
 def sgemm(a, b, trans_a=False, trans_b=False, out=None):
     """op(a) . op(b) in fp32 on the matrix cores; a, b contiguous 2-D. ``out``:
     a contiguous [m, n] tensor (e.g. a row slice of a larger buffer) to write."""

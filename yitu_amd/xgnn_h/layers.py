@@ -145,11 +145,16 @@ class _TypedLinear(torch.autograd.Function):
         for x in xs:
             parts.append(y[off:off + x.size(0)])
             off += x.size(0)
-        graph_ext.sgemm_typed([x.contiguous() for x in xs], [w.contiguous() for w in ws],
-                              trans_b=True, out_list=parts)
-        for part, b in zip(parts, bs):
-            if b is not None:
-                part += b
+        if all(w.shape == ws[0].shape for w in ws):
+            graph_ext.linear_forward_typed(
+                [x.contiguous() for x in xs], [w.contiguous() for w in ws],
+                [None if b is None else b.contiguous() for b in bs], out_list=parts)
+        else:
+            graph_ext.sgemm_typed([x.contiguous() for x in xs], [w.contiguous() for w in ws],
+                                  trans_b=True, out_list=parts)
+            for part, b in zip(parts, bs):
+                if b is not None:
+                    part += b
         ctx.n_parts = n_parts
         ctx.has_bias = [b is not None for b in bs]
         ctx.save_for_backward(*xs, *ws)
