@@ -182,8 +182,8 @@ class _TypedLinear(torch.autograd.Function):
                                                         [xs[i].contiguous() for i in want],
                                                         trans_a=True)):
                 gw[i] = g
-        gb = [gs[i].sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None
-              for i in range(n)]
+        gb = [graph_ext.column_sum(gs[i])
+              if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None for i in range(n)]
         return (None, *gx, *gw, *gb)
 
 
