@@ -730,6 +730,17 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
 
     params = list(model.em.parameters()) + list(l1.parameters()) + list(l2.parameters())
     res["stacked_model_2_layers_fwd_bwd_ms"] = _event_ms(train_step(two_layers, params), steps, warm)
+    del l1, l2, stacked, model, lowered, stitched_flow, params
+    # the reference's 2-layer attention model (4 heads of 64, mean over heads) on the same graph
+    torch.manual_seed(7)
+    model = models.RGATModel(hg, dim, 64, 64, n_heads=4).to(dev)
+    kwargs = {"hgraph": hg, "xs": kwargs["xs"]}
+    lowered = xgnn_h.Optimizer().lower(xgnn_h.Module2IR().transform(model, kwargs), kwargs)
+    stitched_flow = xgnn_h.Stitcher().transform(lowered, kwargs)
+    gy = {n: torch.randn(c, 64, generator=g, device=dev) for n, c in ntypes.items()}
+    for flow, tag in ((lowered, "lowered"), (stitched_flow, "stitched")):
+        res["reference_rgat_2_layers_%s_fwd_bwd_ms" % tag] = _event_ms(
+            train_step(lambda: executor.run(flow, kwargs), list(model.parameters())), steps, warm)
     return res
 
 

@@ -391,8 +391,12 @@ def test_skinny_linear_rejects_wide_outputs(dev):
     assert not graph_ext.skinny_linear_shape(1024, 8) and graph_ext.skinny_linear_shape(1024, 4)
 
 
-@pytest.mark.parametrize("m,n", [(1, 1), (11132, 100), (64, 272), (65, 3), (5000, 1000)])
+@pytest.mark.parametrize("m,n", [(1, 1), (11132, 100), (64, 272), (65, 3), (5000, 1000), (70001, 256),
+                                 (9000, 1024), (8193, 12), (300000, 64), (4097, 1028), (777, 4)])
 def test_column_sum(dev, m, n):
+    """Column counts that are multiples of 4 up to 1024 (16-byte reads, several rows side by
+    side, also where 256 is not a multiple of n / 4) and others (one column per thread); row
+    counts around the chunking's steps; the same bits on a second call."""
     g = torch.Generator().manual_seed(m + n)
     x = torch.randn(m, n, generator=g)
     got = graph_ext.column_sum(x.to(dev))

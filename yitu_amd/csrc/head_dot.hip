@@ -495,6 +495,7 @@ __global__ __launch_bounds__(kBlock) void partial_sum_kernel(float *__restrict__
     const int j = blockIdx.x * kSumCols + c;
     float s = 0.0f;
     if (j < width)
+#pragma unroll 8
         for (int r = g; r < n_rows; r += kSumGroups) s += partial[(size_t)r * width + j];
     red[g][c] = s;
     __syncthreads();
@@ -621,12 +622,13 @@ YITU_API int yitu_skinny_linear_backward(float *grad_x, int accumulate, float *g
 namespace yitu {
 namespace {
 
-// rows per workgroup: 64 on large inputs, fewer on small ones so that a few thousand
-// rows still make a few hundred workgroups (and as many partial rows for the second step) (a function of n_rows alone: the workspace
-// size and the summation order follow from it)
+// rows per workgroup: about a thousand workgroups on large inputs (all resident at once, a few
+// hundred KB of row data each, and a thousand partial rows for the second step), 8 rows on
+// small ones (a function of n_rows alone: the workspace size and the summation order follow
+// from it)
 inline int col_sum_chunk(int64_t n_rows) {
-    const int64_t c = n_rows / 256;
-    return c < 8 ? 8 : (c > 64 ? 64 : (int)c);
+    const int64_t c = ceil_div(n_rows, 1024);
+    return c < 8 ? 8 : (int)c;
 }
 
 __global__ __launch_bounds__(kBlock) void column_chunk_sum_kernel(float *__restrict__ partial,
@@ -638,6 +640,31 @@ __global__ __launch_bounds__(kBlock) void column_chunk_sum_kernel(float *__restr
 #pragma unroll 8
         for (int r = r0; r < r1; r++) s += x[(size_t)r * n_cols + c];
         partial[(size_t)blockIdx.x * n_cols + c] = s;
+    }
+}
+
+// The same for rows of up to 1024 columns, a multiple of 4: a thread reads 16 bytes of a row,
+// 256 / (n_cols / 4) rows are read side by side, and their sums are added in row-group order.
+__global__ __launch_bounds__(kBlock) void column_chunk_sum4_kernel(float *__restrict__ partial,
+                                                                   const float *__restrict__ x,
+                                                                   int n_rows, int n_cols, int chunk) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ f4 red[kBlock];
+    const int vc = n_cols / 4, side = kBlock / vc;
+    const int c4 = threadIdx.x % vc, rg = threadIdx.x / vc;
+    const int r0 = blockIdx.x * chunk, r1 = min(r0 + chunk, n_rows);
+    f4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (rg < side) {
+        const f4 *__restrict__ src = reinterpret_cast<const f4 *>(x) + c4;
+#pragma unroll 8
+        for (int r = r0 + rg; r < r1; r += side)
+            s += __builtin_nontemporal_load(src + (size_t)r * vc);
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if (rg == 0) {
+        for (int q = 1; q < side; q++) s += red[q * vc + c4];
+        reinterpret_cast<f4 *>(partial + (size_t)blockIdx.x * n_cols)[c4] = s;
     }
 }
 
@@ -663,8 +690,12 @@ YITU_API int yitu_column_sum(float *out, const float *x, int64_t n_rows, int64_t
     const int chunk = col_sum_chunk(n_rows);
     const int chunks = (int)ceil_div(n_rows, chunk);
     float *partial = static_cast<float *>(workspace);
-    column_chunk_sum_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows, (int)n_cols,
-                                                           chunk);
+    if (n_cols % 4 == 0 && n_cols <= 4 * kBlock && aligned16(x) && aligned16(partial))
+        column_chunk_sum4_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows,
+                                                                (int)n_cols, chunk);
+    else
+        column_chunk_sum_kernel<<<chunks, kBlock, 0, stream>>>(partial, x, (int)n_rows,
+                                                               (int)n_cols, chunk);
     YITU_LAUNCH_CHECK();
     partial_sum_kernel<<<(int)ceil_div(n_cols, kSumCols), kBlock, 0, stream>>>(
         out, (int)n_cols, nullptr, 0, partial, chunks);
