@@ -725,7 +725,8 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
     stacked = l1.stack(blocks, norms)
 
     def two_layers():
-        hidden = l1(model.em(hg, kwargs["xs"]), stacked)
+        # (all node ids in order: the tables themselves, as the executor passes them on)
+        hidden = l1({n: table.weight for n, table in model.em.embeds.items()}, stacked)
         return l2({n: torch.relu(h) for n, h in hidden.items()}, stacked)
 
     params = list(model.em.parameters()) + list(l1.parameters()) + list(l2.parameters())

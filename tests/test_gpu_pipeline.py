@@ -113,3 +113,46 @@ def test_single_root_stitch_like_the_reference_test(dev):
     # training mode: dropout is live, two runs differ
     executor.train()
     assert not torch.equal(executor.run(dataflow_2, kwargs), executor.run(dataflow_2, kwargs))
+
+
+def test_embedding_of_all_ids_in_order_is_the_table(dev, monkeypatch):
+    """Node ids 0..n-1 in order: the executor hands on the table instead of gathering it, with
+    the same outputs and parameter gradients, bit for bit, as the lookup; ids in another order,
+    or changed in place after the first run, take the lookup."""
+    torch.manual_seed(11)
+    hgraph = cases.hetero_graph(device=dev)
+    kwargs = cases.hetero_kwargs(hgraph, device=dev)
+    model = models.RGCNModel(hgraph, 16, 16, 4).to(dev)
+    lowered = xgnn_h.Optimizer().lower(xgnn_h.Module2IR().transform(model, kwargs), kwargs)
+    weights = {nty: torch.randn(num, 4, device=dev) for nty, num in hgraph.nty2num.items()}
+    params = list(model.parameters())
+    taken = []
+    whole_table = xgnn_h.Executor._whole_table
+
+    def counting(self, node, v):
+        res = whole_table(self, node, v)
+        taken.append(res is not None)
+        return res
+
+    monkeypatch.setattr(xgnn_h.Executor, "_whole_table", counting)
+    short = _run_with_grads(lowered, kwargs, params, weights)
+    assert taken and all(taken)
+    monkeypatch.setattr(xgnn_h.Executor, "_whole_table", lambda self, node, v: None)
+    _compare(short, _run_with_grads(lowered, kwargs, params, weights), rtol=0, atol=0)
+
+    # one executor, ids reversed in place between two runs: the second run looks them up
+    monkeypatch.setattr(xgnn_h.Executor, "_whole_table", counting)
+    executor = xgnn_h.Executor()
+    executor.eval()
+    first = executor.run(lowered, kwargs)
+    for ids in kwargs["xs"].values():
+        ids.copy_(ids.flip(0))
+    del taken[:]
+    second = executor.run(lowered, kwargs)
+    assert taken and not any(taken)
+    want = xgnn_h.Executor()
+    want.eval()
+    monkeypatch.setattr(xgnn_h.Executor, "_whole_table", lambda self, node, v: None)
+    for nty, got in second.items():
+        assert torch.equal(got, want.run(lowered, kwargs)[nty])
+    assert any(not torch.equal(first[nty], second[nty]) for nty in first)

@@ -24,6 +24,7 @@ class Executor:
     def __init__(self):
         self._is_training = None
         self._edge_values = {}  # edge_values node -> (state of its inputs, result, inputs)
+        self._whole_tables = {}  # embedding node -> (state of its index tensor, is arange, tensor)
 
     def eval(self):
         self._is_training = False
@@ -45,12 +46,37 @@ class Executor:
             return value[rest]
         return value[int(rest)]
 
+    def _whole_table(self, node: ir.Node, v: dict):
+        """An embedding lookup of every row in order (the models are fed all node ids,
+        model.py:174-195 with the benchmark's ``arange`` inputs) is the table itself: no gather
+        and, in the backward, no sort-and-segment pass over the incoming gradient. The index
+        tensor is compared with ``arange`` once and remembered for as long as it is unchanged."""
+        args, kw = _fill(node.attrs["args"], v), node.attrs["kwargs"]
+        if len(args) != 2 or kw.get("max_norm") is not None or kw.get("scale_grad_by_freq") or \
+                kw.get("sparse") or kw.get("padding_idx") is not None:
+            return None
+        idx, weight = args
+        if not (torch.is_tensor(idx) and torch.is_tensor(weight)) or idx.dim() != 1 or \
+                weight.dim() != 2 or idx.numel() != weight.size(0) or idx.is_floating_point():
+            return None
+        state = (idx.data_ptr(), idx._version, idx.numel())
+        kept = self._whole_tables.get(id(node))
+        if kept is None or kept[0] != state or kept[2] is not idx:
+            same = torch.equal(idx, torch.arange(idx.numel(), device=idx.device, dtype=idx.dtype))
+            kept = (state, bool(same), idx)
+            self._whole_tables[id(node)] = kept
+        return weight.view_as(weight) if kept[1] else None
+
     # -- one node ------------------------------------------------------------
     def _eval(self, node: ir.Node, v: dict, kwargs: dict):
         op = node.op
         if op in ("input", "graph"):
             return self._lookup(node.name, kwargs)
         if op == "call":
+            if node.attrs["fn"] is F.embedding:
+                whole = self._whole_table(node, v)
+                if whole is not None:
+                    return whole
             return node.attrs["fn"](*_fill(node.attrs["args"], v), **_fill(node.attrs["kwargs"], v))
         if op == "linear":
             return bundle.linear(v["x"], node.attrs["weight"], node.attrs["bias"])
