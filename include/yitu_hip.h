@@ -102,11 +102,17 @@ int yitu_agg_csr(float *out_device, const void *x_device, int x_is_bf16,
  * yitu_agg_csr_noalloc_max_bytes() = 32 MiB inside the library instead of a
  * caller's workspace. No counterpart in the reference. It calls no hipMalloc /
  * hipFree or any allocating routine; problems whose
- * yitu_spmm_workspace_bytes(nnz, dim, 0) exceeds the array are rejected (< 0).
+ * yitu_spmm_workspace_bytes(nnz, dim, 0) exceeds the array are rejected (< 0),
+ * except that a graph which cannot hold a row of 64 edges (nnz < 64, or a stated
+ * 0 <= max_degree < 64) uses no scratch and is accepted at any size.
  * All calls on one GPU share that GPU's array: calls that overlap in time on
  * one GPU (different streams or threads) race and must be serialised by the caller.
+ * yitu_agg_csr_noalloc_init() looks up the array's address on the current device
+ * (hipGetSymbolAddress, once per device); the first call on a device does the same,
+ * so a caller that captures a stream calls init, or the function once, beforehand.
  */
 size_t yitu_agg_csr_noalloc_max_bytes(void);
+int yitu_agg_csr_noalloc_init(void);
 int yitu_agg_csr_noalloc(float *out_device, const void *x_device, int x_is_bf16,
                          const int32_t *row_pointers_device, const int32_t *column_index_device,
                          const float *degrees_device, int64_t n_rows, int64_t n_src, int64_t nnz,

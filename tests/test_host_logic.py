@@ -27,7 +27,8 @@ def test_library_exports_every_declared_symbol():
     missing = [n for n in sorted(names) if not hasattr(lib, n)]
     assert not missing, "declared but not exported: %s" % missing
     lib.yitu_abi_version.restype = ctypes.c_int
-    assert lib.yitu_abi_version() >= 1
+    from yitu_amd import _lib as binding
+    assert lib.yitu_abi_version() == binding.ABI_VERSION == 3
 
 
 def test_host_library_exports_every_declared_symbol():

@@ -259,3 +259,37 @@ def test_printer_lists_nodes_in_evaluation_order():
         "%%3: [%d, 4] = call.squeeze(0: %%2)" % n,
         "%%4: [%d, 4] = call.multiply(0: %%norm, 1: %%3)" % n,
     ]
+
+
+def test_whole_embedding_table_is_aliased_only_under_autograd():
+    """All ids in order make an embedding lookup the table itself. The alias is handed out
+    only where an in-place write to it would raise (gradients on, a table that takes one);
+    under no_grad and for a frozen table the lookup copies, so nothing downstream can write
+    into the parameter."""
+    import torch.nn.functional as F
+    hgraph = cases.hetero_graph()
+    kwargs = cases.hetero_kwargs(hgraph)
+    model = models.RGCNModel(hgraph, 8, 8, 4)
+    dataflow = xgnn_h.Module2IR().transform(model, kwargs)
+    nodes = [n for n in ir.walk(dataflow) if n.op == "call" and n.attrs["fn"] is F.embedding]
+    assert nodes
+    node = nodes[0]
+    executor = xgnn_h.Executor()
+    table = torch.nn.Parameter(torch.randn(6, 3))
+    ids = torch.arange(6)
+    node_like = type("N", (), {"attrs": {"args": (ids, table), "kwargs": {}}})()
+    executor.train()
+    assert executor._whole_table(node_like, {}).data_ptr() == table.data_ptr()
+    with torch.no_grad():
+        assert executor._whole_table(node_like, {}) is None
+    executor.eval()  # no dropout; gradients still flow, so autograd still guards the alias
+    assert executor._whole_table(node_like, {}) is not None
+    with pytest.raises(RuntimeError):
+        executor._whole_table(node_like, {}).add_(1.0)
+    table.requires_grad_(False)
+    assert executor._whole_table(node_like, {}) is None
+    table.requires_grad_(True)
+    shuffled = type("N", (), {"attrs": {"args": (ids.flip(0), table), "kwargs": {}}})()
+    assert executor._whole_table(shuffled, {}) is None
+    executor.forget_tables()
+    assert not executor._whole_tables

@@ -65,3 +65,28 @@ def test_rejects_what_does_not_fit_the_static_array(dev):
                                          _lib.c_f32(1.0), _lib.c_i64(-1), _lib.stream_ptr(dev))
     assert rc < 0
     assert b"static array" in _lib.lib().yitu_last_error()
+
+
+def test_large_graph_of_short_rows_needs_no_scratch(dev):
+    """A graph beyond the static array's worst-case bound is accepted when the caller
+    states that no row reaches the planning threshold: nothing is planned, nothing is
+    staged. (2^17 rows x 12 edges, F = 64: the bound asks for about 37 MiB.)"""
+    assert _lib.lib().yitu_agg_csr_noalloc_init() == 0
+    n, per_row, dim = 1 << 17, 12, 64
+    g = torch.Generator().manual_seed(11)
+    indptr = (torch.arange(n + 1, dtype=torch.int64) * per_row).to(torch.int32)
+    indices = torch.randint(0, n, (n * per_row,), generator=g).to(torch.int32)
+    x = torch.randn(n, dim, generator=g)
+    deg = graphgen.gcn_norm(indptr)
+    need = _lib.size_fn("yitu_spmm_workspace_bytes")(_lib.c_i64(indices.numel()), _lib.c_i64(dim),
+                                                     _lib.c_int(0))
+    assert need > (32 << 20)
+    xd, rp, ci, dg = x.to(dev), indptr.to(dev), indices.to(dev), deg.to(dev)
+    out = torch.empty(n, dim, device=dev)
+    args = (_lib.ptr(out), _lib.ptr(xd), 0, _lib.ptr(rp), _lib.ptr(ci), _lib.ptr(dg), _lib.c_i64(n),
+            _lib.c_i64(n), _lib.c_i64(ci.numel()), _lib.c_i64(dim), _lib.c_f32(1.0))
+    rc = _lib.lib().yitu_agg_csr_noalloc(*args, _lib.c_i64(-1), _lib.stream_ptr(dev))
+    assert rc < 0  # without the hint the worst case does not fit
+    rc = _lib.lib().yitu_agg_csr_noalloc(*args, _lib.c_i64(per_row), _lib.stream_ptr(dev))
+    _lib.check(rc, "yitu_agg_csr_noalloc")
+    assert_close(out, oracle.row_agg(x.numpy(), indptr, indices, deg.numpy(), oracle.MODE_GCN))

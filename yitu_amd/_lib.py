@@ -15,6 +15,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libyitu_hip.so")
 _lib = None
 _lock = threading.Lock()
+# The C ABI these bindings were written for (yitu_abi_version() of include/yitu_hip.h). A
+# library of another version has other argument lists: calling it would hand the kernels
+# shifted pointers, so it is refused at load time.
+ABI_VERSION = 3
 
 c_i64 = ctypes.c_int64
 c_int = ctypes.c_int
@@ -34,6 +38,12 @@ def lib():
                         "libyitu_hip.so is not built; run `python -m yitu_amd.build` "
                         "(there is no CPU fallback)")
                 l = ctypes.CDLL(LIB_PATH)
+                l.yitu_abi_version.restype = ctypes.c_int
+                found = l.yitu_abi_version()
+                if found != ABI_VERSION:
+                    raise RuntimeError(
+                        "libyitu_hip.so has ABI version %d, these bindings need %d; rebuild it "
+                        "with `python -m yitu_amd.build --force`" % (found, ABI_VERSION))
                 l.yitu_last_error.restype = ctypes.c_char_p
                 _lib = l
     return _lib

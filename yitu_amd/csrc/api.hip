@@ -85,12 +85,21 @@ int static_scratch(void **ptr) {
 
 YITU_API size_t yitu_agg_csr_noalloc_max_bytes(void) { return kStaticScratchBytes; }
 
+YITU_API int yitu_agg_csr_noalloc_init(void) {
+    void *ws = nullptr;
+    return static_scratch(&ws);
+}
+
 YITU_API int yitu_agg_csr_noalloc(float *out, const void *x, int x_is_bf16,
                                   const int32_t *row_pointers, const int32_t *column_index,
                                   const float *degrees, int64_t n_rows, int64_t n_src,
                                   int64_t nnz, int64_t dim, float alpha, int64_t max_degree,
                                   void *stream) {
     YITU_REQUIRE(n_rows >= 0 && n_src >= 0 && nnz >= 0 && dim >= 0, "negative size");
+    // no row can reach the planning threshold: no temporary plan, no partial rows, no scratch
+    if (nnz < kPlanThreshold || (max_degree >= 0 && max_degree < kPlanThreshold))
+        return yitu_agg_csr(out, x, x_is_bf16, row_pointers, column_index, degrees, n_rows, n_src,
+                            nnz, dim, alpha, max_degree, nullptr, nullptr, nullptr, 0, stream);
     const size_t need = spmm_workspace_bytes(nnz, dim, false);
     YITU_REQUIRE(need <= kStaticScratchBytes,
                  "problem needs %zu bytes of scratch, the static array holds %zu: use "

@@ -286,6 +286,13 @@ YITU_API size_t yitu_build_part_workspace_bytes(int64_t n_rows) {
            align_up(part_scan_bytes(n_rows), 256);
 }
 
+namespace yitu {
+__global__ void part_empty_kernel(int32_t *part_ptr, long long *n_parts_out) {
+    *n_parts_out = 0;
+    part_ptr[0] = 0;
+}
+}  // namespace yitu
+
 YITU_API int yitu_build_part(int32_t *part_ptr, int32_t *part2node, long long *n_parts_out,
                              const int32_t *indptr, int64_t n_rows, int64_t part_size,
                              int64_t capacity, void *workspace, size_t workspace_bytes,
@@ -301,8 +308,9 @@ YITU_API int yitu_build_part(int32_t *part_ptr, int32_t *part2node, long long *n
                  "workspace too small or misaligned: need %zu bytes, 256-byte aligned",
                  yitu_build_part_workspace_bytes(n_rows));
     if (n_rows == 0) {
-        YITU_HIP(hipMemsetAsync(n_parts_out, 0, sizeof(long long), stream));
-        YITU_HIP(hipMemsetAsync(part_ptr, 0, sizeof(int32_t), stream));
+        // one thread writes the two words: no memset node, so the call may be captured
+        part_empty_kernel<<<1, 1, 0, stream>>>(part_ptr, n_parts_out);
+        YITU_LAUNCH_CHECK();
         return 0;
     }
     char *w = static_cast<char *>(workspace);

@@ -50,7 +50,14 @@ class Executor:
         """An embedding lookup of every row in order (the models are fed all node ids,
         model.py:174-195 with the benchmark's ``arange`` inputs) is the table itself: no gather
         and, in the backward, no sort-and-segment pass over the incoming gradient. The index
-        tensor is compared with ``arange`` once and remembered for as long as it is unchanged."""
+        tensor is compared with ``arange`` once and remembered for as long as it is unchanged
+        (its address, torch version counter and length; an index buffer refilled through its raw
+        pointer must be dropped with ``forget_tables``). The alias is only handed out where
+        autograd guards it: with gradients enabled and a table that takes one, an in-place
+        write to the result raises instead of changing the table. ``no_grad`` runs and frozen
+        tables take ``F.embedding``'s copy."""
+        if not torch.is_grad_enabled():
+            return None
         args, kw = _fill(node.attrs["args"], v), node.attrs["kwargs"]
         if len(args) != 2 or kw.get("max_norm") is not None or kw.get("scale_grad_by_freq") or \
                 kw.get("sparse") or kw.get("padding_idx") is not None:
@@ -59,6 +66,8 @@ class Executor:
         if not (torch.is_tensor(idx) and torch.is_tensor(weight)) or idx.dim() != 1 or \
                 weight.dim() != 2 or idx.numel() != weight.size(0) or idx.is_floating_point():
             return None
+        if not weight.requires_grad:
+            return None
         state = (idx.data_ptr(), idx._version, idx.numel())
         kept = self._whole_tables.get(id(node))
         if kept is None or kept[0] != state or kept[2] is not idx:
@@ -66,6 +75,11 @@ class Executor:
             kept = (state, bool(same), idx)
             self._whole_tables[id(node)] = kept
         return weight.view_as(weight) if kept[1] else None
+
+    def forget_tables(self):
+        """Drops what is remembered about embedding index tensors (call after refilling one
+        through a raw pointer, which leaves its version counter unchanged)."""
+        self._whole_tables.clear()
 
     # -- one node ------------------------------------------------------------
     def _eval(self, node: ir.Node, v: dict, kwargs: dict):
