@@ -144,6 +144,99 @@ def cpu_library_cross_check(rp, ci, deg, x, with_scipy=False):
     return res
 
 
+def _cpu_cores():
+    return int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+
+def _cpu_median_s(fn, reps=3):
+    fn()  # warm-up: page in the operands, spin up the thread team
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2]
+
+
+def cpu_baseline_gat(rp, ci, q, k, x, gy):
+    """The reference's GAT lowering (sddmm_forward, spmm_forward, spmm_backward,
+    sddmm_backward: sparse.py:7-81) as the oracle's float builds on all host cores, full
+    workload. The by-source view that the two gradient sums walk is per-graph preparation
+    and untimed, like the transposed structure of the GPU path."""
+    import oracle
+    rp_h, ci_h = rp.cpu().numpy(), ci.cpu().numpy()
+    q_h, k_h = q.cpu().numpy()[None], k.cpu().numpy()
+    x_h, gy_h = x.cpu().numpy(), gy.cpu().numpy()
+    n = k_h.shape[0]
+    tr = oracle.csr_transpose(rp_h, ci_h, n)
+
+    def step():
+        attn = oracle.sddmm_forward(rp_h, ci_h, q_h, k_h)
+        oracle.mh_spmm_forward(attn, rp_h, ci_h, x_h, f64=False)
+        ga, _ = oracle.mh_spmm_backward_omp(attn, rp_h, ci_h, x_h, gy_h, tr)
+        oracle.sddmm_backward_omp(rp_h, ci_h, q_h, k_h, attn, ga, tr)
+
+    t = _cpu_median_s(step)
+    return {"value": ci_h.shape[0] / t, "unit": "edges/s", "cores": _cpu_cores(), "kind": "port",
+            "sample": "full workload (%d nodes, %d edges, 4 heads x 64), attention fwd+bwd, median "
+                      "of 3, OpenMP float restatement oracle/yitu_oracle.c" % (n, ci_h.shape[0]),
+            "seconds": t}
+
+
+def cpu_baseline_rgcn(xs, wts, values, indptr, indices, d_out, off):
+    """The heterogeneous layer of the fourth configuration on the host cores: per-type
+    products, the stacked edge-weighted aggregation, its by-source backward and the two
+    gradient products, all in float on all cores (oracle/yitu_oracle.c), full workload."""
+    import numpy as np
+    import oracle
+    xs_h = [x.cpu().numpy() for x in xs]
+    ws_h = [w.cpu().numpy() for w in wts]
+    v_h, ip_h, ix_h = values.cpu().numpy(), indptr.cpu().numpy(), indices.cpu().numpy()
+    g_h = d_out.cpu().numpy()
+    n_all, dim = g_h.shape
+    tr = oracle.csr_transpose(ip_h, ix_h, n_all)
+
+    def step():
+        h = np.concatenate([oracle.gemm_omp(x, w) for x, w in zip(xs_h, ws_h)])
+        oracle.mh_spmm_forward(v_h, ip_h, ix_h, h.reshape(n_all, 1, dim), f64=False)
+        _, dh = oracle.mh_spmm_backward_omp(v_h, ip_h, ix_h, h.reshape(n_all, 1, dim),
+                                            g_h.reshape(n_all, 1, dim), tr, need_grad_a=False)
+        dh = dh.reshape(n_all, dim)
+        for t, (x, w) in enumerate(zip(xs_h, ws_h)):
+            part = dh[off[t]:off[t + 1]]
+            oracle.gemm_omp(x, part, trans_a=True)
+            oracle.gemm_omp(part, w, trans_b=True)
+
+    t = _cpu_median_s(step)
+    return {"value": t * 1e3, "unit": "ms per layer fwd+bwd", "cores": _cpu_cores(), "kind": "port",
+            "sample": "full workload (4 node types, %d edges, 256 features, fp32), median of 3, "
+                      "OpenMP float restatement oracle/yitu_oracle.c" % ix_h.shape[0],
+            "seconds": t}
+
+
+def cpu_baseline_temporal(layer, blk, gout, k):
+    """The temporal attention layer as dense masked attention in plain torch on the host
+    cores (oracle/temporal.py, the statement of YiTu_T/layers.py:75-142 that the GPU layer is
+    checked against), forward + backward through autograd on the same batch."""
+    import copy
+    from oracle.temporal import dense_temporal_attention
+    cpu_layer = copy.deepcopy(layer).cpu()
+    h = blk.h.detach().cpu().requires_grad_()
+    row, dt, g = blk.row.cpu(), blk.dt.cpu(), gout.cpu()
+
+    def step():
+        dense_temporal_attention(cpu_layer, h, row, dt, blk.n_dst, k).backward(g)
+        h.grad = None
+        cpu_layer.zero_grad(set_to_none=True)
+
+    t = _cpu_median_s(step, reps=5)
+    return {"value": t * 1e3, "unit": "ms per layer fwd+bwd", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "the same batch (%d roots, %d sampled edges), median of 5, dense masked "
+                      "attention in torch on the host (oracle/temporal.py)" % (blk.n_dst, row.numel()),
+            "seconds": t}
+
+
 def run_spmm(args, dev, bf16):
     from yitu_amd import _lib
     n, rp, ci, deg, info = build_c3(dev)
@@ -346,11 +439,13 @@ def run_gat(args, dev):
         xgnn_h.Optimizer(fuse_gat=False, bundle_gemm=False).lower(captured, m_kwargs))
     alg_sd = 4 * (n + 1) + 4 * nnz + 8 * n * h + 4 * nnz * h
     alg_fwd, alg_bwd = gat_algorithmic_bytes(n, nnz, h, f)
+    cpu = None if args.no_cpu else cpu_baseline_gat(rp, ci, q, k, x, gy)
     return {
         "metric": "GAT attention fwd+bwd (fused SDDMM+LeakyReLU+softmax+aggregate), edges/sec",
         "value": nnz / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "cpu_baseline": cpu,
         "config": {"workload": "c2_gat_f32", "graph": "R-MAT scale 18, 13M draws dedup, CSR by "
                    "destination", "n_nodes": n, "n_edges": nnz, "heads": h, "head_dim": f},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
@@ -651,7 +746,9 @@ def run_c4(args, dev):
     gather = n_edges * dim * 4
     module_ms = _c4_module_ms(sizes, rels, dim, dev, steps, warm)
     peak = 157.3  # fp32 matrix TFLOP/s, published
+    cpu = None if args.no_cpu else cpu_baseline_rgcn(xs, wts, values, indptr, indices, d_out, off)
     return {"value": n_edges / (total * 1e-3), "unit": "edges/s", "ms_per_step": total, "dtype": "f32",
+            "cpu_baseline": cpu,
             "config": {"workload": "c4_rgcn_f32", "node_types": sizes, "relations": 8,
                        "n_edges": n_edges, "feature_dim": dim,
                        "aggregation": "one edge-weighted SpMM over the stacked relations"},
@@ -899,8 +996,9 @@ def run_c5(args, dev):
 
     ms = _event_ms(step, max(args.steps, 20), args.warmup)
     graph_ms = _c5_graph_ms(layer, blk, gout, max(args.steps, 20))
+    cpu = None if args.no_cpu else cpu_baseline_temporal(layer, blk, gout, k)
     return {"value": ms, "unit": "ms", "ms_per_step": ms, "dtype": "f32", "higher_is_better": False,
-            "hip_graph_ms": graph_ms,
+            "hip_graph_ms": graph_ms, "cpu_baseline": cpu,
             "config": {"workload": "c5_temporal_attention_f32", "n_nodes": n_nodes,
                        "n_events": n_events, "batch": batch, "neighbours": k,
                        "sampled_edges": blk.num_edges()},
@@ -1067,19 +1165,29 @@ def main():
         res["copy_calibration"] = calibration_copy(dev)
         if not args.no_extra:
             # the other single-GPU configurations ride along as extra fields
-            args.cpu_cross_check = not args.no_cpu  # the small first configuration keeps its own
-            args.no_cpu = True
+            want_cpu = not args.no_cpu
+            args.cpu_cross_check = want_cpu  # the small first configuration keeps its own
             slim = lambda r: {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "config",
-                                                "roofline", "fwd_ms", "bwd_ms", "layer_fwd_bwd_ms",
+                                                "roofline", "cpu_baseline", "fwd_ms", "bwd_ms",
+                                                "layer_fwd_bwd_ms",
                                                 "reference_gatlayer_fwd_bwd_ms", "gat_model_2_layers",
                                                 "sddmm", "weighted_spmm")
                               if k in r}
-            res["extra"] = {"c3_spmm_bf16": slim(run_spmm(args, dev, bf16=True)),
-                            "c2_gat_f32": slim(run_gat(args, dev)),
-                            "c3_gat_f32": slim(run_gat_c3(args, dev)),
-                            "c1_gcn_f32": run_c1(args, dev),
-                            "c4_rgcn_f32": run_c4(args, dev),
-                            "c5_temporal_attention_f32": run_c5(args, dev)}
+            extra = {}
+            # each configuration's own CPU leg rides along (a few seconds each, about twenty
+            # for the dense products of the fourth); the two that reuse the headline's
+            # graph do without
+            args.no_cpu = True
+            extra["c3_spmm_bf16"] = slim(run_spmm(args, dev, bf16=True))
+            args.no_cpu = not want_cpu
+            extra["c2_gat_f32"] = slim(run_gat(args, dev))
+            args.no_cpu = True
+            extra["c3_gat_f32"] = slim(run_gat_c3(args, dev))
+            extra["c1_gcn_f32"] = run_c1(args, dev)
+            args.no_cpu = not want_cpu
+            extra["c4_rgcn_f32"] = run_c4(args, dev)
+            extra["c5_temporal_attention_f32"] = run_c5(args, dev)
+            res["extra"] = extra
             if args.orders:
                 res["extra"]["c3_vertex_orders"] = run_c3_orders(args, dev)
     elif args.workload == "c3_spmm_bf16":

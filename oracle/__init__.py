@@ -181,6 +181,63 @@ def mh_spmm_backward(values, indptr, indices, feat, grad_out):
     return grad_a, grad_x
 
 
+def csr_transpose(indptr, indices, n_src):
+    """By-source view (t_indptr, t_rows, t_perm) of a CSR: stable sort on the column."""
+    indptr, indices = _i32(indptr), _i32(indices)
+    n_dst = indptr.shape[0] - 1
+    t_indptr = np.zeros(n_src + 1, dtype=np.int32)
+    t_rows = np.zeros(indices.shape[0], dtype=np.int32)
+    t_perm = np.zeros(indices.shape[0], dtype=np.int32)
+    lib().orc_csr_transpose(_p(t_indptr), _p(t_rows), _p(t_perm), _p(indptr), _p(indices),
+                            I64(n_dst), I64(n_src))
+    return t_indptr, t_rows, t_perm
+
+
+def mh_spmm_backward_omp(values, indptr, indices, feat, grad_out, transposed, need_grad_a=True,
+                         need_grad_x=True):
+    """Float, all cores, for timing: the gradients of mh_spmm_backward without atomics
+    (grad_x over the by-source view ``transposed`` = csr_transpose(...))."""
+    values, feat, grad_out = _f32(values), _f32(feat), _f32(grad_out)
+    indptr, indices = _i32(indptr), _i32(indices)
+    t_indptr, t_rows, t_perm = transposed
+    n_dst = indptr.shape[0] - 1
+    n_src, h, f = feat.shape
+    grad_a = np.empty_like(values) if need_grad_a else None
+    grad_x = np.empty_like(feat) if need_grad_x else None
+    lib().orc_mh_spmm_bwd_omp(_p(grad_a) if need_grad_a else None,
+                              _p(grad_x) if need_grad_x else None, _p(values), _p(indptr),
+                              _p(indices), _p(feat), _p(grad_out), _p(t_indptr), _p(t_rows),
+                              _p(t_perm), I64(n_dst), I64(n_src), I64(h), I64(f))
+    return grad_a, grad_x
+
+
+def sddmm_backward_omp(indptr, indices, query, key, attn, grad_out, transposed):
+    """Float, all cores, for timing: sddmm_backward with grad_key summed by source."""
+    query, key, attn, grad_out = _f32(query), _f32(key), _f32(attn), _f32(grad_out)
+    indptr, indices = _i32(indptr), _i32(indices)
+    t_indptr, _, t_perm = transposed
+    gq = np.empty_like(query)
+    gk = np.empty_like(key)
+    scratch = np.empty_like(attn)
+    lib().orc_sddmm_bwd_omp(_p(gq), _p(gk), _p(scratch), _p(indptr), _p(indices), _p(query),
+                            _p(key), _p(attn), _p(grad_out), _p(t_indptr), _p(t_perm),
+                            I64(indptr.shape[0] - 1), I64(key.shape[0]), I64(query.shape[-1]),
+                            I64(query.shape[0]))
+    return gq, gk
+
+
+def gemm_omp(a, b, trans_a=False, trans_b=False):
+    """Float, all cores, for timing: op(a) . op(b)."""
+    a, b = _f32(a), _f32(b)
+    n, k = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    m = b.shape[0] if trans_b else b.shape[1]
+    assert (b.shape[1] if trans_b else b.shape[0]) == k
+    c = np.empty((n, m), dtype=np.float32)
+    lib().orc_gemm_f32_omp(_p(c), _p(a), _p(b), I64(n), I64(m), I64(k),
+                           ctypes.c_int(1 if trans_a else 0), ctypes.c_int(1 if trans_b else 0))
+    return c
+
+
 def sddmm_forward(indptr, indices, query, key):
     """sddmm_cuda.cu:5-33,69-89. query [n_bid,Nd,H], key [Ns,H] -> attn [E,H]."""
     query, key = _f32(query), _f32(key)

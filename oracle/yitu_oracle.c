@@ -267,6 +267,72 @@ ORC_EXPORT void orc_mh_spmm_bwd(float *grad_a, float *grad_x, const float *value
     free(gx);
 }
 
+/*
+ * By-source view of a CSR (stable counting sort on the column): t_indptr [n_src + 1],
+ * t_rows[j] = destination row and t_perm[j] = CSR position of the j-th by-source edge.
+ * Per-graph preparation of the timed _omp gradients below, which must not race on a
+ * source's row the way the reference's atomics do (spmm_cuda.cu:33-38).
+ */
+ORC_EXPORT void orc_csr_transpose(int32_t *t_indptr, int32_t *t_rows, int32_t *t_perm,
+                                  const int32_t *indptr, const int32_t *indices, int64_t n_dst,
+                                  int64_t n_src)
+{
+    for (int64_t c = 0; c <= n_src; c++) t_indptr[c] = 0;
+    for (int64_t i = 0; i < indptr[n_dst]; i++) t_indptr[(indices[i] & COL_MASK) + 1]++;
+    for (int64_t c = 0; c < n_src; c++) t_indptr[c + 1] += t_indptr[c];
+    int32_t *cursor = (int32_t *)malloc(sizeof(int32_t) * (size_t)(n_src + 1));
+    memcpy(cursor, t_indptr, sizeof(int32_t) * (size_t)(n_src + 1));
+    for (int64_t r = 0; r < n_dst; r++)
+        for (int32_t i = indptr[r]; i < indptr[r + 1]; i++) {
+            int32_t j = cursor[indices[i] & COL_MASK]++;
+            t_rows[j] = (int32_t)r;
+            t_perm[j] = i;
+        }
+    free(cursor);
+}
+
+/*
+ * orc_mh_spmm_bwd in float on all cores, for timing only: grad_a row-parallel, grad_x
+ * source-parallel over the by-source view (each source's row has one writer, edges
+ * added in ascending destination order). Either output may be NULL.
+ */
+ORC_EXPORT void orc_mh_spmm_bwd_omp(float *grad_a, float *grad_x, const float *values,
+                                    const int32_t *indptr, const int32_t *indices,
+                                    const float *feat, const float *grad_out,
+                                    const int32_t *t_indptr, const int32_t *t_rows,
+                                    const int32_t *t_perm, int64_t n_dst, int64_t n_src,
+                                    int64_t n_heads, int64_t n_feat)
+{
+    int64_t L = n_heads * n_feat;
+    if (grad_a) {
+#pragma omp parallel for schedule(dynamic, 64)
+        for (int64_t r = 0; r < n_dst; r++) {
+            const float *g = grad_out + r * L;
+            for (int32_t i = indptr[r]; i < indptr[r + 1]; i++) {
+                const float *x = feat + (int64_t)(indices[i] & COL_MASK) * L;
+                for (int64_t h = 0; h < n_heads; h++) {
+                    float dot = 0.0f;
+                    for (int64_t k = 0; k < n_feat; k++) dot += g[h * n_feat + k] * x[h * n_feat + k];
+                    grad_a[(int64_t)i * n_heads + h] = dot;
+                }
+            }
+        }
+    }
+    if (grad_x) {
+#pragma omp parallel for schedule(dynamic, 64)
+        for (int64_t c = 0; c < n_src; c++) {
+            float *o = grad_x + c * L;
+            for (int64_t t = 0; t < L; t++) o[t] = 0.0f;
+            for (int32_t j = t_indptr[c]; j < t_indptr[c + 1]; j++) {
+                const float *g = grad_out + (int64_t)t_rows[j] * L;
+                const float *v = values + (int64_t)t_perm[j] * n_heads;
+                for (int64_t h = 0; h < n_heads; h++)
+                    for (int64_t k = 0; k < n_feat; k++) o[h * n_feat + k] += v[h] * g[h * n_feat + k];
+            }
+        }
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 /* B3/B4: SDDMM(u_add_v) + LeakyReLU(0.2) + edge softmax.                     */
 /* YiTu_GNN/YiTu_H/src/sddmm_cuda.cu, ops.cuh                                 */
@@ -348,6 +414,51 @@ ORC_EXPORT void orc_sddmm_bwd(float *grad_q, float *grad_k, const int32_t *indpt
     free(gk);
 }
 
+/*
+ * orc_sddmm_bwd in float on all cores, for timing only: a row-parallel pass writes the
+ * per-edge logit gradient gv into edge_grad [nnz, H] (caller's scratch) and sums grad_q,
+ * a source-parallel pass sums grad_k over the by-source view.
+ */
+ORC_EXPORT void orc_sddmm_bwd_omp(float *grad_q, float *grad_k, float *edge_grad,
+                                  const int32_t *indptr, const int32_t *indices,
+                                  const float *query, const float *key, const float *attn,
+                                  const float *grad_out, const int32_t *t_indptr,
+                                  const int32_t *t_perm, int64_t n_dst, int64_t n_src,
+                                  int64_t n_heads, int64_t n_bid)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t r = 0; r < n_dst; r++) {
+        for (int64_t h = 0; h < n_heads; h++) {
+            float cache[16] = {0.0f}, gq[16] = {0.0f};
+            for (int32_t j = indptr[r]; j < indptr[r + 1]; j++) {
+                int32_t bid = (int32_t)((uint32_t)indices[j] >> 24);
+                cache[bid] -= attn[(int64_t)j * n_heads + h] * grad_out[(int64_t)j * n_heads + h];
+            }
+            for (int32_t i = indptr[r]; i < indptr[r + 1]; i++) {
+                int32_t bid = (int32_t)((uint32_t)indices[i] >> 24);
+                int64_t c = indices[i] & COL_MASK;
+                float gs = attn[(int64_t)i * n_heads + h] *
+                           (cache[bid] + grad_out[(int64_t)i * n_heads + h]);
+                float x = query[(int64_t)bid * n_dst * n_heads + r * n_heads + h] +
+                          key[c * n_heads + h];
+                float gv = gs * (x < 0.0f ? 0.2f : 1.0f);
+                edge_grad[(int64_t)i * n_heads + h] = gv;
+                gq[bid] += gv;
+            }
+            for (int64_t b = 0; b < n_bid; b++)
+                grad_q[b * n_dst * n_heads + r * n_heads + h] = gq[b];
+        }
+    }
+#pragma omp parallel for schedule(dynamic, 256)
+    for (int64_t c = 0; c < n_src; c++)
+        for (int64_t h = 0; h < n_heads; h++) {
+            float acc = 0.0f;
+            for (int32_t j = t_indptr[c]; j < t_indptr[c + 1]; j++)
+                acc += edge_grad[(int64_t)t_perm[j] * n_heads + h];
+            grad_k[c * n_heads + h] = acc;
+        }
+}
+
 /* ------------------------------------------------------------------------- */
 /* B10: stitch_csr. YiTu_GNN/YiTu_H/xgnn_h/block.py:36-67                      */
 /* ------------------------------------------------------------------------- */
@@ -383,6 +494,59 @@ ORC_EXPORT int orc_stitch_csr(int n_blk, int64_t n_rows, const int32_t *const *i
 /* ------------------------------------------------------------------------- */
 /* B7/B8: two-way bundled GEMM. YiTu_GNN/YiTu_H/src/fc_cuda.cu                */
 /* ------------------------------------------------------------------------- */
+
+/*
+ * c[n,m] (+)= op(a) . op(b) in float on all cores, for timing only (the reference calls
+ * cuBLAS, fc_cuda.cu:61-69, 131, 178; torch::mm in YiTu_GNN_kernel.cu:276, 471-472).
+ * Row-major operands; ta / tb say whether a is stored [k,n] / b is stored [m,k]. Rows of
+ * c are dealt to the threads, the inner loops run over contiguous memory where the
+ * layout allows it, so that the compiler vectorises them.
+ */
+ORC_EXPORT void orc_gemm_f32_omp(float *c, const float *a, const float *b, int64_t n, int64_t m,
+                                 int64_t k, int ta, int tb)
+{
+    if (!ta) {
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n; i++) {
+            float *ci = c + i * m;
+            for (int64_t j = 0; j < m; j++) ci[j] = 0.0f;
+            if (!tb) {
+                for (int64_t t = 0; t < k; t++) {
+                    const float av = a[i * k + t];
+                    const float *bt = b + t * m;
+                    for (int64_t j = 0; j < m; j++) ci[j] += av * bt[j];
+                }
+            } else {
+                for (int64_t j = 0; j < m; j++) {
+                    const float *bj = b + j * k;
+                    float acc = 0.0f;
+                    for (int64_t t = 0; t < k; t++) acc += a[i * k + t] * bj[t];
+                    ci[j] = acc;
+                }
+            }
+        }
+        return;
+    }
+    /* a stored [k, n]: c = a^T . b, a sum over the k rows; threads own output rows in blocks
+       and walk k together so that every row of a and b is streamed once per block */
+#pragma omp parallel for schedule(static)
+    for (int64_t i0 = 0; i0 < n; i0 += 8) {
+        int64_t i1 = i0 + 8 < n ? i0 + 8 : n;
+        for (int64_t i = i0; i < i1; i++)
+            for (int64_t j = 0; j < m; j++) c[i * m + j] = 0.0f;
+        for (int64_t t = 0; t < k; t++) {
+            const float *bt = tb ? NULL : b + t * m;
+            for (int64_t i = i0; i < i1; i++) {
+                const float av = a[t * n + i];
+                float *ci = c + i * m;
+                if (bt)
+                    for (int64_t j = 0; j < m; j++) ci[j] += av * bt[j];
+                else
+                    for (int64_t j = 0; j < m; j++) ci[j] += av * b[j * k + t];
+            }
+        }
+    }
+}
 
 /* y[n,m] = x[n,k] . w[m,k]^T, double accumulate (fc_cuda.cu:61-69, batch member) */
 ORC_EXPORT void orc_gemm_nt_f64(float *y, const float *x, const float *w, int64_t n, int64_t m,

@@ -97,31 +97,4 @@ def powerlaw_graph(scale, m, seed):
     return graphgen.csr_by_destination(src, dst, 1 << scale)
 
 
-def dense_temporal_attention(layer, h, row, dt, n_dst, k_max):
-    """Dense masked attention with the layer's own parameters."""
-    dev = h.device
-    E = row.numel()
-    slot = torch.zeros(E, dtype=torch.long, device=dev)
-    counts = torch.bincount(row, minlength=n_dst)
-    start = torch.cumsum(counts, 0) - counts
-    slot = torch.arange(E, device=dev) - start[row]
-    mask = torch.zeros(n_dst, k_max, dtype=torch.bool, device=dev)
-    mask[row, slot] = True
-    te = torch.cos(dt[:, None] * layer.time_enc.w.weight[:, 0][None, :] + layer.time_enc.w.bias)
-    te0 = torch.cos(layer.time_enc.w.bias)[None, :].expand(n_dst, -1)
-    q = layer.w_q(torch.cat([h[:n_dst], te0], 1))
-    kv_in = torch.cat([h[n_dst:], te], 1)
-    k, v = layer.w_k(kv_in), layer.w_v(kv_in)
-    H, D = layer.num_head, layer.dim_out // layer.num_head
-    Kd = torch.zeros(n_dst, k_max, H, D, device=dev)
-    Vd = torch.zeros(n_dst, k_max, H, D, device=dev)
-    Kd[row, slot] = k.reshape(E, H, D)
-    Vd[row, slot] = v.reshape(E, H, D)
-    logits = torch.einsum("bhd,bkhd->bkh", q.reshape(n_dst, H, D), Kd)
-    logits = torch.nn.functional.leaky_relu(logits, 0.2)
-    logits = logits.masked_fill(~mask[:, :, None], float("-inf"))
-    att = torch.softmax(logits, dim=1)
-    att = torch.nan_to_num(att, nan=0.0)  # roots without neighbours
-    agg = torch.einsum("bkh,bkhd->bhd", att, Vd).reshape(n_dst, H * D)
-    out = layer.w_out(torch.cat([agg, h[:n_dst]], 1))
-    return layer.layer_norm(torch.relu(out))
+from oracle.temporal import dense_temporal_attention  # noqa: E402,F401  (dense masked attention)

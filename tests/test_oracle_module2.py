@@ -233,3 +233,55 @@ def test_stack_blocks_places_every_block_in_the_union_matrix():
     # no scales: unit weights
     _, ones = xblock.stack_blocks(blocks, row_off, col_off, n_rows, n_cols)
     assert torch.equal(ones, torch.ones_like(values))
+
+
+@pytest.mark.parametrize("n_dst,n_src,h,f,n_bid,seed", [(60, 45, 4, 8, 1, 0), (33, 70, 2, 5, 3, 1),
+                                                        (90, 90, 1, 16, 16, 2)])
+def test_all_core_float_builds_equal_the_serial_gradients(n_dst, n_src, h, f, n_bid, seed):
+    """The *_omp functions exist to be timed on all cores; they are the same sums as the
+    serial double-accumulate gradients they stand beside (by-source instead of scattered),
+    and the by-source view they walk is the stable sort on the column."""
+    indptr, indices = random_csr(n_dst, n_src, 0.15, seed, hub_rows=(3,), hub_degree=min(n_src, 40),
+                                 empty_rows=(0,))
+    rng = np.random.default_rng(seed)
+    ip, ix = indptr.numpy(), indices.numpy().copy()
+    ix |= (rng.integers(0, n_bid, ix.shape[0]).astype(np.int32) << 24)
+    # a stitched row lists its blocks in ascending tag order
+    for r in range(n_dst):
+        seg = ix[ip[r]:ip[r + 1]]
+        seg.sort()
+    t_indptr, t_rows, t_perm = tr = oracle.csr_transpose(ip, ix, n_src)
+    col = ix & 0xffffff
+    rows = np.repeat(np.arange(n_dst), np.diff(ip))
+    order = np.argsort(col, kind="stable")
+    assert np.array_equal(t_perm, order) and np.array_equal(t_rows, rows[order])
+    assert np.array_equal(np.diff(t_indptr), np.bincount(col, minlength=n_src))
+    values = rng.standard_normal((ix.shape[0], h)).astype(np.float32)
+    feat = rng.standard_normal((n_src, h, f)).astype(np.float32)
+    gy = rng.standard_normal((n_dst, h, f)).astype(np.float32)
+    ga, gx = oracle.mh_spmm_backward(values, ip, ix, feat, gy)
+    ga2, gx2 = oracle.mh_spmm_backward_omp(values, ip, ix, feat, gy, tr)
+    assert_close(ga2, ga)
+    assert_close(gx2, gx)
+    none_a, gx3 = oracle.mh_spmm_backward_omp(values, ip, ix, feat, gy, tr, need_grad_a=False)
+    assert none_a is None and np.array_equal(gx3, gx2)
+    q = rng.standard_normal((n_bid, n_dst, h)).astype(np.float32)
+    k = rng.standard_normal((n_src, h)).astype(np.float32)
+    attn = oracle.sddmm_forward(ip, ix, q, k)
+    g_attn = rng.standard_normal(attn.shape).astype(np.float32)
+    gq, gk = oracle.sddmm_backward(ip, ix, q, k, attn, g_attn)
+    gq2, gk2 = oracle.sddmm_backward_omp(ip, ix, q, k, attn, g_attn, tr)
+    # rows without an edge of a block keep grad_query 0 in both
+    assert_close(gq2, gq)
+    assert_close(gk2, gk)
+
+
+@pytest.mark.parametrize("n,m,k", [(37, 20, 13), (8, 64, 64), (1, 5, 9)])
+def test_all_core_float_gemm_equals_numpy(n, m, k):
+    rng = np.random.default_rng(n + m + k)
+    for ta in (False, True):
+        for tb in (False, True):
+            a = rng.standard_normal((k, n) if ta else (n, k)).astype(np.float32)
+            b = rng.standard_normal((m, k) if tb else (k, m)).astype(np.float32)
+            want = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+            assert_close(oracle.gemm_omp(a, b, ta, tb), want)
