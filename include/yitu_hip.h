@@ -341,6 +341,14 @@ int yitu_skinny_linear_backward(float *grad_x_device, int accumulate, float *gra
  * cleared accumulator, so the call can be recorded into a HIP graph and replayed.
  */
 size_t yitu_column_sum_workspace_bytes(int64_t n_rows, int64_t n_cols);
+/* The same for a list of short matrices x_i [n_rows_i, n_cols] (row stride ld floats) in one
+ * launch per 32 of them: out_i[j] = sum_r x_i[r, j], rows added by a fixed number of threads
+ * in a fixed order. The bias gradients of the per-relation Linears of a small heterogeneous
+ * graph (test/common/model.py:137-171 over :25-29); meant for matrices of up to a few thousand
+ * rows, longer ones take yitu_column_sum. out, x, n_rows are HOST arrays. */
+int yitu_column_sum_typed(float *const *out_device_ptrs, const float *const *x_device_ptrs,
+                          const int64_t *n_rows, int64_t n_problems, int64_t n_cols, int64_t ld,
+                          void *stream);
 int yitu_column_sum(float *out_device, const float *x_device, int64_t n_rows, int64_t n_cols,
                     void *workspace_device, size_t workspace_bytes, void *stream);
 
@@ -360,6 +368,7 @@ int yitu_column_sum(float *out_device, const float *x_device, int64_t n_rows, in
  * registers; a weight stored [k,n] is first
  * copied as [n,k] into the workspace when that is large enough.
  */
+/* n_problems: how many products a typed call brings (1 for a single product). */
 size_t yitu_sgemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t n_problems);
 int yitu_sgemm(float *c_device, const float *a_device, const float *b_device, int64_t m, int64_t n,
                int64_t k, int trans_a, int trans_b, int64_t lda, int64_t ldb, int64_t ldc,
@@ -378,10 +387,10 @@ int yitu_linear_forward(float *y_device, const float *x_device, const float *w_d
 /*
  * The same for the Linear layers of several node or edge types at once (the
  * per-relation loop of HeteroGraphConv, test/common/model.py:137-171, over layers
- * of model.py:25-29): y_i[m_i,n] = x_i[m_i,k] . w_i^T + bias_i for i < n_problems, eight
- * layers per launch. y, x, w, bias, m are HOST arrays (of device pointers and sizes); the
+ * of model.py:25-29): y_i[m_i,n] = x_i[m_i,k] . w_i^T + bias_i for i < n_problems, up to
+ * 32 layers per launch. y, x, w, bias, m are HOST arrays (of device pointers and sizes); the
  * bias table or single entries of it may be NULL. All y_i are contiguous (row stride n).
- * Workspace as for yitu_sgemm(max m_i, n, k, min(n_problems, 8)).
+ * Workspace: yitu_sgemm_workspace_bytes(max m_i, n, k, n_problems).
  */
 int yitu_linear_forward_typed(float *const *y, const float *const *x, const float *const *w,
                               const float *const *bias, const int64_t *m, int64_t n_problems,
@@ -389,7 +398,7 @@ int yitu_linear_forward_typed(float *const *y, const float *const *x, const floa
                               size_t workspace_bytes, void *stream);
 
 /*
- * Typed products in one launch per 8 problems: C_i[m_i,n] (+)= op(A_i)[m_i,k_i] .
+ * Typed products in one launch per 32 problems: C_i[m_i,n] (+)= op(A_i)[m_i,k_i] .
  * op(B_i)[k_i,n] for i < n_problems, with shared n, transposes and leading
  * dimensions. c, a, b, m, k are HOST arrays (of device pointers and sizes).
  * Replaces the loop of per-relation / per-type Linear layers of the
@@ -397,7 +406,7 @@ int yitu_linear_forward_typed(float *const *y, const float *const *x, const floa
  * its two gradient products): the row tiles of all node types fill the chip
  * together instead of one short launch after another. Workspace for the split
  * products (X_t^T . G_t): yitu_sgemm_workspace_bytes(max m_i, n, max k_i,
- * min(n_problems, 8)); the same workspace serves every group of 8.
+ * n_problems); the same workspace serves every group of 32.
  */
 int yitu_sgemm_typed(float *const *c_device_ptrs, const float *const *a_device_ptrs,
                      const float *const *b_device_ptrs, const int64_t *m, const int64_t *k,

@@ -423,3 +423,44 @@ def test_bundle_linear_matches_torch(dev, n, k, m, bias):
     want = [y2.detach(), x.grad, lin.weight.grad] + ([lin.bias.grad] if bias else [])
     for a, b in zip(got, want):
         assert_close(a, b, rtol=1e-4, atol=2e-4 * (n ** 0.5 if a.dim() < 2 or a.shape == lin.weight.shape else 1))
+
+
+def test_typed_products_of_forty_small_layers(dev):
+    """More layers than one launch takes (32), a few hundred rows each, outputs of 2 and of 32
+    columns: the per-relation Linears and attention projections of a small heterogeneous
+    graph. Forward with biases, both gradient products and the bias gradients in one
+    grouped call each, against float64."""
+    g = torch.Generator().manual_seed(77)
+    for n_out, k in ((32, 32), (2, 64), (4, 24)):
+        ms = [int(v) for v in torch.randint(0, 400, (40,), generator=g)]
+        ms[5] = 0
+        xs = [torch.randn(m, k, generator=g) for m in ms]
+        ws = [torch.randn(n_out, k, generator=g) for _ in ms]
+        bs = [torch.randn(n_out, generator=g) if i % 3 else None for i in range(len(ms))]
+        to = lambda ts: [None if t is None else t.to(dev) for t in ts]
+        got = graph_ext.linear_forward_typed(to(xs), to(ws), to(bs))
+        for x, w, b, y in zip(xs, ws, bs, got):
+            want = x.double() @ w.double().t() + (0 if b is None else b.double())
+            assert_close(y, want, abs_sum=x.double().abs() @ w.double().abs().t())
+        gys = [torch.randn(m, n_out, generator=g) for m in ms]
+        gx = graph_ext.sgemm_typed(to(gys), to(ws))
+        gw = graph_ext.sgemm_typed(to(gys), to(xs), trans_a=True)
+        for gy, x, w, dx, dw in zip(gys, xs, ws, gx, gw):
+            assert_close(dx, gy.double() @ w.double(), abs_sum=gy.double().abs() @ w.double().abs())
+            assert_close(dw, gy.double().t() @ x.double(),
+                         abs_sum=gy.double().abs().t() @ x.double().abs())
+        # bias gradients: row slices of one buffer, one launch per 32 of them
+        buf = torch.cat(gys).to(dev)
+        parts, off = [], 0
+        for m in ms:
+            parts.append(buf[off:off + m])
+            off += m
+        sums = graph_ext.column_sum_typed(parts)
+        for gy, s in zip(gys, sums):
+            assert_close(s, gy.double().sum(0), abs_sum=gy.double().abs().sum(0))
+        again = graph_ext.column_sum_typed(parts)
+        assert all(torch.equal(a, b) for a, b in zip(sums, again))
+    # long matrices take the two-stage sum of one matrix each
+    long_parts = [torch.randn(9000, 8, generator=g).to(dev), torch.randn(10, 8, generator=g).to(dev)]
+    for x, s in zip(long_parts, graph_ext.column_sum_typed(long_parts)):
+        assert_close(s, x.double().sum(0), abs_sum=x.double().abs().sum(0))

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     assert not missing, "declared but not exported: %s" % missing
     lib.yitu_abi_version.restype = ctypes.c_int
     from yitu_amd import _lib as binding
-    assert lib.yitu_abi_version() == binding.ABI_VERSION == 3
+    assert lib.yitu_abi_version() == binding.ABI_VERSION == 4
 
 
 def test_host_library_exports_every_declared_symbol():

@@ -293,3 +293,44 @@ def test_whole_embedding_table_is_aliased_only_under_autograd():
     assert executor._whole_table(shuffled, {}) is None
     executor.forget_tables()
     assert not executor._whole_tables
+
+
+@pytest.mark.parametrize("which", ["rgcn", "rgat"])
+def test_grouped_linears_equal_one_linear_at_a_time(which):
+    """The executor runs the Linears of one depth and one shape as one grouped node
+    (``Optimizer.group_linears``): same outputs and parameter gradients as one Linear at a
+    time, and the per-relation Linears of a layer do end up in few groups."""
+    hgraph = cases.hetero_graph()
+    kwargs = cases.hetero_kwargs(hgraph, with_norms=which == "rgcn")
+    torch.manual_seed(3)
+    model = models.RGCNModel(hgraph, 8, 8, 4) if which == "rgcn" else \
+        models.RGATModel(hgraph, 8, 8, 4, n_heads=2)
+    model.eval()
+    dataflow = xgnn_h.Module2IR().transform(model, kwargs)
+    grouped = xgnn_h.Optimizer.group_linears(dataflow)
+    n_linear = sum(1 for n in ir.walk(dataflow) if n.op == "linear")
+    typed = [n for n in ir.walk(grouped) if n.op == "typed_linear"]
+    left = sum(1 for n in ir.walk(grouped) if n.op == "linear")
+    assert typed and sum(len(t.inputs) for t in typed) + left == n_linear
+    assert len(typed) <= 8 and left <= 2  # a handful of launches for a dozen relations
+    for t in typed:
+        assert sorted(t.inputs) == sorted(str(i) for i in range(len(t.attrs["weights"])))
+        assert sum(t.attrs["split"]) == t.size[0]
+    params = list(model.parameters())
+    results = []
+    for flag in (False, True):
+        for p in params:
+            p.grad = None
+        executor = xgnn_h.Executor(group_linears=flag)
+        executor.eval()
+        out = executor.run(dataflow, kwargs)
+        sum((v * (i + 1.0)).sum() for i, v in enumerate(out.values())).backward()
+        results.append(({k: v.detach().clone() for k, v in out.items()},
+                        [None if p.grad is None else p.grad.clone() for p in params]))
+    (out_a, grads_a), (out_b, grads_b) = results
+    for k in out_a:
+        assert_close(out_b[k], out_a[k], rtol=1e-6, atol=1e-6)
+    for ga, gb in zip(grads_a, grads_b):
+        assert (ga is None) == (gb is None)
+        if ga is not None:
+            assert_close(gb, ga, rtol=1e-5, atol=1e-6)

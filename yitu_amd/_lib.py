@@ -18,7 +18,7 @@ _lock = threading.Lock()
 # The C ABI these bindings were written for (yitu_abi_version() of include/yitu_hip.h). A
 # library of another version has other argument lists: calling it would hand the kernels
 # shifted pointers, so it is refused at load time.
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 c_i64 = ctypes.c_int64
 c_int = ctypes.c_int

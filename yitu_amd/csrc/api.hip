@@ -10,7 +10,7 @@ using namespace yitu;
 #define YITU_API extern "C" __attribute__((visibility("default")))
 
 YITU_API const char *yitu_last_error(void) { return last_error(); }
-YITU_API int yitu_abi_version(void) { return 3; }
+YITU_API int yitu_abi_version(void) { return 4; }
 
 YITU_API size_t yitu_spmm_workspace_bytes(int64_t nnz, int64_t row_len, int with_plan) {
     return spmm_workspace_bytes(nnz, row_len, with_plan != 0);

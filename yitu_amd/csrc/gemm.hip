@@ -5,7 +5,7 @@
 //
 //   C[M,N] (+)= A[M,K] . B[K,N],  element (i,k) of A at A + i*a_si + k*a_sk,
 //                                  element (k,j) of B at B + k*b_sk + j*b_sj,
-// one of each stride pair being 1, C row-major. Up to 8 problems that share
+// one of each stride pair being 1, C row-major. Up to 32 problems that share
 // N and the strides, each with its own M and K, are grouped into one launch
 // (blockIdx.z walks the problems and their K splits).
 //
@@ -21,7 +21,7 @@
 namespace yitu {
 
 constexpr int BK = 16;  // K-step
-constexpr int kMaxGroup = 8;
+constexpr int kMaxGroup = 32;  // problems per launch (their table travels as kernel arguments)
 constexpr int kMinSplitK = 128;  // shortest K range worth a workgroup of its own
 
 typedef float float16v __attribute__((ext_vector_type(16)));
@@ -366,7 +366,7 @@ static int sgemm_launch(const GemmParams &p, int tile, int max_m, int n_z, hipSt
 }
 
 // ---- many rows, inner dimension 64 / 128 / 256: the weight stays in registers -------
-// C_q[M_q, N] = A_q[M_q, K] . B_q for up to 8 problems (node types). The 8 waves of a
+// C_q[M_q, N] = A_q[M_q, K] . B_q for up to 32 problems (node types, relations). The 8 waves of a
 // workgroup hold all of B_q[0 .. K, n0 .. n0 + 256) as MFMA operands (wave w keeps 32
 // columns: K / 2 steps x 1 register), the workgroup walks 32-row tiles of A and reads each
 // as whole rows, two tiles ahead through a ring of registers into a double-buffered LDS
@@ -970,6 +970,16 @@ __global__ __launch_bounds__(256) void bias_add_kernel(float *__restrict__ y,
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
         y[(i / n) * ldy + i % n] += bias[i % n];
 }
+// The same for every problem of a group in one launch (blockIdx.y = problem): the per-relation
+// Linears of a small heterogeneous graph are dozens of products of a few hundred rows.
+__global__ __launch_bounds__(256) void bias_add_group_kernel(GemmParams p) {
+    const GemmProblem &pr = p.prob[blockIdx.y];
+    if (!pr.bias) return;
+    const int n = p.N;
+    const int64_t total = (int64_t)pr.M * n, stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+        pr.C[(i / n) * p.ldc + i % n] += pr.bias[i % n];
+}
 }  // namespace yitu
 
 YITU_API int yitu_linear_forward(float *y, const float *x, const float *w, const float *bias,
@@ -1040,11 +1050,13 @@ YITU_API int yitu_linear_forward_typed(float *const *y, const float *const *x,
         const int rc = sgemm_grouped(p, false, true, (int)k, (int)k, workspace, workspace_bytes,
                                      stream);
         if (rc) return rc;
-        for (int i = 0; i < all.n_prob; i++) {
-            const GemmProblem &pr = all.prob[i];
-            if (!pr.bias) continue;
-            const int grid = (int)std::min<int64_t>(ceil_div((int64_t)pr.M * n, 256), 16384);
-            bias_add_kernel<<<grid, 256, 0, stream>>>(pr.C, pr.bias, pr.M, (int)n, n);
+        int64_t most = 0;
+        for (int i = 0; i < all.n_prob; i++)
+            if (all.prob[i].bias) most = std::max<int64_t>(most, (int64_t)all.prob[i].M * n);
+        if (most > 0) {
+            const dim3 grid((unsigned)std::min<int64_t>(ceil_div(most, 256), 16384),
+                            (unsigned)all.n_prob);
+            bias_add_group_kernel<<<grid, 256, 0, stream>>>(all);
             YITU_LAUNCH_CHECK();
         }
     }

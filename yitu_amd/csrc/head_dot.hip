@@ -671,6 +671,74 @@ __global__ __launch_bounds__(kBlock) void column_chunk_sum4_kernel(float *__rest
 }  // namespace
 }  // namespace yitu
 
+namespace yitu {
+namespace {
+// Column sums of up to 32 short matrices in one launch (blockIdx.y = matrix, blockIdx.x =
+// block of CB columns): the bias gradients of the per-relation Linears of a small
+// heterogeneous graph, where one launch pair per Linear costs more than the sums. A
+// thread adds every (256 / CB)-th row of its column, the thread sums are added in order.
+constexpr int kColSumGroup = 32;
+struct ColSumGroup {
+    const float *src[kColSumGroup];
+    float *out[kColSumGroup];
+    int rows[kColSumGroup];
+    int n_cols;
+    int64_t ld;
+};
+
+template <int CB>
+__global__ __launch_bounds__(kBlock) void column_sum_group_kernel(ColSumGroup g) {
+    constexpr int RG = kBlock / CB;
+    __shared__ float red[RG][CB];
+    const int q = blockIdx.y, c = threadIdx.x % CB, rg = threadIdx.x / CB;
+    const int j = blockIdx.x * CB + c;
+    const float *__restrict__ src = g.src[q];
+    float s = 0.0f;
+    if (j < g.n_cols)
+        for (int r = rg; r < g.rows[q]; r += RG) s += src[(size_t)r * g.ld + j];
+    red[rg][c] = s;
+    __syncthreads();
+    if (rg == 0 && j < g.n_cols) {
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < RG; k++) t += red[k][c];
+        g.out[q][j] = t;
+    }
+}
+}  // namespace
+}  // namespace yitu
+
+YITU_API int yitu_column_sum_typed(float *const *out, const float *const *x, const int64_t *n_rows,
+                                   int64_t n_problems, int64_t n_cols, int64_t ld, void *stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    YITU_REQUIRE(n_problems >= 0 && n_cols >= 0 && n_cols < (1 << 24) && ld >= n_cols,
+                 "size out of range");
+    if (n_problems == 0 || n_cols == 0) return 0;
+    YITU_REQUIRE(out && x && n_rows, "null problem table");
+    for (int64_t first = 0; first < n_problems; first += kColSumGroup) {
+        ColSumGroup g{};
+        const int count = (int)std::min<int64_t>(kColSumGroup, n_problems - first);
+        for (int i = 0; i < count; i++) {
+            const int64_t m = n_rows[first + i];
+            YITU_REQUIRE(m >= 0 && m < INT32_MAX && out[first + i] && (m == 0 || x[first + i]),
+                         "problem %d: null pointer or size out of range", (int)(first + i));
+            g.src[i] = x[first + i];
+            g.out[i] = out[first + i];
+            g.rows[i] = (int)m;
+        }
+        g.n_cols = (int)n_cols;
+        g.ld = ld;
+        if (n_cols <= 32)
+            column_sum_group_kernel<32><<<dim3((unsigned)ceil_div(n_cols, 32), (unsigned)count),
+                                          kBlock, 0, stream>>>(g);
+        else
+            column_sum_group_kernel<64><<<dim3((unsigned)ceil_div(n_cols, 64), (unsigned)count),
+                                          kBlock, 0, stream>>>(g);
+        YITU_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 YITU_API size_t yitu_column_sum_workspace_bytes(int64_t n_rows, int64_t n_cols) {
     return sizeof(float) * (size_t)std::max<int64_t>(ceil_div(n_rows, col_sum_chunk(n_rows)), 1) *
            (size_t)n_cols;

@@ -511,7 +511,7 @@ def linear_forward(x, weight, bias=None):
 
 def linear_forward_typed(x_list, weight_list, bias_list, out_list=None):
     """[x_i . weight_i^T + bias_i] for Linear layers that share both widths (the per-type
-    layers of a heterogeneous model), eight layers per launch. ``bias_list`` entries may be
+    layers of a heterogeneous model), up to 32 layers per launch. ``bias_list`` entries may be
     None. ``out_list``: contiguous [m_i, n] tensors to write (e.g. row slices of one buffer)."""
     import ctypes
     count = len(x_list)
@@ -537,7 +537,7 @@ def linear_forward_typed(x_list, weight_list, bias_list, out_list=None):
             if tuple(c.shape) != (m, n) or c.device != dev:
                 raise RuntimeError("out must be [%d, %d] on the operands' device" % (m, n))
     ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(
-        c_i64(max(ms)), c_i64(n), c_i64(k), c_i64(min(count, 8))), dev)
+        c_i64(max(ms)), c_i64(n), c_i64(k), c_i64(count)), dev)
     pointers = lambda ts: (ctypes.c_void_p * count)(
         *[(t.data_ptr() or None) if t is not None else None for t in ts])
     with torch.cuda.device(dev):
@@ -580,7 +580,7 @@ def sgemm(a, b, trans_a=False, trans_b=False, out=None):
 def sgemm_typed(a_list, b_list, trans_a=False, trans_b=False, out_list=None):
     """[op(a_i) . op(b_i)] for operand pairs that share the output width, the
     transposes and the row strides (the per-type Linear layers of a heterogeneous
-    model and their gradient products), eight products per launch so that the
+    model and their gradient products), up to 32 products per launch so that the
     row tiles of all types fill the chip together. ``out_list``: contiguous
     [m_i, n] tensors to write (e.g. row slices of one buffer)."""
     import ctypes
@@ -612,7 +612,7 @@ def sgemm_typed(a_list, b_list, trans_a=False, trans_b=False, out_list=None):
                 raise RuntimeError("out must be [%d, %d] on the operands' device" % (m, n))
     count = len(a_list)
     ws = _lib.workspace(_size_fn("yitu_sgemm_workspace_bytes")(
-        c_i64(max(ms)), c_i64(n), c_i64(max(ks)), c_i64(min(count, 8))), dev)
+        c_i64(max(ms)), c_i64(n), c_i64(max(ks)), c_i64(count)), dev)
     pointers = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() or None for t in ts])
     sizes = lambda v: (ctypes.c_int64 * count)(*v)
     with torch.cuda.device(dev):
@@ -1005,3 +1005,38 @@ def column_sum(x):
                                         c_size(ws.numel()), stream_ptr(dev))
     check(rc, "yitu_column_sum")
     return out
+
+
+COLUMN_SUM_TYPED_MAX_ROWS = 4096  # above this a matrix takes column_sum's two-stage form
+
+
+def column_sum_typed(x_list):
+    """``[x_i.sum(0)]`` for 2-D fp32 tensors of one width whose rows are one common stride
+    apart (row slices of one buffer): one launch per 32 of them when they are short (the bias
+    gradients of the per-relation Linears of a small heterogeneous graph), otherwise
+    ``column_sum`` each. Fixed summation order, no cleared accumulator."""
+    import ctypes
+    if not x_list:
+        return []
+    n = x_list[0].size(1)
+    ld = x_list[0].stride(0) if x_list[0].size(0) > 1 else n
+    short = True
+    for x in x_list:
+        if x.dtype != torch.float32 or x.dim() != 2 or not x.is_cuda or x.size(1) != n or \
+                (x.size(1) > 1 and x.stride(1) != 1):
+            raise RuntimeError("column_sum_typed takes 2-D fp32 GPU tensors of one width")
+        short = short and x.size(0) <= COLUMN_SUM_TYPED_MAX_ROWS and \
+            (x.size(0) <= 1 or x.stride(0) == ld)
+    if not short or ld < n:
+        return [column_sum(x.contiguous()) for x in x_list]
+    dev = x_list[0].device
+    count = len(x_list)
+    out = torch.empty((count, n), dtype=torch.float32, device=dev)
+    pointers = lambda ts: (ctypes.c_void_p * count)(*[t.data_ptr() or None for t in ts])
+    with torch.cuda.device(dev):
+        rc = _lib.lib().yitu_column_sum_typed(
+            pointers([out[i] for i in range(count)]), pointers(x_list),
+            (ctypes.c_int64 * count)(*[x.size(0) for x in x_list]), c_i64(count), c_i64(n),
+            c_i64(ld), stream_ptr(dev))
+    check(rc, "yitu_column_sum_typed")
+    return list(out.unbind(0))

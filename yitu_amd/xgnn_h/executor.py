@@ -21,7 +21,11 @@ def _fill(template, values):
 
 
 class Executor:
-    def __init__(self):
+    def __init__(self, group_linears: bool = True):
+        """``group_linears``: run the Linears of one depth and one shape as one grouped
+        launch (``Optimizer.group_linears``), decided once per dataflow."""
+        self._group_linears = group_linears
+        self._prepared = {}  # id(dataflow) -> (dataflow, the form that is evaluated, its order)
         self._is_training = None
         self._edge_values = {}  # edge_values node -> (state of its inputs, result, inputs)
         self._whole_tables = {}  # embedding node -> (state of its index tensor, is arange, tensor)
@@ -118,8 +122,15 @@ class Executor:
             return torch.cat(parts, dim=0) if op == "concat" else torch.stack(parts, dim=0)
         if op == "typed_linear":
             count = len(node.inputs)
-            return layers._TypedLinear.apply(count, *[v[str(i)] for i in range(count)],
-                                             *node.attrs["weights"], *node.attrs["biases"])
+            xs = [v[str(i)] for i in range(count)]
+            if all(x.is_cuda and x.dtype == torch.float32 for x in xs):
+                y = layers._TypedLinear.apply(count, *xs, *node.attrs["weights"],
+                                              *node.attrs["biases"])
+            else:  # host tensors: the same rows from torch
+                y = torch.cat([F.linear(x, w, b) for x, w, b in
+                               zip(xs, node.attrs["weights"], node.attrs["biases"])], dim=0)
+            # grouped Linears of a lowered model: every former Linear reads its own rows
+            return y.split(node.attrs["split"], dim=0) if "split" in node.attrs else y
         if op == "edge_values":
             # per-edge weights of a stitched block from the relations' row scales: constants
             # of the graph, so they are kept for as long as the same scale tensors come by
@@ -145,8 +156,15 @@ class Executor:
     def run(self, dataflow: ir.Dataflow, kwargs: dict):
         """Evaluates the root (or every root of a dict) of ``dataflow``; ``kwargs``
         are the model's arguments, plus ``stitch`` when the stitcher has run."""
+        kept = self._prepared.get(id(dataflow))
+        if kept is None or kept[0] is not dataflow:
+            from .optimizer import Optimizer
+            flow = Optimizer.group_linears(dataflow) if self._group_linears else dataflow
+            kept = (dataflow, flow, ir.walk(flow))
+            self._prepared[id(dataflow)] = kept
+        _, dataflow, order = kept
         values = {}
-        for node in ir.walk(dataflow):
+        for node in order:
             ins = {k: values[id(c)] for k, c in node.inputs.items()}
             values[id(node)] = self._eval(node, ins, kwargs)
         if isinstance(dataflow, ir.Node):

@@ -182,8 +182,11 @@ class _TypedLinear(torch.autograd.Function):
                                                         [xs[i].contiguous() for i in want],
                                                         trans_a=True)):
                 gw[i] = g
-        gb = [graph_ext.column_sum(gs[i])
-              if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i] else None for i in range(n)]
+        gb = [None] * n
+        want = [i for i in range(n) if ctx.has_bias[i] and ctx.needs_input_grad[1 + 2 * n + i]]
+        if want:
+            for i, g in zip(want, graph_ext.column_sum_typed([gs[i] for i in want])):
+                gb[i] = g
         return (None, *gx, *gw, *gb)
 
 

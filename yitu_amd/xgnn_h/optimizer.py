@@ -120,6 +120,76 @@ class Optimizer:
 
         return ir.rewrite(dataflow, rule)
 
+    # -- the Linears of one depth and one shape -> one grouped launch ---------
+    @staticmethod
+    def group_linears(dataflow: ir.Dataflow, min_group: int = 2) -> ir.Dataflow:
+        """A heterogeneous model applies one Linear per relation (model.py:137-171 over
+        :25-29, :70-71): at the scale of the reference's own benchmark that is a hundred
+        products of a few hundred rows, each a launch of its own forward and three more
+        backward. Linears (and the two halves of a ``bundle``) that sit at the same depth of
+        the dataflow cannot depend on each other; those of one weight shape become one
+        ``typed_linear`` node, a grouped GEMM launch that writes all their outputs into one
+        buffer, and every former Linear reads its rows back through one ``split`` (whose
+        backward is one concatenation of the incoming gradients). The executor applies this
+        to whatever dataflow it is given (lowered or stitched), once per dataflow."""
+        depth = {}
+        for node in ir.walk(dataflow):
+            depth[id(node)] = 1 + max([depth[id(c)] for c in node.inputs.values()], default=0)
+        # units: (key, original node, which weight of it)
+        groups = {}
+        for node in ir.walk(dataflow):
+            if node.op == "linear":
+                ws = [(node.attrs["weight"], node.attrs["bias"])]
+            elif node.op == "bundle":
+                ws = list(zip(node.attrs["weights"], node.attrs["biases"]))
+            else:
+                continue
+            x = node.inputs["x"]
+            if x.size is None or len(x.size) != 2 or any(w.dim() != 2 for w, _ in ws):
+                continue
+            for which, (w, _) in enumerate(ws):
+                key = (depth[id(node)], node.op, which, tuple(w.shape))
+                groups.setdefault(key, []).append(node)
+        place = {}  # (id(original node), which) -> (typed node, position in it)
+        for key, members in groups.items():
+            if len(members) < min_group:
+                continue
+            which = key[2]
+            sizes = [int(m.inputs["x"].size[0]) for m in members]
+            pick = (lambda m: (m.attrs["weight"], m.attrs["bias"])) if key[1] == "linear" else \
+                (lambda m: (m.attrs["weights"][which], m.attrs["biases"][which]))
+            typed = ir.Node("typed_linear", {},
+                            {"weights": [pick(m)[0] for m in members],
+                             "biases": [pick(m)[1] for m in members], "split": sizes},
+                            size=[sum(sizes), int(key[3][0])])
+            for i, m in enumerate(members):
+                place[(id(m), which)] = (typed, i)
+        if not place:
+            return dataflow
+
+        def piece(typed, i, size):
+            return ir.Node("select", {"x": typed}, {"index": i}, size)
+
+        def rule(node: ir.Node, original: ir.Node) -> ir.Node:
+            if original.op == "linear" and (id(original), 0) in place:
+                typed, i = place[(id(original), 0)]
+                typed.inputs[str(i)] = node.inputs["x"]
+                return piece(typed, i, node.size)
+            if original.op == "bundle":
+                # register the (rewritten) input with both typed nodes; readers follow below
+                for which in (0, 1):
+                    if (id(original), which) in place:
+                        typed, i = place[(id(original), which)]
+                        typed.inputs[str(i)] = node.inputs["x"]
+                return node
+            if original.op == "select" and original.inputs["x"].op == "bundle":
+                hit = place.get((id(original.inputs["x"]), original.attrs["index"]))
+                if hit is not None:
+                    return piece(hit[0], hit[1], node.size)
+            return node
+
+        return ir.rewrite(dataflow, rule)
+
     def lower(self, dataflow: ir.Dataflow, kwargs: dict = None) -> ir.Dataflow:
         dataflow = ir.rewrite(dataflow, self._lower_node)
         if self.fuse_gat:
