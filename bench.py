@@ -1065,22 +1065,6 @@ def run_c3_orders(args, dev):
     return res
 
 
-def planted_partition(n_comm, size, intra, inter, seed, dev):
-    """Planted-partition graph: n_comm communities of `size` vertices; every vertex draws
-    `intra` sources inside its community and `inter` anywhere. Ids as planted (a
-    community is a contiguous id block). Returns (src, dst) int64 on `dev`, self loops
-    included once per vertex."""
-    g = torch.Generator(device=dev).manual_seed(seed)
-    n = n_comm * size
-    dst = torch.arange(n, device=dev).repeat_interleave(intra)
-    base = dst // size * size
-    src = base + torch.randint(0, size, (n * intra,), generator=g, device=dev)
-    dst2 = torch.arange(n, device=dev).repeat_interleave(inter)
-    src2 = torch.randint(0, n, (n * inter,), generator=g, device=dev)
-    loop = torch.arange(n, device=dev)
-    return torch.cat([src, src2, loop]), torch.cat([dst, dst2, loop])
-
-
 def run_planted_orders(args, dev):
     """The reorder on a graph it can help: a planted-partition graph of the third
     configuration's size (2^21 vertices, about 30 sources per vertex, 28 of them inside
@@ -1092,7 +1076,7 @@ def run_planted_orders(args, dev):
     from yitu_amd.data import graphgen
     n_comm, size = 4096, 512
     n = n_comm * size
-    src, dst = planted_partition(n_comm, size, 28, 2, 20244, dev)
+    src, dst = graphgen.planted_partition(n_comm, size, 28, 2, 20244, dev)
     g = torch.Generator(device=dev).manual_seed(20244)
     x = torch.randn(n, 128, generator=g, device=dev)
     res = {"n_nodes": n, "communities": n_comm, "community_size": size}

@@ -86,3 +86,19 @@ def bipartite_uniform(n_dst, n_src, avg_degree, seed, device="cpu"):
     rows = torch.repeat_interleave(torch.arange(n_dst, device=device), cnt)
     cols = torch.randint(0, n_src, (int(cnt.sum()),), generator=g, device=device)
     return csr_from_edges(rows, cols, n_dst, n_src)
+
+
+def planted_partition(n_comm, size, intra, inter, seed, device="cpu"):
+    """Planted-partition graph: n_comm communities of `size` vertices; every vertex draws
+    `intra` sources inside its community and `inter` anywhere. Ids as planted (a
+    community is a contiguous id block). Returns (src, dst) int64 on `device`, self loops
+    included once per vertex."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    n = n_comm * size
+    dst = torch.arange(n, device=device).repeat_interleave(intra)
+    base = dst // size * size
+    src = base + torch.randint(0, size, (n * intra,), generator=g, device=device)
+    dst2 = torch.arange(n, device=device).repeat_interleave(inter)
+    src2 = torch.randint(0, n, (n * inter,), generator=g, device=device)
+    loop = torch.arange(n, device=device)
+    return torch.cat([src, src2, loop]), torch.cat([dst, dst2, loop])
