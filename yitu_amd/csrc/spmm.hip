@@ -158,16 +158,6 @@ int launch_spmm(SpmmParams &p, int wmode, bool bf16_in, int64_t nnz, int64_t max
                           p.col_mask, max_degree_hint, workspace, workspace_bytes, &rest,
                           &rest_bytes, stream);
     if (rc) return rc;
-    // rows that are whole 16-byte units and a table below 2^32 units (64 GB): the 16-byte
-    // gathers address rows by 32-bit unit offsets
-    {
-        const int64_t row_bytes = (int64_t)p.L * (bf16_in ? 2 : 4);
-        p.row16 = 0;
-        if (row_bytes % 16 == 0 && aligned16(p.feat) &&
-            (int64_t)std::max(p.n_src, 1) * (row_bytes / 16) < ((int64_t)1 << 32) &&
-            (!p.cols_are_edges || nnz * (row_bytes / 16) < ((int64_t)1 << 32)))
-            p.row16 = (int)(row_bytes / 16);
-    }
     p.partial = nullptr;
     if (with_hub) {
         const size_t need = sizeof(float) * (size_t)p.plan.max_items * (size_t)p.L;

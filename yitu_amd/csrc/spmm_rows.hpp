@@ -49,9 +49,6 @@ struct SpmmParams {
     float alpha;   // output scale
     int out_bf16;  // nonzero: the output rows are bf16 (round to nearest even); partial rows
                    // stay fp32. Taken by the row / item / reduce kernels of this file.
-    int row16;     // > 0: a feature row is row16 units of 16 bytes and n_src * row16 < 2^32, so the
-                   // kernels whose lanes load 16 bytes address a row by its 32-bit unit offset
-                   // (set by launch_spmm; 0 = 64-bit element offsets)
     PlanView plan;   // long rows: band-ordered 64-edge items (plan.threshold = INT_MAX: none)
     float *partial;  // [plan item id, L] unscaled partial rows of multi-item rows
 };
@@ -93,7 +90,6 @@ struct EdgeWindow {
     int col;
     float w;
     int vrow;
-    uint32_t rofs;  // col * p.row16: where the edge's feature row starts, in 16-byte units
 };
 
 // Loads edges [base, base + 64) clipped to `limit` (exclusive). Lanes past the
@@ -110,8 +106,6 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
     if constexpr (WMODE == W_DEGPROD)
         win.w = p.edge_scale ? __builtin_nontemporal_load(p.edge_scale + e) : p.scale_col[win.col];
     if constexpr (WMODE == W_EDGEHEAD) win.vrow = p.eperm ? __builtin_nontemporal_load(p.eperm + e) : e;
-    // one multiplication per edge here instead of a 64-bit one per edge and lane at the gather
-    win.rofs = (uint32_t)win.col * (uint32_t)p.row16;
 }
 
 // One step of the edge loop: every slot of the wave picks its edge
@@ -157,52 +151,6 @@ __device__ __forceinline__ void gather_step(float (&v)[KT][VEC], float (&w)[KT],
     }
 }
 
-// The same step for lanes that load 16 bytes when rows can be addressed in 16-byte units
-// (p.row16 > 0): the row's unit offset comes out of the window ready made, the lane's
-// own byte offset sits in `base`, so an address costs one shift-and-add. FULL: every
-// slot of the step has an edge (k < n), so nothing is clamped or masked. Lanes past the
-// end of a row (tiles wider than the row) read the row's start and are never stored.
-template <int VEC, int G, int KT, int WMODE, typename TIN, bool FULL>
-__device__ __forceinline__ void gather_units(float (&v)[KT][VEC], float (&w)[KT],
-                                             const SpmmParams &p, const char *const (&base)[KT],
-                                             const EdgeWindow &win, int first, int step, int n,
-                                             const int (&head)[KT]) {
-    constexpr int SLOTS = kWave / G;
-    uint32_t ro;
-    int vrow = 0;
-    float ws = 0.0f;
-    bool valid = true;
-    if constexpr (SLOTS == 1) {
-        const int src = first + step;
-        ro = (uint32_t)__builtin_amdgcn_readlane((int)win.rofs, src);
-        if constexpr (WMODE == W_EDGEHEAD)
-            vrow = __builtin_amdgcn_readlane(win.vrow, src);
-        else
-            ws = __builtin_bit_cast(float,
-                                    __builtin_amdgcn_readlane(__builtin_bit_cast(int, win.w), src));
-    } else {
-        const int k = step + lane_id() / G;
-        int src = first + k;
-        if constexpr (!FULL) {
-            valid = k < n;
-            src = first + min(k, n - 1);
-        }
-        ro = (uint32_t)__shfl((int)win.rofs, src, kWave);
-        if constexpr (WMODE == W_EDGEHEAD)
-            vrow = __shfl(win.vrow, src, kWave);
-        else
-            ws = __shfl(win.w, src, kWave);
-    }
-#pragma unroll
-    for (int t = 0; t < KT; t++) {
-        if constexpr (WMODE == W_EDGEHEAD)
-            w[t] = valid ? p.values[(size_t)vrow * p.H + head[t]] : 0.0f;
-        else
-            w[t] = valid ? ws : 0.0f;
-        RowLoad<VEC, TIN>::ld(reinterpret_cast<const TIN *>(base[t] + ((size_t)ro << 4)), v[t]);
-    }
-}
-
 // Column-tile geometry of this lane for the tile that starts at element c0.
 template <int VEC, int G, int KT, int WMODE>
 struct TileLanes {
@@ -228,54 +176,10 @@ struct TileLanes {
 template <int VEC, int G, int KT, int WMODE, typename TIN,
           int UNROLL = ((KT >= 4 || G <= 16) ? 2 : ((G == kWave && KT == 1) ? 8 : 4))>
 __device__ __forceinline__ void accumulate_window(float (&acc)[KT][VEC], const SpmmParams &p,
-                                                  const EdgeWindow &win, int first_, int n_,
+                                                  const EdgeWindow &win, int first, int n,
                                                   const TileLanes<VEC, G, KT, WMODE> &tl) {
     constexpr int SLOTS = kWave / G;
-    // the same in every lane, but usually the result of a lane shuffle: as scalars they
-    // make the step loop a scalar loop instead of one under a lane mask
-    const int first = __builtin_amdgcn_readfirstlane(first_);
-    const int n = __builtin_amdgcn_readfirstlane(n_);
     const TIN *__restrict__ feat = static_cast<const TIN *>(p.feat);
-    if constexpr (VEC * sizeof(TIN) == 16) {
-        if (p.row16 > 0) {  // the same for the whole launch
-            const char *base[KT];
-#pragma unroll
-            for (int t = 0; t < KT; t++)
-                base[t] = reinterpret_cast<const char *>(feat + tl.off[t]);
-            int s = 0;
-            for (; s + SLOTS * UNROLL <= n; s += SLOTS * UNROLL) {
-                float v[UNROLL][KT][VEC];
-                float w[UNROLL][KT];
-#pragma unroll
-                for (int u = 0; u < UNROLL; u++)
-                    gather_units<VEC, G, KT, WMODE, TIN, true>(v[u], w[u], p, base, win, first,
-                                                               s + u * SLOTS, n, tl.head);
-#pragma unroll
-                for (int u = 0; u < UNROLL; u++)
-#pragma unroll
-                    for (int t = 0; t < KT; t++)
-#pragma unroll
-                        for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
-            }
-            if (s < n) {
-                float v[UNROLL][KT][VEC];
-                float w[UNROLL][KT];
-#pragma unroll
-                for (int u = 0; u < UNROLL; u++)
-                    if (s + u * SLOTS < n)  // wave-uniform
-                        gather_units<VEC, G, KT, WMODE, TIN, false>(v[u], w[u], p, base, win, first,
-                                                                    s + u * SLOTS, n, tl.head);
-#pragma unroll
-                for (int u = 0; u < UNROLL; u++)
-                    if (s + u * SLOTS < n)
-#pragma unroll
-                        for (int t = 0; t < KT; t++)
-#pragma unroll
-                            for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
-            }
-            return;
-        }
-    }
     // full groups of UNROLL steps: all gathers of a group are issued before any FMA
     int s = 0;
     for (; s + SLOTS * UNROLL <= n; s += SLOTS * UNROLL) {
