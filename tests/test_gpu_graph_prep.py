@@ -70,7 +70,7 @@ def test_forget_after_a_raw_pointer_refill(dev):
     on another stream waits for the build."""
     import oracle
     from helpers import assert_close, powerlaw_graph
-    from yitu_amd import _lib, graph_ext
+    from yitu_amd import graph_ext
     n = 1 << 12
     ip_a, ix_a = powerlaw_graph(12, 60000, 1)
     ip_b, ix_b = powerlaw_graph(12, 60000, 2)
