@@ -823,6 +823,14 @@ def _c4_module_ms(sizes, rels, dim, dev, steps, warm):
     executor.train()
     res["reference_model_2_layers_lowered_fwd_bwd_ms"] = _event_ms(
         train_step(lambda: executor.run(lowered, kwargs), list(model.parameters())), steps, warm)
+    # the same with the node ids in a random order: the embedding tables are then gathered
+    # row by row (and their gradients sorted and summed) instead of being passed on whole
+    gp = torch.Generator(device=dev).manual_seed(11)
+    shuffled = dict(kwargs, xs={n: torch.randperm(c, generator=gp, device=dev)
+                                for n, c in ntypes.items()})
+    res["reference_model_2_layers_lowered_shuffled_ids_fwd_bwd_ms"] = _event_ms(
+        train_step(lambda: executor.run(lowered, shuffled), list(model.parameters())), steps, warm)
+    del shuffled
     stitched_flow = xgnn_h.Stitcher().transform(lowered, kwargs)
     res["reference_model_2_layers_stitched_fwd_bwd_ms"] = _event_ms(
         train_step(lambda: executor.run(stitched_flow, kwargs), list(model.parameters())), steps, warm)
