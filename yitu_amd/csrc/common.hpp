@@ -53,6 +53,22 @@ __device__ __forceinline__ float bf16_hi(uint32_t packed) {
     return __uint_as_float(packed & 0xffff0000u);
 }
 
+// Lane exchanges of the gfx950 vector ALU (no trip through the LDS unit). For two
+// registers a, b: pair_sum32 leaves a[l] + a[l + 32] in the lower half of the wave and
+// b[l - 32] + b[l] in the upper half; pair_sum16 leaves, in the four quarters of the
+// wave, a(q0) + a(q1), b(q0) + b(q1), a(q2) + a(q3), b(q2) + b(q3). One exchange and
+// one add thus fold two values at once, each half (quarter pair) keeping one of them.
+__device__ __forceinline__ float pair_sum32(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false,
+                                                    false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float pair_sum16(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false,
+                                                    false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // ---- vector loads: VEC consecutive elements of a feature row -> fp32 -------
 template <int VEC, typename T>
 struct RowLoad;
@@ -142,6 +158,10 @@ __device__ __forceinline__ void store_row_streaming(float *p, const float (&v)[V
             f4 t = {v[i], v[i + 1], v[i + 2], v[i + 3]};
             __builtin_nontemporal_store(t, reinterpret_cast<f4 *>(p + i));
         }
+    } else if constexpr (VEC == 2) {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        f2 t = {v[0], v[1]};
+        __builtin_nontemporal_store(t, reinterpret_cast<f2 *>(p));
     } else {
 #pragma unroll
         for (int i = 0; i < VEC; i++) __builtin_nontemporal_store(v[i], p + i);

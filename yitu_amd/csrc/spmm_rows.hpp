@@ -227,6 +227,31 @@ __device__ __forceinline__ void fold_slots(float (&acc)[KT][VEC]) {
             for (int i = 0; i < VEC; i++) acc[t][i] += __shfl_xor(acc[t][i], o, kWave);
 }
 
+// The same fold for one tile, shared out: the SLOTS partial rows are added in the same
+// pairs as in fold_slots (the same bits), but every slot ends up with its own VEC / SLOTS
+// consecutive elements of the lane's VEC, r[] = elements [slot * OUT, (slot + 1) * OUT).
+// Half the exchanges and adds (two values per exchange), no LDS permutes, and the row is
+// then stored by all 64 lanes.
+template <int VEC, int G>
+__device__ __forceinline__ void fold_scatter(const float (&a)[VEC],
+                                             float (&r)[VEC / (kWave / G)]) {
+    static_assert(G == 16 || G == 32 || G == kWave, "lanes per row");
+    static_assert(VEC % (kWave / G) == 0, "every slot keeps a whole number of elements");
+    if constexpr (G == kWave) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) r[i] = a[i];
+    } else if constexpr (G == 32) {
+#pragma unroll
+        for (int i = 0; i < VEC / 2; i++) r[i] = pair_sum32(a[i], a[i + VEC / 2]);
+    } else {
+        float u[VEC / 2];
+#pragma unroll
+        for (int i = 0; i < VEC / 2; i++) u[i] = pair_sum32(a[i], a[i + VEC / 2]);
+#pragma unroll
+        for (int j = 0; j < VEC / 4; j++) r[j] = pair_sum16(u[j], u[j + VEC / 4]);
+    }
+}
+
 constexpr int kRowsPerWave = 4;  // most consecutive rows one wave of a row kernel handles
 
 // Rows per wave of the row kernels: 4 where that still leaves several thousand
@@ -303,16 +328,29 @@ __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, i
                     load_window<WMODE>(win, p, b, limit);
                 accumulate_window<VEC, G, KT, WMODE, TIN>(acc, p, win, b - win.base, n, tl);
             }
-            if (deg > 0) fold_slots<VEC, G, KT>(acc);
-            if (slot == 0) {
+            if constexpr (G < kWave && KT == 1) {
+                constexpr int OUT = VEC / (kWave / G);
+                float r[OUT];
 #pragma unroll
-                for (int t = 0; t < KT; t++) {
-                    const int o = c0 + (t * G + sub) * VEC;
-                    if (o < p.L) {
-                        float r[VEC];
+                for (int k = 0; k < OUT; k++) r[k] = 0.0f;
+                if (deg > 0) fold_scatter<VEC, G>(acc[0], r);
+                if (c0 + sub * VEC < p.L) {
 #pragma unroll
-                        for (int k = 0; k < VEC; k++) r[k] = acc[t][k] * sr;
-                        store_out<VEC>(p, (size_t)row * p.L + o, r);
+                    for (int k = 0; k < OUT; k++) r[k] *= sr;
+                    store_out<OUT>(p, (size_t)row * p.L + c0 + sub * VEC + slot * OUT, r);
+                }
+            } else {
+                if (deg > 0) fold_slots<VEC, G, KT>(acc);
+                if (slot == 0) {
+#pragma unroll
+                    for (int t = 0; t < KT; t++) {
+                        const int o = c0 + (t * G + sub) * VEC;
+                        if (o < p.L) {
+                            float r[VEC];
+#pragma unroll
+                            for (int k = 0; k < VEC; k++) r[k] = acc[t][k] * sr;
+                            store_out<VEC>(p, (size_t)row * p.L + o, r);
+                        }
                     }
                 }
             }
@@ -359,12 +397,25 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
 #pragma unroll
                 for (int i = 0; i < VEC; i++) acc[t][i] = 0.0f;
             accumulate_window<VEC, G, KT, WMODE, TIN>(acc, p, win[j], 0, n_edges[j], tl);
-            fold_slots<VEC, G, KT>(acc);
             const bool single = row_tag[j] < 0;
             const int row = row_tag[j] & 0x7fffffff;
             float *dst = p.partial + (size_t)item_id[j] * p.L;  // not for single items
             const float sr =
                 single ? (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha : 1.0f;
+            if constexpr (G < kWave && KT == 1) {
+                constexpr int OUT = VEC / (kWave / G);
+                float r[OUT];
+                fold_scatter<VEC, G>(acc[0], r);
+                if (c0 + sub * VEC < p.L) {
+                    const int o = c0 + sub * VEC + slot * OUT;
+#pragma unroll
+                    for (int i = 0; i < OUT; i++) r[i] *= sr;
+                    if (single) store_out<OUT>(p, (size_t)row * p.L + o, r);
+                    else store_row_streaming<OUT>(dst + o, r);
+                }
+                continue;
+            }
+            fold_slots<VEC, G, KT>(acc);
             if (slot == 0) {
 #pragma unroll
                 for (int t = 0; t < KT; t++) {
