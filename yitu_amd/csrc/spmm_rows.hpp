@@ -292,13 +292,17 @@ __device__ __forceinline__ int row_block(const SpmmParams &p, int block, int n_b
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, int n_blocks) {
     const int lane = lane_id();
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int rpw = rows_per_wave(p.n_rows);
     const int r0 = (row_block(p, block, n_blocks) * kWavesPerBlock + wave) * rpw;
     if (r0 >= p.n_rows) return;
     const int n_here = min(rpw, p.n_rows - r0);
     const int my_ptr = p.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);  // end of this wave's edges
+    // the rows' scales with the same round trip as their bounds (a load per row, placed
+    // where the scale is first named, would be waited for before the row's gathers)
+    float my_scale = 1.0f;
+    if constexpr (WMODE == W_DEGPROD) my_scale = p.scale_row[r0 + min(lane, n_here - 1)];
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);  // end of this wave's edges
     const int sub = lane % G;
     const int slot = lane / G;
 
@@ -310,11 +314,13 @@ __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, i
 
     for (int i = 0; i < n_here; i++) {
         const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave);
-        const int end = __shfl(my_ptr, i + 1, kWave);
+        // (scalar reads: the row's bounds and loops stay off the vector ALU)
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i);
+        const int end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         const int deg = end - beg;
         if (deg >= p.plan.threshold) continue;  // a planned row: written by the item kernels
-        const float sr = (WMODE == W_DEGPROD ? p.scale_row[row] : 1.0f) * p.alpha;
+        const float sr = __builtin_bit_cast(float, __builtin_amdgcn_readlane(
+                             __builtin_bit_cast(int, my_scale), i)) * p.alpha;
         for (int c0 = 0; c0 < p.L; c0 += G * VEC * KT) {
             const TileLanes<VEC, G, KT, WMODE> tl(p, c0);
             float acc[KT][VEC];
