@@ -385,10 +385,10 @@ __device__ __forceinline__ void spmm_item_group(const SpmmParams &p, int pos0, i
     int item_id[IPW], n_edges[IPW], row_tag[IPW];
 #pragma unroll
     for (int j = 0; j < IPW; j++) {
-        const int beg = __shfl(my_rec.x, j, kWave);
-        const int end = __shfl(my_rec.y, j, kWave);
-        item_id[j] = __shfl(my_rec.z, j, kWave);
-        row_tag[j] = __shfl(my_rec.w, j, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_rec.x, j);
+        const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+        item_id[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+        row_tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
         n_edges[j] = j < n_here ? end - beg : 0;
         if (n_edges[j] > 0) load_window<WMODE>(win[j], p, beg, end);
     }
@@ -448,7 +448,8 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
     const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
     const int n_groups = (n_items + IPW - 1) / IPW;
     const int stride = gridDim.x * kWavesPerBlock;
-    for (int grp = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; grp < n_groups; grp += stride)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    for (int grp = blockIdx.x * kWavesPerBlock + wave; grp < n_groups; grp += stride)
         spmm_item_group<VEC, G, KT, WMODE, TIN, IPW>(p, grp * IPW,
                                                 min(IPW, n_items - grp * IPW));
 }
