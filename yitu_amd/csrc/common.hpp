@@ -170,6 +170,11 @@ __device__ __forceinline__ void store_row_streaming(float *p, const float (&v)[V
 
 // ---- wave64 helpers ---------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+// The wave's index in its workgroup as a scalar: what is derived from it (row ranges,
+// loop bounds) then stays in scalar registers and scalar branches.
+__device__ __forceinline__ int wave_id() {
+    return __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+}
 
 // Sum over the lanes whose ids differ only in bits >= log2(stride): the
 // butterfly leaves every lane with the total of its residue class mod stride.

@@ -106,18 +106,18 @@ template <int VEC, int G, int KT>
 __device__ __forceinline__ void dot_rows_body(const DotParams &p, int block) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (block * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (block * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     EdgeWindow win;
     win.base = -1;
     win.col = 0;
     win.w = 0.0f;
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         if (end == beg || end - beg >= p.sp.plan.threshold) continue;
         for (int c0 = 0; c0 < p.sp.L; c0 += G * VEC * KT) {
             const TileLanes<VEC, G, KT, W_EDGEHEAD> tl(p.sp, c0);

@@ -137,11 +137,11 @@ template <int VEC, int G, int KT>
 __global__ __launch_bounds__(kBlock) void gat_rows_kernel(GatParams p) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     const int sub = lane % G, slot = lane / G;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H, L = p.sp.L;
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kBlock) void gat_rows_kernel(GatParams p) {
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
         const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         const int deg = end - beg;
         if (deg >= p.sp.plan.threshold) continue;
         float qv = 0.0f, m = 0.0f, inv = 0.0f;
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_stats_kernel(GatParams p) {
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -218,9 +218,9 @@ __global__ __launch_bounds__(kBlock) void gat_item_stats_kernel(GatParams p) {
         float qv[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            const int beg = __shfl(my_rec.x, j, kWave), end = __shfl(my_rec.y, j, kWave);
-            item[j] = __shfl(my_rec.z, j, kWave);
-            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            const int beg = __builtin_amdgcn_readlane(my_rec.x, j), end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            const int row = __builtin_amdgcn_readlane(my_rec.w, j) & 0x7fffffff;
             n[j] = j < n_here ? end - beg : 0;
             qv[j] = 0.0f;
             if (n[j] > 0) {
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kBlock) void gat_row_combine_kernel(GatParams p) {
     // one wave per planned row: lane = (item slot, head), merged by a fixed butterfly
     const int hl = lane & (p.HP - 1), c0 = lane / p.HP, step = kWave / p.HP;
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int slot = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; slot < n_rows;
+    for (int slot = blockIdx.x * kWavesPerBlock + wave_id(); slot < n_rows;
          slot += n_waves) {
         const int4 r = p.sp.plan.rows[slot];
         MaxSum a = ms_init();
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_apply_kernel(GatParams p) {
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H, L = p.sp.L;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -286,10 +286,10 @@ __global__ __launch_bounds__(kBlock) void gat_item_apply_kernel(GatParams p) {
             row_tag[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            e_beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item_id[j] = __shfl(my_rec.z, j, kWave);
-            row_tag[j] = __shfl(my_rec.w, j, kWave);
+            e_beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item_id[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            row_tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
             n_edges[j] = j < n_here ? end - e_beg[j] : 0;
             if (n_edges[j] > 0) load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
         }
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_kernel(GatParams p) {
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H, L = p.sp.L;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -353,10 +353,10 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_kernel(GatParams p) {
         float qv[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            e_beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item_id[j] = __shfl(my_rec.z, j, kWave);
-            row_tag[j] = __shfl(my_rec.w, j, kWave);
+            e_beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item_id[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            row_tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
             n_edges[j] = j < n_here ? end - e_beg[j] : 0;
             qv[j] = 0.0f;
             if (n_edges[j] > 0) {
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
     const int hl = lane & (HP - 1), esub = lane / HP;
     const int H = p.sp.H, L = p.sp.L;
     const float *__restrict__ feat = static_cast<const float *>(p.sp.feat);
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kLocalItems;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kLocalItems;
          pos0 < n_items; pos0 += n_waves * kLocalItems) {
         const int n_here = min(kLocalItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -590,7 +590,7 @@ __global__ __launch_bounds__(kBlock) void gat_scaled_reduce_kernel(GatParams p) 
         const int slots = kWave / lanes;
         const int slot = lane / lanes, sub = lane % lanes;
         const int stride = half * kWavesPerBlock;
-        for (int h = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; h < n_hub; h += stride) {
+        for (int h = blockIdx.x * kWavesPerBlock + wave_id(); h < n_hub; h += stride) {
             const int4 r = p.sp.plan.rows[h];
             if (r.z <= 1 || r.z > kReduceWaveItems) continue;
             for (int l0 = 0; l0 < lanes_total; l0 += lanes) {
@@ -680,7 +680,7 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_combine_kernel(GatBwdParams p)
     const int H = p.sp.H;
     const int h = lane & (p.HP - 1), c0 = lane / p.HP, step = kWave / p.HP;
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int slot = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave; slot < n_rows;
+    for (int slot = blockIdx.x * kWavesPerBlock + wave_id(); slot < n_rows;
          slot += n_waves) {
         const int4 r = p.sp.plan.rows[slot];
         float s = 0.0f, a1 = 0.0f, a2 = 0.0f;
@@ -712,7 +712,7 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_apply_kernel(GatBwdParams p) {
     const int H = p.sp.H;
     const int hl = lane & (p.HP - 1), esub = lane / p.HP, eps = kWave / p.HP;
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -721,9 +721,9 @@ __global__ __launch_bounds__(kBlock) void gat_bwd_apply_kernel(GatBwdParams p) {
         float qv[kItemsPerWave], S[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            const int row = __builtin_amdgcn_readlane(my_rec.w, j) & 0x7fffffff;
             n[j] = j < n_here ? end - beg[j] : 0;
             qv[j] = S[j] = 0.0f;
             if (n[j] > 0) {
@@ -794,11 +794,11 @@ __device__ __forceinline__ void attn_write_window(const GatParams &p, const Edge
 __global__ __launch_bounds__(kBlock) void attn_rows_kernel(GatParams p) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
     EdgeWindow win;
@@ -807,7 +807,7 @@ __global__ __launch_bounds__(kBlock) void attn_rows_kernel(GatParams p) {
     win.w = 0.0f;
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         const int n = end - beg;
         if (n == 0 || n >= p.sp.plan.threshold) continue;
         const float qv = hl < H ? p.query[(size_t)(r0 + i) * H + hl] : 0.0f;
@@ -841,7 +841,7 @@ __global__ __launch_bounds__(kBlock) void attn_item_write_kernel(GatParams p) {
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -850,9 +850,9 @@ __global__ __launch_bounds__(kBlock) void attn_item_write_kernel(GatParams p) {
         float qv[kItemsPerWave], m[kItemsPerWave], inv[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            const int row = __builtin_amdgcn_readlane(my_rec.w, j) & 0x7fffffff;
             n[j] = j < n_here ? end - beg[j] : 0;
             qv[j] = m[j] = inv[j] = 0.0f;
             if (n[j] > 0) {
@@ -945,11 +945,11 @@ __device__ __forceinline__ void attn_bwd_reduce(float &S, float &A1, float &A2, 
 __global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
     EdgeWindow win;
@@ -959,7 +959,7 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_rows_kernel(GatBwdParams p) {
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
         const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         const int n = end - beg;
         if (n >= p.sp.plan.threshold) continue;
         if (n == 0) {
@@ -1000,7 +1000,7 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int hl = lane & (p.HP - 1);
     const int H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -1009,10 +1009,10 @@ __global__ __launch_bounds__(kBlock) void attn_bwd_item_sums_kernel(GatBwdParams
         float qv[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item[j] = __shfl(my_rec.z, j, kWave);
-            const int row = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            const int row = __builtin_amdgcn_readlane(my_rec.w, j) & 0x7fffffff;
             n[j] = j < n_here ? end - beg[j] : 0;
             qv[j] = 0.0f;
             if (n[j] > 0) {
@@ -1090,7 +1090,7 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float4 *__restrict_
     constexpr int HPT = kWave / LPH, H = HPT * KT, L = 256 * KT, U = KT == 1 ? 4 : 2;
     const int lane = lane_id();
     const int g_lane = (head_mean ? lane % LPH : lane) * 4, g_tile = head_mean ? 0 : 256;
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kRowsPerWave;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kRowsPerWave;
     for (int i0 = 0; i0 < kRowsPerWave && r0 + i0 < n_rows; i0 += U) {
         float d[U][KT];
 #pragma unroll
@@ -1294,11 +1294,11 @@ template <int LPH, int KT, bool FULL>
 __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     EdgeWindow win;
     win.base = -1;
     win.col = 0;
@@ -1306,7 +1306,7 @@ __global__ __launch_bounds__(kBlock) void gat_src_rows_kernel(GatSrcParams p) {
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
         const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
         float xt[KT][4], acc[KT][4], kc[KT], gk[KT];
         gat_src_begin<LPH, KT, FULL>(p, row, end > beg, xt, acc, kc, gk);
@@ -1328,7 +1328,7 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
     const int L = p.sp.L, H = p.sp.H;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kSrcItems;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kSrcItems;
          pos0 < n_items; pos0 += n_waves * kSrcItems) {
         const int n_here = min(kSrcItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -1336,10 +1336,10 @@ __global__ __launch_bounds__(kBlock) void gat_src_items_kernel(GatSrcParams p) {
         int n_edges[kSrcItems], tag[kSrcItems], item[kSrcItems];
 #pragma unroll
         for (int j = 0; j < kSrcItems; j++) {
-            const int beg = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item[j] = __shfl(my_rec.z, j, kWave);
-            tag[j] = __shfl(my_rec.w, j, kWave);
+            const int beg = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
             n_edges[j] = j < n_here ? end - beg : 0;
             if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
         }
@@ -1499,11 +1499,11 @@ __global__ __launch_bounds__(kBlock) void gat_slot_rows_kernel(GatSrcParams p) {
     constexpr int H = kWave / LPH;
     const int lane = lane_id();
     const int rpw = rows_per_wave(p.sp.n_rows);
-    const int r0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * rpw;
+    const int r0 = (blockIdx.x * kWavesPerBlock + wave_id()) * rpw;
     if (r0 >= p.sp.n_rows) return;
     const int n_here = min(rpw, p.sp.n_rows - r0);
     const int my_ptr = p.sp.indptr[r0 + min(lane, n_here)];
-    const int limit = __shfl(my_ptr, n_here, kWave);
+    const int limit = __builtin_amdgcn_readlane(my_ptr, n_here);
     EdgeWindow win;
     win.base = -1;
     win.col = 0;
@@ -1511,7 +1511,7 @@ __global__ __launch_bounds__(kBlock) void gat_slot_rows_kernel(GatSrcParams p) {
     win.vrow = 0;
     for (int i = 0; i < n_here; i++) {
         const int row = r0 + i;
-        const int beg = __shfl(my_ptr, i, kWave), end = __shfl(my_ptr, i + 1, kWave);
+        const int beg = __builtin_amdgcn_readlane(my_ptr, i), end = __builtin_amdgcn_readlane(my_ptr, i + 1);
         if (end - beg >= p.sp.plan.threshold) continue;  // a planned row: the item kernel
         SlotRow<LPH> acc;
         slot_begin<LPH>(acc, p, row, end > beg);
@@ -1532,7 +1532,7 @@ __global__ __launch_bounds__(kBlock) void gat_slot_items_kernel(GatSrcParams p) 
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kSrcItems;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kSrcItems;
          pos0 < n_items; pos0 += n_waves * kSrcItems) {
         const int n_here = min(kSrcItems, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -1540,10 +1540,10 @@ __global__ __launch_bounds__(kBlock) void gat_slot_items_kernel(GatSrcParams p) 
         int n_edges[kSrcItems], tag[kSrcItems], item[kSrcItems];
 #pragma unroll
         for (int j = 0; j < kSrcItems; j++) {
-            const int beg = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            item[j] = __shfl(my_rec.z, j, kWave);
-            tag[j] = __shfl(my_rec.w, j, kWave);
+            const int beg = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            item[j] = __builtin_amdgcn_readlane(my_rec.z, j);
+            tag[j] = __builtin_amdgcn_readlane(my_rec.w, j);
             n_edges[j] = j < n_here ? end - beg : 0;
             if (n_edges[j] > 0) load_window<W_EDGEHEAD>(win[j], p.sp, beg, end);
         }

@@ -16,7 +16,7 @@ __global__ __launch_bounds__(kBlock) void dot_items_kernel(DotParams p) {
     if (p.sp.plan.counters->overflow) return;
     const int n_items = min(p.sp.plan.counters->n_items, p.sp.plan.max_items);
     const int n_waves = gridDim.x * kWavesPerBlock;
-    for (int pos0 = (blockIdx.x * kWavesPerBlock + threadIdx.x / kWave) * kItemsPerWave;
+    for (int pos0 = (blockIdx.x * kWavesPerBlock + wave_id()) * kItemsPerWave;
          pos0 < n_items; pos0 += n_waves * kItemsPerWave) {
         const int n_here = min(kItemsPerWave, n_items - pos0);
         const int4 my_rec = p.sp.plan.records[pos0 + min(lane, n_here - 1)];
@@ -24,9 +24,9 @@ __global__ __launch_bounds__(kBlock) void dot_items_kernel(DotParams p) {
         int e_beg[kItemsPerWave], n_edges[kItemsPerWave], row[kItemsPerWave];
 #pragma unroll
         for (int j = 0; j < kItemsPerWave; j++) {
-            e_beg[j] = __shfl(my_rec.x, j, kWave);
-            const int end = __shfl(my_rec.y, j, kWave);
-            row[j] = __shfl(my_rec.w, j, kWave) & 0x7fffffff;
+            e_beg[j] = __builtin_amdgcn_readlane(my_rec.x, j);
+            const int end = __builtin_amdgcn_readlane(my_rec.y, j);
+            row[j] = __builtin_amdgcn_readlane(my_rec.w, j) & 0x7fffffff;
             n_edges[j] = j < n_here ? end - e_beg[j] : 0;
             if (n_edges[j] > 0) load_window<W_NONE>(win[j], p.sp, e_beg[j], end);
         }

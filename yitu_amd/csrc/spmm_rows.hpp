@@ -292,7 +292,7 @@ __device__ __forceinline__ int row_block(const SpmmParams &p, int block, int n_b
 template <int VEC, int G, int KT, int WMODE, typename TIN>
 __device__ __forceinline__ void spmm_rows_body(const SpmmParams &p, int block, int n_blocks) {
     const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int wave = wave_id();
     const int rpw = rows_per_wave(p.n_rows);
     const int r0 = (row_block(p, block, n_blocks) * kWavesPerBlock + wave) * rpw;
     if (r0 >= p.n_rows) return;
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(SpmmParams p) {
     const int n_items = min(p.plan.counters->n_items, p.plan.max_items);
     const int n_groups = (n_items + IPW - 1) / IPW;
     const int stride = gridDim.x * kWavesPerBlock;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int wave = wave_id();
     for (int grp = blockIdx.x * kWavesPerBlock + wave; grp < n_groups; grp += stride)
         spmm_item_group<VEC, G, KT, WMODE, TIN, IPW>(p, grp * IPW,
                                                 min(IPW, n_items - grp * IPW));
