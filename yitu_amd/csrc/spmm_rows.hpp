@@ -112,7 +112,8 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
 // (window lane first + step + slot) and loads that neighbour's row tile. Slots
 // whose edge lies past the n edges of the range carry weight 0 and load the
 // (valid) tile of the range's last edge.
-template <int VEC, int G, int KT, int WMODE, typename TIN>
+// WHOLE: every slot of the step has an edge (step + SLOTS <= n): no clamp, no mask.
+template <int VEC, int G, int KT, int WMODE, typename TIN, bool WHOLE = false>
 __device__ __forceinline__ void gather_step(float (&v)[KT][VEC], float (&w)[KT],
                                             const SpmmParams &p, const TIN *__restrict__ feat,
                                             const EdgeWindow &win, int first, int step, int n,
@@ -133,8 +134,8 @@ __device__ __forceinline__ void gather_step(float (&v)[KT][VEC], float (&w)[KT],
                                     __builtin_amdgcn_readlane(__builtin_bit_cast(int, win.w), src));
     } else {
         const int k = step + lane_id() / G;
-        valid = k < n;
-        const int src = first + min(k, n - 1);
+        valid = WHOLE || k < n;
+        const int src = WHOLE ? first + k : first + min(k, n - 1);
         c = __shfl(win.col, src, kWave);
         if constexpr (WMODE == W_EDGEHEAD)
             vrow = __shfl(win.vrow, src, kWave);
@@ -187,8 +188,8 @@ __device__ __forceinline__ void accumulate_window(float (&acc)[KT][VEC], const S
         float w[UNROLL][KT];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++)
-            gather_step<VEC, G, KT, WMODE, TIN>(v[u], w[u], p, feat, win, first, s + u * SLOTS, n,
-                                                tl.off, tl.head, tl.live);
+            gather_step<VEC, G, KT, WMODE, TIN, true>(v[u], w[u], p, feat, win, first,
+                                                      s + u * SLOTS, n, tl.off, tl.head, tl.live);
 #pragma unroll
         for (int u = 0; u < UNROLL; u++)
 #pragma unroll
