@@ -1098,9 +1098,12 @@ __global__ __launch_bounds__(kBlock) void gat_row_dot_kernel(float4 *__restrict_
             const int r = min(r0 + i0 + u, n_rows - 1);
 #pragma unroll
             for (int t = 0; t < KT; t++) {
-                float a[4], b[4];
-                RowLoad<4, float>::ld(grad_out + (size_t)r * g_ld + t * g_tile + g_lane, a);
-                RowLoad<4, float>::ld(out + (size_t)r * L + t * 256 + lane * 4, b);
+                // both arrays are read once, front to back: streaming loads
+                typedef float f4 __attribute__((ext_vector_type(4)));
+                const f4 a = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(
+                    grad_out + (size_t)r * g_ld + t * g_tile + g_lane));
+                const f4 b = __builtin_nontemporal_load(
+                    reinterpret_cast<const f4 *>(out + (size_t)r * L + t * 256 + lane * 4));
                 d[u][t] = (a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3]) * g_scale;
             }
         }
