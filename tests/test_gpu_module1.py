@@ -90,7 +90,7 @@ def test_gin_forward_backward(dev):
     assert_close(dw, want_dw, abs_sum=abs_dw)
 
 
-@pytest.mark.parametrize("dim", [8, 128, 100, 264])
+@pytest.mark.parametrize("dim", [8, 64, 128, 100, 256, 264])
 def test_bf16_input_fp32_accumulate(dev, dim):
     indptr, indices = powerlaw_graph(12, 80000, 5)
     n = indptr.numel() - 1

@@ -85,7 +85,7 @@ def test_spmm_power_law_with_hub_rows_and_columns(dev, h, f):
     assert torch.equal(ga, ga2) and torch.equal(gx, gx2)  # no atomics: reproducible
 
 
-@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24), (3, 5), (1, 8)])
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 64), (1, 64), (2, 24), (3, 5), (1, 8)])
 def test_spmm_bf16_features(dev, h, f):
     """bf16 feature rows, fp32 edge values and accumulation: equal to the fp32 op on the
     rounded features (tolerance of the bf16 bar; in fact only the order of the fp32 sums
@@ -104,7 +104,7 @@ def test_spmm_bf16_features(dev, h, f):
     assert_close(got, same, rtol=1e-5, atol=1e-4)
 
 
-@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24)])
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 64), (1, 64), (2, 24)])
 def test_spmm_backward_bf16_rows(dev, h, f):
     """grad_x of the product from bf16 gradient rows (fp32 weights, fp32 sums, fp32 out):
     equal to the fp32 op on the same (exactly representable) rows, hence to the oracle,
@@ -127,7 +127,7 @@ def test_spmm_backward_bf16_rows(dev, h, f):
         graph_ext.spmm_backward(*args, x.to(dev), gy16.to(dev))
 
 
-@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 24), (1, 8)])
+@pytest.mark.parametrize("h,f", [(1, 256), (4, 64), (2, 64), (1, 64), (1, 32), (2, 24), (1, 8)])
 def test_spmm_bf16_rows_in_and_out(dev, h, f):
     """bf16 rows out: exactly the fp32-out result of the same call rounded once to nearest
     even (short rows, single-item rows and reduced rows all take the same store), forward
