@@ -10,8 +10,9 @@
 //     with one coalesced load (an "edge window"), then broadcast lane-to-lane, so
 //     the feature gathers of one round are independent and UNROLL of them are
 //     in flight per wave;
-//   * slots are folded with a fixed butterfly and a row is written once:
-//     no atomics, bitwise reproducible;
+//   * slots are folded in fixed pairs (lane swaps of the vector ALU, every slot keeping
+//     its share of the row) and a row is written once, by all 64 lanes: no atomics,
+//     bitwise reproducible;
 //   * rows below the plan threshold (64 edges): a wave walks 4 consecutive rows
 //     through a sliding window; longer rows: the row plan's items of at most 64
 //     edges in band order, four per wave, whose partial rows a third kernel adds
