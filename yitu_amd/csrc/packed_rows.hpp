@@ -94,6 +94,7 @@ template <typename Chunk, typename Big, typename Empty>
 __device__ __forceinline__ void packed_walk(const SpmmParams &sp, int R, int wave_id, Chunk chunk,
                                             Big big, Empty empty) {
     const int lane = lane_id();
+    wave_id = __builtin_amdgcn_readfirstlane(wave_id);  // what follows from it stays scalar
     const long long first = (long long)wave_id * R;
     if (first >= sp.n_rows) return;
     const int r0 = (int)first;
@@ -109,20 +110,20 @@ __device__ __forceinline__ void packed_walk(const SpmmParams &sp, int R, int wav
     empty(r0, __ballot(is_row && deg == 0));
     int cur = 0;
     while (cur < n_here) {
-        const int base = __shfl(my_ptr, cur, kWave);
+        const int base = __builtin_amdgcn_readlane(my_ptr, cur);
         const bool over = is_row && lane >= cur && next_ptr - base > kWave;
         const unsigned long long m = (__ballot(over) | stop) & (~0ull << cur);
         const int r_end = __ffsll((long long)m) - 1;  // the chunk is rows [cur, r_end)
         if (r_end == cur) {
             if (!((planned_mask >> cur) & 1ull))
-                big(r0 + cur, base, __shfl(my_ptr, cur + 1, kWave));
+                big(r0 + cur, base, __builtin_amdgcn_readlane(my_ptr, cur + 1));
             cur++;
             continue;
         }
         PackedChunk c;
         c.r0 = r0;
         c.base = base;
-        c.n = __shfl(my_ptr, r_end, kWave) - base;
+        c.n = __builtin_amdgcn_readlane(my_ptr, r_end) - base;
         if (c.n > 0) {
             const int e = base + lane;
             int pos = cur;  // the largest row index whose first edge is <= e
