@@ -78,6 +78,32 @@ def test_gat_shapes(dev, h, f):
     assert torch.all(out[0] == 0) and torch.all(out[202] == 0)
 
 
+@pytest.mark.parametrize("h,f", [(4, 64), (2, 16), (4, 8), (1, 128), (8, 32)])
+def test_gat_forward_of_an_infinite_source_row(dev, h, f):
+    """One source's feature row is +inf. Destinations that have it as a neighbour come out
+    +inf (probabilities here are far from underflow), every other row is bitwise untouched:
+    a padded lane that loads the row again must not turn it into 0 x inf = NaN."""
+    n = 600
+    indptr, indices = random_csr(n, n, 0.01, h * 100 + f, hub_rows=(3, 400), hub_degree=200,
+                                 empty_rows=(9,))
+    g = torch.Generator().manual_seed(f)
+    q = torch.randn(n, h, generator=g) * 0.3
+    k = torch.randn(n, h, generator=g) * 0.3
+    x = torch.rand(n, h, f, generator=g) + 0.5
+    src = int(indices[indptr[4] - 1])  # the last neighbour of a hub row
+    x_inf = x.clone()
+    x_inf[src] = float("inf")
+    d = lambda t: t.to(dev)
+    base = graph_ext.gat_forward(d(indptr), d(indices), d(q), d(k), d(x))[0].cpu()
+    got = graph_ext.gat_forward(d(indptr), d(indices), d(q), d(k), d(x_inf))[0].cpu()
+    rows = torch.repeat_interleave(torch.arange(n), (indptr[1:] - indptr[:-1]).long())
+    hit = torch.zeros(n, dtype=torch.bool)
+    hit[rows[indices.long() == src]] = True
+    assert hit.sum() >= 2 and not hit.all()
+    assert torch.all(torch.isposinf(got[hit])), "a neighbour of the infinite row is not +inf"
+    assert torch.equal(got[~hit], base[~hit])
+
+
 @pytest.mark.parametrize("h,f", [(4, 64), (8, 8), (1, 32), (8, 64), (8, 128)])
 def test_gat_power_law_hub_rows(dev, h, f):
     indptr, indices = powerlaw_graph(13, 150000, 11 * h + f)

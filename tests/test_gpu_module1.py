@@ -31,6 +31,34 @@ def test_sag_all_row_widths(dev, dim):
     assert torch.all(got[0] == 0) and torch.all(got[5] == 0)
 
 
+@pytest.mark.parametrize("dim,bf16", [(64, False), (128, False), (128, True), (256, True), (33, False)])
+def test_an_infinite_source_row_stays_infinite(dev, dim, bf16):
+    """One source row holds +inf. Every destination that has it as a neighbour gets +inf (the
+    IEEE sum, what a plain loop over the neighbours gives: never NaN, which 0 x inf from a
+    padded lane would make of it), every other row is untouched. Rows of 1, 2, 3 ... edges
+    and rows of several items are among the neighbours."""
+    n = 600
+    indptr, indices = random_csr(n, n, 0.01, 7, hub_rows=(3, 400), hub_degree=200, empty_rows=(9,))
+    x = torch.rand(n, dim, generator=torch.Generator().manual_seed(dim)) + 0.5
+    if bf16:
+        x = x.to(torch.bfloat16).float()
+    # the last neighbour of the first hub row: where the columns of a row ascend it is the
+    # last edge of most rows that hold it, the edge that padded lanes load again
+    src = int(indices[indptr[4] - 1])
+    x_inf = x.clone()
+    x_inf[src] = float("inf")
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    feed = (lambda t: t.to(torch.bfloat16)) if bf16 else (lambda t: t)
+    base = K.SAG(feed(x).to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB).float().cpu()
+    got = K.SAG(feed(x_inf).to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB).float().cpu()
+    rows = torch.repeat_interleave(torch.arange(n), (indptr[1:] - indptr[:-1]).long())
+    hit = torch.zeros(n, dtype=torch.bool)
+    hit[rows[indices.long() == src]] = True
+    assert hit.sum() >= 2 and not hit.all()
+    assert torch.all(torch.isposinf(got[hit])), "a neighbour of the infinite row is not +inf"
+    assert torch.equal(got[~hit], base[~hit])
+
+
 @pytest.mark.parametrize("hub_degree", [63, 64, 65, 127, 128, 129, 511, 1025, 3000])
 @pytest.mark.parametrize("dim", [64, 128, 36])
 def test_long_rows_take_the_planned_item_path(dev, hub_degree, dim):

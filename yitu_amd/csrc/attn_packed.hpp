@@ -132,9 +132,13 @@ struct PackedGat {
                             if (tl.head[t] == g * HV + h) w[u][t] = ph;
                     }
                 }
-                if (k + u > last) {
+                if (k + u > last) {  // (0 x value is not 0 for every value: drop the row too)
 #pragma unroll
-                    for (int t = 0; t < KT; t++) w[u][t] = 0.0f;
+                    for (int t = 0; t < KT; t++) {
+                        w[u][t] = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) v[u][t][i] = 0.0f;
+                    }
                 }
 #pragma unroll
                 for (int t = 0; t < KT; t++)

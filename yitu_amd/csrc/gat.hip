@@ -112,8 +112,13 @@ __device__ __forceinline__ void gat_apply_window(float (&acc)[KT][VEC], const Ga
                 }
                 if (j0 + u * SLOTS < nb) {  // wave-uniform: steps past the sub-batch load nothing
 #pragma unroll
-                    for (int t = 0; t < KT; t++)
+                    for (int t = 0; t < KT; t++) {
                         RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                        if constexpr (SLOTS > 1) {  // a slot without an edge: 0 x value is not 0
+#pragma unroll
+                            for (int i = 0; i < VEC; i++) v[u][t][i] = valid ? v[u][t][i] : 0.0f;
+                        }
+                    }
                 } else {
 #pragma unroll
                     for (int t = 0; t < KT; t++)
@@ -513,8 +518,14 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
                             }
                             if (j0 + u * SLOTS < nb) {  // wave-uniform
 #pragma unroll
-                                for (int t = 0; t < KT; t++)
+                                for (int t = 0; t < KT; t++) {
                                     RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                                    if constexpr (SLOTS > 1) {  // a slot without an edge
+#pragma unroll
+                                        for (int i = 0; i < VEC; i++)
+                                            v[u][t][i] = valid ? v[u][t][i] : 0.0f;
+                                    }
+                                }
                             } else {
 #pragma unroll
                                 for (int t = 0; t < KT; t++)
