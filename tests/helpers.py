@@ -92,6 +92,24 @@ def random_csr(n_dst, n_src, density, seed, hub_rows=(), hub_degree=0, empty_row
     return indptr, indices
 
 
+def scrambled_csr(indptr, indices, seed, repeat=0.15):
+    """The same rows with their edges in random order and a share of them repeated (a
+    multigraph): what the reference's loops accept (YiTu_GNN_kernel.cu:186-199 walks
+    whatever the row holds), though most builders emit sorted, unique columns."""
+    rng = np.random.default_rng(seed)
+    ip = indptr.numpy().astype(np.int64)
+    ix = indices.numpy()
+    rows = np.repeat(np.arange(len(ip) - 1), np.diff(ip))
+    extra = rng.random(len(ix)) < repeat
+    rows = np.concatenate([rows, rows[extra]])
+    cols = np.concatenate([ix, ix[extra]])
+    order = np.lexsort((rng.random(len(rows)), rows))  # rows together, edges shuffled inside
+    rows, cols = rows[order], cols[order]
+    new_ip = np.zeros(len(ip), dtype=np.int64)
+    np.cumsum(np.bincount(rows, minlength=len(ip) - 1), out=new_ip[1:])
+    return torch.from_numpy(new_ip.astype(np.int32)), torch.from_numpy(cols.astype(np.int32))
+
+
 def powerlaw_graph(scale, m, seed):
     src, dst = graphgen.rmat(scale, m, seed, self_loops=True)
     return graphgen.csr_by_destination(src, dst, 1 << scale)

@@ -5,8 +5,8 @@ import pytest
 import torch
 
 import oracle
-from helpers import (assert_close, powerlaw_graph, random_csr, softmax_backward_abs_sums,
-                     spmm_abs_sums)
+from helpers import (assert_close, powerlaw_graph, random_csr, scrambled_csr,
+                     softmax_backward_abs_sums, spmm_abs_sums)
 from yitu_amd import graph_ext
 from yitu_amd.xgnn_h import block as xblock
 from yitu_amd.xgnn_h import sparse
@@ -76,6 +76,18 @@ def test_gat_shapes(dev, h, f):
                                  empty_rows=(0, 202))
     out = _run(dev, indptr, indices, n_dst, n_src, h, f, seed=h + f)
     assert torch.all(out[0] == 0) and torch.all(out[202] == 0)
+
+
+@pytest.mark.parametrize("h,f", [(4, 64), (2, 16), (8, 32)])
+def test_gat_rows_with_unsorted_and_repeated_edges(dev, h, f):
+    """The fused attention, forward and every gradient, on a multigraph whose rows hold
+    their edges in random order (a repeated edge takes part in the softmax twice, as in
+    the reference's loops, sddmm_cuda.cu:11-31)."""
+    n = 1 << 12
+    indptr, indices = random_csr(n, n, 0.002, 11 * h + f, hub_rows=(5, 2000, 4095),
+                                 hub_degree=1500, empty_rows=(2,))
+    indptr, indices = scrambled_csr(indptr, indices, h + f)
+    _run(dev, indptr, indices, n, n, h, f, seed=h * f)
 
 
 @pytest.mark.parametrize("h,f", [(4, 64), (2, 16), (4, 8), (1, 128), (8, 32)])

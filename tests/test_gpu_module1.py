@@ -5,7 +5,8 @@ import pytest
 import torch
 
 import oracle
-from helpers import ATOL_BF16, RTOL_BF16, assert_close, powerlaw_graph, random_csr
+from helpers import (ATOL_BF16, RTOL_BF16, assert_close, powerlaw_graph, random_csr,
+                     scrambled_csr)
 from yitu_amd import YiTu_GNN_kernel as K
 from yitu_amd.data import graphgen
 
@@ -57,6 +58,26 @@ def test_an_infinite_source_row_stays_infinite(dev, dim, bf16):
     assert hit.sum() >= 2 and not hit.all()
     assert torch.all(torch.isposinf(got[hit])), "a neighbour of the infinite row is not +inf"
     assert torch.equal(got[~hit], base[~hit])
+
+
+@pytest.mark.parametrize("dim", [64, 128, 100])
+def test_rows_with_unsorted_and_repeated_edges(dev, dim):
+    """Edges of a row in any order, some of them twice: the sums are those of the loops
+    over whatever the row holds, for short rows and for rows that the plan cuts at band
+    crossings (which are then out of order)."""
+    n = 1 << 13
+    indptr, indices = random_csr(n, n, 0.001, dim, hub_rows=(5, 4000, 8191), hub_degree=3000,
+                                 empty_rows=(2,))
+    indptr, indices = scrambled_csr(indptr, indices, dim)
+    g = torch.Generator().manual_seed(dim)
+    x = torch.randn(n, dim, generator=g)
+    rp, ci, deg, pp, p2n = _graph_args(indptr, indices, dev)
+    got = K.SAG(x.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)
+    assert_close(got, oracle.sag(x.numpy(), indptr, indices), what="SAG dim=%d" % dim)
+    w = torch.eye(dim)
+    got = K.forward(x.to(dev), w.to(dev), rp, ci, deg, pp, p2n, PS, DW, WPB)[0]
+    want = oracle.gcn_forward(x.numpy(), w.numpy(), indptr, indices, deg.cpu().numpy())
+    assert_close(got, want, what="GCN dim=%d" % dim)
 
 
 @pytest.mark.parametrize("hub_degree", [63, 64, 65, 127, 128, 129, 511, 1025, 3000])
