@@ -113,11 +113,17 @@ struct PackedGat {
             float v[U][KT][4], w[U][KT];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int ek = min(k + u, last);  // past the end: the last edge again, weight 0
+                const bool past = k + u > last;  // wave-uniform: no edge, no load
+                const int ek = min(k + u, last);
                 const int c = __builtin_amdgcn_readlane(col, ek);
 #pragma unroll
                 for (int t = 0; t < KT; t++) {
-                    RowLoad<4, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                    if (!past) {
+                        RowLoad<4, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) v[u][t][i] = 0.0f;
+                    }
                     w[u][t] = 0.0f;
                 }
 #pragma unroll
@@ -132,13 +138,9 @@ struct PackedGat {
                             if (tl.head[t] == g * HV + h) w[u][t] = ph;
                     }
                 }
-                if (k + u > last) {  // (0 x value is not 0 for every value: drop the row too)
+                if (past) {
 #pragma unroll
-                    for (int t = 0; t < KT; t++) {
-                        w[u][t] = 0.0f;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) v[u][t][i] = 0.0f;
-                    }
+                    for (int t = 0; t < KT; t++) w[u][t] = 0.0f;
                 }
 #pragma unroll
                 for (int t = 0; t < KT; t++)

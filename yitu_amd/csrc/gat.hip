@@ -112,13 +112,8 @@ __device__ __forceinline__ void gat_apply_window(float (&acc)[KT][VEC], const Ga
                 }
                 if (j0 + u * SLOTS < nb) {  // wave-uniform: steps past the sub-batch load nothing
 #pragma unroll
-                    for (int t = 0; t < KT; t++) {
+                    for (int t = 0; t < KT; t++)
                         RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
-                        if constexpr (SLOTS > 1) {  // a slot without an edge: 0 x value is not 0
-#pragma unroll
-                            for (int i = 0; i < VEC; i++) v[u][t][i] = valid ? v[u][t][i] : 0.0f;
-                        }
-                    }
                 } else {
 #pragma unroll
                     for (int t = 0; t < KT; t++)
@@ -127,11 +122,16 @@ __device__ __forceinline__ void gat_apply_window(float (&acc)[KT][VEC], const Ga
                 }
             }
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++)
+            for (int u = 0; u < UNROLL; u++) {
+                // a slot without an edge has loaded edge 0's row: 0 x value is not 0 for
+                // every value, so the row is dropped (here, after the loads are out)
+                const bool valid = SLOTS == 1 || j0 + u * SLOTS + slot < nb;
 #pragma unroll
                 for (int t = 0; t < KT; t++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
+                    for (int i = 0; i < VEC; i++)
+                        acc[t][i] += w[u][t] * (valid ? v[u][t][i] : 0.0f);
+            }
         }
     }
 }
@@ -518,14 +518,8 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
                             }
                             if (j0 + u * SLOTS < nb) {  // wave-uniform
 #pragma unroll
-                                for (int t = 0; t < KT; t++) {
+                                for (int t = 0; t < KT; t++)
                                     RowLoad<VEC, float>::ld(feat + (size_t)c * L + tl.off[t], v[u][t]);
-                                    if constexpr (SLOTS > 1) {  // a slot without an edge
-#pragma unroll
-                                        for (int i = 0; i < VEC; i++)
-                                            v[u][t][i] = valid ? v[u][t][i] : 0.0f;
-                                    }
-                                }
                             } else {
 #pragma unroll
                                 for (int t = 0; t < KT; t++)
@@ -534,11 +528,14 @@ __global__ __launch_bounds__(kBlock) void gat_item_local_hp_kernel(GatParams p) 
                             }
                         }
 #pragma unroll
-                        for (int u = 0; u < UNROLL; u++)
+                        for (int u = 0; u < UNROLL; u++) {
+                            const bool valid = SLOTS == 1 || j0 + u * SLOTS + slot < nb;  // as above
 #pragma unroll
                             for (int t = 0; t < KT; t++)
 #pragma unroll
-                                for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
+                                for (int i = 0; i < VEC; i++)
+                                    acc[t][i] += w[u][t] * (valid ? v[u][t][i] : 0.0f);
+                        }
                     }
                 }
                 fold_slots<VEC, G, KT>(acc);

@@ -111,8 +111,8 @@ __device__ __forceinline__ void load_window(EdgeWindow &win, const SpmmParams &p
 
 // One step of the edge loop: every slot of the wave picks its edge
 // (window lane first + step + slot) and loads that neighbour's row tile. Slots
-// whose edge lies past the n edges of the range carry weight 0 and value 0 (they load
-// the valid tile of the range's last edge and drop it).
+// whose edge lies past the n edges of the range carry weight 0 and load the (valid)
+// tile of the range's last edge, which the caller must drop (0 x inf is not 0).
 // WHOLE: every slot of the step has an edge (step + SLOTS <= n): no clamp, no mask.
 template <int VEC, int G, int KT, int WMODE, typename TIN, bool WHOLE = false>
 __device__ __forceinline__ void gather_step(float (&v)[KT][VEC], float (&w)[KT],
@@ -150,12 +150,6 @@ __device__ __forceinline__ void gather_step(float (&v)[KT][VEC], float (&w)[KT],
         else
             w[t] = (valid && live[t]) ? ws : 0.0f;
         RowLoad<VEC, TIN>::ld(feat + (size_t)c * p.L + off[t], v[t]);
-        if constexpr (!WHOLE && SLOTS > 1) {
-            // a slot without an edge has loaded the range's last row again: its values
-            // must not reach the sum even as 0 x value (0 x inf is not 0)
-#pragma unroll
-            for (int i = 0; i < VEC; i++) v[t][i] = valid ? v[t][i] : 0.0f;
-        }
     }
 }
 
@@ -216,11 +210,17 @@ __device__ __forceinline__ void accumulate_window(float (&acc)[KT][VEC], const S
                                                     n, tl.off, tl.head, tl.live);
 #pragma unroll
         for (int u = 0; u < UNROLL; u++)
-            if (s + u * SLOTS < n)
+            if (s + u * SLOTS < n) {
+                // a slot without an edge has loaded the range's last row again: its values
+                // must not reach the sum even as 0 x value. (Selected here, after all the
+                // group's loads have been issued, not where the row is loaded.)
+                const bool valid = SLOTS == 1 || s + u * SLOTS + lane_id() / G < n;
 #pragma unroll
                 for (int t = 0; t < KT; t++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) acc[t][i] += w[u][t] * v[u][t][i];
+                    for (int i = 0; i < VEC; i++)
+                        acc[t][i] += w[u][t] * (valid ? v[u][t][i] : 0.0f);
+            }
     }
 }
 
